@@ -1,0 +1,61 @@
+"""Build the CPU oracle (test infrastructure, not the product).
+
+  python oracle/build.py          builds oracle/liboracle.so from oracle/oracle.c
+  python oracle/build.py --ref    additionally compiles the reference's own CPU
+                                  sources (where they lie under /root/reference)
+                                  into oracle/_ref/, when that tree is present.
+"""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+REFERENCE_BACKEND = "/root/reference/torchsparse/backend"
+REF_MODULE = "tsref_cpu"
+
+
+def build_oracle(verbose: bool = False) -> str:
+    out = os.path.join(HERE, "liboracle.so")
+    cmd = ["gcc", "-O3", "-march=native", "-fopenmp", "-fPIC", "-shared", "-std=c11",
+           "-fvisibility=hidden", os.path.join(HERE, "oracle.c"), "-o", out, "-lm"]
+    if verbose:
+        print(" ".join(cmd))
+    subprocess.check_call(cmd)
+    return out
+
+
+def build_ref(verbose: bool = False):
+    """Compile convolution_gather_scatter_cpu.cpp + hash_cpu.cpp of the reference
+    behind oracle/ref_bind.cpp.  Returns the path of the built module or None
+    when the reference tree is absent."""
+    if not os.path.isdir(REFERENCE_BACKEND):
+        return None
+    from torch.utils import cpp_extension
+
+    out_dir = os.path.join(HERE, "_ref")
+    os.makedirs(out_dir, exist_ok=True)
+    cpp_extension.load(
+        name=REF_MODULE,
+        sources=[
+            os.path.join(HERE, "ref_bind.cpp"),
+            os.path.join(REFERENCE_BACKEND, "convolution", "convolution_gather_scatter_cpu.cpp"),
+            os.path.join(REFERENCE_BACKEND, "hash", "hash_cpu.cpp"),
+        ],
+        extra_include_paths=[REFERENCE_BACKEND],
+        extra_cflags=["-O3", "-fopenmp"],
+        extra_ldflags=["-lgomp"],
+        build_directory=out_dir,
+        verbose=verbose,
+        is_python_module=False,
+    )
+    # keep only the shared object; the intermediate files are not needed
+    for f in os.listdir(out_dir):
+        if not f.endswith(".so"):
+            os.remove(os.path.join(out_dir, f))
+    return os.path.join(out_dir, REF_MODULE + ".so")
+
+
+if __name__ == "__main__":
+    print(build_oracle(verbose=True))
+    if "--ref" in sys.argv:
+        print(build_ref(verbose=True))

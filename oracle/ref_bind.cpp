@@ -1,0 +1,13 @@
+// Python binding for the reference's own CPU sources (compiled where they lie
+// under /root/reference; nothing is copied).  Test infrastructure only: used
+// to validate oracle.c and, optionally, as the cpu_baseline of the benchmark.
+#include <torch/extension.h>
+
+#include "convolution/convolution_gather_scatter_cpu.h"
+#include "hash/hash_cpu.h"
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.def("conv_forward_gather_scatter_cpu", &conv_forward_gather_scatter_cpu);
+  m.def("hash_cpu", &hash_cpu);
+  m.def("kernel_hash_cpu", &kernel_hash_cpu);
+}
