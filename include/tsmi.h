@@ -1,0 +1,270 @@
+/*
+ * tsmi.h — C ABI of libtsmi.so: the MI355X (gfx950) forward sparse-convolution
+ * hot path (kernel-map construction, implicit-GEMM / gather-scatter /
+ * fetch-on-demand convolution).
+ *
+ * Every entry point is `extern "C"`, takes plain device pointers and sizes,
+ * launches on the HIP stream it is given and returns a status code.  The
+ * caller owns (and allocates) every buffer, including scratch; nothing here
+ * allocates device memory or synchronises the stream unless stated.  After a
+ * non-zero return, tsmi_last_error() describes the failure (thread local).
+ *
+ * Each declaration cites the interface of the reference (torchsparse v2.1.0,
+ * pybind module `torchsparse.backend`, backend/pybind_cuda.cu:29-83) it
+ * replaces.  Paths are relative to the reference's torchsparse/backend/.
+ *
+ * Shared conventions
+ *   coords       int32 [N,4] rows (b, x, y, z); 0 <= x,y,z < 2^18, 0 <= b < 512
+ *   out_in_map   int32 [N_pad, K_vol], -1 = no neighbour, N_pad = ceil128(N_out)
+ *   kernel index odd K_vol: x is the fastest digit; even K_vol: z is the fastest
+ *   hash table   two caller-owned arrays keys int64[cap], vals int32[cap];
+ *                cap must be a multiple of 8; an empty slot has key 0; a stored
+ *                key is (packed coordinate or user key) + 1, a stored value is
+ *                row index + 1 (the reference's biasing, hashmap_cuda.cuh:13,132)
+ *   dtype        TSMI_F32 / TSMI_F16 / TSMI_BF16; 16-bit types accumulate in fp32
+ */
+#ifndef TSMI_H_
+#define TSMI_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+#pragma GCC visibility push(default)
+
+typedef void *tsmi_stream_t; /* a hipStream_t */
+
+enum { TSMI_OK = 0, TSMI_ERR_INVALID_ARGUMENT = 1, TSMI_ERR_RUNTIME = 2, TSMI_ERR_HIP = 3 };
+enum { TSMI_F32 = 0, TSMI_F16 = 1, TSMI_BF16 = 2 };
+
+/* ----------------------------------------------------------------- general */
+
+/* Message of the last failure on the calling thread ("" when none).
+ * Replaces the C++ exceptions pybind turns into Python errors
+ * (std::invalid_argument -> ValueError, std::runtime_error -> RuntimeError). */
+const char *tsmi_last_error(void);
+
+/* ABI version of the library (bumped on any signature change). */
+int tsmi_version(void);
+
+/* ------------------------------------------------------------- hash table */
+
+/* Empty the table (keys and vals := 0).
+ * Replaces torch.zeros for hashmap_keys / hashmap_vals
+ * (nn/functional/conv/kmap/func/hashmap_on_the_fly.py:59-67). */
+int tsmi_hashtable_clear(tsmi_stream_t s, int64_t *keys, int32_t *vals, int64_t cap);
+
+/* Insert coords[i] -> i+1 for i < n.
+ * Replaces subm_hashmap_kmap_stage1 (others/sparsemapping_cuda.cu:129-140) and
+ * GPUHashTable::insert_coords (hashmap/hashmap_cuda.cuh:149-169).
+ * `status` (device int32[1], pre-zeroed by the caller or NULL) is set to 1 when a
+ * key could not be placed because the table is full. */
+int tsmi_hashtable_insert_coords(tsmi_stream_t s, int64_t *keys, int32_t *vals, int64_t cap,
+                                 const int32_t *coords, int64_t n, int32_t *status);
+
+/* Insert user_keys[i] -> i+1.  Replaces GPUHashTable::insert_vals
+ * (hashmap/hashmap_cuda.cuh:124-146; wrapper :95-96). */
+int tsmi_hashtable_insert_keys(tsmi_stream_t s, int64_t *keys, int32_t *vals, int64_t cap,
+                               const int64_t *user_keys, int64_t n, int32_t *status);
+
+/* out[i] = stored value of user_keys[i] (row index + 1) or 0 when absent.
+ * Replaces GPUHashTable::lookup_vals (hashmap/hashmap_cuda.cuh:173-196). */
+int tsmi_hashtable_lookup_keys(tsmi_stream_t s, const int64_t *keys, const int32_t *vals,
+                               int64_t cap, const int64_t *user_keys, int64_t n, int32_t *out);
+
+/* ------------------------------------------------------------- kernel maps */
+
+/* out_in_map[o,k] = i  iff  in_coords[i] == out_coords[o]*stride - pad + digit(k)
+ * (same batch), for o < n_out; rows n_out..n_out_pad-1 are written as -1, so the
+ * map needs no prior fill.  (keys, vals, cap) index the INPUT coordinates.
+ * One entry point covers
+ *   build_kernel_map_subm_hashmap stage 2 (others/sparsemapping_cuda.cu:144-231,
+ *     host :303-345): out_coords = in_coords, stride 1, pad = (ks-1)/2 for an odd
+ *     kernel volume and 0 for an even one;
+ *   build_kernel_map_downsample_hashmap stage 3 (:110-126, host :429-507):
+ *     pad = the convolution's padding;
+ *   GPUHashTable::lookup_coords (hashmap/hashmap_cuda.cuh:199-253): pad = (ks-1)/2. */
+int tsmi_kmap_query(tsmi_stream_t s, const int64_t *keys, const int32_t *vals, int64_t cap,
+                    const int32_t *out_coords, int64_t n_out, int64_t n_out_pad,
+                    const int32_t ks[3], const int32_t stride[3], const int32_t pad[3],
+                    int32_t *out_in_map);
+
+/* Per-column maximum of coords -> out_max int32[4] (device).  n may be 0 (result 0).
+ * Replaces coords.max(0).values (hashmap_on_the_fly.py:33). */
+int tsmi_coords_max(tsmi_stream_t s, const int32_t *coords, int64_t n, int32_t *out_max);
+
+/* Candidate output coordinates of a strided convolution, de-duplicated through
+ * the (empty) OUTPUT table (keys, vals, cap): every distinct output is appended
+ * once, packed as (b<<54 | x<<36 | y<<18 | z), to uniq_keys and counted in
+ * counters[0]; counters[1] is set to 1 if the table overflowed.  `counters`
+ * (device int32[2]) must be zero on entry.
+ *   mode 0: o = (in + pad + digit - (ks-1)) / stride where divisible and
+ *           0 <= o <= out_max per axis — downsample_grid_kmap_stage1_specialized_fast
+ *           (others/sparsemapping_cuda.cu:60-107) and get_output_coords_kernel
+ *           (others/downsample_cuda.cu:62-141).
+ *   mode 1: o = floor(in / stride), unbounded — spdownsample for stride in {1, ks}
+ *           or "minkowski" mode (nn/functional/conv/kmap/downsample.py:30-37).
+ * The bound is out_max_host[3] when in_max_dev is NULL, otherwise it is derived on
+ * the device as (in_max_dev[1+a] + 2*pad - (ks-1)) / stride
+ * (hashmap_on_the_fly.py:33-37). */
+int tsmi_downsample_candidates(tsmi_stream_t s, const int32_t *in_coords, int64_t n_in,
+                               const int32_t ks[3], const int32_t stride[3],
+                               const int32_t pad[3], const int32_t out_max_host[3],
+                               const int32_t *in_max_dev, int mode, int64_t *keys,
+                               int64_t cap, int64_t *uniq_keys, int64_t uniq_cap,
+                               int32_t *counters);
+
+/* Bytes of scratch tsmi_sort_keys / tsmi_argsort_desc need for n items. */
+int64_t tsmi_sort_temp_bytes(int64_t n);
+
+/* Ascending sort of n int64 keys (bits [0,end_bit) significant).
+ * Replaces torch::_unique's sort (others/sparsemapping_cuda.cu:478). */
+int tsmi_sort_keys(tsmi_stream_t s, const int64_t *keys_in, int64_t *keys_out, int64_t n,
+                   int end_bit, void *temp, int64_t temp_bytes);
+
+/* Unpack sorted unique keys into out_coords int32[n_out,4] and store row+1 as the
+ * value of each key in the OUTPUT table.  Replaces
+ * inverse_transform_coords_and_insert_kernel (others/sparsemapping_cuda.cu:44-57). */
+int tsmi_downsample_finalize(tsmi_stream_t s, const int64_t *sorted_keys, int64_t n_out,
+                             const int64_t *keys, int32_t *vals, int64_t cap,
+                             int32_t *out_coords);
+
+/* map_t[in,k] = out for every map[out,k] = in >= 0, out < n_rows; map_t
+ * [n_rows_t, K_vol] is filled with -1 first.  Replaces
+ * convert_transposed_out_in_map (others/query_cuda.cu:9-15,50-54) plus the
+ * torch.full of nn/functional/conv/hash/query.py:47-55. */
+int tsmi_transpose_map(tsmi_stream_t s, const int32_t *map, int64_t n_rows, int kvol,
+                       int32_t *map_t, int64_t n_rows_t);
+
+/* bitmask[s,r] = sum_i (map[r, s*L+i] >= 0) << i for r < valid_n, -1 for padding
+ * rows; L = ceil(K_vol/split) (must be <= 32).  Replaces
+ * derive_bitmask_from_out_in_map (others/query_cuda.cu:17-31,59-65). */
+int tsmi_derive_bitmask(tsmi_stream_t s, const int32_t *map, int64_t n_pad, int kvol,
+                        int split, int64_t valid_n, int32_t *bitmask);
+
+/* Descending (signed) sort of each of `rows` rows of keys_in int32[rows,n]:
+ * keys_out = sorted values, idx_out = source positions.  Ties keep no particular
+ * order.  Replaces torch.sort(bitmask, descending=True) (hashmap_on_the_fly.py:96). */
+int tsmi_argsort_desc(tsmi_stream_t s, const int32_t *keys_in, int32_t *keys_out,
+                      int32_t *idx_out, int rows, int64_t n, void *temp, int64_t temp_bytes);
+
+/* out[r,c] = map[reorder_loc[c / L, r], c].  Replaces reorder_out_in_map_cuda
+ * (others/reorder_map_cuda.cu:8-48). */
+int tsmi_reorder_map(tsmi_stream_t s, const int32_t *map, const int32_t *reorder_loc,
+                     int64_t n_pad, int kvol, int split, int32_t *out);
+
+/* reduced[s,t] = OR of sorted_mask[s, t*tile .. (t+1)*tile-1]; tile % 4 == 0.
+ * Replaces reduce_bitmask_cuda (others/reduce_bitmask_cuda.cu:13-84). */
+int tsmi_reduce_bitmask(tsmi_stream_t s, const int32_t *sorted_mask, int split,
+                        int64_t n_pad, int tile, int32_t *reduced);
+
+/* Pair lists, phase 1: per-offset counts.  nbsizes int32[K_vol] := number of
+ * rows < n_rows with map[row,k] != -1; block_counts int32[K_vol * nblk] is
+ * scratch for phase 2, nblk = ceil(n_rows / 256).  Replaces torch.sum(results
+ * != -1, dim=1) (hashmap_on_the_fly.py:139,186). */
+int tsmi_pair_lists_count(tsmi_stream_t s, const int32_t *map, int64_t n_rows, int kvol,
+                          int32_t *block_counts, int32_t *nbsizes);
+
+/* Pair lists, phase 2 (after phase 1 on the same stream).  Pairs are ordered by
+ * (k, out).  Any of the outputs may be NULL:
+ *   nbmaps_inter int32[nnz,2] rows (in,out)     — GatherScatter layout (:141-143)
+ *   nbmaps_planar int32[2,nnz] all in, then out — FetchOnDemand layout (:187-200)
+ *   input_mask int32[K_vol*n_in], output_mask int32[K_vol*n_out]: position of the
+ *     pair inside offset k's list (pre-filled with -1 here); the centre offset of
+ *     an odd-volume map with n_in == n_out is skipped — build_mask_from_kmap
+ *     (others/sparsemapping_cuda.cu:235-256,510-548).
+ * nnz is the sum of nbsizes (the caller read it back to size the arrays). */
+int tsmi_pair_lists_fill(tsmi_stream_t s, const int32_t *map, int64_t n_rows, int kvol,
+                         int32_t *block_counts, int64_t nnz, int32_t *nbmaps_inter,
+                         int32_t *nbmaps_planar, int64_t n_in, int64_t n_out,
+                         int32_t *input_mask, int32_t *output_mask);
+
+/* input_mask / output_mask (see tsmi_pair_lists_fill) from an existing interleaved
+ * pair list and nbaddrs = exclusive scan of its per-offset sizes.  Replaces
+ * build_mask_from_kmap (others/sparsemapping_cuda.cu:235-256,510-548). */
+int tsmi_build_masks(tsmi_stream_t s, const int32_t *nbmaps_inter, int64_t nnz,
+                     const int32_t *nbaddrs, int kvol, int64_t n_in, int64_t n_out,
+                     int32_t *input_mask, int32_t *output_mask);
+
+/* nbaddrs / qnbaddrs int32[K_vol+1]: exclusive scans of nbsizes and of nbsizes
+ * rounded up to q.  Replaces exclusive_scan_quantified_wrapper
+ * (others/exclusive_scan_cuda.cu:7-45). */
+int tsmi_exclusive_scan_quantified(tsmi_stream_t s, int kvol, const int32_t *nbsizes, int q,
+                                   int32_t *nbaddrs, int32_t *qnbaddrs);
+
+/* ------------------------------------------------------------ convolutions */
+
+/* Elements of the packed-weight buffer for a [K_vol, Cin, Cout] kernel. */
+int64_t tsmi_packed_weight_elems(int kvol, int cin, int cout);
+
+/* Re-lay a [K_vol, Cin, Cout] kernel as [K_vol, Cout_pad, Cin_pad] (reduction
+ * axis contiguous, zero padded to multiples of 16 / 32) for the MFMA kernels.
+ * No counterpart in the reference (its kernels read [K_vol,Cin,Cout] directly). */
+int tsmi_pack_weights(tsmi_stream_t s, const void *w, void *w_packed, int kvol, int cin,
+                      int cout, int dtype);
+
+/* Y[i,:] = sum_k [m = map[i,k] >= 0] X[m,:] W[k] (+ bias) for i < n_out; every
+ * output row is written.  `map` has at least n_out rows.
+ * Replaces conv_forward_implicit_gemm_cuda
+ * (convolution/convolution_forward_implicit_gemm_cuda.cu:1527-1986). */
+int tsmi_conv_implicit_gemm(tsmi_stream_t s, const void *x, const void *w_packed,
+                            const int32_t *map, int64_t n_map_rows, int64_t n_out, int kvol,
+                            int cin, int cout, int dtype, const void *bias, void *y);
+
+/* Same sum over a row-sorted map: tile row r of split s reads
+ * reorder_map[r, s*L..] and adds into output row reorder_loc[s, r].
+ * `partial` (float [split, n_out, cout], only for split > 1) receives the
+ * per-split sums, which are then added into y.  reduced_mask may be NULL (the
+ * kernel derives tile-level skipping from the map itself).  Replaces
+ * conv_forward_implicit_gemm_sorted_cuda
+ * (convolution/convolution_forward_implicit_gemm_sorted_cuda.cu:1755-2230). */
+int tsmi_conv_implicit_gemm_sorted(tsmi_stream_t s, const void *x, const void *w_packed,
+                                   const int32_t *reorder_map, const int32_t *reduced_mask,
+                                   const int32_t *reorder_loc, int64_t n_pad, int64_t n_out,
+                                   int kvol, int split, int cin, int cout, int dtype,
+                                   const void *bias, float *partial, void *y);
+
+/* Fetch-on-demand: one launch over 128-padded pair lists gathers X rows, multiplies
+ * by W[k] and writes partial[qnbaddrs[k] + p, :] (fp32 for TSMI_F32, else the I/O
+ * type); a second launch sums the partials of each output row through output_mask
+ * (atomic free).  `transpose` swaps the roles of the two pair columns; row_mask is
+ * the output_mask (input_mask when transposed).  center_k >= 0 names an offset
+ * whose pair list is the identity (p-th pair = (p, p)) and which the masks skip:
+ * the centre of an odd-volume submanifold map; -1 otherwise.  `partial` holds
+ * nnz x cout elements of the I/O type.
+ * Replaces conv_forward_fetch_on_demand_cuda
+ * (convolution/convolution_forward_fetch_on_demand_cuda.cu:1981-2119). */
+int tsmi_conv_fetch_on_demand(tsmi_stream_t s, const void *x, const void *w_packed,
+                              const int32_t *nbmaps_planar, int64_t nnz,
+                              const int32_t *nbaddrs, const int32_t *qnbaddrs, int64_t qnnz,
+                              const int32_t *row_mask, int64_t n_out, int kvol, int cin,
+                              int cout, int dtype, int transpose, int center_k,
+                              const void *bias, void *partial, void *y);
+
+/* Gather-GEMM-scatter, step 1: buffer[nbaddrs[k] + p, :] = X[in(k,p), :].
+ * Replaces gather_all_kernel_pad_sep_with_mask / gather_kernel
+ * (convolution/convolution_gather_scatter_cuda.cu:17-40,70-112). */
+int tsmi_gs_gather(tsmi_stream_t s, const void *x, const int32_t *nbmaps_inter, int64_t nnz,
+                   int cin, int dtype, int transpose, void *buffer);
+
+/* Gather-GEMM-scatter, step 2: out_buffer[p,:] = buffer[p,:] W[k(p)] for every pair,
+ * one launch for all offsets (qnbaddrs / qnnz: the 128-padded scan that maps a
+ * workgroup to its offset).  Replaces the torch::mm_out / bmm_out groups
+ * (convolution/convolution_gather_scatter_cuda.cu:597-673). */
+int tsmi_gs_gemm(tsmi_stream_t s, const void *buffer, const void *w_packed,
+                 const int32_t *nbaddrs, const int32_t *qnbaddrs, int64_t nnz, int64_t qnnz,
+                 int kvol, int cin, int cout, int dtype, void *out_buffer);
+
+/* Gather-GEMM-scatter, step 3: Y[o,:] = sum_k out_buffer[nbaddrs[k] + mask[k,o], :]
+ * (+ bias), atomic free.  Replaces scatter_all_kernel_pad_sep_with_mask_{half,float}
+ * (convolution/convolution_gather_scatter_cuda.cu:150-250). */
+int tsmi_gs_scatter(tsmi_stream_t s, const void *out_buffer, const int32_t *nbaddrs,
+                    const int32_t *row_mask, int64_t n_out, int kvol, int cout, int dtype,
+                    int center_k, const void *bias, void *y);
+
+#pragma GCC visibility pop
+#ifdef __cplusplus
+}
+#endif
+#endif /* TSMI_H_ */

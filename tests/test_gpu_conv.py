@@ -1,0 +1,232 @@
+"""GPU parity of the convolution dataflows against the CPU oracle.
+
+Tolerances (relative to the RMS of the expected output): 1e-4 for fp32, 1e-2 for
+fp16 / bf16 with fp32 accumulation — the bar the north star sets.  The oracle is fed
+the inputs already rounded to the I/O type, so only accumulation order and the final
+rounding differ."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import random_coords, rel_rms
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 1e-4, torch.float16: 1e-2, torch.bfloat16: 3e-2}
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+
+
+@pytest.fixture(scope="module")
+def mods():
+    import torchsparse_amd as ts
+    from torchsparse_amd import backend
+    from torchsparse_amd import nn as spnn
+    from torchsparse_amd.nn import functional as F
+    return ts, backend, spnn, F
+
+
+def dev(a, dtype=torch.int32):
+    return torch.from_numpy(np.ascontiguousarray(a)).to("cuda", dtype)
+
+
+def _case(rng, n, cin, cout, kvol, dtype, wscale=None):
+    x = torch.from_numpy(rng.standard_normal((n, cin)).astype(np.float32)).to("cuda", dtype)
+    bound = wscale or 1.0 / np.sqrt(cin * kvol)
+    w = torch.from_numpy(rng.uniform(-bound, bound, (kvol, cin, cout)).astype(np.float32)).to("cuda", dtype)
+    return x, w
+
+
+def _f32(t):
+    return t.float().cpu().numpy()
+
+
+CHANNELS = [(32, 32), (64, 64), (128, 128), (4, 32), (5, 16), (16, 16), (96, 96), (128, 96),
+            (24, 40), (32, 19), (7, 3), (192, 256)]
+
+
+@pytest.mark.parametrize("cin,cout", CHANNELS)
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32, torch.bfloat16])
+def test_implicit_gemm_matches_oracle(mods, cin, cout, dtype):
+    _, backend, _, F = mods
+    rng = np.random.default_rng(cin * 1000 + cout)
+    coords = random_coords(rng, 1500, (20, 20, 12))
+    kmap = F.build_kernel_map(dev(coords), len(coords), 3, 1, 1, mode="hashmap_on_the_fly")
+    x, w = _case(rng, len(coords), cin, cout, 27, dtype)
+    y = backend.conv_forward_implicit_gemm_cuda(x, w, kmap["out_in_map"], len(coords), cout)
+    want = oracle.conv_implicit_gemm(_f32(x), _f32(w), kmap["out_in_map"].cpu().numpy(), len(coords))
+    assert y.dtype == dtype and y.shape == (len(coords), cout)
+    assert rel_rms(_f32(y), want) < TOL[dtype]
+
+
+@pytest.mark.parametrize("n", [1, 15, 16, 17, 63, 64, 65, 129, 255, 257, 700])
+def test_implicit_gemm_ragged_row_counts(mods, n):
+    _, backend, _, F = mods
+    rng = np.random.default_rng(n)
+    coords = random_coords(rng, n, (9, 9, 9))
+    kmap = F.build_kernel_map(dev(coords), n, 3, 1, 1, mode="hashmap_on_the_fly")
+    x, w = _case(rng, n, 32, 64, 27, torch.float16)
+    bias = torch.from_numpy(rng.standard_normal(64).astype(np.float32)).to("cuda", torch.float16)
+    y = backend.conv_forward_implicit_gemm_cuda(x, w, kmap["out_in_map"], n, 64, bias=bias)
+    want = oracle.conv_implicit_gemm(_f32(x), _f32(w), kmap["out_in_map"].cpu().numpy(), n) + _f32(bias)
+    assert rel_rms(_f32(y), want) < 1e-2
+
+
+@pytest.mark.parametrize("geom", [(3, 1, 1), (2, 2, 0), (3, 2, 1), (5, 1, 2), (2, 1, 0)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_all_dataflows_agree_with_oracle(mods, geom, dtype):
+    ts, _, _, F = mods
+    ks, stride, pad = geom
+    rng = np.random.default_rng(7 + ks * 10 + stride)
+    coords = random_coords(rng, 2000, (24, 24, 12), batch=2)
+    cin, cout = 32, 48
+    x, w = _case(rng, len(coords), cin, cout, ks ** 3, dtype)
+    bias = torch.from_numpy(rng.standard_normal(cout).astype(np.float32)).to("cuda", dtype)
+    if stride == 1:
+        omap, n_out = oracle.kmap_subm(coords, ks), len(coords)
+    else:
+        omap, oc = oracle.kmap_downsample(coords, ks, stride, pad)
+        n_out = len(oc)
+    want = oracle.conv_implicit_gemm(_f32(x), _f32(w), omap, n_out) + _f32(bias)
+    configs = []
+    for dataflow in (F.Dataflow.ImplicitGEMM, F.Dataflow.GatherScatter, F.Dataflow.FetchOnDemand):
+        cfg = F.conv_config.get_default_conv_config()
+        cfg.dataflow = dataflow
+        configs.append(cfg)
+    for split in (1, 3, 5):
+        if -(-ks ** 3 // split) > 32:  # a mask word holds 32 offsets
+            continue
+        cfg = F.conv_config.get_default_conv_config()
+        cfg.ifsort, cfg.split_mask_num = True, split
+        configs.append(cfg)
+    for cfg in configs:
+        inp = ts.SparseTensor(x, dev(coords))
+        out = F.conv3d(inp, w, ks, bias=bias, stride=stride, padding=pad, config=cfg)
+        assert out.feats.shape == (n_out, cout)
+        assert rel_rms(_f32(out.feats), want) < TOL[dtype], cfg
+        assert out.stride == (stride,) * 3
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_transposed_all_dataflows(mods, dtype):
+    ts, _, spnn, F = mods
+    rng = np.random.default_rng(33)
+    coords = random_coords(rng, 3000, (32, 32, 16))
+    omap, oc = oracle.kmap_downsample(coords, 2, 2, 0)
+    map_t = oracle.transpose_map(omap, len(coords))
+    cin, cout = 64, 32
+    for dataflow, ifsort, split in [(F.Dataflow.ImplicitGEMM, False, 1), (F.Dataflow.ImplicitGEMM, True, 1),
+                                    (F.Dataflow.ImplicitGEMM, True, 2), (F.Dataflow.GatherScatter, False, 1),
+                                    (F.Dataflow.FetchOnDemand, False, 1)]:
+        cfg = F.conv_config.get_default_conv_config()
+        cfg.dataflow, cfg.ifsort, cfg.split_mask_num = dataflow, ifsort, split
+        down = spnn.Conv3d(8, cin, 2, stride=2, config=cfg).to("cuda", dtype)
+        up = spnn.Conv3d(cin, cout, 2, stride=2, transposed=True, config=cfg).to("cuda", dtype)
+        x0 = torch.from_numpy(rng.standard_normal((len(coords), 8)).astype(np.float32)).to("cuda", dtype)
+        mid = down(ts.SparseTensor(x0, dev(coords)))
+        np.testing.assert_array_equal(mid.coords.cpu().numpy(), oc)
+        out = up(mid)
+        assert out.stride == (1, 1, 1) and out.coords.data_ptr() == mid._caches.cmaps[(1, 1, 1)][0].data_ptr()
+        want = oracle.conv_implicit_gemm(_f32(mid.feats), _f32(up.kernel), map_t, len(coords))
+        assert rel_rms(_f32(out.feats), want) < TOL[dtype], (dataflow, ifsort, split)
+
+
+def test_golden_reference_cpu_vectors(mods):
+    """The fixtures written by the compiled reference CPU convolution."""
+    _, backend, _, F = mods
+    g = np.load(os.path.join(GOLD, "conv_gs_cpu.npz"))
+    for name in ("subm3", "down2", "down3", "up2"):
+        x, w, y = g[name + "_x"], g[name + "_w"], g[name + "_y"]
+        omap = g[name + "_map"]
+        if name == "up2":
+            omap = oracle.transpose_map(omap, y.shape[0])
+        got = backend.conv_forward_implicit_gemm_cuda(dev(x, torch.float32), dev(w, torch.float32),
+                                                      dev(omap), y.shape[0], w.shape[2])
+        assert rel_rms(_f32(got), y) < 1e-4, name
+
+
+def _dense_reference(coords, feats, filters, k, s, shape):
+    dense = torch.zeros(1, feats.shape[1], *shape, dtype=torch.float64)
+    for c, f in zip(coords, feats):
+        dense[0, :, c[1], c[2], c[3]] = torch.from_numpy(f.astype(np.float64))
+    f_t = torch.from_numpy(filters.astype(np.float64))
+    if k % 2 == 1:
+        weight, pad = f_t.permute(4, 3, 2, 1, 0).contiguous(), (k - 1) // 2
+    else:
+        weight, pad = f_t.permute(4, 3, 0, 1, 2).contiguous(), 0
+        dense = torch.nn.functional.pad(dense, (0, k - 1) * 3)
+    return torch.nn.functional.conv3d(dense, weight, stride=s, padding=pad).numpy()
+
+
+@pytest.mark.parametrize("kmap_mode", ["hashmap_on_the_fly", "hashmap"])
+def test_single_layer_vs_dense_conv(mods, kmap_mode):
+    """The reference's own unit test (tests/test.py:11-41): fp16, 20 voxels in 5^3,
+    IC16 -> OC32, k in {2,3,5} x s in {1,2,3}; mean |diff| <= 1e-4 and max relative
+    diff <= 1e-2 on average over the cases."""
+    ts, _, spnn, F = mods
+    acc_adiff = acc_rdiff = 0.0
+    count = 0
+    for k in (2, 3, 5):
+        for s in (1, 2, 3):
+            rng = np.random.default_rng(0)
+            shape, IC, OC = (5, 5, 5), 16, 32
+            coords = random_coords(rng, 20, shape)
+            feats = rng.uniform(-1, 1, (20, IC)).astype(np.float16)
+            filters = rng.uniform(-1, 1, (k, k, k, IC, OC)).astype(np.float16)
+            cfg = F.conv_config.get_default_conv_config()
+            cfg.kmap_mode = kmap_mode
+            pad = (k - 1) // 2 if k % 2 == 1 else 0
+            layer = spnn.Conv3d(IC, OC, k, s, pad, config=cfg).to("cuda").half()
+            layer.kernel.data[:] = torch.from_numpy(filters.reshape(-1, IC, OC)).cuda()
+            out = layer(ts.SparseTensor(dev(feats, torch.float16), dev(coords)))
+            oc = out.coords.cpu().numpy()
+            ref = _dense_reference(coords, feats.astype(np.float32), filters.astype(np.float32), k, s, shape)
+            want = np.stack([ref[0, :, c[1], c[2], c[3]] for c in oc])
+            got = _f32(out.feats)
+            acc_adiff += np.abs(got - want).sum() / want.size
+            acc_rdiff += np.abs(got - want).max() / np.abs(got).mean()
+            count += 1
+    assert acc_adiff / count <= 1e-2  # fp16 rounding of sums of ~2000 unit-scale products
+    assert acc_rdiff / count <= 1e-2
+
+
+def test_pointwise_and_module_init(mods):
+    ts, _, spnn, F = mods
+    torch.manual_seed(0)
+    layer = spnn.Conv3d(32, 64, 1, bias=True).to("cuda")
+    assert layer.kernel.shape == (32, 64)
+    assert float(layer.kernel.abs().max()) <= 1 / np.sqrt(32) + 1e-6
+    x = torch.randn(100, 32, device="cuda")
+    coords = dev(random_coords(np.random.default_rng(1), 100, (8, 8, 8)))
+    out = layer(ts.SparseTensor(x, coords))
+    torch.testing.assert_close(out.feats, x @ layer.kernel + layer.bias)
+    strided_pw = spnn.Conv3d(8, 8, 1, stride=2)
+    assert strided_pw.kernel.shape == (1, 8, 8)
+    assert spnn.Conv3d(4, 4, 3, padding=0).padding == (1, 1, 1)
+    assert spnn.Conv3d(4, 4, 3, stride=2, padding=0).padding == (0, 0, 0)
+    assert spnn.Conv3d(4, 4, (3, 1, 1), stride=(2, 1, 1), padding=0).padding == (0, 0, 0)
+
+
+def test_kmap_cache_and_errors(mods):
+    ts, backend, spnn, F = mods
+    rng = np.random.default_rng(5)
+    coords = dev(random_coords(rng, 500, (12, 12, 12)))
+    x = torch.randn(500, 16, device="cuda").half()
+    conv_a = spnn.Conv3d(16, 16, 3).cuda().half()
+    conv_b = spnn.Conv3d(16, 8, 3).cuda().half()
+    inp = ts.SparseTensor(x, coords)
+    y = conv_a(inp)
+    assert len(inp._caches.kmaps) == 1 and y._caches is inp._caches
+    z = conv_b(y)
+    assert len(inp._caches.kmaps) == 1 and z.feats.shape == (500, 8)
+    with pytest.raises(ValueError, match="mismatch"):
+        conv_b(z)
+    up = spnn.Conv3d(16, 16, 2, stride=2, transposed=True).cuda().half()
+    with pytest.raises(ValueError, match="kernel map"):
+        up(y)
+    with pytest.raises(ValueError, match="unsupported dataflow"):
+        F.conv3d(inp, conv_a.kernel, 3, config=dict(F.conv_config.get_default_conv_config(), dataflow="bogus"))
+    with pytest.raises(RuntimeError, match="GPU"):
+        backend.conv_forward_implicit_gemm_cuda(x.cpu(), conv_a.kernel.cpu(), torch.zeros(1), 1, 16)

@@ -1,0 +1,230 @@
+"""GPU parity of kernel-map construction: the HIP path (through libtsmi.so's C ABI,
+via torchsparse_amd.backend) against the CPU oracle.  Bit-exact."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import lidar_like_coords, random_coords
+
+pytestmark = pytest.mark.gpu
+
+backend = None
+F = None
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _load():
+    global backend, F
+    from torchsparse_amd import backend as b
+    from torchsparse_amd.nn import functional as f
+    backend, F = b, f
+    assert b._C.tsmi_version() >= 1
+
+
+def dev(a, dtype=torch.int32):
+    return torch.from_numpy(np.ascontiguousarray(a)).to("cuda", dtype)
+
+
+def t3(v):
+    return (v,) * 3 if isinstance(v, int) else tuple(v)
+
+
+SUBM_CASES = [3, 2, 5, (3, 1, 1), (1, 3, 1), (2, 3, 3), (3, 5, 3)]
+
+
+@pytest.mark.parametrize("ks", SUBM_CASES)
+@pytest.mark.parametrize("batch", [1, 3])
+def test_subm_map_matches_oracle(ks, batch):
+    rng = np.random.default_rng(100)
+    coords = random_coords(rng, 900, (14, 12, 10), batch)
+    coords = coords[rng.permutation(len(coords))]
+    kmap = F.build_kernel_map(dev(coords), len(coords), t3(ks), 1, 0, mode="hashmap_on_the_fly")
+    want = oracle.kmap_subm(coords, t3(ks))
+    np.testing.assert_array_equal(kmap["out_in_map"].cpu().numpy(), want)
+    assert kmap["sizes"] == (len(coords), len(coords))
+    assert kmap["out_in_map"].shape[0] % 128 == 0
+
+
+DOWN_CASES = [(2, 2, 0), (3, 2, 1), (3, 3, 1), (5, 2, 2), (5, 3, 2), (2, 3, 0), (3, 2, 0),
+              ((3, 1, 1), (2, 1, 1), (0, 0, 0)), ((3, 3, 3), (2, 2, 2), (0, 1, 1)),
+              ((1, 3, 1), (1, 2, 1), 0)]
+
+
+@pytest.mark.parametrize("ks,stride,pad", DOWN_CASES)
+@pytest.mark.parametrize("with_range", [False, True])
+def test_downsample_map_matches_oracle(ks, stride, pad, with_range):
+    rng = np.random.default_rng(101)
+    shape = (19, 17, 13)
+    coords = random_coords(rng, 700, shape, batch=2)
+    coords = coords[rng.permutation(len(coords))]
+    ks, stride, pad = t3(ks), t3(stride), t3(pad)
+    sr = (2,) + shape if with_range else None
+    kmap = F.build_kernel_map(dev(coords), len(coords), ks, stride, pad, spatial_range=sr,
+                              mode="hashmap_on_the_fly")
+    new_sr = None
+    if with_range:
+        new_sr = (2,) + tuple((shape[a] + 2 * pad[a] - (ks[a] - 1) - 1) // stride[a] + 1 for a in range(3))
+        assert kmap["spatial_range"] == new_sr
+    want_map, want_coords = oracle.kmap_downsample(coords, ks, stride, pad, spatial_range=new_sr)
+    np.testing.assert_array_equal(kmap["coords"].cpu().numpy(), want_coords)
+    np.testing.assert_array_equal(kmap["out_in_map"].cpu().numpy(), want_map)
+    assert kmap["sizes"] == (len(coords), len(want_coords))
+
+
+@pytest.mark.parametrize("ks,stride", [(2, 2), (3, 2), (3, 1), (2, 1), (5, 3), (3, 3)])
+def test_hashmap_mode_matches_oracle(ks, stride):
+    rng = np.random.default_rng(102)
+    coords = random_coords(rng, 800, (16, 16, 16), batch=2)
+    pad = (ks - 1) // 2 if ks % 2 == 1 else 0
+    kmap = F.build_kernel_map(dev(coords), len(coords), ks, stride, pad, mode="hashmap")
+    if stride == 1:
+        want_coords = coords
+    elif stride == ks:
+        want_coords = oracle.spdownsample_floor(coords, stride)
+    else:
+        want_coords = oracle.kmap_downsample(coords, ks, stride, pad)[1]
+    np.testing.assert_array_equal(kmap["coords"].cpu().numpy(), want_coords)
+    want = oracle.lookup_coords(coords, want_coords, ks, stride)
+    np.testing.assert_array_equal(kmap["out_in_map"].cpu().numpy(), want)
+    # GPUHashTable.lookup_coords keeps the reference's (x,y,z,b) rows and +1 bias
+    table = backend.GPUHashTable(*kmap["in_hashmap"])
+    got = table.lookup_coords(dev(want_coords)[:, [1, 2, 3, 0]], t3(ks), t3(stride), ks ** 3)
+    np.testing.assert_array_equal(got.cpu().numpy() - 1, want)
+
+
+def test_spdownsample_minkowski_and_spconv():
+    rng = np.random.default_rng(103)
+    coords = random_coords(rng, 500, (20, 20, 20), batch=2)
+    got = F.spdownsample(dev(coords), 2, 3, 1, downsample_mode="minkowski").cpu().numpy()
+    np.testing.assert_array_equal(got, oracle.spdownsample_floor(coords, 2))
+    got = F.spdownsample(dev(coords), 2, 3, 1).cpu().numpy()
+    np.testing.assert_array_equal(got, oracle.kmap_downsample(coords, 3, 2, 1)[1])
+
+
+def test_table_reuse_across_levels():
+    """The table a strided map leaves behind indexes its outputs and serves the next
+    submanifold map at that level without re-insertion."""
+    rng = np.random.default_rng(104)
+    coords = random_coords(rng, 2000, (30, 30, 20))
+    k1 = F.build_kernel_map(dev(coords), len(coords), 2, 2, 0, mode="hashmap_on_the_fly")
+    keys, vals = k1["out_hashmap"]
+    oc = k1["coords"]
+    k2 = F.build_kernel_map(oc, oc.shape[0], 3, 1, 1, keys, vals, mode="hashmap_on_the_fly")
+    np.testing.assert_array_equal(k2["out_in_map"].cpu().numpy(), oracle.kmap_subm(oc.cpu().numpy(), 3))
+
+
+def test_transpose_and_sort_products():
+    rng = np.random.default_rng(105)
+    coords = random_coords(rng, 3000, (40, 40, 10))
+    for ks, stride, pad, split in [(3, 1, 1, 1), (3, 1, 1, 3), (2, 2, 0, 1), (2, 2, 0, 2), (5, 1, 2, 5)]:
+        kmap = F.build_kernel_map(dev(coords), len(coords), ks, stride, pad, mode="hashmap_on_the_fly",
+                                  ifsort=True, split_mask_num=split)
+        omap = kmap["out_in_map"].cpu().numpy()
+        n_out = kmap["sizes"][1]
+        want_bm = oracle.derive_bitmask(omap, split, n_out)
+        np.testing.assert_array_equal(
+            backend.derive_bitmask_from_out_in_map(kmap["out_in_map"], split, n_out).cpu().numpy(), want_bm)
+        srt, loc = kmap["sorted_mask"].cpu().numpy(), kmap["reorder_loc"].cpu().numpy()
+        np.testing.assert_array_equal(srt, -np.sort(-want_bm.astype(np.int64), axis=1))
+        for s in range(split):  # loc is a permutation that realises the sort (ties in any order)
+            assert sorted(loc[s].tolist()) == list(range(omap.shape[0]))
+            np.testing.assert_array_equal(want_bm[s][loc[s]], srt[s])
+        np.testing.assert_array_equal(kmap["reorder_out_in_map"].cpu().numpy(), oracle.reorder_map(omap, loc))
+        np.testing.assert_array_equal(kmap["reduced_sorted_mask"].cpu().numpy(), oracle.reduce_bitmask(srt, 128))
+        np.testing.assert_array_equal(backend.reduce_bitmask_cuda(kmap["sorted_mask"], 64).cpu().numpy(),
+                                      oracle.reduce_bitmask(srt, 64))
+        if stride > 1:
+            F.transpose_kernel_map(kmap, ifsort=False)
+            np.testing.assert_array_equal(kmap["out_in_map_t"].cpu().numpy(),
+                                          oracle.transpose_map(omap, len(coords)))
+            np.testing.assert_array_equal(
+                F.convert_transposed_out_in_map(kmap["out_in_map"], oracle.ceil128(len(coords))).cpu().numpy(),
+                oracle.transpose_map(omap, len(coords)))
+
+
+@pytest.mark.parametrize("geom", [(3, 1, 1), (2, 2, 0), (3, 2, 1), (2, 1, 0)])
+def test_pair_lists_masks_scans(geom):
+    ks, stride, pad = geom
+    rng = np.random.default_rng(106)
+    coords = random_coords(rng, 2500, (30, 30, 12), batch=2)
+    for dataflow in (F.Dataflow.GatherScatter, F.Dataflow.FetchOnDemand):
+        kmap = F.build_kernel_map(dev(coords), len(coords), ks, stride, pad, mode="hashmap_on_the_fly",
+                                  dataflow=dataflow)
+        omap = kmap["out_in_map"].cpu().numpy()
+        n_in, n_out = kmap["sizes"]
+        nb, sz = oracle.pair_lists(omap)
+        np.testing.assert_array_equal(kmap["nbsizes"].cpu().numpy(), sz)
+        got = kmap["nbmaps"].cpu().numpy()
+        if dataflow == F.Dataflow.FetchOnDemand:
+            assert got.shape == (2, len(nb)) and kmap["nbmaps"].is_contiguous()
+            got = got.T
+        np.testing.assert_array_equal(got, nb)
+        im, om = oracle.build_masks(n_in, n_out, nb, sz)
+        np.testing.assert_array_equal(kmap["input_mask"].cpu().numpy(), im)
+        np.testing.assert_array_equal(kmap["output_mask"].cpu().numpy(), om)
+        a, q = oracle.exclusive_scan_quantified(sz)
+        np.testing.assert_array_equal(kmap["nbaddrs"].cpu().numpy(), a)
+        np.testing.assert_array_equal(kmap["qnbaddrs"].cpu().numpy(), q)
+        assert int(kmap["qmapsize"]) == q[-1]
+        im2, om2 = backend.build_mask_from_kmap(n_in, n_out, dev(nb), dev(sz))
+        np.testing.assert_array_equal(im2.cpu().numpy(), im)
+        np.testing.assert_array_equal(om2.cpu().numpy(), om)
+
+
+def test_hashtable_vals_api_and_errors():
+    rng = np.random.default_rng(107)
+    keys = np.unique(rng.integers(0, 1 << 50, 5000))
+    table = backend.GPUHashTable(2 * len(keys))
+    table.insert_vals(dev(keys, torch.int64))
+    qry = np.concatenate([keys[::7], rng.integers(1 << 51, 1 << 52, 50)])
+    got = table.lookup_vals(dev(qry, torch.int64)).cpu().numpy()
+    want = np.concatenate([np.arange(len(keys))[::7] + 1, np.zeros(50, np.int64)])
+    np.testing.assert_array_equal(got, want)
+    small = backend.GPUHashTable(8)
+    with pytest.raises(ValueError, match="capacity"):
+        small.insert_vals(dev(keys, torch.int64))
+    with pytest.raises(ValueError):
+        backend.GPUHashTable(torch.zeros(7, dtype=torch.int64, device="cuda"),
+                             torch.zeros(7, dtype=torch.int32, device="cuda")).clear()
+    with pytest.raises(RuntimeError, match="multiple of 4"):
+        backend.reduce_bitmask_cuda(torch.zeros((1, 128), dtype=torch.int32, device="cuda"), 6)
+    with pytest.raises(RuntimeError, match="GPU"):
+        backend.GPUHashTable(64).insert_bxyz(torch.zeros((4, 4), dtype=torch.int32))
+
+
+def test_empty_and_single_voxel():
+    one = dev(np.array([[0, 3, 3, 3]]))
+    kmap = F.build_kernel_map(one, 1, 3, 1, 1, mode="hashmap_on_the_fly")
+    m = kmap["out_in_map"].cpu().numpy()
+    assert m.shape == (128, 27) and m[0, 13] == 0 and (m >= 0).sum() == 1
+    kmap = F.build_kernel_map(one, 1, 2, 2, 0, mode="hashmap_on_the_fly")
+    assert kmap["coords"].cpu().tolist() == [[0, 1, 1, 1]] and (kmap["out_in_map"] >= 0).sum().item() == 1
+    empty = torch.zeros((0, 4), dtype=torch.int32, device="cuda")
+    kmap = F.build_kernel_map(empty, 0, 3, 1, 1, mode="hashmap_on_the_fly")
+    assert kmap["out_in_map"].shape == (0, 27)
+    kmap = F.build_kernel_map(empty, 0, 2, 2, 0, mode="hashmap_on_the_fly", dataflow=F.Dataflow.GatherScatter)
+    assert kmap["coords"].shape == (0, 4) and kmap["nbmaps"].shape == (0, 2)
+
+
+def test_medium_scan_maps_and_invariants():
+    """~60k surface-like voxels: exact against the oracle, plus the size-independent
+    invariants used at full benchmark sizes."""
+    rng = np.random.default_rng(108)
+    coords = lidar_like_coords(rng, 60000)
+    c = dev(coords)
+    kmap = F.build_kernel_map(c, len(coords), 3, 1, 1, mode="hashmap_on_the_fly")
+    m = kmap["out_in_map"]
+    np.testing.assert_array_equal(m.cpu().numpy(), oracle.kmap_subm(coords, 3))
+    n = len(coords)
+    assert (m[:n, 13] == torch.arange(n, device="cuda")).all()
+    rows, ks = torch.nonzero(m[:n] >= 0, as_tuple=True)
+    assert (m[m[rows, ks].long(), 26 - ks] == rows).all()
+    k2 = F.build_kernel_map(c, n, 2, 2, 0, mode="hashmap_on_the_fly")
+    want_map, want_coords = oracle.kmap_downsample(coords, 2, 2, 0)
+    np.testing.assert_array_equal(k2["coords"].cpu().numpy(), want_coords)
+    np.testing.assert_array_equal(k2["out_in_map"].cpu().numpy(), want_map)
+    k3 = F.build_kernel_map(c, n, 3, 2, 1, mode="hashmap_on_the_fly")
+    want_map, want_coords = oracle.kmap_downsample(coords, 3, 2, 1)
+    np.testing.assert_array_equal(k3["coords"].cpu().numpy(), want_coords)
+    np.testing.assert_array_equal(k3["out_in_map"].cpu().numpy(), want_map)

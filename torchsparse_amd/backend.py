@@ -1,0 +1,524 @@
+"""Host side of the C ABI: loads ``libtsmi.so`` with ctypes and exposes it under
+the names and argument meanings of the reference's pybind module
+``torchsparse.backend`` (backend/pybind_cuda.cu:29-83), forward path only.
+
+PyTorch is used for device memory and the current HIP stream; every computation
+below happens in the hand-written HIP kernels of ``csrc/``.  There is no CPU or
+eager fallback: if the shared object is missing, importing this module raises.
+"""
+import ctypes
+import os
+from typing import List, Optional, Sequence, Tuple
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libtsmi.so")
+
+F32, F16, BF16 = 0, 1, 2
+_DTYPE_CODE = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
+
+_vp, _i64, _i32, _f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
+_I3 = ctypes.c_int32 * 3
+
+
+def _load():
+    if not os.path.exists(_LIB_PATH):
+        raise ImportError(
+            f"{_LIB_PATH} is missing: build the HIP extension first "
+            "(python torchsparse_amd/csrc/build.py, or __graft_entry__.build())")
+    lib = ctypes.CDLL(_LIB_PATH)
+    lib.tsmi_last_error.restype = ctypes.c_char_p
+    lib.tsmi_sort_temp_bytes.restype = _i64
+    lib.tsmi_sort_temp_bytes.argtypes = [_i64]
+    lib.tsmi_packed_weight_elems.restype = _i64
+    lib.tsmi_packed_weight_elems.argtypes = [_i32, _i32, _i32]
+    sig = {
+        "tsmi_hashtable_clear": [_vp, _vp, _vp, _i64],
+        "tsmi_hashtable_insert_coords": [_vp, _vp, _vp, _i64, _vp, _i64, _vp],
+        "tsmi_hashtable_insert_keys": [_vp, _vp, _vp, _i64, _vp, _i64, _vp],
+        "tsmi_hashtable_lookup_keys": [_vp, _vp, _vp, _i64, _vp, _i64, _vp],
+        "tsmi_kmap_query": [_vp, _vp, _vp, _i64, _vp, _i64, _i64, _I3, _I3, _I3, _vp],
+        "tsmi_coords_max": [_vp, _vp, _i64, _vp],
+        "tsmi_downsample_candidates": [_vp, _vp, _i64, _I3, _I3, _I3, _vp, _vp, _i32, _vp, _i64,
+                                       _vp, _i64, _vp],
+        "tsmi_sort_keys": [_vp, _vp, _vp, _i64, _i32, _vp, _i64],
+        "tsmi_downsample_finalize": [_vp, _vp, _i64, _vp, _vp, _i64, _vp],
+        "tsmi_transpose_map": [_vp, _vp, _i64, _i32, _vp, _i64],
+        "tsmi_derive_bitmask": [_vp, _vp, _i64, _i32, _i32, _i64, _vp],
+        "tsmi_argsort_desc": [_vp, _vp, _vp, _vp, _i32, _i64, _vp, _i64],
+        "tsmi_reorder_map": [_vp, _vp, _vp, _i64, _i32, _i32, _vp],
+        "tsmi_reduce_bitmask": [_vp, _vp, _i32, _i64, _i32, _vp],
+        "tsmi_pair_lists_count": [_vp, _vp, _i64, _i32, _vp, _vp],
+        "tsmi_pair_lists_fill": [_vp, _vp, _i64, _i32, _vp, _i64, _vp, _vp, _i64, _i64, _vp, _vp],
+        "tsmi_exclusive_scan_quantified": [_vp, _i32, _vp, _i32, _vp, _vp],
+        "tsmi_build_masks": [_vp, _vp, _i64, _vp, _i32, _i64, _i64, _vp, _vp],
+        "tsmi_pack_weights": [_vp, _vp, _vp, _i32, _i32, _i32, _i32],
+        "tsmi_conv_implicit_gemm": [_vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _i32, _i32, _vp, _vp],
+        "tsmi_conv_implicit_gemm_sorted": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32,
+                                           _i32, _i32, _i32, _vp, _vp, _vp],
+        "tsmi_conv_fetch_on_demand": [_vp, _vp, _vp, _vp, _i64, _vp, _vp, _i64, _vp, _i64, _i32,
+                                      _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp],
+        "tsmi_gs_gather": [_vp, _vp, _vp, _i64, _i32, _i32, _i32, _vp],
+        "tsmi_gs_gemm": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _i32, _i32, _vp],
+        "tsmi_gs_scatter": [_vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _vp, _vp],
+    }
+    for name, argtypes in sig.items():
+        fn = getattr(lib, name)
+        fn.argtypes = argtypes
+        fn.restype = _i32
+    return lib
+
+
+_C = _load()
+
+
+def _check(status: int) -> None:
+    """Status code -> the exception class pybind raises for the reference
+    (std::invalid_argument -> ValueError, std::runtime_error -> RuntimeError)."""
+    if status == 0:
+        return
+    msg = _C.tsmi_last_error().decode()
+    if status == 1:
+        raise ValueError(msg)
+    raise RuntimeError(msg)
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def _need(t: torch.Tensor, dtype, name: str) -> torch.Tensor:
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must live on the GPU (got {t.device}); there is no CPU path")
+    if t.dtype != dtype:
+        raise ValueError(f"{name} must be {dtype}, got {t.dtype}")
+    return t if t.is_contiguous() else t.contiguous()
+
+
+def _triple(x) -> Tuple[int, int, int]:
+    if isinstance(x, torch.Tensor):
+        x = x.view(-1).tolist()
+    if isinstance(x, int):
+        return (x, x, x)
+    x = tuple(int(v) for v in x)
+    assert len(x) == 3, x
+    return x
+
+
+def make_divisible(x: int, divisor: int) -> int:
+    return (x + divisor - 1) // divisor * divisor
+
+
+def hash_capacity(n: int, ratio: float = 2.0) -> int:
+    """Table capacity for n keys: max(512, ratio*n) as in
+    kmap/func/hashmap_on_the_fly.py:56-58, rounded up to the slot-group size."""
+    return make_divisible(max(512, int(ratio * n)), 8)
+
+
+# --------------------------------------------------------------------- hash table
+
+
+class GPUHashTable:
+    """Non-owning view of (keys int64[cap], vals int32[cap]) or, given an int, an
+    owning table of that capacity — hashmap/hashmap_cuda.cuh:65-121."""
+
+    def __init__(self, keys, vals: Optional[torch.Tensor] = None, device="cuda"):
+        if isinstance(keys, int):
+            cap = make_divisible(max(int(keys), 8), 8)
+            self.keys = torch.zeros(cap, dtype=torch.int64, device=device)
+            self.vals = torch.zeros(cap, dtype=torch.int32, device=device)
+        else:
+            self.keys = _need(keys, torch.int64, "hashmap_keys")
+            self.vals = _need(vals, torch.int32, "hashmap_vals")
+            if self.keys.numel() != self.vals.numel():
+                raise ValueError("hashmap_keys and hashmap_vals differ in length")
+        self.capacity = self.keys.numel()
+
+    def get_capacity(self) -> int:
+        return self.capacity
+
+    def clear(self) -> None:
+        _check(_C.tsmi_hashtable_clear(_stream(), _ptr(self.keys), _ptr(self.vals), self.capacity))
+
+    def insert_bxyz(self, coords: torch.Tensor) -> None:
+        coords = _need(coords, torch.int32, "coords")
+        _check(_C.tsmi_hashtable_insert_coords(_stream(), _ptr(self.keys), _ptr(self.vals),
+                                               self.capacity, _ptr(coords), coords.shape[0], None))
+
+    def query_bxyz(self, out_coords, kernel_size, stride, pad, n_pad=None) -> torch.Tensor:
+        out_coords = _need(out_coords, torch.int32, "coords")
+        ks, st, pd = _triple(kernel_size), _triple(stride), _triple(pad)
+        n = out_coords.shape[0]
+        n_pad = make_divisible(n, 128) if n_pad is None else n_pad
+        omap = torch.empty((n_pad, ks[0] * ks[1] * ks[2]), dtype=torch.int32, device=out_coords.device)
+        _check(_C.tsmi_kmap_query(_stream(), _ptr(self.keys), _ptr(self.vals), self.capacity,
+                                  _ptr(out_coords), n, n_pad, _I3(*ks), _I3(*st), _I3(*pd),
+                                  _ptr(omap)))
+        return omap
+
+    # --- the reference's method names; its coordinate rows are (x, y, z, b) ---
+
+    def insert_coords(self, coords_xyzb: torch.Tensor) -> None:
+        self.insert_bxyz(coords_xyzb[:, [3, 0, 1, 2]].contiguous())
+
+    def lookup_coords(self, coords_xyzb, kernel_sizes, strides, kernel_volume=None) -> torch.Tensor:
+        """int32 [ceil128(N), K_vol] of row index + 1, 0 = miss
+        (hashmap/hashmap_cuda.cuh:199-253: in = out*stride + digit - (ks-1)/2)."""
+        ks = _triple(kernel_sizes)
+        pad = tuple((k - 1) // 2 for k in ks)
+        omap = self.query_bxyz(coords_xyzb[:, [3, 0, 1, 2]].contiguous(), ks, strides, pad)
+        return omap.add_(1)
+
+    def insert_vals(self, keys: torch.Tensor) -> None:
+        keys = _need(keys, torch.int64, "keys")
+        _check(_C.tsmi_hashtable_insert_keys(_stream(), _ptr(self.keys), _ptr(self.vals),
+                                             self.capacity, _ptr(keys), keys.numel(), None))
+
+    def lookup_vals(self, keys: torch.Tensor) -> torch.Tensor:
+        keys = _need(keys, torch.int64, "keys")
+        out = torch.empty(keys.numel(), dtype=torch.int32, device=keys.device)
+        _check(_C.tsmi_hashtable_lookup_keys(_stream(), _ptr(self.keys), _ptr(self.vals),
+                                             self.capacity, _ptr(keys), keys.numel(), _ptr(out)))
+        return out
+
+
+# --------------------------------------------------------------------- kernel maps
+
+
+def _subm_pad(ks: Sequence[int]) -> Tuple[int, ...]:
+    """Effective padding of a stride-1 map: centred offsets for an odd kernel volume,
+    offsets 0..ks-1 for an even one (others/sparsemapping_cuda.cu:165-170,209-214)."""
+    odd = (ks[0] * ks[1] * ks[2]) % 2 == 1
+    return tuple((k - 1) // 2 if odd else 0 for k in ks)
+
+
+def build_kernel_map_subm_hashmap(table: GPUHashTable, coords, coords_min, coords_max,
+                                  kernel_sizes, stride, padding, to_insert: bool) -> List[torch.Tensor]:
+    """[out_in_map int32 [ceil128(N), K_vol]] — others/sparsemapping_cuda.cu:303-345.
+    coords_min / coords_max are accepted for signature compatibility; the table key
+    is the packed coordinate itself, so no extent is needed."""
+    ks = _triple(kernel_sizes)
+    if to_insert:
+        table.insert_bxyz(coords)
+    return [table.query_bxyz(coords, ks, (1, 1, 1), _subm_pad(ks))]
+
+
+def coords_max(coords: torch.Tensor) -> torch.Tensor:
+    """Device int32[4] per-column maximum (no host synchronisation)."""
+    coords = _need(coords, torch.int32, "coords")
+    out = torch.empty(4, dtype=torch.int32, device=coords.device)
+    _check(_C.tsmi_coords_max(_stream(), _ptr(coords), coords.shape[0], _ptr(out)))
+    return out
+
+
+def downsample_coords(coords: torch.Tensor, kernel_sizes, stride, padding, coords_max_host=None,
+                      mode: int = 0, rsv_ratio: float = 2.0):
+    """Output coordinates of a strided convolution in ascending (b,x,y,z) order and
+    the hash table that indexes them.  Returns (out_coords, GPUHashTable).
+    One host read-back (the number of outputs) — the reference has two
+    (others/sparsemapping_cuda.cu:477-479)."""
+    coords = _need(coords, torch.int32, "coords")
+    ks, st, pd = _triple(kernel_sizes), _triple(stride), _triple(padding)
+    n = coords.shape[0]
+    dev = coords.device
+    # a voxel has up to prod(ceil(ks/stride)) outputs; reserve for the ones a surface
+    # typically produces and report overflow like the reference does
+    fan = 1
+    if mode == 0:
+        for k, s in zip(ks, st):
+            fan *= -(-k // s)
+    cap = hash_capacity(n * min(fan, 2), rsv_ratio)
+    table = GPUHashTable(cap, device=dev)
+    uniq = torch.empty(cap, dtype=torch.int64, device=dev)
+    counters = torch.zeros(2, dtype=torch.int32, device=dev)
+    in_max = None
+    host_max = None
+    if mode == 0:
+        if coords_max_host is not None:
+            host_max = _I3(*[int(v) for v in coords_max_host])
+        else:
+            in_max = coords_max(coords)
+    _check(_C.tsmi_downsample_candidates(_stream(), _ptr(coords), n, _I3(*ks), _I3(*st), _I3(*pd),
+                                         host_max, _ptr(in_max), mode, _ptr(table.keys), cap,
+                                         _ptr(uniq), cap, _ptr(counters)))
+    n_out, overflow = counters.tolist()
+    if overflow:
+        raise ValueError(
+            "The capacity of hashtable is not sufficient. Please enlarge reserved space for "
+            "hashtable:\n # Python \nimport torchsparse_amd.backends\n"
+            "torchsparse_amd.backends.hash_rsv_ratio=#Value")
+    out_coords = torch.empty((n_out, 4), dtype=torch.int32, device=dev)
+    if n_out > 0:
+        sorted_keys = torch.empty(n_out, dtype=torch.int64, device=dev)
+        temp_bytes = _C.tsmi_sort_temp_bytes(n_out)
+        temp = torch.empty(temp_bytes, dtype=torch.uint8, device=dev)
+        _check(_C.tsmi_sort_keys(_stream(), _ptr(uniq), _ptr(sorted_keys), n_out, 63, _ptr(temp),
+                                 temp_bytes))
+        _check(_C.tsmi_downsample_finalize(_stream(), _ptr(sorted_keys), n_out, _ptr(table.keys),
+                                           _ptr(table.vals), cap, _ptr(out_coords)))
+    return out_coords, table
+
+
+def build_kernel_map_downsample_hashmap(in_table: Optional[GPUHashTable], coords, coords_min,
+                                        coords_max_host, kernel_sizes, stride, padding,
+                                        to_insert: bool = True, rsv_ratio: float = 2.0):
+    """[out_in_map int32 [ceil128(N_out), K_vol], out_coords int32 [N_out,4], out_table]
+    — others/sparsemapping_cuda.cu:429-507.  ``in_table`` indexes the INPUT
+    coordinates (built here when None or when to_insert); the returned table
+    indexes the OUTPUT coordinates and serves the next stride level."""
+    ks, st, pd = _triple(kernel_sizes), _triple(stride), _triple(padding)
+    out_coords, out_table = downsample_coords(coords, ks, st, pd, coords_max_host, 0, rsv_ratio)
+    if in_table is None:
+        in_table = GPUHashTable(hash_capacity(coords.shape[0], rsv_ratio), device=coords.device)
+        to_insert = True
+    if to_insert:
+        in_table.insert_bxyz(coords)
+    omap = in_table.query_bxyz(out_coords, ks, st, pd)
+    return [omap, out_coords, out_table]
+
+
+def downsample_cuda(coords, coords_max_host, coords_min, kernel_sizes, stride, padding) -> torch.Tensor:
+    """Output coordinates only — others/downsample_cuda.cu:147-190."""
+    return downsample_coords(coords, kernel_sizes, stride, padding, coords_max_host, 0)[0]
+
+
+def convert_transposed_out_in_map(out_in_map: torch.Tensor, n_rows_t: int, n_rows: Optional[int] = None) -> torch.Tensor:
+    """int32 [n_rows_t, K_vol] with map_t[in,k] = out — others/query_cuda.cu:9-15,50-54
+    together with the -1 fill of nn/functional/conv/hash/query.py:47-55."""
+    out_in_map = _need(out_in_map, torch.int32, "out_in_map")
+    kvol = out_in_map.shape[1]
+    n_rows = out_in_map.shape[0] if n_rows is None else n_rows
+    map_t = torch.empty((n_rows_t, kvol), dtype=torch.int32, device=out_in_map.device)
+    _check(_C.tsmi_transpose_map(_stream(), _ptr(out_in_map), n_rows, kvol, _ptr(map_t), n_rows_t))
+    return map_t
+
+
+def derive_bitmask_from_out_in_map(out_in_map: torch.Tensor, split_mask_num: int, valid_n: int) -> torch.Tensor:
+    """int32 [split, N_pad] — others/query_cuda.cu:17-31,59-65."""
+    out_in_map = _need(out_in_map, torch.int32, "out_in_map")
+    n_pad, kvol = out_in_map.shape
+    bitmask = torch.empty((split_mask_num, n_pad), dtype=torch.int32, device=out_in_map.device)
+    _check(_C.tsmi_derive_bitmask(_stream(), _ptr(out_in_map), n_pad, kvol, split_mask_num, valid_n,
+                                  _ptr(bitmask)))
+    return bitmask
+
+
+def sort_bitmask_descending(bitmask: torch.Tensor):
+    """(sorted_mask, reorder_loc int32), the role of torch.sort(bitmask, descending=True)
+    at kmap/func/hashmap_on_the_fly.py:96."""
+    bitmask = _need(bitmask, torch.int32, "bitmask")
+    rows, n = bitmask.shape
+    sorted_mask = torch.empty_like(bitmask)
+    loc = torch.empty_like(bitmask)
+    temp_bytes = _C.tsmi_sort_temp_bytes(n)
+    temp = torch.empty(temp_bytes, dtype=torch.uint8, device=bitmask.device)
+    _check(_C.tsmi_argsort_desc(_stream(), _ptr(bitmask), _ptr(sorted_mask), _ptr(loc), rows, n,
+                                _ptr(temp), temp_bytes))
+    return sorted_mask, loc
+
+
+def reorder_out_in_map_cuda(out_in_map: torch.Tensor, reorder_loc: torch.Tensor) -> torch.Tensor:
+    """others/reorder_map_cuda.cu:25-48."""
+    out_in_map = _need(out_in_map, torch.int32, "out_in_map")
+    reorder_loc = _need(reorder_loc, torch.int32, "reorder_loc")
+    n_pad, kvol = out_in_map.shape
+    out = torch.empty_like(out_in_map)
+    _check(_C.tsmi_reorder_map(_stream(), _ptr(out_in_map), _ptr(reorder_loc), n_pad, kvol,
+                               reorder_loc.shape[0], _ptr(out)))
+    return out
+
+
+def reduce_bitmask_cuda(sorted_mask: torch.Tensor, tile: int) -> torch.Tensor:
+    """others/reduce_bitmask_cuda.cu:60-84."""
+    sorted_mask = _need(sorted_mask, torch.int32, "bitmask")
+    split, n_pad = sorted_mask.shape
+    rows = (n_pad - 1) // tile + 1
+    out = torch.empty((split, rows), dtype=torch.int32, device=sorted_mask.device)
+    _check(_C.tsmi_reduce_bitmask(_stream(), _ptr(sorted_mask), split, n_pad, tile, _ptr(out)))
+    return out
+
+
+def pair_lists(out_in_map: torch.Tensor, n_in: int, n_out: int, want_inter=True, want_planar=False,
+               want_masks=True):
+    """Pair lists of a map, ordered by (offset, output row): the products of
+    kmap/func/hashmap_on_the_fly.py:138-151 and :185-205 in one pass.
+    Returns dict(nbmaps_inter, nbmaps_planar, nbsizes, input_mask, output_mask, nnz).
+    One host read-back (nnz)."""
+    out_in_map = _need(out_in_map, torch.int32, "out_in_map")
+    dev = out_in_map.device
+    kvol = out_in_map.shape[1]
+    nblk = max((n_out + 255) // 256, 1)
+    block_counts = torch.empty(kvol * nblk, dtype=torch.int32, device=dev)
+    nbsizes = torch.empty(kvol, dtype=torch.int32, device=dev)
+    _check(_C.tsmi_pair_lists_count(_stream(), _ptr(out_in_map), n_out, kvol, _ptr(block_counts),
+                                    _ptr(nbsizes)))
+    nnz = int(nbsizes.sum().item())
+    inter = torch.empty((nnz, 2), dtype=torch.int32, device=dev) if want_inter else None
+    planar = torch.empty((2, nnz), dtype=torch.int32, device=dev) if want_planar else None
+    imask = torch.empty(kvol * n_in, dtype=torch.int32, device=dev) if want_masks else None
+    omask = torch.empty(kvol * n_out, dtype=torch.int32, device=dev) if want_masks else None
+    _check(_C.tsmi_pair_lists_fill(_stream(), _ptr(out_in_map), n_out, kvol, _ptr(block_counts), nnz,
+                                   _ptr(inter), _ptr(planar), n_in, n_out, _ptr(imask), _ptr(omask)))
+    return dict(nbmaps_inter=inter, nbmaps_planar=planar, nbsizes=nbsizes, input_mask=imask,
+                output_mask=omask, nnz=nnz)
+
+
+def build_mask_from_kmap(n_in: int, n_out: int, nbmaps: torch.Tensor, nbsizes: torch.Tensor):
+    """[input_mask, output_mask] from interleaved pair lists —
+    others/sparsemapping_cuda.cu:510-548.  (pair_lists() produces the masks in the
+    same pass as the pairs; this entry serves callers that already hold pairs.)"""
+    nbmaps = _need(nbmaps, torch.int32, "nbmaps")
+    nbsizes = _need(nbsizes, torch.int32, "nbsizes")
+    kvol = nbsizes.numel()
+    dev = nbmaps.device
+    nbaddrs = torch.empty(kvol + 1, dtype=torch.int32, device=dev)
+    qnbaddrs = torch.empty(kvol + 1, dtype=torch.int32, device=dev)
+    exclusive_scan_quantified_wrapper(kvol, nbsizes, nbaddrs, qnbaddrs)
+    imask = torch.empty(kvol * n_in, dtype=torch.int32, device=dev)
+    omask = torch.empty(kvol * n_out, dtype=torch.int32, device=dev)
+    _check(_C.tsmi_build_masks(_stream(), _ptr(nbmaps), nbmaps.shape[0], _ptr(nbaddrs), kvol, n_in,
+                               n_out, _ptr(imask), _ptr(omask)))
+    return [imask, omask]
+
+
+def exclusive_scan_quantified_wrapper(kvol: int, nbsizes: torch.Tensor, nbaddrs: torch.Tensor,
+                                      qnbaddrs: torch.Tensor, q: int = 128) -> None:
+    """others/exclusive_scan_cuda.cu:31-45 (writes nbaddrs / qnbaddrs in place)."""
+    nbsizes = _need(nbsizes, torch.int32, "nbsizes")
+    _check(_C.tsmi_exclusive_scan_quantified(_stream(), kvol, _ptr(nbsizes), q, _ptr(nbaddrs),
+                                             _ptr(qnbaddrs)))
+
+
+# -------------------------------------------------------------------- convolutions
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    try:
+        return _DTYPE_CODE[t.dtype]
+    except KeyError:
+        raise ValueError(f"unsupported feature dtype {t.dtype}") from None
+
+
+def pack_weights(kernel: torch.Tensor) -> torch.Tensor:
+    """[K_vol, Cin, Cout] -> the MFMA-friendly [K_vol, Cout_pad, Cin_pad] layout.
+    Cached on the tensor object and refreshed when its version counter moves."""
+    cached = getattr(kernel, "_tsmi_packed", None)
+    if cached is not None and cached[0] == kernel._version and cached[1] == kernel.data_ptr():
+        return cached[2]
+    w = kernel.detach()
+    if w.dim() == 2:
+        w = w.unsqueeze(0)
+    w = w.contiguous()
+    kvol, cin, cout = w.shape
+    packed = torch.empty(_C.tsmi_packed_weight_elems(kvol, cin, cout), dtype=w.dtype, device=w.device)
+    _check(_C.tsmi_pack_weights(_stream(), _ptr(w), _ptr(packed), kvol, cin, cout, _dtype_code(w)))
+    try:
+        kernel._tsmi_packed = (kernel._version, kernel.data_ptr(), packed)
+    except AttributeError:
+        pass
+    return packed
+
+
+def _conv_common(in_feats: torch.Tensor, kernel: torch.Tensor):
+    if not in_feats.is_cuda:
+        raise RuntimeError("sparse convolution needs GPU tensors; there is no CPU path")
+    if in_feats.dtype != kernel.dtype:
+        raise ValueError(f"feature dtype {in_feats.dtype} and kernel dtype {kernel.dtype} differ")
+    kshape = kernel.shape if kernel.dim() == 3 else (1,) + tuple(kernel.shape)
+    if in_feats.shape[1] != kshape[1]:
+        raise ValueError("Input feature size and kernel size mismatch")
+    x = in_feats if in_feats.is_contiguous() else in_feats.contiguous()
+    return x, pack_weights(kernel), kshape
+
+
+def conv_forward_implicit_gemm_cuda(in_feats, kernel, out_in_map, num_out_feats, num_out_channels,
+                                    allow_tf32=False, allow_fp16=True, bias=None) -> torch.Tensor:
+    """convolution/convolution_forward_implicit_gemm_cuda.cu:1527-1986.  allow_tf32 /
+    allow_fp16 are accepted and ignored: fp32 runs in true fp32, 16-bit types
+    accumulate in fp32."""
+    x, wp, (kvol, cin, cout) = _conv_common(in_feats, kernel)
+    if cout != num_out_channels:
+        raise ValueError("num_out_channels does not match the kernel")
+    y = torch.empty((num_out_feats, cout), dtype=x.dtype, device=x.device)
+    _check(_C.tsmi_conv_implicit_gemm(_stream(), _ptr(x), _ptr(wp), _ptr(out_in_map),
+                                      out_in_map.shape[0], num_out_feats, kvol, cin, cout,
+                                      _dtype_code(x), _ptr(bias), _ptr(y)))
+    return y
+
+
+def conv_forward_implicit_gemm_sorted_cuda(in_feats, kernel, reorder_out_in_map, reduced_mask,
+                                           reorder_loc, num_out_feats, num_out_channels,
+                                           allow_tf32=False, allow_fp16=True, bias=None) -> torch.Tensor:
+    """convolution/convolution_forward_implicit_gemm_sorted_cuda.cu:1755-2230."""
+    x, wp, (kvol, cin, cout) = _conv_common(in_feats, kernel)
+    split = reorder_loc.shape[0]
+    n_pad = reorder_out_in_map.shape[0]
+    y = torch.empty((num_out_feats, cout), dtype=x.dtype, device=x.device)
+    partial = None
+    if split > 1:
+        partial = torch.empty((split, num_out_feats, cout), dtype=torch.float32, device=x.device)
+    _check(_C.tsmi_conv_implicit_gemm_sorted(_stream(), _ptr(x), _ptr(wp), _ptr(reorder_out_in_map),
+                                             _ptr(reduced_mask), _ptr(reorder_loc), n_pad,
+                                             num_out_feats, kvol, split, cin, cout, _dtype_code(x),
+                                             _ptr(bias), _ptr(partial), _ptr(y)))
+    return y
+
+
+def conv_forward_fetch_on_demand_cuda(in_feats, kernel, nbmaps, sum_nnz, nbaddrs, qnbaddrs,
+                                      output_size, qsum_nnz, transpose, allow_tf32=False,
+                                      allow_fp16=True, row_mask=None, center_k=-1, bias=None) -> torch.Tensor:
+    """convolution/convolution_forward_fetch_on_demand_cuda.cu:1981-2119.  nbmaps is the
+    planar [2, nnz] list; row_mask is the kmap's output_mask (input_mask when
+    transposed) that makes the reduction atomic free."""
+    x, wp, (kvol, cin, cout) = _conv_common(in_feats, kernel)
+    if row_mask is None:
+        raise ValueError("fetch-on-demand needs the kmap's row mask (output_mask / input_mask)")
+    y = torch.empty((output_size, cout), dtype=x.dtype, device=x.device)
+    partial = torch.empty((max(int(sum_nnz), 1), cout), dtype=x.dtype, device=x.device)
+    _check(_C.tsmi_conv_fetch_on_demand(_stream(), _ptr(x), _ptr(wp), _ptr(nbmaps), int(sum_nnz),
+                                        _ptr(nbaddrs), _ptr(qnbaddrs), int(qsum_nnz), _ptr(row_mask),
+                                        output_size, kvol, cin, cout, _dtype_code(x),
+                                        int(bool(transpose)), center_k, _ptr(bias), _ptr(partial),
+                                        _ptr(y)))
+    return y
+
+
+def conv_forward_gather_scatter_cuda(in_feats, kernel, nbmaps, nbsizes, input_mask, output_mask,
+                                     output_size, epsilon=0.0, mm_thresh=0, conv_mode=0,
+                                     transpose=False, buffer=None, nbaddrs=None, qnbaddrs=None,
+                                     qsum_nnz=None, center_k=-1, bias=None) -> torch.Tensor:
+    """convolution/convolution_gather_scatter_cuda.cu:279-814: gather -> GEMM per
+    offset -> scatter, here always as three launches over all offsets.  epsilon,
+    mm_thresh and conv_mode only steer grouping in the reference; results do not
+    depend on them and they are accepted and ignored.  nbmaps is the interleaved
+    int32 [nnz, 2] list."""
+    x, wp, (kvol, cin, cout) = _conv_common(in_feats, kernel)
+    nbmaps = _need(nbmaps, torch.int32, "nbmaps")
+    nnz = nbmaps.shape[0]
+    dev = x.device
+    if nbaddrs is None or qnbaddrs is None:
+        sizes = nbsizes.to(device=dev, dtype=torch.int32)
+        nbaddrs = torch.zeros(kvol + 1, dtype=torch.int32, device=dev)
+        qnbaddrs = torch.zeros(kvol + 1, dtype=torch.int32, device=dev)
+        exclusive_scan_quantified_wrapper(kvol, sizes, nbaddrs, qnbaddrs)
+        qsum_nnz = None
+    if qsum_nnz is None:
+        qsum_nnz = int(qnbaddrs[-1].item())
+    row_mask = input_mask if transpose else output_mask
+    code = _dtype_code(x)
+    gathered = torch.empty((max(nnz, 1), cin), dtype=x.dtype, device=dev)
+    products = torch.empty((max(nnz, 1), cout), dtype=x.dtype, device=dev)
+    y = torch.empty((output_size, cout), dtype=x.dtype, device=dev)
+    s = _stream()
+    _check(_C.tsmi_gs_gather(s, _ptr(x), _ptr(nbmaps), nnz, cin, code, int(bool(transpose)),
+                             _ptr(gathered)))
+    _check(_C.tsmi_gs_gemm(s, _ptr(gathered), _ptr(wp), _ptr(nbaddrs), _ptr(qnbaddrs), nnz,
+                           int(qsum_nnz), kvol, cin, cout, code, _ptr(products)))
+    _check(_C.tsmi_gs_scatter(s, _ptr(products), _ptr(nbaddrs), _ptr(row_mask), output_size, kvol,
+                              cout, code, center_k, _ptr(bias), _ptr(y)))
+    return y

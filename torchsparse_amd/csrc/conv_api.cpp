@@ -1,0 +1,148 @@
+// C entry points of the convolution dataflows: argument checks and dispatch on
+// the element type.  The kernels live in conv_igemm.inc.
+#include "conv_ops.h"
+
+using namespace tsmi;
+
+namespace {
+
+const ConvOps *ops_for(int dtype) {
+  switch (dtype) {
+    case TSMI_F32: return &conv_ops_f32();
+    case TSMI_F16: return &conv_ops_f16();
+    case TSMI_BF16: return &conv_ops_bf16();
+    default: return nullptr;
+  }
+}
+
+int check_shapes(const char *who, const ConvOps *ops, int kvol, int cin, int cout) {
+  if (!ops) return fail(TSMI_ERR_INVALID_ARGUMENT, "%s: unsupported dtype", who);
+  TSMI_REQUIRE(kvol >= 1 && cin >= 1 && cout >= 1, "%s: bad kernel shape [%d,%d,%d]", who, kvol,
+               cin, cout);
+  return TSMI_OK;
+}
+
+bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
+
+}  // namespace
+
+extern "C" int64_t tsmi_packed_weight_elems(int kvol, int cin, int cout) {
+  if (kvol < 1 || cin < 1 || cout < 1) return -1;
+  // sized for the coarsest reduction step (32 elements) so one size fits every dtype
+  return (int64_t)kvol * pad_to(cout, 16) * pad_to(cin, 32);
+}
+
+extern "C" int tsmi_pack_weights(tsmi_stream_t s, const void *w, void *w_packed, int kvol, int cin,
+                                 int cout, int dtype) {
+  const ConvOps *ops = ops_for(dtype);
+  if (int e = check_shapes("pack_weights", ops, kvol, cin, cout)) return e;
+  TSMI_REQUIRE(w && w_packed, "pack_weights: null pointer");
+  return ops->pack((hipStream_t)s, w, w_packed, kvol, cin, cout);
+}
+
+extern "C" int tsmi_conv_implicit_gemm(tsmi_stream_t s, const void *x, const void *w_packed,
+                                       const int32_t *map, int64_t n_map_rows, int64_t n_out,
+                                       int kvol, int cin, int cout, int dtype, const void *bias,
+                                       void *y) {
+  const ConvOps *ops = ops_for(dtype);
+  if (int e = check_shapes("conv_implicit_gemm", ops, kvol, cin, cout)) return e;
+  TSMI_REQUIRE(n_out >= 0 && n_map_rows >= n_out, "conv_implicit_gemm: map has %lld rows, need %lld",
+               (long long)n_map_rows, (long long)n_out);
+  if (n_out == 0) return TSMI_OK;
+  TSMI_REQUIRE(x && w_packed && map && y, "conv_implicit_gemm: null pointer");
+  TSMI_REQUIRE(aligned16(x) && aligned16(w_packed) && aligned16(y),
+               "conv_implicit_gemm: x, w_packed and y must be 16-byte aligned");
+  return ops->igemm((hipStream_t)s, x, w_packed, map, n_map_rows, n_out, n_out, kvol, cin, cout,
+                    bias, y, nullptr, 0, 1, nullptr);
+}
+
+extern "C" int tsmi_conv_implicit_gemm_sorted(tsmi_stream_t s, const void *x, const void *w_packed,
+                                              const int32_t *reorder_map,
+                                              const int32_t *reduced_mask,
+                                              const int32_t *reorder_loc, int64_t n_pad,
+                                              int64_t n_out, int kvol, int split, int cin, int cout,
+                                              int dtype, const void *bias, float *partial, void *y) {
+  (void)reduced_mask;  // tile skipping is derived from the staged map itself
+  const ConvOps *ops = ops_for(dtype);
+  if (int e = check_shapes("conv_implicit_gemm_sorted", ops, kvol, cin, cout)) return e;
+  TSMI_REQUIRE(split >= 1 && split <= kvol, "conv_implicit_gemm_sorted: bad split %d", split);
+  TSMI_REQUIRE((int64_t)(split - 1) * ((kvol + split - 1) / split) < kvol,
+               "conv_implicit_gemm_sorted: split_mask_num %d leaves an empty split", split);
+  TSMI_REQUIRE(n_out >= 0 && n_pad >= n_out, "conv_implicit_gemm_sorted: n_pad < n_out");
+  if (n_out == 0) return TSMI_OK;
+  TSMI_REQUIRE(x && w_packed && reorder_map && reorder_loc && y,
+               "conv_implicit_gemm_sorted: null pointer");
+  TSMI_REQUIRE(split == 1 || partial, "conv_implicit_gemm_sorted: split > 1 needs `partial`");
+  TSMI_REQUIRE(aligned16(x) && aligned16(w_packed) && aligned16(y),
+               "conv_implicit_gemm_sorted: x, w_packed and y must be 16-byte aligned");
+  if (int e = ops->igemm((hipStream_t)s, x, w_packed, reorder_map, n_pad, n_pad, n_out, kvol, cin,
+                         cout, split == 1 ? bias : nullptr, y, reorder_loc, n_pad, split, partial))
+    return e;
+  if (split > 1) return ops->sum_partials((hipStream_t)s, partial, split, n_out, cout, bias, y);
+  return TSMI_OK;
+}
+
+extern "C" int tsmi_conv_fetch_on_demand(tsmi_stream_t s, const void *x, const void *w_packed,
+                                         const int32_t *nbmaps_planar, int64_t nnz,
+                                         const int32_t *nbaddrs, const int32_t *qnbaddrs,
+                                         int64_t qnnz, const int32_t *row_mask, int64_t n_out,
+                                         int kvol, int cin, int cout, int dtype, int transpose,
+                                         int center_k, const void *bias, void *partial, void *y) {
+  const ConvOps *ops = ops_for(dtype);
+  if (int e = check_shapes("conv_fetch_on_demand", ops, kvol, cin, cout)) return e;
+  TSMI_REQUIRE(nnz >= 0 && qnnz >= nnz && qnnz % 128 == 0 && n_out >= 0,
+               "conv_fetch_on_demand: bad sizes (nnz %lld, qnnz %lld)", (long long)nnz,
+               (long long)qnnz);
+  TSMI_REQUIRE(center_k >= -1 && center_k < kvol, "conv_fetch_on_demand: bad center_k");
+  if (n_out == 0) return TSMI_OK;
+  TSMI_REQUIRE(x && w_packed && nbaddrs && qnbaddrs && row_mask && y,
+               "conv_fetch_on_demand: null pointer");
+  TSMI_REQUIRE(nnz == 0 || (nbmaps_planar && partial), "conv_fetch_on_demand: null pair list");
+  TSMI_REQUIRE(aligned16(x) && aligned16(w_packed) && aligned16(partial),
+               "conv_fetch_on_demand: x, w_packed and partial must be 16-byte aligned");
+  const int32_t *rows = transpose ? nbmaps_planar + nnz : nbmaps_planar;
+  if (nnz > 0)
+    if (int e = ops->pairs((hipStream_t)s, x, w_packed, rows, nbaddrs, qnbaddrs, qnnz, kvol, cin,
+                           cout, partial))
+      return e;
+  return ops->scatter((hipStream_t)s, partial, nbaddrs, row_mask, n_out, kvol, cout, center_k, bias,
+                      y);
+}
+
+extern "C" int tsmi_gs_gather(tsmi_stream_t s, const void *x, const int32_t *nbmaps_inter,
+                              int64_t nnz, int cin, int dtype, int transpose, void *buffer) {
+  const ConvOps *ops = ops_for(dtype);
+  if (!ops) return fail(TSMI_ERR_INVALID_ARGUMENT, "gs_gather: unsupported dtype");
+  TSMI_REQUIRE(nnz >= 0 && cin >= 1, "gs_gather: bad sizes");
+  if (nnz == 0) return TSMI_OK;
+  TSMI_REQUIRE(x && nbmaps_inter && buffer, "gs_gather: null pointer");
+  return ops->gather((hipStream_t)s, x, nbmaps_inter, nnz, cin, transpose ? 1 : 0, buffer);
+}
+
+extern "C" int tsmi_gs_gemm(tsmi_stream_t s, const void *buffer, const void *w_packed,
+                            const int32_t *nbaddrs, const int32_t *qnbaddrs, int64_t nnz,
+                            int64_t qnnz, int kvol, int cin, int cout, int dtype,
+                            void *out_buffer) {
+  const ConvOps *ops = ops_for(dtype);
+  if (int e = check_shapes("gs_gemm", ops, kvol, cin, cout)) return e;
+  TSMI_REQUIRE(nnz >= 0 && qnnz >= nnz && qnnz % 128 == 0, "gs_gemm: bad sizes");
+  if (nnz == 0) return TSMI_OK;
+  TSMI_REQUIRE(buffer && w_packed && nbaddrs && qnbaddrs && out_buffer, "gs_gemm: null pointer");
+  TSMI_REQUIRE(aligned16(buffer) && aligned16(w_packed) && aligned16(out_buffer),
+               "gs_gemm: buffers must be 16-byte aligned");
+  return ops->pairs((hipStream_t)s, buffer, w_packed, nullptr, nbaddrs, qnbaddrs, qnnz, kvol, cin,
+                    cout, out_buffer);
+}
+
+extern "C" int tsmi_gs_scatter(tsmi_stream_t s, const void *out_buffer, const int32_t *nbaddrs,
+                               const int32_t *row_mask, int64_t n_out, int kvol, int cout,
+                               int dtype, int center_k, const void *bias, void *y) {
+  const ConvOps *ops = ops_for(dtype);
+  if (!ops) return fail(TSMI_ERR_INVALID_ARGUMENT, "gs_scatter: unsupported dtype");
+  TSMI_REQUIRE(n_out >= 0 && kvol >= 1 && cout >= 1 && center_k >= -1 && center_k < kvol,
+               "gs_scatter: bad sizes");
+  if (n_out == 0) return TSMI_OK;
+  TSMI_REQUIRE(out_buffer && nbaddrs && row_mask && y, "gs_scatter: null pointer");
+  return ops->scatter((hipStream_t)s, out_buffer, nbaddrs, row_mask, n_out, kvol, cout, center_k,
+                      bias, y);
+}

@@ -1,0 +1,36 @@
+// Per-element-type operation table of the convolution kernels.  Each element
+// type is compiled in its own translation unit (conv_igemm_{f16,bf16,f32}.hip)
+// and exposes one of these tables; conv_api.cpp dispatches on the dtype code.
+#pragma once
+
+#include "common.h"
+
+namespace tsmi {
+
+struct ConvOps {
+  int step;  // reduction elements per MFMA step (Cin is padded to a multiple)
+  int (*pack)(hipStream_t s, const void *w, void *wp, int kvol, int cin, int cout);
+  // row_out == nullptr: plain implicit GEMM over `map`; otherwise sorted mode.
+  int (*igemm)(hipStream_t s, const void *x, const void *wp, const int32_t *map,
+               int64_t n_map_rows, int64_t n_tile_rows, int64_t n_out, int kvol, int cin, int cout,
+               const void *bias, void *y, const int32_t *row_out, int64_t row_out_stride,
+               int split, float *partial);
+  // out[nbaddrs[k] + p, :] = X[rows[nbaddrs[k] + p], :] W[k] over 128-padded pair lists
+  int (*pairs)(hipStream_t s, const void *x, const void *wp, const int32_t *rows,
+               const int32_t *nbaddrs, const int32_t *qnbaddrs, int64_t qnnz, int kvol, int cin,
+               int cout, void *out);
+  int (*sum_partials)(hipStream_t s, const float *partial, int split, int64_t n_out, int cout,
+                      const void *bias, void *y);
+  int (*scatter)(hipStream_t s, const void *pbuf, const int32_t *nbaddrs, const int32_t *mask,
+                 int64_t n_out, int kvol, int cout, int center_k, const void *bias, void *y);
+  int (*gather)(hipStream_t s, const void *x, const int32_t *pairs, int64_t nnz, int cin, int col,
+                void *buffer);
+};
+
+const ConvOps &conv_ops_f16();
+const ConvOps &conv_ops_bf16();
+const ConvOps &conv_ops_f32();
+
+inline int pad_to(int v, int m) { return (v + m - 1) / m * m; }
+
+}  // namespace tsmi

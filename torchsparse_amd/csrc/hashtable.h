@@ -1,0 +1,89 @@
+// Open-addressing hash table over two caller-owned arrays (keys int64, vals int32).
+//
+// Slot layout: groups of 4 consecutive slots.  The group is chosen by a mixed
+// hash of (key >> 2) and the slot inside the group by the low two key bits, so
+// the packed coordinates z-1, z, z+1 of one column land in the same or the next
+// 32-byte key segment and a 3-wide neighbourhood touches 9 cache lines instead
+// of 27.  Collisions resolve by linear probing over the whole table.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace tsmi {
+
+constexpr int kCoordBits = 18;            // x, y, z each in [0, 2^18)
+constexpr int kCoordLimit = 1 << kCoordBits;
+constexpr int kBatchLimit = 512;          // keeps key + 1 positive in int64
+
+struct TableView {
+  unsigned long long *keys;  // 0 = empty, otherwise key + 1
+  int32_t *vals;             // row index + 1
+  uint32_t cap;              // multiple of 8
+  uint32_t groups;           // cap / 4
+};
+
+__device__ __forceinline__ bool coords_packable(int b, int x, int y, int z) {
+  return (unsigned)x < (unsigned)kCoordLimit && (unsigned)y < (unsigned)kCoordLimit &&
+         (unsigned)z < (unsigned)kCoordLimit && (unsigned)b < (unsigned)kBatchLimit;
+}
+
+__device__ __forceinline__ unsigned long long pack_coords(int b, int x, int y, int z) {
+  return ((unsigned long long)(unsigned)b << (3 * kCoordBits)) |
+         ((unsigned long long)(unsigned)x << (2 * kCoordBits)) |
+         ((unsigned long long)(unsigned)y << kCoordBits) | (unsigned long long)(unsigned)z;
+}
+
+__device__ __forceinline__ void unpack_coords(unsigned long long key, int *c) {
+  const unsigned mask = kCoordLimit - 1;
+  c[3] = (int)(key & mask);
+  c[2] = (int)((key >> kCoordBits) & mask);
+  c[1] = (int)((key >> (2 * kCoordBits)) & mask);
+  c[0] = (int)(key >> (3 * kCoordBits));
+}
+
+__device__ __forceinline__ uint32_t home_slot(const TableView &t, unsigned long long key) {
+  unsigned long long h = key >> 2;
+  h ^= h >> 33;
+  h *= 0xff51afd7ed558ccdULL;
+  h ^= h >> 33;
+  uint32_t g = (uint32_t)(((h >> 32) * (unsigned long long)t.groups) >> 32);
+  return (g << 2) | (uint32_t)(key & 3);
+}
+
+// Returns the slot holding `key` (inserting it if absent) or 0xFFFFFFFF when the
+// table is full.  *fresh tells whether this call created the entry.
+__device__ __forceinline__ uint32_t table_insert(const TableView &t, unsigned long long key,
+                                                 bool *fresh) {
+  const unsigned long long stored = key + 1;
+  uint32_t slot = home_slot(t, key);
+  for (uint32_t probe = 0; probe < t.cap; ++probe) {
+    unsigned long long prev = atomicCAS(&t.keys[slot], 0ULL, stored);
+    if (prev == 0ULL) {
+      *fresh = true;
+      return slot;
+    }
+    if (prev == stored) {
+      *fresh = false;
+      return slot;
+    }
+    slot = slot + 1 == t.cap ? 0 : slot + 1;
+  }
+  *fresh = false;
+  return 0xFFFFFFFFu;
+}
+
+// Returns the slot holding `key` or 0xFFFFFFFF when absent.
+__device__ __forceinline__ uint32_t table_find(const TableView &t, unsigned long long key) {
+  const unsigned long long stored = key + 1;
+  uint32_t slot = home_slot(t, key);
+  for (uint32_t probe = 0; probe < t.cap; ++probe) {
+    unsigned long long cur = t.keys[slot];
+    if (cur == stored) return slot;
+    if (cur == 0ULL) return 0xFFFFFFFFu;
+    slot = slot + 1 == t.cap ? 0 : slot + 1;
+  }
+  return 0xFFFFFFFFu;
+}
+
+}  // namespace tsmi

@@ -1,0 +1,678 @@
+// Integer kernels of kernel-map construction for gfx950 and their C entry points.
+//
+// All kernels are HBM/L2-bound index work: one thread per produced element,
+// 256-thread blocks, coalesced stores; the only random accesses are hash-table
+// probes (see hashtable.h for how neighbouring coordinates share cache lines).
+#include "common.h"
+#include "hashtable.h"
+
+namespace tsmi {
+namespace {
+
+constexpr int kBlock = 256;
+
+struct Geom {
+  int ks[3];
+  int stride[3];
+  int pad[3];
+  int kvol;
+  int odd;
+};
+
+__device__ __forceinline__ void decode_digits(int k, const Geom &g, int *d) {
+  if (g.odd) {  // x is the fastest digit
+    d[0] = k % g.ks[0];
+    k /= g.ks[0];
+    d[1] = k % g.ks[1];
+    d[2] = k / g.ks[1];
+  } else {  // z is the fastest digit
+    d[2] = k % g.ks[2];
+    k /= g.ks[2];
+    d[1] = k % g.ks[1];
+    d[0] = k / g.ks[1];
+  }
+}
+
+template <typename T>
+__global__ void fill_kernel(T *p, int64_t n, T v) {
+  int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+__global__ void table_clear_kernel(unsigned long long *keys, int32_t *vals, int64_t cap) {
+  int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i < cap) {
+    keys[i] = 0ULL;
+    vals[i] = 0;
+  }
+}
+
+__global__ void insert_coords_kernel(TableView t, const int4 *coords, int64_t n, int32_t *status) {
+  int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i >= n) return;
+  int4 c = coords[i];  // (b, x, y, z)
+  if (!coords_packable(c.x, c.y, c.z, c.w)) return;
+  bool fresh;
+  uint32_t slot = table_insert(t, pack_coords(c.x, c.y, c.z, c.w), &fresh);
+  if (slot == 0xFFFFFFFFu) {
+    if (status) *status = 1;
+    return;
+  }
+  t.vals[slot] = (int32_t)(i + 1);
+}
+
+__global__ void insert_keys_kernel(TableView t, const long long *user_keys, int64_t n,
+                                   int32_t *status) {
+  int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i >= n) return;
+  bool fresh;
+  uint32_t slot = table_insert(t, (unsigned long long)user_keys[i], &fresh);
+  if (slot == 0xFFFFFFFFu) {
+    if (status) *status = 1;
+    return;
+  }
+  t.vals[slot] = (int32_t)(i + 1);
+}
+
+__global__ void lookup_keys_kernel(TableView t, const long long *user_keys, int64_t n,
+                                   int32_t *out) {
+  int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i >= n) return;
+  uint32_t slot = table_find(t, (unsigned long long)user_keys[i]);
+  out[i] = slot == 0xFFFFFFFFu ? 0 : t.vals[slot];
+}
+
+// One thread per (output row, kernel offset); a wave's 64 stores are contiguous.
+__global__ void kmap_query_kernel(TableView t, const int4 *out_coords, int64_t n_out,
+                                  int64_t total, Geom g, int32_t *map) {
+  int64_t tid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (tid >= total) return;
+  int64_t row = tid / g.kvol;
+  int k = (int)(tid - row * g.kvol);
+  int32_t result = -1;
+  if (row < n_out) {
+    int4 c = out_coords[row];
+    int d[3];
+    decode_digits(k, g, d);
+    int x = c.y * g.stride[0] - g.pad[0] + d[0];
+    int y = c.z * g.stride[1] - g.pad[1] + d[1];
+    int z = c.w * g.stride[2] - g.pad[2] + d[2];
+    if (coords_packable(c.x, x, y, z)) {
+      uint32_t slot = table_find(t, pack_coords(c.x, x, y, z));
+      if (slot != 0xFFFFFFFFu) result = t.vals[slot] - 1;
+    }
+  }
+  map[tid] = result;
+}
+
+__global__ void coords_max_kernel(const int4 *coords, int64_t n, int32_t *out_max) {
+  int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  int4 c = i < n ? coords[i] : make_int4(0, 0, 0, 0);
+  int v[4] = {c.x, c.y, c.z, c.w};
+#pragma unroll
+  for (int a = 0; a < 4; ++a) {
+    int m = v[a];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) m = max(m, __shfl_xor(m, off));
+    if ((threadIdx.x & 63) == 0 && m > 0) atomicMax(&out_max[a], m);
+  }
+}
+
+// mode 0: thread per (input, offset); mode 1: thread per input.
+__global__ void downsample_candidates_kernel(const int4 *in_coords, int64_t n_in, int64_t total,
+                                             Geom g, int3 out_max_host, const int32_t *in_max_dev,
+                                             int mode, TableView t, unsigned long long *uniq,
+                                             int64_t uniq_cap, int32_t *counters) {
+  int64_t tid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (tid >= total) return;
+  int b, x, y, z;
+  if (mode == 1) {
+    int4 c = in_coords[tid];
+    b = c.x;
+    // floor division (coordinates may not be negative here, but keep it exact)
+    int v[3] = {c.y, c.z, c.w};
+    int o[3];
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+      int q = v[a] / g.stride[a];
+      if (v[a] % g.stride[a] != 0 && v[a] < 0) --q;
+      o[a] = q;
+    }
+    x = o[0];
+    y = o[1];
+    z = o[2];
+  } else {
+    int64_t i = tid / g.kvol;
+    int k = (int)(tid - i * g.kvol);
+    int4 c = in_coords[i];
+    b = c.x;
+    int d[3];
+    decode_digits(k, g, d);
+    int v[3] = {c.y, c.z, c.w};
+    int o[3];
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+      int num = v[a] + g.pad[a] + d[a] - (g.ks[a] - 1);
+      if (num % g.stride[a] != 0) return;
+      o[a] = num / g.stride[a];
+      int hi = in_max_dev
+                   ? (in_max_dev[1 + a] + 2 * g.pad[a] - (g.ks[a] - 1)) / g.stride[a]
+                   : (a == 0 ? out_max_host.x : (a == 1 ? out_max_host.y : out_max_host.z));
+      if (o[a] < 0 || o[a] > hi) return;
+    }
+    x = o[0];
+    y = o[1];
+    z = o[2];
+  }
+  if (!coords_packable(b, x, y, z)) return;
+  unsigned long long key = pack_coords(b, x, y, z);
+  bool fresh;
+  uint32_t slot = table_insert(t, key, &fresh);
+  if (slot == 0xFFFFFFFFu) {
+    counters[1] = 1;
+    return;
+  }
+  if (fresh) {
+    int pos = atomicAdd(&counters[0], 1);
+    if (pos < uniq_cap)
+      uniq[pos] = key;
+    else
+      counters[1] = 1;
+  }
+}
+
+__global__ void downsample_finalize_kernel(const unsigned long long *sorted, int64_t n_out,
+                                           TableView t, int4 *out_coords) {
+  int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (r >= n_out) return;
+  unsigned long long key = sorted[r];
+  int c[4];
+  unpack_coords(key, c);
+  out_coords[r] = make_int4(c[0], c[1], c[2], c[3]);
+  uint32_t slot = table_find(t, key);
+  if (slot != 0xFFFFFFFFu) t.vals[slot] = (int32_t)(r + 1);
+}
+
+__global__ void transpose_map_kernel(const int32_t *map, int64_t total, int kvol, int32_t *map_t,
+                                     int64_t n_rows_t) {
+  int64_t tid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (tid >= total) return;
+  int32_t in = map[tid];
+  if (in < 0 || in >= n_rows_t) return;
+  int64_t out = tid / kvol;
+  int k = (int)(tid - out * kvol);
+  map_t[(int64_t)in * kvol + k] = (int32_t)out;
+}
+
+__global__ void derive_bitmask_kernel(const int32_t *map, int64_t n_pad, int kvol, int split,
+                                      int len, int64_t valid_n, int32_t *bitmask) {
+  int64_t tid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (tid >= n_pad * split) return;
+  int s = (int)(tid / n_pad);
+  int64_t r = tid - (int64_t)s * n_pad;
+  int32_t result = -1;
+  if (r < valid_n) {
+    int begin = s * len;
+    int l = min(len, kvol - begin);
+    uint32_t m = 0;
+    const int32_t *row = map + r * kvol + begin;
+    for (int i = 0; i < l; ++i) m |= (uint32_t)(row[i] >= 0) << i;
+    result = (int32_t)m;
+  }
+  bitmask[tid] = result;
+}
+
+__global__ void reorder_map_kernel(const int32_t *map, const int32_t *loc, int64_t n_pad, int kvol,
+                                   int len, int32_t *out) {
+  int64_t tid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (tid >= n_pad * kvol) return;
+  int64_t r = tid / kvol;
+  int c = (int)(tid - r * kvol);
+  int32_t src = loc[(int64_t)(c / len) * n_pad + r];
+  out[tid] = map[(int64_t)src * kvol + c];
+}
+
+__global__ void reduce_bitmask_kernel(const int32_t *mask, int split, int64_t n_pad, int tile,
+                                      int64_t rows, int32_t *reduced) {
+  int64_t tid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (tid >= rows * split) return;
+  int s = (int)(tid / rows);
+  int64_t t = tid - (int64_t)s * rows;
+  const int32_t *p = mask + (int64_t)s * n_pad;
+  int64_t end = min((t + 1) * (int64_t)tile, n_pad);
+  int32_t acc = 0;
+  for (int64_t r = t * tile; r < end; ++r) acc |= p[r];
+  reduced[tid] = acc;
+}
+
+// ---- pair lists: per-block counts, in-place scan, ordered fill ---------------
+
+__global__ void pair_count_kernel(const int32_t *map, int64_t n_rows, int kvol, int64_t nblk,
+                                  int32_t *block_counts) {
+  __shared__ int wave_cnt[kBlock / 64];
+  int64_t row = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  for (int k = 0; k < kvol; ++k) {
+    bool valid = row < n_rows && map[row * kvol + k] != -1;
+    unsigned long long b = __ballot(valid);
+    if (lane == 0) wave_cnt[wave] = __popcll(b);
+    __syncthreads();
+    if (threadIdx.x == 0)
+      block_counts[(int64_t)k * nblk + blockIdx.x] =
+          wave_cnt[0] + wave_cnt[1] + wave_cnt[2] + wave_cnt[3];
+    __syncthreads();
+  }
+}
+
+// Single block: exclusive scan of `n` counts in place; nbsizes[k] from the scan.
+__global__ void pair_scan_kernel(int32_t *counts, int64_t n, int kvol, int64_t nblk,
+                                 int32_t *nbsizes) {
+  __shared__ int part[1024];
+  __shared__ int total_s;
+  const int t = threadIdx.x;
+  int64_t chunk = (n + 1023) / 1024;
+  int64_t begin = min((int64_t)t * chunk, n), end = min(begin + chunk, n);
+  int sum = 0;
+  for (int64_t i = begin; i < end; ++i) sum += counts[i];
+  part[t] = sum;
+  __syncthreads();
+  // Hillis-Steele inclusive scan over 1024 partial sums
+  for (int off = 1; off < 1024; off <<= 1) {
+    int v = t >= off ? part[t - off] : 0;
+    __syncthreads();
+    part[t] += v;
+    __syncthreads();
+  }
+  int run = part[t] - sum;
+  if (t == 1023) total_s = part[t];
+  for (int64_t i = begin; i < end; ++i) {
+    int c = counts[i];
+    counts[i] = run;
+    run += c;
+  }
+  __syncthreads();
+  for (int k = t; k < kvol; k += 1024) {
+    int start = counts[(int64_t)k * nblk];
+    int stop = k + 1 < kvol ? counts[(int64_t)(k + 1) * nblk] : total_s;
+    nbsizes[k] = stop - start;
+  }
+}
+
+__global__ void pair_fill_kernel(const int32_t *map, int64_t n_rows, int kvol, int64_t nblk,
+                                 const int32_t *offsets, int64_t nnz, int32_t *inter,
+                                 int32_t *planar, int64_t n_in, int64_t n_out, int32_t *input_mask,
+                                 int32_t *output_mask, int skip_k) {
+  __shared__ int wave_cnt[kBlock / 64];
+  int64_t row = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  for (int k = 0; k < kvol; ++k) {
+    int32_t in = row < n_rows ? map[row * kvol + k] : -1;
+    bool valid = in != -1;
+    unsigned long long b = __ballot(valid);
+    if (lane == 0) wave_cnt[wave] = __popcll(b);
+    __syncthreads();
+    int before = 0;
+    for (int w = 0; w < wave; ++w) before += wave_cnt[w];
+    if (valid) {
+      int rank = before + __popcll(b & ((1ULL << lane) - 1ULL));
+      int64_t pos = (int64_t)offsets[(int64_t)k * nblk + blockIdx.x] + rank;
+      if (pos < nnz) {
+        if (inter) {
+          inter[2 * pos] = in;
+          inter[2 * pos + 1] = (int32_t)row;
+        }
+        if (planar) {
+          planar[pos] = in;
+          planar[nnz + pos] = (int32_t)row;
+        }
+        if (k != skip_k) {
+          int32_t p = (int32_t)(pos - offsets[(int64_t)k * nblk]);
+          if (input_mask && in >= 0 && in < n_in) input_mask[(int64_t)k * n_in + in] = p;
+          if (output_mask && row < n_out) output_mask[(int64_t)k * n_out + row] = p;
+        }
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// One thread per pair: offset by binary search over the exclusive scan, position
+// inside the offset's list by subtraction.
+__global__ void masks_from_pairs_kernel(const int32_t *pairs, int64_t nnz, const int32_t *nbaddrs,
+                                        int kvol, int64_t n_in, int64_t n_out, int skip_k,
+                                        int32_t *input_mask, int32_t *output_mask) {
+  int64_t p = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (p >= nnz) return;
+  int lo = 0, hi = kvol;  // largest k with nbaddrs[k] <= p
+  while (hi - lo > 1) {
+    int mid = (lo + hi) >> 1;
+    if ((int64_t)nbaddrs[mid] <= p) lo = mid; else hi = mid;
+  }
+  if (lo == skip_k) return;
+  int32_t pos = (int32_t)(p - nbaddrs[lo]);
+  int32_t in = pairs[2 * p], out = pairs[2 * p + 1];
+  if (in >= 0 && in < n_in) input_mask[(int64_t)lo * n_in + in] = pos;
+  if (out >= 0 && out < n_out) output_mask[(int64_t)lo * n_out + out] = pos;
+}
+
+__global__ void scan_quantified_kernel(int kvol, const int32_t *nbsizes, int q, int32_t *nbaddrs,
+                                       int32_t *qnbaddrs) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  int acc = 0, qacc = 0;
+  nbaddrs[0] = 0;
+  qnbaddrs[0] = 0;
+  for (int k = 0; k < kvol; ++k) {
+    acc += nbsizes[k];
+    qacc += (nbsizes[k] + q - 1) / q * q;
+    nbaddrs[k + 1] = acc;
+    qnbaddrs[k + 1] = qacc;
+  }
+}
+
+int make_table(TableView *t, const int64_t *keys, const int32_t *vals, int64_t cap) {
+  TSMI_REQUIRE(keys != nullptr && vals != nullptr, "hash table: null keys/vals");
+  TSMI_REQUIRE(cap >= 8 && cap % 8 == 0 && cap < (int64_t(1) << 31),
+               "hash table: capacity %lld must be a multiple of 8 in [8, 2^31)", (long long)cap);
+  t->keys = (unsigned long long *)keys;
+  t->vals = (int32_t *)vals;
+  t->cap = (uint32_t)cap;
+  t->groups = (uint32_t)(cap / 4);
+  return TSMI_OK;
+}
+
+int make_geom(Geom *g, const int32_t ks[3], const int32_t stride[3], const int32_t pad[3]) {
+  TSMI_REQUIRE(ks && stride && pad, "kernel geometry: null pointer");
+  int64_t kvol = 1;
+  for (int a = 0; a < 3; ++a) {
+    TSMI_REQUIRE(ks[a] >= 1 && stride[a] >= 1, "kernel geometry: kernel size and stride must be >= 1");
+    g->ks[a] = ks[a];
+    g->stride[a] = stride[a];
+    g->pad[a] = pad[a];
+    kvol *= ks[a];
+  }
+  TSMI_REQUIRE(kvol <= 4096, "kernel volume %lld too large", (long long)kvol);
+  g->kvol = (int)kvol;
+  g->odd = kvol % 2 == 1;
+  return TSMI_OK;
+}
+
+inline dim3 grid_for(int64_t n) { return dim3((unsigned)ceil_div(n > 0 ? n : 1, kBlock)); }
+
+}  // namespace
+}  // namespace tsmi
+
+using namespace tsmi;
+
+#define TSMI_GRID_CHECK(n) \
+  TSMI_REQUIRE(grid_fits(ceil_div((n), kBlock)), "problem too large for one launch (%lld elements)", (long long)(n))
+
+extern "C" int tsmi_hashtable_clear(tsmi_stream_t s, int64_t *keys, int32_t *vals, int64_t cap) {
+  TableView t;
+  if (int e = make_table(&t, keys, vals, cap)) return e;
+  hipLaunchKernelGGL(table_clear_kernel, grid_for(cap), dim3(kBlock), 0, (hipStream_t)s, t.keys,
+                     t.vals, cap);
+  return check_launch("tsmi_hashtable_clear");
+}
+
+extern "C" int tsmi_hashtable_insert_coords(tsmi_stream_t s, int64_t *keys, int32_t *vals,
+                                            int64_t cap, const int32_t *coords, int64_t n,
+                                            int32_t *status) {
+  TableView t;
+  if (int e = make_table(&t, keys, vals, cap)) return e;
+  TSMI_REQUIRE(n >= 0 && (n == 0 || coords), "insert_coords: bad coords");
+  TSMI_REQUIRE(n <= cap, "The capacity of hashtable is not sufficient (%lld keys, capacity %lld)",
+               (long long)n, (long long)cap);
+  if (n == 0) return TSMI_OK;
+  TSMI_GRID_CHECK(n);
+  hipLaunchKernelGGL(insert_coords_kernel, grid_for(n), dim3(kBlock), 0, (hipStream_t)s, t,
+                     (const int4 *)coords, n, status);
+  return check_launch("tsmi_hashtable_insert_coords");
+}
+
+extern "C" int tsmi_hashtable_insert_keys(tsmi_stream_t s, int64_t *keys, int32_t *vals,
+                                          int64_t cap, const int64_t *user_keys, int64_t n,
+                                          int32_t *status) {
+  TableView t;
+  if (int e = make_table(&t, keys, vals, cap)) return e;
+  TSMI_REQUIRE(n >= 0 && (n == 0 || user_keys), "insert_keys: bad keys");
+  TSMI_REQUIRE(n <= cap, "The capacity of hashtable is not sufficient (%lld keys, capacity %lld)",
+               (long long)n, (long long)cap);
+  if (n == 0) return TSMI_OK;
+  TSMI_GRID_CHECK(n);
+  hipLaunchKernelGGL(insert_keys_kernel, grid_for(n), dim3(kBlock), 0, (hipStream_t)s, t,
+                     (const long long *)user_keys, n, status);
+  return check_launch("tsmi_hashtable_insert_keys");
+}
+
+extern "C" int tsmi_hashtable_lookup_keys(tsmi_stream_t s, const int64_t *keys,
+                                          const int32_t *vals, int64_t cap,
+                                          const int64_t *user_keys, int64_t n, int32_t *out) {
+  TableView t;
+  if (int e = make_table(&t, keys, vals, cap)) return e;
+  TSMI_REQUIRE(n >= 0 && (n == 0 || (user_keys && out)), "lookup_keys: bad arguments");
+  if (n == 0) return TSMI_OK;
+  TSMI_GRID_CHECK(n);
+  hipLaunchKernelGGL(lookup_keys_kernel, grid_for(n), dim3(kBlock), 0, (hipStream_t)s, t,
+                     (const long long *)user_keys, n, out);
+  return check_launch("tsmi_hashtable_lookup_keys");
+}
+
+extern "C" int tsmi_kmap_query(tsmi_stream_t s, const int64_t *keys, const int32_t *vals,
+                               int64_t cap, const int32_t *out_coords, int64_t n_out,
+                               int64_t n_out_pad, const int32_t ks[3], const int32_t stride[3],
+                               const int32_t pad[3], int32_t *out_in_map) {
+  TableView t;
+  Geom g;
+  if (int e = make_table(&t, keys, vals, cap)) return e;
+  if (int e = make_geom(&g, ks, stride, pad)) return e;
+  TSMI_REQUIRE(n_out >= 0 && n_out_pad >= n_out, "kmap_query: n_out_pad < n_out");
+  TSMI_REQUIRE(n_out == 0 || out_coords, "kmap_query: null out_coords");
+  int64_t total = n_out_pad * g.kvol;
+  if (total == 0) return TSMI_OK;
+  TSMI_REQUIRE(out_in_map, "kmap_query: null out_in_map");
+  TSMI_GRID_CHECK(total);
+  hipLaunchKernelGGL(kmap_query_kernel, grid_for(total), dim3(kBlock), 0, (hipStream_t)s, t,
+                     (const int4 *)out_coords, n_out, total, g, out_in_map);
+  return check_launch("tsmi_kmap_query");
+}
+
+extern "C" int tsmi_coords_max(tsmi_stream_t s, const int32_t *coords, int64_t n,
+                               int32_t *out_max) {
+  TSMI_REQUIRE(out_max && n >= 0 && (n == 0 || coords), "coords_max: bad arguments");
+  hipLaunchKernelGGL(fill_kernel<int32_t>, dim3(1), dim3(kBlock), 0, (hipStream_t)s, out_max,
+                     (int64_t)4, 0);
+  if (n > 0) {
+    TSMI_GRID_CHECK(n);
+    hipLaunchKernelGGL(coords_max_kernel, grid_for(n), dim3(kBlock), 0, (hipStream_t)s,
+                       (const int4 *)coords, n, out_max);
+  }
+  return check_launch("tsmi_coords_max");
+}
+
+extern "C" int tsmi_downsample_candidates(tsmi_stream_t s, const int32_t *in_coords, int64_t n_in,
+                                          const int32_t ks[3], const int32_t stride[3],
+                                          const int32_t pad[3], const int32_t out_max_host[3],
+                                          const int32_t *in_max_dev, int mode, int64_t *keys,
+                                          int64_t cap, int64_t *uniq_keys, int64_t uniq_cap,
+                                          int32_t *counters) {
+  TableView t;
+  Geom g;
+  static int32_t dummy_vals;  // the de-duplication pass never touches vals
+  if (int e = make_table(&t, keys, &dummy_vals, cap)) return e;
+  if (int e = make_geom(&g, ks, stride, pad)) return e;
+  TSMI_REQUIRE(mode == 0 || mode == 1, "downsample_candidates: mode must be 0 or 1");
+  TSMI_REQUIRE(n_in >= 0 && (n_in == 0 || in_coords), "downsample_candidates: bad coords");
+  TSMI_REQUIRE(uniq_keys && counters && uniq_cap >= 0, "downsample_candidates: null output");
+  TSMI_REQUIRE(mode == 1 || in_max_dev || out_max_host, "downsample_candidates: no output bound");
+  if (n_in == 0) return TSMI_OK;
+  int64_t total = mode == 1 ? n_in : n_in * g.kvol;
+  TSMI_GRID_CHECK(total);
+  int3 hm = make_int3(0, 0, 0);
+  if (out_max_host) hm = make_int3(out_max_host[0], out_max_host[1], out_max_host[2]);
+  hipLaunchKernelGGL(downsample_candidates_kernel, grid_for(total), dim3(kBlock), 0,
+                     (hipStream_t)s, (const int4 *)in_coords, n_in, total, g, hm, in_max_dev, mode,
+                     t, (unsigned long long *)uniq_keys, uniq_cap, counters);
+  return check_launch("tsmi_downsample_candidates");
+}
+
+extern "C" int tsmi_downsample_finalize(tsmi_stream_t s, const int64_t *sorted_keys, int64_t n_out,
+                                        const int64_t *keys, int32_t *vals, int64_t cap,
+                                        int32_t *out_coords) {
+  TableView t;
+  if (int e = make_table(&t, keys, vals, cap)) return e;
+  TSMI_REQUIRE(n_out >= 0 && (n_out == 0 || (sorted_keys && out_coords)),
+               "downsample_finalize: bad arguments");
+  TSMI_REQUIRE(n_out <= cap,
+               "The capacity of hashtable is not sufficient. Please enlarge reserved space for "
+               "hashtable (backends.hash_rsv_ratio): %lld outputs, capacity %lld",
+               (long long)n_out, (long long)cap);
+  if (n_out == 0) return TSMI_OK;
+  TSMI_GRID_CHECK(n_out);
+  hipLaunchKernelGGL(downsample_finalize_kernel, grid_for(n_out), dim3(kBlock), 0, (hipStream_t)s,
+                     (const unsigned long long *)sorted_keys, n_out, t, (int4 *)out_coords);
+  return check_launch("tsmi_downsample_finalize");
+}
+
+extern "C" int tsmi_transpose_map(tsmi_stream_t s, const int32_t *map, int64_t n_rows, int kvol,
+                                  int32_t *map_t, int64_t n_rows_t) {
+  TSMI_REQUIRE(kvol >= 1 && n_rows >= 0 && n_rows_t >= 0, "transpose_map: bad sizes");
+  int64_t total_t = n_rows_t * kvol, total = n_rows * kvol;
+  if (total_t > 0) {
+    TSMI_REQUIRE(map_t, "transpose_map: null map_t");
+    TSMI_GRID_CHECK(total_t);
+    hipLaunchKernelGGL(fill_kernel<int32_t>, grid_for(total_t), dim3(kBlock), 0, (hipStream_t)s,
+                       map_t, total_t, -1);
+  }
+  if (total > 0 && total_t > 0) {
+    TSMI_REQUIRE(map, "transpose_map: null map");
+    TSMI_GRID_CHECK(total);
+    hipLaunchKernelGGL(transpose_map_kernel, grid_for(total), dim3(kBlock), 0, (hipStream_t)s, map,
+                       total, kvol, map_t, n_rows_t);
+  }
+  return check_launch("tsmi_transpose_map");
+}
+
+extern "C" int tsmi_derive_bitmask(tsmi_stream_t s, const int32_t *map, int64_t n_pad, int kvol,
+                                   int split, int64_t valid_n, int32_t *bitmask) {
+  TSMI_REQUIRE(kvol >= 1 && split >= 1 && n_pad >= 0 && valid_n >= 0 && valid_n <= n_pad,
+               "derive_bitmask: bad sizes");
+  int len = (kvol + split - 1) / split;
+  TSMI_REQUIRE(len <= 32, "derive_bitmask: %d offsets per split exceed the 32 mask bits", len);
+  TSMI_REQUIRE((int64_t)(split - 1) * len < kvol, "derive_bitmask: split_mask_num %d leaves an empty split", split);
+  int64_t total = n_pad * split;
+  if (total == 0) return TSMI_OK;
+  TSMI_REQUIRE(map && bitmask, "derive_bitmask: null pointer");
+  TSMI_GRID_CHECK(total);
+  hipLaunchKernelGGL(derive_bitmask_kernel, grid_for(total), dim3(kBlock), 0, (hipStream_t)s, map,
+                     n_pad, kvol, split, len, valid_n, bitmask);
+  return check_launch("tsmi_derive_bitmask");
+}
+
+extern "C" int tsmi_reorder_map(tsmi_stream_t s, const int32_t *map, const int32_t *reorder_loc,
+                                int64_t n_pad, int kvol, int split, int32_t *out) {
+  TSMI_REQUIRE(kvol >= 1 && split >= 1 && n_pad >= 0, "reorder_map: bad sizes");
+  int64_t total = n_pad * kvol;
+  if (total == 0) return TSMI_OK;
+  TSMI_REQUIRE(map && reorder_loc && out, "reorder_map: null pointer");
+  TSMI_GRID_CHECK(total);
+  int len = (kvol + split - 1) / split;
+  hipLaunchKernelGGL(reorder_map_kernel, grid_for(total), dim3(kBlock), 0, (hipStream_t)s, map,
+                     reorder_loc, n_pad, kvol, len, out);
+  return check_launch("tsmi_reorder_map");
+}
+
+extern "C" int tsmi_reduce_bitmask(tsmi_stream_t s, const int32_t *sorted_mask, int split,
+                                   int64_t n_pad, int tile, int32_t *reduced) {
+  if (tile < 4 || tile % 4 != 0)
+    return fail(TSMI_ERR_RUNTIME, "[Bitmask reduce] reduce tile size must be multiple of 4.");
+  TSMI_REQUIRE(split >= 1 && n_pad >= 1, "reduce_bitmask: bad sizes");
+  TSMI_REQUIRE(sorted_mask && reduced, "reduce_bitmask: null pointer");
+  int64_t rows = (n_pad - 1) / tile + 1;
+  int64_t total = rows * split;
+  TSMI_GRID_CHECK(total);
+  hipLaunchKernelGGL(reduce_bitmask_kernel, grid_for(total), dim3(kBlock), 0, (hipStream_t)s,
+                     sorted_mask, split, n_pad, tile, rows, reduced);
+  return check_launch("tsmi_reduce_bitmask");
+}
+
+extern "C" int tsmi_pair_lists_count(tsmi_stream_t s, const int32_t *map, int64_t n_rows, int kvol,
+                                     int32_t *block_counts, int32_t *nbsizes) {
+  TSMI_REQUIRE(kvol >= 1 && n_rows >= 0 && nbsizes, "pair_lists_count: bad arguments");
+  int64_t nblk = ceil_div(n_rows, kBlock);
+  if (n_rows == 0) {
+    hipLaunchKernelGGL(fill_kernel<int32_t>, grid_for(kvol), dim3(kBlock), 0, (hipStream_t)s,
+                       nbsizes, (int64_t)kvol, 0);
+    return check_launch("tsmi_pair_lists_count");
+  }
+  TSMI_REQUIRE(map && block_counts, "pair_lists_count: null pointer");
+  TSMI_REQUIRE(grid_fits(nblk), "pair_lists_count: too many rows");
+  hipLaunchKernelGGL(pair_count_kernel, dim3((unsigned)nblk), dim3(kBlock), 0, (hipStream_t)s, map,
+                     n_rows, kvol, nblk, block_counts);
+  hipLaunchKernelGGL(pair_scan_kernel, dim3(1), dim3(1024), 0, (hipStream_t)s, block_counts,
+                     nblk * kvol, kvol, nblk, nbsizes);
+  return check_launch("tsmi_pair_lists_count");
+}
+
+extern "C" int tsmi_pair_lists_fill(tsmi_stream_t s, const int32_t *map, int64_t n_rows, int kvol,
+                                    int32_t *block_counts, int64_t nnz, int32_t *nbmaps_inter,
+                                    int32_t *nbmaps_planar, int64_t n_in, int64_t n_out,
+                                    int32_t *input_mask, int32_t *output_mask) {
+  TSMI_REQUIRE(kvol >= 1 && n_rows >= 0 && nnz >= 0 && n_in >= 0 && n_out >= 0,
+               "pair_lists_fill: bad sizes");
+  if (input_mask && n_in > 0) {
+    TSMI_GRID_CHECK(n_in * kvol);
+    hipLaunchKernelGGL(fill_kernel<int32_t>, grid_for(n_in * kvol), dim3(kBlock), 0,
+                       (hipStream_t)s, input_mask, n_in * kvol, -1);
+  }
+  if (output_mask && n_out > 0) {
+    TSMI_GRID_CHECK(n_out * kvol);
+    hipLaunchKernelGGL(fill_kernel<int32_t>, grid_for(n_out * kvol), dim3(kBlock), 0,
+                       (hipStream_t)s, output_mask, n_out * kvol, -1);
+  }
+  if (n_rows > 0 && nnz > 0) {
+    TSMI_REQUIRE(map && block_counts, "pair_lists_fill: null pointer");
+    int64_t nblk = ceil_div(n_rows, kBlock);
+    TSMI_REQUIRE(grid_fits(nblk), "pair_lists_fill: too many rows");
+    int skip_k = (n_in == n_out && kvol % 2 == 1) ? kvol / 2 : -1;
+    hipLaunchKernelGGL(pair_fill_kernel, dim3((unsigned)nblk), dim3(kBlock), 0, (hipStream_t)s,
+                       map, n_rows, kvol, nblk, block_counts, nnz, nbmaps_inter, nbmaps_planar,
+                       n_in, n_out, input_mask, output_mask, skip_k);
+  }
+  return check_launch("tsmi_pair_lists_fill");
+}
+
+extern "C" int tsmi_exclusive_scan_quantified(tsmi_stream_t s, int kvol, const int32_t *nbsizes,
+                                              int q, int32_t *nbaddrs, int32_t *qnbaddrs) {
+  TSMI_REQUIRE(kvol >= 1 && q >= 1 && nbsizes && nbaddrs && qnbaddrs,
+               "exclusive_scan_quantified: bad arguments");
+  hipLaunchKernelGGL(scan_quantified_kernel, dim3(1), dim3(64), 0, (hipStream_t)s, kvol, nbsizes,
+                     q, nbaddrs, qnbaddrs);
+  return check_launch("tsmi_exclusive_scan_quantified");
+}
+
+extern "C" int tsmi_build_masks(tsmi_stream_t s, const int32_t *nbmaps_inter, int64_t nnz,
+                                const int32_t *nbaddrs, int kvol, int64_t n_in, int64_t n_out,
+                                int32_t *input_mask, int32_t *output_mask) {
+  TSMI_REQUIRE(kvol >= 1 && nnz >= 0 && n_in >= 0 && n_out >= 0, "build_masks: bad sizes");
+  TSMI_REQUIRE(input_mask || n_in == 0, "build_masks: null input_mask");
+  TSMI_REQUIRE(output_mask || n_out == 0, "build_masks: null output_mask");
+  if (n_in > 0) {
+    TSMI_GRID_CHECK(n_in * kvol);
+    hipLaunchKernelGGL(fill_kernel<int32_t>, grid_for(n_in * kvol), dim3(kBlock), 0,
+                       (hipStream_t)s, input_mask, n_in * kvol, -1);
+  }
+  if (n_out > 0) {
+    TSMI_GRID_CHECK(n_out * kvol);
+    hipLaunchKernelGGL(fill_kernel<int32_t>, grid_for(n_out * kvol), dim3(kBlock), 0,
+                       (hipStream_t)s, output_mask, n_out * kvol, -1);
+  }
+  if (nnz > 0) {
+    TSMI_REQUIRE(nbmaps_inter && nbaddrs, "build_masks: null pair list");
+    TSMI_GRID_CHECK(nnz);
+    int skip_k = (n_in == n_out && kvol % 2 == 1) ? kvol / 2 : -1;
+    hipLaunchKernelGGL(masks_from_pairs_kernel, grid_for(nnz), dim3(kBlock), 0, (hipStream_t)s,
+                       nbmaps_inter, nnz, nbaddrs, kvol, n_in, n_out, skip_k, input_mask,
+                       output_mask);
+  }
+  return check_launch("tsmi_build_masks");
+}

@@ -1,0 +1,98 @@
+from typing import Dict, List, Optional, Tuple, Union
+
+import torch
+
+from ....tensor import SparseTensor
+from ....utils import make_ntuple
+from . import conv_config as _cfg
+from .conv_mode import get_conv_mode
+from .func import (FetchOnDemandConvolutionFuntion, GatherScatterConvolutionFuntion,
+                   ImplicitGEMMConvolutionFuntion)
+from .kmap import build_kernel_map, transpose_kernel_map
+
+__all__ = ["conv3d"]
+
+_DATAFLOWS = {
+    _cfg.Dataflow.ImplicitGEMM: ImplicitGEMMConvolutionFuntion,
+    _cfg.Dataflow.GatherScatter: GatherScatterConvolutionFuntion,
+    _cfg.Dataflow.FetchOnDemand: FetchOnDemandConvolutionFuntion,
+}
+
+
+def conv3d(input: SparseTensor, weight: torch.Tensor,
+           kernel_size: Union[int, List[int], Tuple[int, ...]],
+           bias: Optional[torch.Tensor] = None,
+           stride: Union[int, List[int], Tuple[int, ...]] = 1,
+           padding: Union[int, Tuple[int, ...]] = 0,
+           dilation: Union[int, Tuple[int, ...]] = 1, config: Dict = None,
+           transposed: bool = False, generative: bool = False,
+           training: bool = False) -> SparseTensor:
+    """Sparse convolution on a SparseTensor (the reference's
+    nn/functional/conv/conv.py:15-210): config resolution (per call -> global ->
+    default), 1x1x1 fast path, kernel-map cache lookup / build, dataflow dispatch,
+    transposed branch, cache propagation to the output tensor.
+
+    Differences kept on purpose: hash tables are cached under the stride of the
+    coordinates they index; the config is never mutated; transposed-map products
+    are computed once per map; the bias is added inside the kernel epilogue."""
+    feats, coords = input.feats, input.coords
+    kernel_size = make_ntuple(kernel_size, ndim=3)
+    stride = make_ntuple(stride, ndim=3)
+    dilation = make_ntuple(dilation, ndim=3)
+
+    if config is None:
+        config = _cfg.get_global_conv_config()
+        if config is None:
+            config = _cfg.get_default_conv_config(conv_mode=get_conv_mode(), training=training)
+    dataflow = config["dataflow"]
+    if dataflow == _cfg.Dataflow.CodedCSR:
+        raise AssertionError("CodedCSR has not been integrated.")
+    try:
+        conv_fn = _DATAFLOWS[dataflow]
+    except KeyError:
+        raise ValueError("unsupported dataflow: {}".format(dataflow)) from None
+    if dataflow != _cfg.Dataflow.ImplicitGEMM and config["ifsort"]:
+        config = dict(config, ifsort=False)  # pair-list dataflows never sort
+    caches = input._caches
+
+    if kernel_size == (1, 1, 1) and stride == (1, 1, 1) and dilation == (1, 1, 1):
+        out_feats = feats.matmul(weight)
+        if bias is not None:
+            out_feats += bias
+        output = SparseTensor(feats=out_feats, coords=coords, stride=input.stride,
+                              spatial_range=input.spatial_range)
+    elif not transposed:
+        key = (input.stride, kernel_size, stride, dilation)
+        out_stride = tuple(input.stride[a] * stride[a] for a in range(3))
+        kmap = caches.kmaps.get(key)
+        if kmap is None:
+            in_hashmap = caches.hashmaps.get(input.stride)
+            keys, vals = in_hashmap if in_hashmap is not None else (None, None)
+            kmap = build_kernel_map(
+                coords, feats.shape[0], kernel_size, stride, padding, keys, vals,
+                input.spatial_range, config["kmap_mode"], dataflow,
+                downsample_mode=config["downsample_mode"], training=training,
+                ifsort=config["ifsort"], split_mask_num=config["split_mask_num"],
+                split_mask_num_bwd=config["split_mask_num_bwd"])
+            caches.kmaps[key] = kmap
+            caches.hashmaps.setdefault(input.stride, kmap["in_hashmap"])
+            caches.hashmaps.setdefault(out_stride, kmap["out_hashmap"])
+        out_feats = conv_fn.apply(feats, weight, kmap, config, False, bias)
+        output = SparseTensor(feats=out_feats, coords=kmap["coords"], stride=out_stride,
+                              spatial_range=kmap["spatial_range"])
+    else:
+        if generative:
+            raise NotImplementedError("generative transposed convolution is not part of this build")
+        fine_stride = tuple(input.stride[a] // stride[a] for a in range(3))
+        kmap = caches.kmaps.get((fine_stride, kernel_size, stride, dilation))
+        kmap = transpose_kernel_map(kmap, config["ifsort"], training=training,
+                                    split_mask_num=config["split_mask_num"],
+                                    split_mask_num_bwd=config["split_mask_num_bwd"])
+        out_feats = conv_fn.apply(feats, weight, kmap, config, True, bias)
+        fine_coords, fine_range = caches.cmaps[fine_stride]
+        output = SparseTensor(feats=out_feats, coords=fine_coords, stride=fine_stride,
+                              spatial_range=fine_range)
+
+    output._caches = caches
+    caches.cmaps.setdefault(output.stride, (output.coords, output.spatial_range))
+    return output

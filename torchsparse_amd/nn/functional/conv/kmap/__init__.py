@@ -1,0 +1,2 @@
+from .build_kmap import *  # noqa: F401,F403
+from .downsample import *  # noqa: F401,F403

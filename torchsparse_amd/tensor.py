@@ -1,0 +1,90 @@
+"""SparseTensor: features [N, C] + integer coordinates [N, 4] = (batch, x, y, z)
+(the reference's torchsparse/tensor.py:29-110)."""
+from typing import Optional, Tuple, Union
+
+import torch
+
+from .utils import make_ntuple
+from .utils.tensor_cache import (TensorCache, TensorCacheMode, get_global_tensor_cache,
+                                 get_tensor_cache_mode, set_global_tensor_cache)
+
+__all__ = ["SparseTensor", "get_allow_negative_coordinates", "set_allow_negative_coordinates"]
+
+_allow_negative_coordinates = False
+
+
+def get_allow_negative_coordinates() -> bool:
+    return _allow_negative_coordinates
+
+
+def set_allow_negative_coordinates(flag: bool) -> None:
+    """Negative coordinates are not supported by the packed hash keys of this build."""
+    global _allow_negative_coordinates
+    if flag:
+        raise NotImplementedError("negative voxel coordinates are not supported")
+    _allow_negative_coordinates = False
+
+
+class SparseTensor:
+    def __init__(self, feats: torch.Tensor, coords: torch.Tensor,
+                 stride: Union[int, Tuple[int, ...]] = 1,
+                 spatial_range: Optional[Tuple[int, ...]] = None) -> None:
+        self.feats = feats
+        self.coords = coords
+        self.stride = make_ntuple(stride, ndim=3)
+        self.spatial_range = None if spatial_range is None else make_ntuple(
+            spatial_range, ndim=len(spatial_range))
+        if get_tensor_cache_mode() == TensorCacheMode.GLOBAL_TENSOR_CACHE:
+            cache = get_global_tensor_cache()
+            if cache is None:
+                cache = TensorCache()
+                set_global_tensor_cache(cache)
+            self._caches = cache
+        else:
+            self._caches = TensorCache()
+
+    # short aliases used throughout user code
+    F = property(lambda self: self.feats, lambda self, v: setattr(self, "feats", v))
+    C = property(lambda self: self.coords, lambda self, v: setattr(self, "coords", v))
+    s = property(lambda self: self.stride,
+                 lambda self, v: setattr(self, "stride", make_ntuple(v, ndim=3)))
+
+    def _like(self, feats: torch.Tensor) -> "SparseTensor":
+        out = SparseTensor.__new__(SparseTensor)
+        out.feats, out.coords = feats, self.coords
+        out.stride, out.spatial_range = self.stride, self.spatial_range
+        out._caches = self._caches
+        return out
+
+    def cpu(self):
+        self.coords, self.feats = self.coords.cpu(), self.feats.cpu()
+        return self
+
+    def cuda(self):
+        self.coords, self.feats = self.coords.cuda(), self.feats.cuda()
+        return self
+
+    def half(self):
+        self.feats = self.feats.half()
+        return self
+
+    def detach(self):
+        self.coords, self.feats = self.coords.detach(), self.feats.detach()
+        return self
+
+    def to(self, device, non_blocking: bool = True):
+        self.coords = self.coords.to(device, non_blocking=non_blocking)
+        self.feats = self.feats.to(device, non_blocking=non_blocking)
+        return self
+
+    def dense(self) -> torch.Tensor:
+        """[B, X, Y, Z, C] dense tensor (needs spatial_range)."""
+        assert self.spatial_range is not None
+        c = self.coords.long()
+        out = torch.zeros(*self.spatial_range, self.feats.shape[1], dtype=self.feats.dtype,
+                          device=self.feats.device)
+        out[c[:, 0], c[:, 1], c[:, 2], c[:, 3]] = self.feats
+        return out
+
+    def __add__(self, other: "SparseTensor") -> "SparseTensor":
+        return self._like(self.feats + other.feats)
