@@ -40,7 +40,7 @@ def _case(rng, n, cin, cout, kvol, dtype, wscale=None):
 
 
 def _f32(t):
-    return t.float().cpu().numpy()
+    return t.detach().float().cpu().numpy()
 
 
 CHANNELS = [(32, 32), (64, 64), (128, 128), (4, 32), (5, 16), (16, 16), (96, 96), (128, 96),
@@ -96,7 +96,8 @@ def test_all_dataflows_agree_with_oracle(mods, geom, dtype):
         cfg.dataflow = dataflow
         configs.append(cfg)
     for split in (1, 3, 5):
-        if -(-ks ** 3 // split) > 32:  # a mask word holds 32 offsets
+        length = -(-ks ** 3 // split)
+        if length > 32 or (split - 1) * length >= ks ** 3:  # 32 offsets per mask word, no empty split
             continue
         cfg = F.conv_config.get_default_conv_config()
         cfg.ifsort, cfg.split_mask_num = True, split

@@ -54,6 +54,9 @@ def conv3d(input: SparseTensor, weight: torch.Tensor,
     if dataflow != _cfg.Dataflow.ImplicitGEMM and config["ifsort"]:
         config = dict(config, ifsort=False)  # pair-list dataflows never sort
     caches = input._caches
+    # the input's own level is registered too, so a transposed layer can return to a
+    # level no earlier layer produced (the reference only registers outputs)
+    caches.cmaps.setdefault(input.stride, (coords, input.spatial_range))
 
     if kernel_size == (1, 1, 1) and stride == (1, 1, 1) and dilation == (1, 1, 1):
         out_feats = feats.matmul(weight)
