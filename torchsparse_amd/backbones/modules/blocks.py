@@ -1,0 +1,56 @@
+"""Building blocks of the sparse backbones.  Sub-module names and order follow the
+reference (backbones/modules/blocks.py) so its state dicts load unchanged:
+ConvBlock / ConvTransposeBlock are Sequential(conv, norm, relu) with indices 0-2;
+ResBlock has ``main`` (conv, norm, relu, conv, norm), ``shortcut`` and ``relu``."""
+from typing import List, Tuple, Union
+
+import numpy as np
+from torch import nn
+
+from ... import nn as spnn
+from ...tensor import SparseTensor
+
+__all__ = ["SparseConvBlock", "SparseConvTransposeBlock", "SparseResBlock"]
+
+_Size = Union[int, List[int], Tuple[int, ...]]
+
+
+def _conv_bn(cin: int, cout: int, kernel_size: _Size, act: bool, **conv_kwargs):
+    layers = [spnn.Conv3d(cin, cout, kernel_size, **conv_kwargs), spnn.BatchNorm(cout)]
+    if act:
+        layers.append(spnn.ReLU(True))
+    return layers
+
+
+class SparseConvBlock(nn.Sequential):
+    def __init__(self, in_channels: int, out_channels: int, kernel_size: _Size, stride: _Size = 1,
+                 dilation: int = 1) -> None:
+        super().__init__(*_conv_bn(in_channels, out_channels, kernel_size, True, stride=stride,
+                                   dilation=dilation))
+
+
+class SparseConvTransposeBlock(nn.Sequential):
+    def __init__(self, in_channels: int, out_channels: int, kernel_size: _Size, stride: _Size = 1,
+                 dilation: int = 1) -> None:
+        super().__init__(*_conv_bn(in_channels, out_channels, kernel_size, True, stride=stride,
+                                   dilation=dilation, transposed=True))
+
+
+class SparseResBlock(nn.Module):
+    """relu(main(x) + shortcut(x)); the shortcut is a 1x1x1 conv + norm when the
+    channel count or the stride changes, the identity otherwise."""
+
+    def __init__(self, in_channels: int, out_channels: int, kernel_size: _Size, stride: _Size = 1,
+                 dilation: int = 1) -> None:
+        super().__init__()
+        self.main = nn.Sequential(
+            *_conv_bn(in_channels, out_channels, kernel_size, True, stride=stride, dilation=dilation),
+            *_conv_bn(out_channels, out_channels, kernel_size, False, dilation=dilation))
+        if in_channels != out_channels or int(np.prod(stride)) != 1:
+            self.shortcut = nn.Sequential(*_conv_bn(in_channels, out_channels, 1, False, stride=stride))
+        else:
+            self.shortcut = nn.Identity()
+        self.relu = spnn.ReLU(True)
+
+    def forward(self, x: SparseTensor) -> SparseTensor:
+        return self.relu(self.main(x) + self.shortcut(x))
