@@ -204,26 +204,38 @@ int64_t tsmi_packed_weight_elems(int kvol, int cin, int cout);
 int tsmi_pack_weights(tsmi_stream_t s, const void *w, void *w_packed, int kvol, int cin,
                       int cout, int dtype);
 
+/* Floats of scratch the implicit-GEMM entry points want for a problem of
+ * n_tile_rows map rows (n_out for the unsorted call, n_pad for the sorted one) and
+ * `split` mask splits; 0 when none is needed.  Small problems cut the kernel offsets
+ * into ranges that run as separate workgroups and add their fp32 partial sums, the
+ * role split-K plays in the reference's wgrad kernels
+ * (convolution/convolution_backward_wgrad_implicit_gemm_cuda.cu:1614-2042). */
+int64_t tsmi_conv_workspace_elems(int64_t n_tile_rows, int64_t n_out, int kvol, int split,
+                                  int cin, int cout, int dtype);
+
 /* Y[i,:] = sum_k [m = map[i,k] >= 0] X[m,:] W[k] (+ bias) for i < n_out; every
- * output row is written.  `map` has at least n_out rows.
+ * output row is written.  `map` has at least n_out rows.  `workspace` (float
+ * [workspace_elems], may be NULL) enables the offset split described above.
  * Replaces conv_forward_implicit_gemm_cuda
  * (convolution/convolution_forward_implicit_gemm_cuda.cu:1527-1986). */
 int tsmi_conv_implicit_gemm(tsmi_stream_t s, const void *x, const void *w_packed,
                             const int32_t *map, int64_t n_map_rows, int64_t n_out, int kvol,
-                            int cin, int cout, int dtype, const void *bias, void *y);
+                            int cin, int cout, int dtype, const void *bias, float *workspace,
+                            int64_t workspace_elems, void *y);
 
 /* Same sum over a row-sorted map: tile row r of split s reads
  * reorder_map[r, s*L..] and adds into output row reorder_loc[s, r].
- * `partial` (float [split, n_out, cout], only for split > 1) receives the
- * per-split sums, which are then added into y.  reduced_mask may be NULL (the
- * kernel derives tile-level skipping from the map itself).  Replaces
+ * `workspace` (tsmi_conv_workspace_elems floats; required for split > 1) receives
+ * the per-split fp32 sums, which are then added into y.  reduced_mask may be NULL
+ * (the kernel derives its skipping from the map itself).  Replaces
  * conv_forward_implicit_gemm_sorted_cuda
  * (convolution/convolution_forward_implicit_gemm_sorted_cuda.cu:1755-2230). */
 int tsmi_conv_implicit_gemm_sorted(tsmi_stream_t s, const void *x, const void *w_packed,
                                    const int32_t *reorder_map, const int32_t *reduced_mask,
                                    const int32_t *reorder_loc, int64_t n_pad, int64_t n_out,
                                    int kvol, int split, int cin, int cout, int dtype,
-                                   const void *bias, float *partial, void *y);
+                                   const void *bias, float *workspace, int64_t workspace_elems,
+                                   void *y);
 
 /* Fetch-on-demand: one launch over 128-padded pair lists gathers X rows, multiplies
  * by W[k] and writes partial[qnbaddrs[k] + p, :] (fp32 for TSMI_F32, else the I/O

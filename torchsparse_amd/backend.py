@@ -33,6 +33,8 @@ def _load():
     lib.tsmi_sort_temp_bytes.argtypes = [_i64]
     lib.tsmi_packed_weight_elems.restype = _i64
     lib.tsmi_packed_weight_elems.argtypes = [_i32, _i32, _i32]
+    lib.tsmi_conv_workspace_elems.restype = _i64
+    lib.tsmi_conv_workspace_elems.argtypes = [_i64, _i64, _i32, _i32, _i32, _i32, _i32]
     sig = {
         "tsmi_hashtable_clear": [_vp, _vp, _vp, _i64],
         "tsmi_hashtable_insert_coords": [_vp, _vp, _vp, _i64, _vp, _i64, _vp],
@@ -54,9 +56,10 @@ def _load():
         "tsmi_exclusive_scan_quantified": [_vp, _i32, _vp, _i32, _vp, _vp],
         "tsmi_build_masks": [_vp, _vp, _i64, _vp, _i32, _i64, _i64, _vp, _vp],
         "tsmi_pack_weights": [_vp, _vp, _vp, _i32, _i32, _i32, _i32],
-        "tsmi_conv_implicit_gemm": [_vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _i32, _i32, _vp, _vp],
+        "tsmi_conv_implicit_gemm": [_vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _i32, _i32, _vp, _vp,
+                                    _i64, _vp],
         "tsmi_conv_implicit_gemm_sorted": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32,
-                                           _i32, _i32, _i32, _vp, _vp, _vp],
+                                           _i32, _i32, _i32, _vp, _vp, _i64, _vp],
         "tsmi_conv_fetch_on_demand": [_vp, _vp, _vp, _vp, _i64, _vp, _vp, _i64, _vp, _i64, _i32,
                                       _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp],
         "tsmi_gs_gather": [_vp, _vp, _vp, _i64, _i32, _i32, _i32, _vp],
@@ -445,9 +448,12 @@ def conv_forward_implicit_gemm_cuda(in_feats, kernel, out_in_map, num_out_feats,
     if cout != num_out_channels:
         raise ValueError("num_out_channels does not match the kernel")
     y = torch.empty((num_out_feats, cout), dtype=x.dtype, device=x.device)
+    code = _dtype_code(x)
+    ws_elems = _C.tsmi_conv_workspace_elems(num_out_feats, num_out_feats, kvol, 1, cin, cout, code)
+    ws = torch.empty(ws_elems, dtype=torch.float32, device=x.device) if ws_elems > 0 else None
     _check(_C.tsmi_conv_implicit_gemm(_stream(), _ptr(x), _ptr(wp), _ptr(out_in_map),
-                                      out_in_map.shape[0], num_out_feats, kvol, cin, cout,
-                                      _dtype_code(x), _ptr(bias), _ptr(y)))
+                                      out_in_map.shape[0], num_out_feats, kvol, cin, cout, code,
+                                      _ptr(bias), _ptr(ws), ws_elems, _ptr(y)))
     return y
 
 
@@ -459,13 +465,13 @@ def conv_forward_implicit_gemm_sorted_cuda(in_feats, kernel, reorder_out_in_map,
     split = reorder_loc.shape[0]
     n_pad = reorder_out_in_map.shape[0]
     y = torch.empty((num_out_feats, cout), dtype=x.dtype, device=x.device)
-    partial = None
-    if split > 1:
-        partial = torch.empty((split, num_out_feats, cout), dtype=torch.float32, device=x.device)
+    code = _dtype_code(x)
+    ws_elems = _C.tsmi_conv_workspace_elems(n_pad, num_out_feats, kvol, split, cin, cout, code)
+    ws = torch.empty(ws_elems, dtype=torch.float32, device=x.device) if ws_elems > 0 else None
     _check(_C.tsmi_conv_implicit_gemm_sorted(_stream(), _ptr(x), _ptr(wp), _ptr(reorder_out_in_map),
                                              _ptr(reduced_mask), _ptr(reorder_loc), n_pad,
-                                             num_out_feats, kvol, split, cin, cout, _dtype_code(x),
-                                             _ptr(bias), _ptr(partial), _ptr(y)))
+                                             num_out_feats, kvol, split, cin, cout, code,
+                                             _ptr(bias), _ptr(ws), ws_elems, _ptr(y)))
     return y
 
 

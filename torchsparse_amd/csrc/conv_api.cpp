@@ -40,10 +40,17 @@ extern "C" int tsmi_pack_weights(tsmi_stream_t s, const void *w, void *w_packed,
   return ops->pack((hipStream_t)s, w, w_packed, kvol, cin, cout);
 }
 
+extern "C" int64_t tsmi_conv_workspace_elems(int64_t n_tile_rows, int64_t n_out, int kvol,
+                                             int split, int cin, int cout, int dtype) {
+  const ConvOps *ops = ops_for(dtype);
+  if (!ops || n_tile_rows < 0 || n_out < 0 || kvol < 1 || split < 1 || cin < 1 || cout < 1) return -1;
+  return ops->workspace(n_tile_rows, n_out, kvol, split, cin, cout);
+}
+
 extern "C" int tsmi_conv_implicit_gemm(tsmi_stream_t s, const void *x, const void *w_packed,
                                        const int32_t *map, int64_t n_map_rows, int64_t n_out,
                                        int kvol, int cin, int cout, int dtype, const void *bias,
-                                       void *y) {
+                                       float *workspace, int64_t workspace_elems, void *y) {
   const ConvOps *ops = ops_for(dtype);
   if (int e = check_shapes("conv_implicit_gemm", ops, kvol, cin, cout)) return e;
   TSMI_REQUIRE(n_out >= 0 && n_map_rows >= n_out, "conv_implicit_gemm: map has %lld rows, need %lld",
@@ -53,7 +60,7 @@ extern "C" int tsmi_conv_implicit_gemm(tsmi_stream_t s, const void *x, const voi
   TSMI_REQUIRE(aligned16(x) && aligned16(w_packed) && aligned16(y),
                "conv_implicit_gemm: x, w_packed and y must be 16-byte aligned");
   return ops->igemm((hipStream_t)s, x, w_packed, map, n_map_rows, n_out, n_out, kvol, cin, cout,
-                    bias, y, nullptr, 0, 1, nullptr);
+                    bias, y, nullptr, 0, 1, workspace, workspace_elems);
 }
 
 extern "C" int tsmi_conv_implicit_gemm_sorted(tsmi_stream_t s, const void *x, const void *w_packed,
@@ -61,7 +68,8 @@ extern "C" int tsmi_conv_implicit_gemm_sorted(tsmi_stream_t s, const void *x, co
                                               const int32_t *reduced_mask,
                                               const int32_t *reorder_loc, int64_t n_pad,
                                               int64_t n_out, int kvol, int split, int cin, int cout,
-                                              int dtype, const void *bias, float *partial, void *y) {
+                                              int dtype, const void *bias, float *workspace,
+                                              int64_t workspace_elems, void *y) {
   (void)reduced_mask;  // tile skipping is derived from the staged map itself
   const ConvOps *ops = ops_for(dtype);
   if (int e = check_shapes("conv_implicit_gemm_sorted", ops, kvol, cin, cout)) return e;
@@ -72,14 +80,11 @@ extern "C" int tsmi_conv_implicit_gemm_sorted(tsmi_stream_t s, const void *x, co
   if (n_out == 0) return TSMI_OK;
   TSMI_REQUIRE(x && w_packed && reorder_map && reorder_loc && y,
                "conv_implicit_gemm_sorted: null pointer");
-  TSMI_REQUIRE(split == 1 || partial, "conv_implicit_gemm_sorted: split > 1 needs `partial`");
+  TSMI_REQUIRE(split == 1 || workspace, "conv_implicit_gemm_sorted: split > 1 needs a workspace");
   TSMI_REQUIRE(aligned16(x) && aligned16(w_packed) && aligned16(y),
                "conv_implicit_gemm_sorted: x, w_packed and y must be 16-byte aligned");
-  if (int e = ops->igemm((hipStream_t)s, x, w_packed, reorder_map, n_pad, n_pad, n_out, kvol, cin,
-                         cout, split == 1 ? bias : nullptr, y, reorder_loc, n_pad, split, partial))
-    return e;
-  if (split > 1) return ops->sum_partials((hipStream_t)s, partial, split, n_out, cout, bias, y);
-  return TSMI_OK;
+  return ops->igemm((hipStream_t)s, x, w_packed, reorder_map, n_pad, n_pad, n_out, kvol, cin, cout,
+                    bias, y, reorder_loc, n_pad, split, workspace, workspace_elems);
 }
 
 extern "C" int tsmi_conv_fetch_on_demand(tsmi_stream_t s, const void *x, const void *w_packed,

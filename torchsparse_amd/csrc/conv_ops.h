@@ -3,6 +3,8 @@
 // and exposes one of these tables; conv_api.cpp dispatches on the dtype code.
 #pragma once
 
+#include <algorithm>
+
 #include "common.h"
 
 namespace tsmi {
@@ -10,11 +12,13 @@ namespace tsmi {
 struct ConvOps {
   int step;  // reduction elements per MFMA step (Cin is padded to a multiple)
   int (*pack)(hipStream_t s, const void *w, void *wp, int kvol, int cin, int cout);
+  // floats of scratch igemm wants for this problem (0 = none)
+  int64_t (*workspace)(int64_t n_tile_rows, int64_t n_out, int kvol, int split, int cin, int cout);
   // row_out == nullptr: plain implicit GEMM over `map`; otherwise sorted mode.
   int (*igemm)(hipStream_t s, const void *x, const void *wp, const int32_t *map,
                int64_t n_map_rows, int64_t n_tile_rows, int64_t n_out, int kvol, int cin, int cout,
                const void *bias, void *y, const int32_t *row_out, int64_t row_out_stride,
-               int split, float *partial);
+               int split, float *partial, int64_t partial_elems);
   // out[nbaddrs[k] + p, :] = X[rows[nbaddrs[k] + p], :] W[k] over 128-padded pair lists
   int (*pairs)(hipStream_t s, const void *x, const void *wp, const int32_t *rows,
                const int32_t *nbaddrs, const int32_t *qnbaddrs, int64_t qnnz, int kvol, int cin,
