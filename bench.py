@@ -5,7 +5,10 @@
 One step = one MinkUNet (SparseResUNet42 + 19-class linear head) forward in fp16 on a
 synthetic 64-beam LiDAR scan (~90k voxels, 4 input channels), starting from a fresh
 SparseTensor, so every step rebuilds its 9 kernel maps.  Inputs and weights are
-resident in HBM before the timed region.  Prints ONE JSON line.
+resident in HBM before the timed region.  The network runs in inference form:
+eval-mode BatchNorm folded into the convolutions, ReLU and shortcut adds in the
+convolution epilogues (nn.utils.fuse_inference; same function, checked in the tests);
+the unfused module-by-module time is reported beside it.  Prints ONE JSON line.
 
 Also measured (same JSON line):
   layers        the five single layers of the layer sweep on the same scan: kernel-map
@@ -38,6 +41,10 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-layers", action="store_true", help="skip the single-layer sweep")
+    ap.add_argument("--no-roofline", action="store_true", help="skip the per-kernel roofline timing")
+    ap.add_argument("--sorted", type=int, default=-1,
+                    help="1: run the implicit GEMM over row-sorted maps (conv_mode 1); 0: unsorted; "
+                         "-1: the default of this benchmark")
     return ap.parse_args()
 
 
@@ -263,28 +270,36 @@ def main():
     n = coords_np.shape[0]
     coords = torch.from_numpy(coords_np).cuda()
     feats = torch.randn(n, 4, device="cuda", dtype=torch.float16)
-    model = SparseResUNet42(in_channels=4).cuda().half().eval()
+    import copy
+    from torchsparse_amd.nn.utils import fuse_inference
+    unfused = SparseResUNet42(in_channels=4).cuda().half().eval()
+    model = fuse_inference(copy.deepcopy(unfused))
     head = torch.nn.Linear(96, 19).cuda().half().eval()
+    if args.sorted == 1:
+        F.set_conv_mode(1)
 
-    def step():
-        with torch.no_grad():
-            x = ts.SparseTensor(feats, coords)
-            return head(model(x)[-1].feats)
+    def timed(net, steps, warmup):
+        def step():
+            with torch.no_grad():
+                x = ts.SparseTensor(feats, coords)
+                return head(net(x)[-1].feats)
+        for _ in range(warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / steps
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms_per_step = timed(model, args.steps, args.warmup)
+    ms_unfused = timed(unfused, max(args.steps // 2, 1), 2)
 
     with torch.no_grad():
         inp = ts.SparseTensor(feats, coords)
         records, outs = network_layers(model, inp)
         warm_ms = event_ms(lambda: model(inp), iters=10, warm=2)  # kernel maps cached
-        roof = dominant_layer_roofline(ts, F, records, inp._caches)
+        roof = None if args.no_roofline else dominant_layer_roofline(ts, F, records, inp._caches)
         level_coords = {lvl: c[0].cpu().numpy() for lvl, c in inp._caches.cmaps.items()}
         layers = None if args.no_layers else layer_sweep(ts, spnn, F, backend, coords, n)
     cpu = None if args.no_cpu else cpu_baseline(records, level_coords)
@@ -297,7 +312,9 @@ def main():
         "config": {"workload": "MinkUNet (SparseResUNet42, cr=1.0) + Linear(96,19) forward, batch 1, "
                                f"synthetic 64-beam scan seed 1, {n} voxels, 4 input channels, "
                                "kernel maps rebuilt every step",
-                   "voxels": n, "warm_map_ms_per_step": round(warm_ms, 4)},
+                   "voxels": n, "warm_map_ms_per_step": round(warm_ms, 4),
+                   "unfused_ms_per_step": round(ms_unfused, 4),
+                   "conv_mode": F.get_conv_mode().value},
         "roofline": roof, "cpu_baseline": cpu, "layers": layers,
     }
     print(json.dumps(result))

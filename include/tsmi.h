@@ -216,12 +216,17 @@ int64_t tsmi_conv_workspace_elems(int64_t n_tile_rows, int64_t n_out, int kvol, 
 /* Y[i,:] = sum_k [m = map[i,k] >= 0] X[m,:] W[k] (+ bias) for i < n_out; every
  * output row is written.  `map` has at least n_out rows.  `workspace` (float
  * [workspace_elems], may be NULL) enables the offset split described above.
+ * Epilogue, shared by every convolution entry point: y = act(sum + bias +
+ * residual), with bias [cout] and residual [n_out, cout] of the I/O type (either
+ * may be NULL) and act = max(., 0) when relu != 0 — the bias add of
+ * nn/functional/conv/conv.py:123-124 and the BatchNorm-folded / ReLU / shortcut
+ * adds of the residual blocks, fused into the producing kernel.
  * Replaces conv_forward_implicit_gemm_cuda
  * (convolution/convolution_forward_implicit_gemm_cuda.cu:1527-1986). */
 int tsmi_conv_implicit_gemm(tsmi_stream_t s, const void *x, const void *w_packed,
                             const int32_t *map, int64_t n_map_rows, int64_t n_out, int kvol,
-                            int cin, int cout, int dtype, const void *bias, float *workspace,
-                            int64_t workspace_elems, void *y);
+                            int cin, int cout, int dtype, const void *bias, const void *residual,
+                            int relu, float *workspace, int64_t workspace_elems, void *y);
 
 /* Same sum over a row-sorted map: tile row r of split s reads
  * reorder_map[r, s*L..] and adds into output row reorder_loc[s, r].
@@ -234,8 +239,8 @@ int tsmi_conv_implicit_gemm_sorted(tsmi_stream_t s, const void *x, const void *w
                                    const int32_t *reorder_map, const int32_t *reduced_mask,
                                    const int32_t *reorder_loc, int64_t n_pad, int64_t n_out,
                                    int kvol, int split, int cin, int cout, int dtype,
-                                   const void *bias, float *workspace, int64_t workspace_elems,
-                                   void *y);
+                                   const void *bias, const void *residual, int relu,
+                                   float *workspace, int64_t workspace_elems, void *y);
 
 /* Fetch-on-demand: one launch over 128-padded pair lists gathers X rows, multiplies
  * by W[k] and writes partial[qnbaddrs[k] + p, :] (fp32 for TSMI_F32, else the I/O
@@ -252,7 +257,8 @@ int tsmi_conv_fetch_on_demand(tsmi_stream_t s, const void *x, const void *w_pack
                               const int32_t *nbaddrs, const int32_t *qnbaddrs, int64_t qnnz,
                               const int32_t *row_mask, int64_t n_out, int kvol, int cin,
                               int cout, int dtype, int transpose, int center_k,
-                              const void *bias, void *partial, void *y);
+                              const void *bias, const void *residual, int relu, void *partial,
+                              void *y);
 
 /* Gather-GEMM-scatter, step 1: buffer[nbaddrs[k] + p, :] = X[in(k,p), :].
  * Replaces gather_all_kernel_pad_sep_with_mask / gather_kernel
@@ -273,7 +279,7 @@ int tsmi_gs_gemm(tsmi_stream_t s, const void *buffer, const void *w_packed,
  * (convolution/convolution_gather_scatter_cuda.cu:150-250). */
 int tsmi_gs_scatter(tsmi_stream_t s, const void *out_buffer, const int32_t *nbaddrs,
                     const int32_t *row_mask, int64_t n_out, int kvol, int cout, int dtype,
-                    int center_k, const void *bias, void *y);
+                    int center_k, const void *bias, const void *residual, int relu, void *y);
 
 #pragma GCC visibility pop
 #ifdef __cplusplus

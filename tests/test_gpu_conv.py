@@ -231,3 +231,57 @@ def test_kmap_cache_and_errors(mods):
         F.conv3d(inp, conv_a.kernel, 3, config=dict(F.conv_config.get_default_conv_config(), dataflow="bogus"))
     with pytest.raises(RuntimeError, match="GPU"):
         backend.conv_forward_implicit_gemm_cuda(x.cpu(), conv_a.kernel.cpu(), torch.zeros(1), 1, 16)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("n", [300, 5000])
+def test_fused_epilogue_bias_residual_relu(mods, dtype, n):
+    """y = relu(conv + bias + residual) in every dataflow (small n takes the offset-split path)."""
+    ts, backend, _, F = mods
+    rng = np.random.default_rng(n)
+    coords = random_coords(rng, n, (30, 30, 10))
+    cin, cout = 64, 128
+    x, w = _case(rng, n, cin, cout, 27, dtype)
+    bias = torch.from_numpy(rng.standard_normal(cout).astype(np.float32)).to("cuda", dtype)
+    res = torch.from_numpy(rng.standard_normal((n, cout)).astype(np.float32)).to("cuda", dtype)
+    omap = oracle.kmap_subm(coords, 3)
+    want = np.maximum(oracle.conv_implicit_gemm(_f32(x), _f32(w), omap, n) + _f32(bias) + _f32(res), 0)
+    for dataflow, ifsort in [(F.Dataflow.ImplicitGEMM, False), (F.Dataflow.ImplicitGEMM, True),
+                             (F.Dataflow.GatherScatter, False), (F.Dataflow.FetchOnDemand, False)]:
+        cfg = F.conv_config.get_default_conv_config()
+        cfg.dataflow, cfg.ifsort = dataflow, ifsort
+        out = F.conv3d(ts.SparseTensor(x, dev(coords)), w, 3, bias=bias, padding=1, config=cfg,
+                       residual=res, activation="relu")
+        assert rel_rms(_f32(out.feats), want) < TOL[dtype], (dataflow, ifsort)
+    with pytest.raises(ValueError, match="activation"):
+        F.conv3d(ts.SparseTensor(x, dev(coords)), w, 3, activation="gelu")
+
+
+def test_fuse_inference_matches_unfused_unet(mods):
+    """BatchNorm folding + fused ReLU / shortcut add leave the network function unchanged."""
+    ts, _, _, F = mods
+    from torchsparse_amd.backbones import SparseResUNet42
+    from torchsparse_amd.nn.utils import fuse_inference
+    import copy
+    torch.manual_seed(1)
+    rng = np.random.default_rng(11)
+    coords = dev(random_coords(rng, 6000, (48, 48, 16)))
+    x = torch.randn(6000, 4, device="cuda")
+    model = SparseResUNet42(in_channels=4).cuda().eval()
+    for m in model.modules():  # non-trivial norm statistics
+        if isinstance(m, torch.nn.BatchNorm1d):
+            m.running_mean.normal_(0, 0.3)
+            m.running_var.uniform_(0.5, 1.5)
+            m.weight.data.uniform_(0.5, 1.5)
+            m.bias.data.normal_(0, 0.2)
+    fused = fuse_inference(copy.deepcopy(model))
+    with torch.no_grad():
+        ref = model(ts.SparseTensor(x, coords))
+        got = fused(ts.SparseTensor(x, coords))
+        assert len(ref) == len(got) == 9
+        for a, b in zip(ref, got):
+            assert a.coords.data_ptr() != 0 and torch.equal(a.coords, b.coords)
+            assert rel_rms(_f32(b.feats), _f32(a.feats)) < 1e-3
+        # and in half precision, against the fp32 network
+        got16 = copy.deepcopy(fused).half()(ts.SparseTensor(x.half(), coords))
+        assert rel_rms(_f32(got16[-1].feats), _f32(ref[-1].feats)) < 3e-2

@@ -53,4 +53,12 @@ class SparseResBlock(nn.Module):
         self.relu = spnn.ReLU(True)
 
     def forward(self, x: SparseTensor) -> SparseTensor:
+        if getattr(self, "_fused_tail", False):
+            # after nn.utils.fuse_inference(): norms are folded into the convolutions and the
+            # shortcut add + ReLU run in the epilogue of the block's last convolution
+            shortcut = self.shortcut(x)
+            y = x
+            for layer in list(self.main)[:-2]:
+                y = layer(y)
+            return self.main[-2](y, residual=shortcut.feats)
         return self.relu(self.main(x) + self.shortcut(x))

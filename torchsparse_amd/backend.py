@@ -57,14 +57,14 @@ def _load():
         "tsmi_build_masks": [_vp, _vp, _i64, _vp, _i32, _i64, _i64, _vp, _vp],
         "tsmi_pack_weights": [_vp, _vp, _vp, _i32, _i32, _i32, _i32],
         "tsmi_conv_implicit_gemm": [_vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _i32, _i32, _vp, _vp,
-                                    _i64, _vp],
+                                    _i32, _vp, _i64, _vp],
         "tsmi_conv_implicit_gemm_sorted": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32,
-                                           _i32, _i32, _i32, _vp, _vp, _i64, _vp],
+                                           _i32, _i32, _i32, _vp, _vp, _i32, _vp, _i64, _vp],
         "tsmi_conv_fetch_on_demand": [_vp, _vp, _vp, _vp, _i64, _vp, _vp, _i64, _vp, _i64, _i32,
-                                      _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp],
+                                      _i32, _i32, _i32, _i32, _i32, _vp, _vp, _i32, _vp, _vp],
         "tsmi_gs_gather": [_vp, _vp, _vp, _i64, _i32, _i32, _i32, _vp],
         "tsmi_gs_gemm": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _i32, _i32, _vp],
-        "tsmi_gs_scatter": [_vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _vp, _vp],
+        "tsmi_gs_scatter": [_vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _vp, _vp, _i32, _vp],
     }
     for name, argtypes in sig.items():
         fn = getattr(lib, name)
@@ -131,10 +131,14 @@ class GPUHashTable:
     owning table of that capacity — hashmap/hashmap_cuda.cuh:65-121."""
 
     def __init__(self, keys, vals: Optional[torch.Tensor] = None, device="cuda"):
+        self.counters = None
         if isinstance(keys, int):
+            # one zero-filled allocation: keys (int64 view), vals, 8 spare counters
             cap = make_divisible(max(int(keys), 8), 8)
-            self.keys = torch.zeros(cap, dtype=torch.int64, device=device)
-            self.vals = torch.zeros(cap, dtype=torch.int32, device=device)
+            buf = torch.zeros(3 * cap + 8, dtype=torch.int32, device=device)
+            self.keys = buf[:2 * cap].view(torch.int64)
+            self.vals = buf[2 * cap:3 * cap]
+            self.counters = buf[3 * cap:]
         else:
             self.keys = _need(keys, torch.int64, "hashmap_keys")
             self.vals = _need(vals, torch.int32, "hashmap_vals")
@@ -238,7 +242,7 @@ def downsample_coords(coords: torch.Tensor, kernel_sizes, stride, padding, coord
     cap = hash_capacity(n * min(fan, 2), rsv_ratio)
     table = GPUHashTable(cap, device=dev)
     uniq = torch.empty(cap, dtype=torch.int64, device=dev)
-    counters = torch.zeros(2, dtype=torch.int32, device=dev)
+    counters = table.counters  # zero on a fresh table
     in_max = None
     host_max = None
     if mode == 0:
@@ -249,7 +253,7 @@ def downsample_coords(coords: torch.Tensor, kernel_sizes, stride, padding, coord
     _check(_C.tsmi_downsample_candidates(_stream(), _ptr(coords), n, _I3(*ks), _I3(*st), _I3(*pd),
                                          host_max, _ptr(in_max), mode, _ptr(table.keys), cap,
                                          _ptr(uniq), cap, _ptr(counters)))
-    n_out, overflow = counters.tolist()
+    n_out, overflow = counters[:2].tolist()
     if overflow:
         raise ValueError(
             "The capacity of hashtable is not sufficient. Please enlarge reserved space for "
@@ -439,8 +443,17 @@ def _conv_common(in_feats: torch.Tensor, kernel: torch.Tensor):
     return x, pack_weights(kernel), kshape
 
 
+def _epilogue_args(bias, residual, x, n_out, cout):
+    for name, t, shape in (("bias", bias, (cout,)), ("residual", residual, (n_out, cout))):
+        if t is not None:
+            if t.dtype != x.dtype or tuple(t.shape) != shape or not t.is_contiguous():
+                raise ValueError(f"{name} must be a contiguous {x.dtype} tensor of shape {shape}")
+    return _ptr(bias), _ptr(residual)
+
+
 def conv_forward_implicit_gemm_cuda(in_feats, kernel, out_in_map, num_out_feats, num_out_channels,
-                                    allow_tf32=False, allow_fp16=True, bias=None) -> torch.Tensor:
+                                    allow_tf32=False, allow_fp16=True, bias=None, residual=None,
+                                    relu=False) -> torch.Tensor:
     """convolution/convolution_forward_implicit_gemm_cuda.cu:1527-1986.  allow_tf32 /
     allow_fp16 are accepted and ignored: fp32 runs in true fp32, 16-bit types
     accumulate in fp32."""
@@ -451,15 +464,17 @@ def conv_forward_implicit_gemm_cuda(in_feats, kernel, out_in_map, num_out_feats,
     code = _dtype_code(x)
     ws_elems = _C.tsmi_conv_workspace_elems(num_out_feats, num_out_feats, kvol, 1, cin, cout, code)
     ws = torch.empty(ws_elems, dtype=torch.float32, device=x.device) if ws_elems > 0 else None
+    pb, pr = _epilogue_args(bias, residual, x, num_out_feats, cout)
     _check(_C.tsmi_conv_implicit_gemm(_stream(), _ptr(x), _ptr(wp), _ptr(out_in_map),
                                       out_in_map.shape[0], num_out_feats, kvol, cin, cout, code,
-                                      _ptr(bias), _ptr(ws), ws_elems, _ptr(y)))
+                                      pb, pr, int(relu), _ptr(ws), ws_elems, _ptr(y)))
     return y
 
 
 def conv_forward_implicit_gemm_sorted_cuda(in_feats, kernel, reorder_out_in_map, reduced_mask,
                                            reorder_loc, num_out_feats, num_out_channels,
-                                           allow_tf32=False, allow_fp16=True, bias=None) -> torch.Tensor:
+                                           allow_tf32=False, allow_fp16=True, bias=None,
+                                           residual=None, relu=False) -> torch.Tensor:
     """convolution/convolution_forward_implicit_gemm_sorted_cuda.cu:1755-2230."""
     x, wp, (kvol, cin, cout) = _conv_common(in_feats, kernel)
     split = reorder_loc.shape[0]
@@ -468,16 +483,18 @@ def conv_forward_implicit_gemm_sorted_cuda(in_feats, kernel, reorder_out_in_map,
     code = _dtype_code(x)
     ws_elems = _C.tsmi_conv_workspace_elems(n_pad, num_out_feats, kvol, split, cin, cout, code)
     ws = torch.empty(ws_elems, dtype=torch.float32, device=x.device) if ws_elems > 0 else None
+    pb, pr = _epilogue_args(bias, residual, x, num_out_feats, cout)
     _check(_C.tsmi_conv_implicit_gemm_sorted(_stream(), _ptr(x), _ptr(wp), _ptr(reorder_out_in_map),
                                              _ptr(reduced_mask), _ptr(reorder_loc), n_pad,
                                              num_out_feats, kvol, split, cin, cout, code,
-                                             _ptr(bias), _ptr(ws), ws_elems, _ptr(y)))
+                                             pb, pr, int(relu), _ptr(ws), ws_elems, _ptr(y)))
     return y
 
 
 def conv_forward_fetch_on_demand_cuda(in_feats, kernel, nbmaps, sum_nnz, nbaddrs, qnbaddrs,
                                       output_size, qsum_nnz, transpose, allow_tf32=False,
-                                      allow_fp16=True, row_mask=None, center_k=-1, bias=None) -> torch.Tensor:
+                                      allow_fp16=True, row_mask=None, center_k=-1, bias=None,
+                                      residual=None, relu=False) -> torch.Tensor:
     """convolution/convolution_forward_fetch_on_demand_cuda.cu:1981-2119.  nbmaps is the
     planar [2, nnz] list; row_mask is the kmap's output_mask (input_mask when
     transposed) that makes the reduction atomic free."""
@@ -486,18 +503,20 @@ def conv_forward_fetch_on_demand_cuda(in_feats, kernel, nbmaps, sum_nnz, nbaddrs
         raise ValueError("fetch-on-demand needs the kmap's row mask (output_mask / input_mask)")
     y = torch.empty((output_size, cout), dtype=x.dtype, device=x.device)
     partial = torch.empty((max(int(sum_nnz), 1), cout), dtype=x.dtype, device=x.device)
+    pb, pr = _epilogue_args(bias, residual, x, output_size, cout)
     _check(_C.tsmi_conv_fetch_on_demand(_stream(), _ptr(x), _ptr(wp), _ptr(nbmaps), int(sum_nnz),
                                         _ptr(nbaddrs), _ptr(qnbaddrs), int(qsum_nnz), _ptr(row_mask),
                                         output_size, kvol, cin, cout, _dtype_code(x),
-                                        int(bool(transpose)), center_k, _ptr(bias), _ptr(partial),
-                                        _ptr(y)))
+                                        int(bool(transpose)), center_k, pb, pr, int(relu),
+                                        _ptr(partial), _ptr(y)))
     return y
 
 
 def conv_forward_gather_scatter_cuda(in_feats, kernel, nbmaps, nbsizes, input_mask, output_mask,
                                      output_size, epsilon=0.0, mm_thresh=0, conv_mode=0,
                                      transpose=False, buffer=None, nbaddrs=None, qnbaddrs=None,
-                                     qsum_nnz=None, center_k=-1, bias=None) -> torch.Tensor:
+                                     qsum_nnz=None, center_k=-1, bias=None, residual=None,
+                                     relu=False) -> torch.Tensor:
     """convolution/convolution_gather_scatter_cuda.cu:279-814: gather -> GEMM per
     offset -> scatter, here always as three launches over all offsets.  epsilon,
     mm_thresh and conv_mode only steer grouping in the reference; results do not
@@ -525,6 +544,7 @@ def conv_forward_gather_scatter_cuda(in_feats, kernel, nbmaps, nbsizes, input_ma
                              _ptr(gathered)))
     _check(_C.tsmi_gs_gemm(s, _ptr(gathered), _ptr(wp), _ptr(nbaddrs), _ptr(qnbaddrs), nnz,
                            int(qsum_nnz), kvol, cin, cout, code, _ptr(products)))
+    pb, pr = _epilogue_args(bias, residual, x, output_size, cout)
     _check(_C.tsmi_gs_scatter(s, _ptr(products), _ptr(nbaddrs), _ptr(row_mask), output_size, kvol,
-                              cout, code, center_k, _ptr(bias), _ptr(y)))
+                              cout, code, center_k, pb, pr, int(relu), _ptr(y)))
     return y

@@ -50,7 +50,8 @@ extern "C" int64_t tsmi_conv_workspace_elems(int64_t n_tile_rows, int64_t n_out,
 extern "C" int tsmi_conv_implicit_gemm(tsmi_stream_t s, const void *x, const void *w_packed,
                                        const int32_t *map, int64_t n_map_rows, int64_t n_out,
                                        int kvol, int cin, int cout, int dtype, const void *bias,
-                                       float *workspace, int64_t workspace_elems, void *y) {
+                                       const void *residual, int relu, float *workspace,
+                                       int64_t workspace_elems, void *y) {
   const ConvOps *ops = ops_for(dtype);
   if (int e = check_shapes("conv_implicit_gemm", ops, kvol, cin, cout)) return e;
   TSMI_REQUIRE(n_out >= 0 && n_map_rows >= n_out, "conv_implicit_gemm: map has %lld rows, need %lld",
@@ -60,7 +61,7 @@ extern "C" int tsmi_conv_implicit_gemm(tsmi_stream_t s, const void *x, const voi
   TSMI_REQUIRE(aligned16(x) && aligned16(w_packed) && aligned16(y),
                "conv_implicit_gemm: x, w_packed and y must be 16-byte aligned");
   return ops->igemm((hipStream_t)s, x, w_packed, map, n_map_rows, n_out, n_out, kvol, cin, cout,
-                    bias, y, nullptr, 0, 1, workspace, workspace_elems);
+                    bias, residual, relu, y, nullptr, 0, 1, workspace, workspace_elems);
 }
 
 extern "C" int tsmi_conv_implicit_gemm_sorted(tsmi_stream_t s, const void *x, const void *w_packed,
@@ -68,8 +69,9 @@ extern "C" int tsmi_conv_implicit_gemm_sorted(tsmi_stream_t s, const void *x, co
                                               const int32_t *reduced_mask,
                                               const int32_t *reorder_loc, int64_t n_pad,
                                               int64_t n_out, int kvol, int split, int cin, int cout,
-                                              int dtype, const void *bias, float *workspace,
-                                              int64_t workspace_elems, void *y) {
+                                              int dtype, const void *bias, const void *residual,
+                                              int relu, float *workspace, int64_t workspace_elems,
+                                              void *y) {
   (void)reduced_mask;  // tile skipping is derived from the staged map itself
   const ConvOps *ops = ops_for(dtype);
   if (int e = check_shapes("conv_implicit_gemm_sorted", ops, kvol, cin, cout)) return e;
@@ -84,7 +86,7 @@ extern "C" int tsmi_conv_implicit_gemm_sorted(tsmi_stream_t s, const void *x, co
   TSMI_REQUIRE(aligned16(x) && aligned16(w_packed) && aligned16(y),
                "conv_implicit_gemm_sorted: x, w_packed and y must be 16-byte aligned");
   return ops->igemm((hipStream_t)s, x, w_packed, reorder_map, n_pad, n_pad, n_out, kvol, cin, cout,
-                    bias, y, reorder_loc, n_pad, split, workspace, workspace_elems);
+                    bias, residual, relu, y, reorder_loc, n_pad, split, workspace, workspace_elems);
 }
 
 extern "C" int tsmi_conv_fetch_on_demand(tsmi_stream_t s, const void *x, const void *w_packed,
@@ -92,7 +94,8 @@ extern "C" int tsmi_conv_fetch_on_demand(tsmi_stream_t s, const void *x, const v
                                          const int32_t *nbaddrs, const int32_t *qnbaddrs,
                                          int64_t qnnz, const int32_t *row_mask, int64_t n_out,
                                          int kvol, int cin, int cout, int dtype, int transpose,
-                                         int center_k, const void *bias, void *partial, void *y) {
+                                         int center_k, const void *bias, const void *residual,
+                                         int relu, void *partial, void *y) {
   const ConvOps *ops = ops_for(dtype);
   if (int e = check_shapes("conv_fetch_on_demand", ops, kvol, cin, cout)) return e;
   TSMI_REQUIRE(nnz >= 0 && qnnz >= nnz && qnnz % 128 == 0 && n_out >= 0,
@@ -111,7 +114,7 @@ extern "C" int tsmi_conv_fetch_on_demand(tsmi_stream_t s, const void *x, const v
                            cout, partial))
       return e;
   return ops->scatter((hipStream_t)s, partial, nbaddrs, row_mask, n_out, kvol, cout, center_k, bias,
-                      y);
+                      residual, relu, y);
 }
 
 extern "C" int tsmi_gs_gather(tsmi_stream_t s, const void *x, const int32_t *nbmaps_inter,
@@ -141,7 +144,8 @@ extern "C" int tsmi_gs_gemm(tsmi_stream_t s, const void *buffer, const void *w_p
 
 extern "C" int tsmi_gs_scatter(tsmi_stream_t s, const void *out_buffer, const int32_t *nbaddrs,
                                const int32_t *row_mask, int64_t n_out, int kvol, int cout,
-                               int dtype, int center_k, const void *bias, void *y) {
+                               int dtype, int center_k, const void *bias, const void *residual,
+                               int relu, void *y) {
   const ConvOps *ops = ops_for(dtype);
   if (!ops) return fail(TSMI_ERR_INVALID_ARGUMENT, "gs_scatter: unsupported dtype");
   TSMI_REQUIRE(n_out >= 0 && kvol >= 1 && cout >= 1 && center_k >= -1 && center_k < kvol,
@@ -149,5 +153,5 @@ extern "C" int tsmi_gs_scatter(tsmi_stream_t s, const void *out_buffer, const in
   if (n_out == 0) return TSMI_OK;
   TSMI_REQUIRE(out_buffer && nbaddrs && row_mask && y, "gs_scatter: null pointer");
   return ops->scatter((hipStream_t)s, out_buffer, nbaddrs, row_mask, n_out, kvol, cout, center_k,
-                      bias, y);
+                      bias, residual, relu, y);
 }

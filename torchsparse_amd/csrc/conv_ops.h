@@ -17,16 +17,17 @@ struct ConvOps {
   // row_out == nullptr: plain implicit GEMM over `map`; otherwise sorted mode.
   int (*igemm)(hipStream_t s, const void *x, const void *wp, const int32_t *map,
                int64_t n_map_rows, int64_t n_tile_rows, int64_t n_out, int kvol, int cin, int cout,
-               const void *bias, void *y, const int32_t *row_out, int64_t row_out_stride,
-               int split, float *partial, int64_t partial_elems);
+               const void *bias, const void *residual, int relu, void *y, const int32_t *row_out,
+               int64_t row_out_stride, int split, float *partial, int64_t partial_elems);
   // out[nbaddrs[k] + p, :] = X[rows[nbaddrs[k] + p], :] W[k] over 128-padded pair lists
   int (*pairs)(hipStream_t s, const void *x, const void *wp, const int32_t *rows,
                const int32_t *nbaddrs, const int32_t *qnbaddrs, int64_t qnnz, int kvol, int cin,
                int cout, void *out);
   int (*sum_partials)(hipStream_t s, const float *partial, int split, int64_t n_out, int cout,
-                      const void *bias, void *y);
+                      const void *bias, const void *residual, int relu, void *y);
   int (*scatter)(hipStream_t s, const void *pbuf, const int32_t *nbaddrs, const int32_t *mask,
-                 int64_t n_out, int kvol, int cout, int center_k, const void *bias, void *y);
+                 int64_t n_out, int kvol, int cout, int center_k, const void *bias,
+                 const void *residual, int relu, void *y);
   int (*gather)(hipStream_t s, const void *x, const int32_t *pairs, int64_t nnz, int cin, int col,
                 void *buffer);
 };

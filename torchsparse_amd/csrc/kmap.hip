@@ -106,6 +106,7 @@ __global__ void kmap_query_kernel(TableView t, const int4 *out_coords, int64_t n
 }
 
 __global__ void coords_max_kernel(const int4 *coords, int64_t n, int32_t *out_max) {
+  __shared__ int smax[kBlock / 64][4];
   int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   int4 c = i < n ? coords[i] : make_int4(0, 0, 0, 0);
   int v[4] = {c.x, c.y, c.z, c.w};
@@ -114,7 +115,13 @@ __global__ void coords_max_kernel(const int4 *coords, int64_t n, int32_t *out_ma
     int m = v[a];
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) m = max(m, __shfl_xor(m, off));
-    if ((threadIdx.x & 63) == 0 && m > 0) atomicMax(&out_max[a], m);
+    if ((threadIdx.x & 63) == 0) smax[threadIdx.x >> 6][a] = m;
+  }
+  __syncthreads();
+  if (threadIdx.x < 4) {  // one atomic per block and column
+    int m = max(max(smax[0][threadIdx.x], smax[1][threadIdx.x]),
+                max(smax[2][threadIdx.x], smax[3][threadIdx.x]));
+    if (m > 0) atomicMax(&out_max[threadIdx.x], m);
   }
 }
 
@@ -172,8 +179,15 @@ __global__ void downsample_candidates_kernel(const int4 *in_coords, int64_t n_in
     counters[1] = 1;
     return;
   }
+  // append the new keys of this wavefront with one atomic for all of them
+  const unsigned long long fresh_mask = __ballot(fresh);
   if (fresh) {
-    int pos = atomicAdd(&counters[0], 1);
+    const int lane = threadIdx.x & 63;
+    const int leader = __ffsll((long long)fresh_mask) - 1;
+    int base = 0;
+    if (lane == leader) base = atomicAdd(&counters[0], __popcll(fresh_mask));
+    base = __shfl(base, leader);
+    const int pos = base + __popcll(fresh_mask & ((1ULL << lane) - 1ULL));
     if (pos < uniq_cap)
       uniq[pos] = key;
     else

@@ -26,7 +26,8 @@ def conv3d(input: SparseTensor, weight: torch.Tensor,
            padding: Union[int, Tuple[int, ...]] = 0,
            dilation: Union[int, Tuple[int, ...]] = 1, config: Dict = None,
            transposed: bool = False, generative: bool = False,
-           training: bool = False) -> SparseTensor:
+           training: bool = False, residual: Optional[torch.Tensor] = None,
+           activation: Optional[str] = None) -> SparseTensor:
     """Sparse convolution on a SparseTensor (the reference's
     nn/functional/conv/conv.py:15-210): config resolution (per call -> global ->
     default), 1x1x1 fast path, kernel-map cache lookup / build, dataflow dispatch,
@@ -34,7 +35,14 @@ def conv3d(input: SparseTensor, weight: torch.Tensor,
 
     Differences kept on purpose: hash tables are cached under the stride of the
     coordinates they index; the config is never mutated; transposed-map products
-    are computed once per map; the bias is added inside the kernel epilogue."""
+    are computed once per map; the bias is added inside the kernel epilogue.
+
+    Two optional extras fuse what usually follows a convolution into its epilogue:
+    ``residual`` (a [N_out, Cout] tensor added to the result) and ``activation``
+    (None or "relu"): output = act(conv(input) + bias + residual)."""
+    if activation not in (None, "relu"):
+        raise ValueError(f"unsupported fused activation: {activation}")
+    relu = activation == "relu"
     feats, coords = input.feats, input.coords
     kernel_size = make_ntuple(kernel_size, ndim=3)
     stride = make_ntuple(stride, ndim=3)
@@ -59,9 +67,11 @@ def conv3d(input: SparseTensor, weight: torch.Tensor,
     caches.cmaps.setdefault(input.stride, (coords, input.spatial_range))
 
     if kernel_size == (1, 1, 1) and stride == (1, 1, 1) and dilation == (1, 1, 1):
-        out_feats = feats.matmul(weight)
-        if bias is not None:
-            out_feats += bias
+        out_feats = feats.matmul(weight) if bias is None else torch.addmm(bias, feats, weight)
+        if residual is not None:
+            out_feats += residual
+        if relu:
+            out_feats = torch.relu_(out_feats)
         output = SparseTensor(feats=out_feats, coords=coords, stride=input.stride,
                               spatial_range=input.spatial_range)
     elif not transposed:
@@ -80,7 +90,7 @@ def conv3d(input: SparseTensor, weight: torch.Tensor,
             caches.kmaps[key] = kmap
             caches.hashmaps.setdefault(input.stride, kmap["in_hashmap"])
             caches.hashmaps.setdefault(out_stride, kmap["out_hashmap"])
-        out_feats = conv_fn.apply(feats, weight, kmap, config, False, bias)
+        out_feats = conv_fn.apply(feats, weight, kmap, config, False, bias, residual, relu)
         output = SparseTensor(feats=out_feats, coords=kmap["coords"], stride=out_stride,
                               spatial_range=kmap["spatial_range"])
     else:
@@ -91,7 +101,7 @@ def conv3d(input: SparseTensor, weight: torch.Tensor,
         kmap = transpose_kernel_map(kmap, config["ifsort"], training=training,
                                     split_mask_num=config["split_mask_num"],
                                     split_mask_num_bwd=config["split_mask_num_bwd"])
-        out_feats = conv_fn.apply(feats, weight, kmap, config, True, bias)
+        out_feats = conv_fn.apply(feats, weight, kmap, config, True, bias, residual, relu)
         fine_coords, fine_range = caches.cmaps[fine_stride]
         output = SparseTensor(feats=out_feats, coords=fine_coords, stride=fine_stride,
                               spatial_range=fine_range)

@@ -17,12 +17,15 @@ class FetchOnDemandConvolutionFuntion:
 
     @staticmethod
     def apply(input: torch.Tensor, weight: torch.Tensor, kmap: Dict, config: Dict,
-              transposed: bool = False, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+              transposed: bool = False, bias: Optional[torch.Tensor] = None,
+              residual: Optional[torch.Tensor] = None, relu: bool = False) -> torch.Tensor:
         sizes = kmap["sizes"]
         out_dtype = weight.dtype
         input, weight = _coerce(input, weight)
         if bias is not None and bias.dtype != input.dtype:
             bias = bias.to(input.dtype)
+        if residual is not None and residual.dtype != input.dtype:
+            residual = residual.to(input.dtype)
         nbmaps = kmap["nbmaps"]  # int32 [2, nnz]
         kvol = weight.shape[0] if weight.dim() == 3 else 1
         out = backend.conv_forward_fetch_on_demand_cuda(
@@ -30,5 +33,5 @@ class FetchOnDemandConvolutionFuntion:
             sizes[0] if transposed else sizes[1], int(kmap["qmapsize"]), transposed,
             backends.allow_tf32, backends.allow_fp16,
             row_mask=kmap["input_mask"] if transposed else kmap["output_mask"],
-            center_k=_center_offset(kmap, kvol), bias=bias)
+            center_k=_center_offset(kmap, kvol), bias=bias, residual=residual, relu=relu)
         return out if out.dtype == out_dtype else out.to(out_dtype)

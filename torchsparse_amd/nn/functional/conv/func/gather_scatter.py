@@ -21,12 +21,15 @@ class GatherScatterConvolutionFuntion:
 
     @staticmethod
     def apply(input: torch.Tensor, weight: torch.Tensor, kmap: Dict, config: Dict,
-              transposed: bool = False, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+              transposed: bool = False, bias: Optional[torch.Tensor] = None,
+              residual: Optional[torch.Tensor] = None, relu: bool = False) -> torch.Tensor:
         sizes = kmap["sizes"]
         out_dtype = weight.dtype
         input, weight = _coerce(input, weight)
         if bias is not None and bias.dtype != input.dtype:
             bias = bias.to(input.dtype)
+        if residual is not None and residual.dtype != input.dtype:
+            residual = residual.to(input.dtype)
         nbmaps = kmap["nbmaps"]
         if nbmaps.dtype != torch.int32:
             nbmaps = nbmaps.int()
@@ -36,5 +39,5 @@ class GatherScatterConvolutionFuntion:
             sizes[0] if transposed else sizes[1], config["epsilon"], int(config["mm_thresh"]), 0,
             transposed, None, nbaddrs=kmap.get("nbaddrs"), qnbaddrs=kmap.get("qnbaddrs"),
             qsum_nnz=None if kmap.get("qmapsize") is None else int(kmap["qmapsize"]),
-            center_k=_center_offset(kmap, kvol), bias=bias)
+            center_k=_center_offset(kmap, kvol), bias=bias, residual=residual, relu=relu)
         return out if out.dtype == out_dtype else out.to(out_dtype)

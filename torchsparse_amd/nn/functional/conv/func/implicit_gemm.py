@@ -25,7 +25,8 @@ class ImplicitGEMMConvolutionFuntion:
 
     @staticmethod
     def apply(input: torch.Tensor, weight: torch.Tensor, kmap: Dict, config: Dict,
-              transposed: bool = False, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+              transposed: bool = False, bias: Optional[torch.Tensor] = None,
+              residual: Optional[torch.Tensor] = None, relu: bool = False) -> torch.Tensor:
         sizes = kmap["sizes"]
         sfx = "_t" if transposed else ""
         num_out_feats = sizes[0] if transposed else sizes[1]
@@ -33,13 +34,15 @@ class ImplicitGEMMConvolutionFuntion:
         input, weight = _coerce(input, weight)
         if bias is not None and bias.dtype != input.dtype:
             bias = bias.to(input.dtype)
+        if residual is not None and residual.dtype != input.dtype:
+            residual = residual.to(input.dtype)
         if not config["ifsort"]:
             out = backend.conv_forward_implicit_gemm_cuda(
                 input, weight, kmap["out_in_map" + sfx], num_out_feats, weight.shape[-1],
-                backends.allow_tf32, backends.allow_fp16, bias=bias)
+                backends.allow_tf32, backends.allow_fp16, bias=bias, residual=residual, relu=relu)
         else:
             out = backend.conv_forward_implicit_gemm_sorted_cuda(
                 input, weight, kmap["reorder_out_in_map" + sfx], kmap["reduced_sorted_mask" + sfx],
                 kmap["reorder_loc" + sfx], num_out_feats, weight.shape[-1],
-                backends.allow_tf32, backends.allow_fp16, bias=bias)
+                backends.allow_tf32, backends.allow_fp16, bias=bias, residual=residual, relu=relu)
         return out if out.dtype == out_dtype else out.to(out_dtype)

@@ -37,6 +37,7 @@ class Conv3d(nn.Module):
         if generative:
             assert transposed
         self._config = config
+        self.activation = None  # "relu" once a following ReLU has been fused in (see nn.utils.fuse)
         self.kernel_volume = self.kernel_size[0] * self.kernel_size[1] * self.kernel_size[2]
         pointwise = self.kernel_volume == 1 and self.stride == (1, 1, 1)
         shape = (in_channels, out_channels) if pointwise else (self.kernel_volume, in_channels, out_channels)
@@ -69,8 +70,9 @@ class Conv3d(nn.Module):
             parts.append("generative=True")
         return ", ".join(parts)
 
-    def forward(self, input: SparseTensor) -> SparseTensor:
+    def forward(self, input: SparseTensor, residual: torch.Tensor = None) -> SparseTensor:
         return F.conv3d(input, weight=self.kernel, kernel_size=self.kernel_size, bias=self.bias,
                         stride=self.stride, padding=self.padding, dilation=self.dilation,
                         transposed=self.transposed, generative=self.generative,
-                        config=self._config, training=self.training)
+                        config=self._config, training=self.training, residual=residual,
+                        activation=self.activation)

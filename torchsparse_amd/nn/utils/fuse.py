@@ -1,0 +1,66 @@
+"""Inference-time fusion: fold eval-mode BatchNorm into the preceding sparse
+convolution and move a following ReLU (and, in residual blocks, the shortcut add)
+into that convolution's kernel epilogue.
+
+    model.eval()
+    fuse_inference(model)      # in place; parameters change, module names do not
+
+The folded model computes the same function (BatchNorm in eval mode is a
+per-channel affine map):  bn(conv(x)) = conv(x; W * g) + (b - mean) * g + beta,
+g = gamma / sqrt(var + eps).  Folding happens in fp32 and the result is cast back
+to the parameter dtype.
+"""
+import torch
+from torch import nn
+
+__all__ = ["fuse_inference"]
+
+
+def _fold(conv, bn) -> None:
+    with torch.no_grad():
+        g = bn.weight.float() if bn.affine else torch.ones_like(bn.running_var, dtype=torch.float32)
+        beta = bn.bias.float() if bn.affine else torch.zeros_like(g)
+        g = g * torch.rsqrt(bn.running_var.float() + bn.eps)
+        shift = beta - bn.running_mean.float() * g
+        if conv.bias is not None:
+            shift = shift + conv.bias.float() * g
+        conv.kernel.copy_((conv.kernel.float() * g).to(conv.kernel.dtype))
+        new_bias = shift.to(conv.kernel.dtype)
+        if conv.bias is None:
+            conv.bias = nn.Parameter(new_bias, requires_grad=False)
+        else:
+            conv.bias.copy_(new_bias)
+
+
+def _fuse_sequential(seq: nn.Sequential) -> None:
+    from ..modules import BatchNorm, Conv3d, ReLU
+    mods = list(seq.named_children())
+    for i, (_, conv) in enumerate(mods):
+        if not isinstance(conv, Conv3d) or i + 1 >= len(mods):
+            continue
+        name_bn, bn = mods[i + 1]
+        if not isinstance(bn, BatchNorm) or bn.training or not bn.track_running_stats:
+            continue
+        _fold(conv, bn)
+        setattr(seq, name_bn, nn.Identity())
+        if i + 2 < len(mods) and isinstance(mods[i + 2][1], ReLU):
+            conv.activation = "relu"
+            setattr(seq, mods[i + 2][0], nn.Identity())
+
+
+def fuse_inference(model: nn.Module) -> nn.Module:
+    """Fold every (Conv3d, eval BatchNorm[, ReLU]) run found inside nn.Sequential
+    containers of `model`, and fuse the tail of the residual blocks."""
+    from ...backbones.modules.blocks import SparseResBlock
+    from ..modules import Conv3d
+    for m in model.modules():
+        if isinstance(m, nn.Sequential):
+            _fuse_sequential(m)
+    for m in model.modules():
+        if isinstance(m, SparseResBlock) and not getattr(m, "_fused_tail", False):
+            last_conv, last_norm = m.main[-2], m.main[-1]
+            if isinstance(last_conv, Conv3d) and isinstance(last_norm, nn.Identity) \
+                    and last_conv.kernel.dim() == 3 and last_conv.activation is None:
+                last_conv.activation = "relu"  # relu(main(x) + shortcut(x)) in one epilogue
+                m._fused_tail = True
+    return model
