@@ -205,13 +205,13 @@ int tsmi_pack_weights(tsmi_stream_t s, const void *w, void *w_packed, int kvol, 
                       int cout, int dtype);
 
 /* Floats of scratch the implicit-GEMM entry points want for a problem of
- * n_tile_rows map rows (n_out for the unsorted call, n_pad for the sorted one) and
- * `split` mask splits; 0 when none is needed.  Small problems cut the kernel offsets
+ * n_tile_rows map rows (n_out for the unsorted call, n_pad and sorted = 1 for the
+ * sorted one) and `split` mask splits; 0 when none is needed.  Small problems cut the kernel offsets
  * into ranges that run as separate workgroups and add their fp32 partial sums, the
  * role split-K plays in the reference's wgrad kernels
  * (convolution/convolution_backward_wgrad_implicit_gemm_cuda.cu:1614-2042). */
 int64_t tsmi_conv_workspace_elems(int64_t n_tile_rows, int64_t n_out, int kvol, int split,
-                                  int cin, int cout, int dtype);
+                                  int cin, int cout, int dtype, int sorted);
 
 /* Y[i,:] = sum_k [m = map[i,k] >= 0] X[m,:] W[k] (+ bias) for i < n_out; every
  * output row is written.  `map` has at least n_out rows.  `workspace` (float

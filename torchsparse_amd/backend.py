@@ -34,7 +34,7 @@ def _load():
     lib.tsmi_packed_weight_elems.restype = _i64
     lib.tsmi_packed_weight_elems.argtypes = [_i32, _i32, _i32]
     lib.tsmi_conv_workspace_elems.restype = _i64
-    lib.tsmi_conv_workspace_elems.argtypes = [_i64, _i64, _i32, _i32, _i32, _i32, _i32]
+    lib.tsmi_conv_workspace_elems.argtypes = [_i64, _i64, _i32, _i32, _i32, _i32, _i32, _i32]
     sig = {
         "tsmi_hashtable_clear": [_vp, _vp, _vp, _i64],
         "tsmi_hashtable_insert_coords": [_vp, _vp, _vp, _i64, _vp, _i64, _vp],
@@ -462,7 +462,7 @@ def conv_forward_implicit_gemm_cuda(in_feats, kernel, out_in_map, num_out_feats,
         raise ValueError("num_out_channels does not match the kernel")
     y = torch.empty((num_out_feats, cout), dtype=x.dtype, device=x.device)
     code = _dtype_code(x)
-    ws_elems = _C.tsmi_conv_workspace_elems(num_out_feats, num_out_feats, kvol, 1, cin, cout, code)
+    ws_elems = _C.tsmi_conv_workspace_elems(num_out_feats, num_out_feats, kvol, 1, cin, cout, code, 0)
     ws = torch.empty(ws_elems, dtype=torch.float32, device=x.device) if ws_elems > 0 else None
     pb, pr = _epilogue_args(bias, residual, x, num_out_feats, cout)
     _check(_C.tsmi_conv_implicit_gemm(_stream(), _ptr(x), _ptr(wp), _ptr(out_in_map),
@@ -481,7 +481,7 @@ def conv_forward_implicit_gemm_sorted_cuda(in_feats, kernel, reorder_out_in_map,
     n_pad = reorder_out_in_map.shape[0]
     y = torch.empty((num_out_feats, cout), dtype=x.dtype, device=x.device)
     code = _dtype_code(x)
-    ws_elems = _C.tsmi_conv_workspace_elems(n_pad, num_out_feats, kvol, split, cin, cout, code)
+    ws_elems = _C.tsmi_conv_workspace_elems(n_pad, num_out_feats, kvol, split, cin, cout, code, 1)
     ws = torch.empty(ws_elems, dtype=torch.float32, device=x.device) if ws_elems > 0 else None
     pb, pr = _epilogue_args(bias, residual, x, num_out_feats, cout)
     _check(_C.tsmi_conv_implicit_gemm_sorted(_stream(), _ptr(x), _ptr(wp), _ptr(reorder_out_in_map),

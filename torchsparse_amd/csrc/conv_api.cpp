@@ -41,10 +41,10 @@ extern "C" int tsmi_pack_weights(tsmi_stream_t s, const void *w, void *w_packed,
 }
 
 extern "C" int64_t tsmi_conv_workspace_elems(int64_t n_tile_rows, int64_t n_out, int kvol,
-                                             int split, int cin, int cout, int dtype) {
+                                             int split, int cin, int cout, int dtype, int sorted) {
   const ConvOps *ops = ops_for(dtype);
   if (!ops || n_tile_rows < 0 || n_out < 0 || kvol < 1 || split < 1 || cin < 1 || cout < 1) return -1;
-  return ops->workspace(n_tile_rows, n_out, kvol, split, cin, cout);
+  return ops->workspace(n_tile_rows, n_out, kvol, split, cin, cout, sorted);
 }
 
 extern "C" int tsmi_conv_implicit_gemm(tsmi_stream_t s, const void *x, const void *w_packed,

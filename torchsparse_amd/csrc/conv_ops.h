@@ -4,6 +4,7 @@
 #pragma once
 
 #include <algorithm>
+#include <cstdlib>
 
 #include "common.h"
 
@@ -13,7 +14,8 @@ struct ConvOps {
   int step;  // reduction elements per MFMA step (Cin is padded to a multiple)
   int (*pack)(hipStream_t s, const void *w, void *wp, int kvol, int cin, int cout);
   // floats of scratch igemm wants for this problem (0 = none)
-  int64_t (*workspace)(int64_t n_tile_rows, int64_t n_out, int kvol, int split, int cin, int cout);
+  int64_t (*workspace)(int64_t n_tile_rows, int64_t n_out, int kvol, int split, int cin, int cout,
+                       int sorted);
   // row_out == nullptr: plain implicit GEMM over `map`; otherwise sorted mode.
   int (*igemm)(hipStream_t s, const void *x, const void *wp, const int32_t *map,
                int64_t n_map_rows, int64_t n_tile_rows, int64_t n_out, int kvol, int cin, int cout,
