@@ -1,0 +1,138 @@
+"""CPU-side checks: the C-ABI library loads and exports every symbol include/tsmi.h
+declares (no compute calls), and the host logic mirrors the reference's formulas."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "tsmi.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(tsmi_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    path = os.path.join(ROOT, "torchsparse_amd", "libtsmi.so")
+    assert os.path.exists(path), "build first: python torchsparse_amd/csrc/build.py"
+    lib = ctypes.CDLL(path)
+    names = _declared_symbols()
+    assert len(names) >= 30
+    for name in names:
+        assert hasattr(lib, name), f"{name} is declared in include/tsmi.h but not exported"
+    lib.tsmi_version.restype = ctypes.c_int
+    assert lib.tsmi_version() >= 1
+    lib.tsmi_last_error.restype = ctypes.c_char_p
+    assert lib.tsmi_last_error() == b""
+
+
+def test_host_side_argument_errors_without_gpu():
+    """Entry points validate sizes before touching the device."""
+    lib = ctypes.CDLL(os.path.join(ROOT, "torchsparse_amd", "libtsmi.so"))
+    lib.tsmi_last_error.restype = ctypes.c_char_p
+    lib.tsmi_packed_weight_elems.restype = ctypes.c_int64
+    assert lib.tsmi_packed_weight_elems(27, 96, 96) == 27 * 96 * 96
+    assert lib.tsmi_packed_weight_elems(27, 4, 19) == 27 * 32 * 32
+    assert lib.tsmi_packed_weight_elems(0, 4, 4) == -1
+    lib.tsmi_reduce_bitmask.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int64,
+                                        ctypes.c_int, ctypes.c_void_p]
+    assert lib.tsmi_reduce_bitmask(None, None, 1, 128, 6, None) == 2  # runtime_error in the reference
+    assert b"multiple of 4" in lib.tsmi_last_error()
+    lib.tsmi_hashtable_clear.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64]
+    assert lib.tsmi_hashtable_clear(None, None, None, 64) == 1
+    lib.tsmi_derive_bitmask.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int,
+                                        ctypes.c_int, ctypes.c_int64, ctypes.c_void_p]
+    assert lib.tsmi_derive_bitmask(None, None, 128, 125, 1, 100, None) == 1
+    assert b"32 mask bits" in lib.tsmi_last_error()
+
+
+def test_python_front_end_mirrors_reference_rules():
+    import torchsparse_amd as ts
+    from torchsparse_amd import nn as spnn
+    from torchsparse_amd.nn import functional as F
+    from torchsparse_amd.nn.functional.conv.kmap.build_kmap import _strided_range
+    from torchsparse_amd.nn.utils import get_kernel_offsets
+
+    # padding override (nn/modules/conv.py:42-48)
+    assert spnn.Conv3d(4, 4, 3, padding=0).padding == (1, 1, 1)
+    assert spnn.Conv3d(4, 4, (3, 1, 3), stride=(1, 1, 2), padding=(0, 5, 7)).padding == (1, 0, 7)
+    # kernel shapes and init bound (conv.py:56-66, 87-94)
+    assert spnn.Conv3d(8, 16, 3).kernel.shape == (27, 8, 16)
+    assert spnn.Conv3d(8, 16, 1).kernel.shape == (8, 16)
+    assert spnn.Conv3d(8, 16, 1, stride=2).kernel.shape == (1, 8, 16)
+    torch.manual_seed(0)
+    up = spnn.Conv3d(8, 16, 2, stride=2, transposed=True, bias=True)
+    assert float(up.kernel.detach().abs().max()) <= 1 / np.sqrt(16 * 8)
+    assert set(up.state_dict().keys()) == {"kernel", "bias"}
+    # strided spatial range (build_kmap.py:65-72)
+    assert _strided_range((2, 41, 1440, 1440), (3, 3, 3), (2, 2, 2), (1, 1, 1)) == (2, 21, 720, 720)
+    assert _strided_range((1, 5, 5, 5), (2, 2, 2), (2, 2, 2), (0, 0, 0)) == (1, 2, 2, 2)
+    assert _strided_range(None, (3, 3, 3), (1, 1, 1), (1, 1, 1)) is None
+    # offset tables equal the oracle's (nn/utils/kernel.py:21-35)
+    for size in (3, 2, 5, (3, 1, 1), (2, 3, 3), 4):
+        np.testing.assert_array_equal(get_kernel_offsets(size).numpy(), oracle.kernel_offsets(size))
+    np.testing.assert_array_equal(get_kernel_offsets(3, 2, 3).numpy(), oracle.kernel_offsets(3, 2, 3))
+    # config knobs
+    cfg = F.conv_config.get_default_conv_config()
+    assert cfg.dataflow == F.Dataflow.ImplicitGEMM and cfg["kmap_mode"] == "hashmap_on_the_fly"
+    assert (cfg.ifsort, cfg.split_mask_num, cfg.epsilon, cfg.mm_thresh, cfg.FOD_fusion) == (False, 1, 0.0, 0, True)
+    cfg.ifsort = True
+    assert F.conv_config.get_default_conv_config().ifsort is False  # copies, not one shared object
+    assert F.conv_config.get_default_conv_config(F.ConvMode.mode2).split_mask_num == 3
+    partial = F.conv_config.AttributeDict(dataflow=F.Dataflow.GatherScatter)
+    F.conv_config.set_global_conv_config(partial)
+    assert F.conv_config.get_global_conv_config()["epsilon"] == 0.0
+    F.conv_config.clear_global_conv_config()
+    with pytest.raises(AssertionError):
+        F.set_kmap_mode("grid")
+    F.set_conv_mode(1)
+    assert F.get_conv_mode() == F.ConvMode.mode1
+    F.set_conv_mode(0)
+    # tensor container and caches
+    x = ts.SparseTensor(torch.zeros(3, 2), torch.zeros(3, 4, dtype=torch.int32), stride=2)
+    assert x.stride == (2, 2, 2) and x.s == (2, 2, 2) and x.F is x.feats and x.C is x.coords
+    y = x + x
+    assert y._caches is x._caches
+    z = ts.cat([x, y])
+    assert z.feats.shape == (3, 4) and z._caches is x._caches
+    from torchsparse_amd.utils import TensorCacheMode, clear_global_tensor_cache, set_tensor_cache_mode
+    set_tensor_cache_mode(TensorCacheMode.GLOBAL_TENSOR_CACHE)
+    a = ts.SparseTensor(torch.zeros(1, 1), torch.zeros(1, 4, dtype=torch.int32))
+    b = ts.SparseTensor(torch.zeros(1, 1), torch.zeros(1, 4, dtype=torch.int32))
+    assert a._caches is b._caches
+    set_tensor_cache_mode(TensorCacheMode.SEPARATE_TENSOR_CACHE)
+    clear_global_tensor_cache()
+    # no CPU path: convolutions refuse host tensors loudly
+    with pytest.raises(RuntimeError, match="GPU"):
+        spnn.Conv3d(2, 2, 3)(ts.SparseTensor(torch.zeros(3, 2), torch.zeros(3, 4, dtype=torch.int32)))
+
+
+def test_fuse_inference_on_cpu_modules():
+    """Folding is pure parameter arithmetic; check it against the unfused affine map."""
+    from torchsparse_amd import nn as spnn
+    from torchsparse_amd.nn.utils.fuse import _fold
+    torch.manual_seed(0)
+    conv, bn = spnn.Conv3d(5, 7, 3, bias=True), spnn.BatchNorm(7).eval()
+    bn.running_mean.normal_(); bn.running_var.uniform_(0.5, 2); bn.weight.data.uniform_(0.5, 2); bn.bias.data.normal_()
+    w0, b0 = conv.kernel.detach().clone(), conv.bias.detach().clone()
+    _fold(conv, bn)
+    g = bn.weight / torch.sqrt(bn.running_var + bn.eps)
+    torch.testing.assert_close(conv.kernel.detach(), w0 * g)
+    torch.testing.assert_close(conv.bias.detach(), (b0 - bn.running_mean) * g + bn.bias)
+
+
+def test_synthetic_workloads_are_seeded_and_sized():
+    from torchsparse_amd.utils.synthetic import lidar_scan_voxels, uniform_voxels
+    a, b = lidar_scan_voxels(seed=1), lidar_scan_voxels(seed=1)
+    np.testing.assert_array_equal(a, b)
+    assert 80_000 < len(a) < 100_000 and a.min() >= 0 and a.dtype == np.int32
+    assert len(np.unique(a, axis=0)) == len(a)
+    c = uniform_voxels(20000, 128, seed=0)
+    assert c.shape == (20000, 4) and len(np.unique(c, axis=0)) == 20000 and c[:, 1:].max() < 128

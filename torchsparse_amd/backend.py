@@ -87,8 +87,13 @@ def _check(status: int) -> None:
     raise RuntimeError(msg)
 
 
+_raw_stream = torch._C._cuda_getCurrentRawStream
+_cur_device = torch._C._cuda_getDevice
+
+
 def _stream() -> int:
-    return torch.cuda.current_stream().cuda_stream
+    """hipStream_t of torch's current stream on the current device (as an int)."""
+    return _raw_stream(_cur_device())
 
 
 def _ptr(t: Optional[torch.Tensor]):
@@ -462,8 +467,11 @@ def conv_forward_implicit_gemm_cuda(in_feats, kernel, out_in_map, num_out_feats,
         raise ValueError("num_out_channels does not match the kernel")
     y = torch.empty((num_out_feats, cout), dtype=x.dtype, device=x.device)
     code = _dtype_code(x)
-    ws_elems = _C.tsmi_conv_workspace_elems(num_out_feats, num_out_feats, kvol, 1, cin, cout, code, 0)
-    ws = torch.empty(ws_elems, dtype=torch.float32, device=x.device) if ws_elems > 0 else None
+    ws, ws_elems = None, 0
+    if num_out_feats < 65536:  # only maps with few row tiles use the offset split
+        ws_elems = _C.tsmi_conv_workspace_elems(num_out_feats, num_out_feats, kvol, 1, cin, cout, code, 0)
+        if ws_elems > 0:
+            ws = torch.empty(ws_elems, dtype=torch.float32, device=x.device)
     pb, pr = _epilogue_args(bias, residual, x, num_out_feats, cout)
     _check(_C.tsmi_conv_implicit_gemm(_stream(), _ptr(x), _ptr(wp), _ptr(out_in_map),
                                       out_in_map.shape[0], num_out_feats, kvol, cin, cout, code,
@@ -481,8 +489,11 @@ def conv_forward_implicit_gemm_sorted_cuda(in_feats, kernel, reorder_out_in_map,
     n_pad = reorder_out_in_map.shape[0]
     y = torch.empty((num_out_feats, cout), dtype=x.dtype, device=x.device)
     code = _dtype_code(x)
-    ws_elems = _C.tsmi_conv_workspace_elems(n_pad, num_out_feats, kvol, split, cin, cout, code, 1)
-    ws = torch.empty(ws_elems, dtype=torch.float32, device=x.device) if ws_elems > 0 else None
+    ws, ws_elems = None, 0
+    if split > 1 or n_pad < 65536:
+        ws_elems = _C.tsmi_conv_workspace_elems(n_pad, num_out_feats, kvol, split, cin, cout, code, 1)
+        if ws_elems > 0:
+            ws = torch.empty(ws_elems, dtype=torch.float32, device=x.device)
     pb, pr = _epilogue_args(bias, residual, x, num_out_feats, cout)
     _check(_C.tsmi_conv_implicit_gemm_sorted(_stream(), _ptr(x), _ptr(wp), _ptr(reorder_out_in_map),
                                              _ptr(reduced_mask), _ptr(reorder_loc), n_pad,

@@ -51,7 +51,7 @@ def conv3d(input: SparseTensor, weight: torch.Tensor,
     if config is None:
         config = _cfg.get_global_conv_config()
         if config is None:
-            config = _cfg.get_default_conv_config(conv_mode=get_conv_mode(), training=training)
+            config = _cfg._shared_default_config(get_conv_mode())
     dataflow = config["dataflow"]
     if dataflow == _cfg.Dataflow.CodedCSR:
         raise AssertionError("CodedCSR has not been integrated.")
@@ -64,7 +64,8 @@ def conv3d(input: SparseTensor, weight: torch.Tensor,
     caches = input._caches
     # the input's own level is registered too, so a transposed layer can return to a
     # level no earlier layer produced (the reference only registers outputs)
-    caches.cmaps.setdefault(input.stride, (coords, input.spatial_range))
+    if input.stride not in caches.cmaps:
+        caches.cmaps[input.stride] = (coords, input.spatial_range)
 
     if kernel_size == (1, 1, 1) and stride == (1, 1, 1) and dilation == (1, 1, 1):
         out_feats = feats.matmul(weight) if bias is None else torch.addmm(bias, feats, weight)
@@ -72,11 +73,11 @@ def conv3d(input: SparseTensor, weight: torch.Tensor,
             out_feats += residual
         if relu:
             out_feats = torch.relu_(out_feats)
-        output = SparseTensor(feats=out_feats, coords=coords, stride=input.stride,
-                              spatial_range=input.spatial_range)
+        output = SparseTensor._make(out_feats, coords, input.stride, input.spatial_range, caches)
     elif not transposed:
         key = (input.stride, kernel_size, stride, dilation)
-        out_stride = tuple(input.stride[a] * stride[a] for a in range(3))
+        ist = input.stride
+        out_stride = (ist[0] * stride[0], ist[1] * stride[1], ist[2] * stride[2])
         kmap = caches.kmaps.get(key)
         if kmap is None:
             in_hashmap = caches.hashmaps.get(input.stride)
@@ -91,8 +92,7 @@ def conv3d(input: SparseTensor, weight: torch.Tensor,
             caches.hashmaps.setdefault(input.stride, kmap["in_hashmap"])
             caches.hashmaps.setdefault(out_stride, kmap["out_hashmap"])
         out_feats = conv_fn.apply(feats, weight, kmap, config, False, bias, residual, relu)
-        output = SparseTensor(feats=out_feats, coords=kmap["coords"], stride=out_stride,
-                              spatial_range=kmap["spatial_range"])
+        output = SparseTensor._make(out_feats, kmap["coords"], out_stride, kmap["spatial_range"], caches)
     else:
         if generative:
             raise NotImplementedError("generative transposed convolution is not part of this build")
@@ -103,9 +103,8 @@ def conv3d(input: SparseTensor, weight: torch.Tensor,
                                     split_mask_num_bwd=config["split_mask_num_bwd"])
         out_feats = conv_fn.apply(feats, weight, kmap, config, True, bias, residual, relu)
         fine_coords, fine_range = caches.cmaps[fine_stride]
-        output = SparseTensor(feats=out_feats, coords=fine_coords, stride=fine_stride,
-                              spatial_range=fine_range)
+        output = SparseTensor._make(out_feats, fine_coords, fine_stride, fine_range, caches)
 
-    output._caches = caches
-    caches.cmaps.setdefault(output.stride, (output.coords, output.spatial_range))
+    if output.stride not in caches.cmaps:
+        caches.cmaps[output.stride] = (output.coords, output.spatial_range)
     return output

@@ -82,6 +82,18 @@ def clear_global_conv_config() -> None:
     _global_conv_config = None
 
 
+_SHARED_DEFAULTS = {}
+
+
+def _shared_default_config(conv_mode: ConvMode):
+    """One read-only default config per conv mode for conv3d's own use (never handed
+    to callers, never mutated)."""
+    cfg = _SHARED_DEFAULTS.get(conv_mode)
+    if cfg is None:
+        cfg = _SHARED_DEFAULTS[conv_mode] = get_default_conv_config(conv_mode)
+    return cfg
+
+
 def get_default_conv_config(conv_mode: ConvMode = ConvMode.mode0, training: bool = False):
     config = AttributeDict(_DEFAULTS)
     if conv_mode == ConvMode.mode1:

@@ -49,6 +49,15 @@ class SparseTensor:
     s = property(lambda self: self.stride,
                  lambda self, v: setattr(self, "stride", make_ntuple(v, ndim=3)))
 
+    @classmethod
+    def _make(cls, feats, coords, stride, spatial_range, caches) -> "SparseTensor":
+        """Constructor for already-normalised fields (used on the convolution path)."""
+        out = cls.__new__(cls)
+        out.feats, out.coords = feats, coords
+        out.stride, out.spatial_range = stride, spatial_range
+        out._caches = caches
+        return out
+
     def _like(self, feats: torch.Tensor) -> "SparseTensor":
         out = SparseTensor.__new__(SparseTensor)
         out.feats, out.coords = feats, self.coords

@@ -9,6 +9,8 @@ __all__ = ["make_ntuple", "make_tensor", "make_divisible"]
 
 def make_ntuple(x, ndim: int) -> Tuple[int, ...]:
     """int -> (x,)*ndim; list / tuple / tensor -> tuple of python ints of length ndim."""
+    if type(x) is tuple and len(x) == ndim:
+        return x
     if isinstance(x, torch.Tensor):
         x = x.reshape(-1).tolist()
     if isinstance(x, (list, tuple)):
