@@ -94,15 +94,16 @@ int tsmi_kmap_query(tsmi_stream_t s, const int64_t *keys, const int32_t *vals, i
  * Replaces coords.max(0).values (hashmap_on_the_fly.py:33). */
 int tsmi_coords_max(tsmi_stream_t s, const int32_t *coords, int64_t n, int32_t *out_max);
 
-/* Candidate output coordinates of a strided convolution, de-duplicated through
- * the (empty) OUTPUT table (keys, vals, cap): every distinct output is appended
- * once, packed as (b<<54 | x<<36 | y<<18 | z), to uniq_keys and counted in
- * counters[0]; counters[1] is set to 1 if the table overflowed.  `counters`
- * (device int32[2]) must be zero on entry.
+/* Candidate output coordinates of a strided convolution, de-duplicated by inserting
+ * them, packed as (b<<54 | x<<36 | y<<18 | z), into the (empty) OUTPUT table
+ * (keys, cap); vals are not touched.  counters[1] (device int32[2], zero on entry) is
+ * set to 1 if the table overflowed.
  *   mode 0: o = (in + pad + digit - (ks-1)) / stride where divisible and
  *           0 <= o <= out_max per axis — downsample_grid_kmap_stage1_specialized_fast
  *           (others/sparsemapping_cuda.cu:60-107) and get_output_coords_kernel
- *           (others/downsample_cuda.cu:62-141).
+ *           (others/downsample_cuda.cu:62-141).  When ks == stride and pad == 0 every
+ *           input has exactly one candidate, floor(in / stride), and one thread per
+ *           input is launched instead of one per (input, offset).
  *   mode 1: o = floor(in / stride), unbounded — spdownsample for stride in {1, ks}
  *           or "minkowski" mode (nn/functional/conv/kmap/downsample.py:30-37).
  * The bound is out_max_host[3] when in_max_dev is NULL, otherwise it is derived on
@@ -112,8 +113,17 @@ int tsmi_downsample_candidates(tsmi_stream_t s, const int32_t *in_coords, int64_
                                const int32_t ks[3], const int32_t stride[3],
                                const int32_t pad[3], const int32_t out_max_host[3],
                                const int32_t *in_max_dev, int mode, int64_t *keys,
-                               int64_t cap, int64_t *uniq_keys, int64_t uniq_cap,
-                               int32_t *counters);
+                               int64_t cap, int32_t *counters);
+
+/* Gather the non-empty slots of a table: stored_keys_out[0..count) = the stored keys
+ * (key + 1) in slot order, *count_out = their number (device int32).  Scratch:
+ * tsmi_sort_temp_bytes(cap).  Together with tsmi_sort_keys this is the de-duplicated,
+ * sorted candidate list torch::_unique returns (others/sparsemapping_cuda.cu:478);
+ * a stream compaction replaces the reference's one-atomic-per-candidate append
+ * (others/sparsemapping_cuda.cu:103-105). */
+int tsmi_hashtable_compact_keys(tsmi_stream_t s, const int64_t *keys, int64_t cap,
+                                int64_t *stored_keys_out, int32_t *count_out, void *temp,
+                                int64_t temp_bytes);
 
 /* Bytes of scratch tsmi_sort_keys / tsmi_argsort_desc need for n items. */
 int64_t tsmi_sort_temp_bytes(int64_t n);
@@ -123,8 +133,9 @@ int64_t tsmi_sort_temp_bytes(int64_t n);
 int tsmi_sort_keys(tsmi_stream_t s, const int64_t *keys_in, int64_t *keys_out, int64_t n,
                    int end_bit, void *temp, int64_t temp_bytes);
 
-/* Unpack sorted unique keys into out_coords int32[n_out,4] and store row+1 as the
- * value of each key in the OUTPUT table.  Replaces
+/* Unpack sorted unique STORED keys (key + 1, as tsmi_hashtable_compact_keys emits
+ * them) into out_coords int32[n_out,4] and store row+1 as the value of each key in
+ * the OUTPUT table.  Replaces
  * inverse_transform_coords_and_insert_kernel (others/sparsemapping_cuda.cu:44-57). */
 int tsmi_downsample_finalize(tsmi_stream_t s, const int64_t *sorted_keys, int64_t n_out,
                              const int64_t *keys, int32_t *vals, int64_t cap,

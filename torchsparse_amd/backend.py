@@ -42,8 +42,8 @@ def _load():
         "tsmi_hashtable_lookup_keys": [_vp, _vp, _vp, _i64, _vp, _i64, _vp],
         "tsmi_kmap_query": [_vp, _vp, _vp, _i64, _vp, _i64, _i64, _I3, _I3, _I3, _vp],
         "tsmi_coords_max": [_vp, _vp, _i64, _vp],
-        "tsmi_downsample_candidates": [_vp, _vp, _i64, _I3, _I3, _I3, _vp, _vp, _i32, _vp, _i64,
-                                       _vp, _i64, _vp],
+        "tsmi_downsample_candidates": [_vp, _vp, _i64, _I3, _I3, _I3, _vp, _vp, _i32, _vp, _i64, _vp],
+        "tsmi_hashtable_compact_keys": [_vp, _vp, _i64, _vp, _vp, _vp, _i64],
         "tsmi_sort_keys": [_vp, _vp, _vp, _i64, _i32, _vp, _i64],
         "tsmi_downsample_finalize": [_vp, _vp, _i64, _vp, _vp, _i64, _vp],
         "tsmi_transpose_map": [_vp, _vp, _i64, _i32, _vp, _i64],
@@ -246,7 +246,6 @@ def downsample_coords(coords: torch.Tensor, kernel_sizes, stride, padding, coord
             fan *= -(-k // s)
     cap = hash_capacity(n * min(fan, 2), rsv_ratio)
     table = GPUHashTable(cap, device=dev)
-    uniq = torch.empty(cap, dtype=torch.int64, device=dev)
     counters = table.counters  # zero on a fresh table
     in_max = None
     host_max = None
@@ -255,9 +254,15 @@ def downsample_coords(coords: torch.Tensor, kernel_sizes, stride, padding, coord
             host_max = _I3(*[int(v) for v in coords_max_host])
         else:
             in_max = coords_max(coords)
-    _check(_C.tsmi_downsample_candidates(_stream(), _ptr(coords), n, _I3(*ks), _I3(*st), _I3(*pd),
-                                         host_max, _ptr(in_max), mode, _ptr(table.keys), cap,
-                                         _ptr(uniq), cap, _ptr(counters)))
+    s = _stream()
+    _check(_C.tsmi_downsample_candidates(s, _ptr(coords), n, _I3(*ks), _I3(*st), _I3(*pd), host_max,
+                                         _ptr(in_max), mode, _ptr(table.keys), cap, _ptr(counters)))
+    # unique keys = the occupied slots of the table: compact, read the count back, sort
+    temp_bytes = _C.tsmi_sort_temp_bytes(cap)
+    scratch = torch.empty(2 * cap + temp_bytes // 8 + 1, dtype=torch.int64, device=dev)
+    uniq, sorted_keys, temp = scratch[:cap], scratch[cap:2 * cap], scratch[2 * cap:]
+    _check(_C.tsmi_hashtable_compact_keys(s, _ptr(table.keys), cap, _ptr(uniq), _ptr(counters),
+                                          _ptr(temp), temp_bytes))
     n_out, overflow = counters[:2].tolist()
     if overflow:
         raise ValueError(
@@ -266,12 +271,8 @@ def downsample_coords(coords: torch.Tensor, kernel_sizes, stride, padding, coord
             "torchsparse_amd.backends.hash_rsv_ratio=#Value")
     out_coords = torch.empty((n_out, 4), dtype=torch.int32, device=dev)
     if n_out > 0:
-        sorted_keys = torch.empty(n_out, dtype=torch.int64, device=dev)
-        temp_bytes = _C.tsmi_sort_temp_bytes(n_out)
-        temp = torch.empty(temp_bytes, dtype=torch.uint8, device=dev)
-        _check(_C.tsmi_sort_keys(_stream(), _ptr(uniq), _ptr(sorted_keys), n_out, 63, _ptr(temp),
-                                 temp_bytes))
-        _check(_C.tsmi_downsample_finalize(_stream(), _ptr(sorted_keys), n_out, _ptr(table.keys),
+        _check(_C.tsmi_sort_keys(s, _ptr(uniq), _ptr(sorted_keys), n_out, 63, _ptr(temp), temp_bytes))
+        _check(_C.tsmi_downsample_finalize(s, _ptr(sorted_keys), n_out, _ptr(table.keys),
                                            _ptr(table.vals), cap, _ptr(out_coords)))
     return out_coords, table
 

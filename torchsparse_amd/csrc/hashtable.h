@@ -58,7 +58,11 @@ __device__ __forceinline__ uint32_t table_insert(const TableView &t, unsigned lo
   const unsigned long long stored = key + 1;
   uint32_t slot = home_slot(t, key);
   for (uint32_t probe = 0; probe < t.cap; ++probe) {
-    unsigned long long prev = atomicCAS(&t.keys[slot], 0ULL, stored);
+    // A plain load first: device-scope atomics are an order of magnitude slower than
+    // loads here, and a slot never changes once it is non-empty, so only slots that
+    // read as empty (possibly stale) need the compare-and-swap.
+    unsigned long long prev = t.keys[slot];
+    if (prev == 0ULL) prev = atomicCAS(&t.keys[slot], 0ULL, stored);
     if (prev == 0ULL) {
       *fresh = true;
       return slot;

@@ -125,18 +125,19 @@ __global__ void coords_max_kernel(const int4 *coords, int64_t n, int32_t *out_ma
   }
 }
 
-// mode 0: thread per (input, offset); mode 1: thread per input.
+// mode 0: thread per (input, offset); modes 1 and 2: thread per input.
 __global__ void downsample_candidates_kernel(const int4 *in_coords, int64_t n_in, int64_t total,
                                              Geom g, int3 out_max_host, const int32_t *in_max_dev,
-                                             int mode, TableView t, unsigned long long *uniq,
-                                             int64_t uniq_cap, int32_t *counters) {
+                                             int mode, TableView t, int32_t *counters) {
   int64_t tid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (tid >= total) return;
   int b, x, y, z;
-  if (mode == 1) {
+  if (mode != 0) {
+    // one candidate per input: o = floor(in / stride).  mode 1 keeps it unbounded; mode 2
+    // is the strided-convolution rule specialised to kernel size == stride, zero padding
+    // (o*s <= in < o*s + k has exactly one solution), bounded like mode 0.
     int4 c = in_coords[tid];
     b = c.x;
-    // floor division (coordinates may not be negative here, but keep it exact)
     int v[3] = {c.y, c.z, c.w};
     int o[3];
 #pragma unroll
@@ -144,6 +145,12 @@ __global__ void downsample_candidates_kernel(const int4 *in_coords, int64_t n_in
       int q = v[a] / g.stride[a];
       if (v[a] % g.stride[a] != 0 && v[a] < 0) --q;
       o[a] = q;
+      if (mode == 2) {
+        int hi = in_max_dev
+                     ? (in_max_dev[1 + a] + 2 * g.pad[a] - (g.ks[a] - 1)) / g.stride[a]
+                     : (a == 0 ? out_max_host.x : (a == 1 ? out_max_host.y : out_max_host.z));
+        if (o[a] < 0 || o[a] > hi) return;
+      }
     }
     x = o[0];
     y = o[1];
@@ -179,27 +186,14 @@ __global__ void downsample_candidates_kernel(const int4 *in_coords, int64_t n_in
     counters[1] = 1;
     return;
   }
-  // append the new keys of this wavefront with one atomic for all of them
-  const unsigned long long fresh_mask = __ballot(fresh);
-  if (fresh) {
-    const int lane = threadIdx.x & 63;
-    const int leader = __ffsll((long long)fresh_mask) - 1;
-    int base = 0;
-    if (lane == leader) base = atomicAdd(&counters[0], __popcll(fresh_mask));
-    base = __shfl(base, leader);
-    const int pos = base + __popcll(fresh_mask & ((1ULL << lane) - 1ULL));
-    if (pos < uniq_cap)
-      uniq[pos] = key;
-    else
-      counters[1] = 1;
-  }
+  (void)fresh;
 }
 
 __global__ void downsample_finalize_kernel(const unsigned long long *sorted, int64_t n_out,
                                            TableView t, int4 *out_coords) {
   int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (r >= n_out) return;
-  unsigned long long key = sorted[r];
+  unsigned long long key = sorted[r] - 1ULL;  // the table stores key + 1
   int c[4];
   unpack_coords(key, c);
   out_coords[r] = make_int4(c[0], c[1], c[2], c[3]);
@@ -507,25 +501,28 @@ extern "C" int tsmi_downsample_candidates(tsmi_stream_t s, const int32_t *in_coo
                                           const int32_t ks[3], const int32_t stride[3],
                                           const int32_t pad[3], const int32_t out_max_host[3],
                                           const int32_t *in_max_dev, int mode, int64_t *keys,
-                                          int64_t cap, int64_t *uniq_keys, int64_t uniq_cap,
-                                          int32_t *counters) {
+                                          int64_t cap, int32_t *counters) {
   TableView t;
   Geom g;
   static int32_t dummy_vals;  // the de-duplication pass never touches vals
   if (int e = make_table(&t, keys, &dummy_vals, cap)) return e;
   if (int e = make_geom(&g, ks, stride, pad)) return e;
   TSMI_REQUIRE(mode == 0 || mode == 1, "downsample_candidates: mode must be 0 or 1");
+  // kernel size == stride and zero padding: every input has exactly one candidate
+  if (mode == 0 && ks[0] == stride[0] && ks[1] == stride[1] && ks[2] == stride[2] &&
+      pad[0] == 0 && pad[1] == 0 && pad[2] == 0)
+    mode = 2;
   TSMI_REQUIRE(n_in >= 0 && (n_in == 0 || in_coords), "downsample_candidates: bad coords");
-  TSMI_REQUIRE(uniq_keys && counters && uniq_cap >= 0, "downsample_candidates: null output");
+  TSMI_REQUIRE(counters, "downsample_candidates: null counters");
   TSMI_REQUIRE(mode == 1 || in_max_dev || out_max_host, "downsample_candidates: no output bound");
   if (n_in == 0) return TSMI_OK;
-  int64_t total = mode == 1 ? n_in : n_in * g.kvol;
+  int64_t total = mode != 0 ? n_in : n_in * g.kvol;
   TSMI_GRID_CHECK(total);
   int3 hm = make_int3(0, 0, 0);
   if (out_max_host) hm = make_int3(out_max_host[0], out_max_host[1], out_max_host[2]);
   hipLaunchKernelGGL(downsample_candidates_kernel, grid_for(total), dim3(kBlock), 0,
                      (hipStream_t)s, (const int4 *)in_coords, n_in, total, g, hm, in_max_dev, mode,
-                     t, (unsigned long long *)uniq_keys, uniq_cap, counters);
+                     t, counters);
   return check_launch("tsmi_downsample_candidates");
 }
 
