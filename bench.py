@@ -42,6 +42,9 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-layers", action="store_true", help="skip the single-layer sweep")
     ap.add_argument("--no-roofline", action="store_true", help="skip the per-kernel roofline timing")
+    ap.add_argument("--pmc-target", action="store_true",
+                    help="run only a 256 MiB device copy (5 launches) and the roofline kernel "
+                         "(5 launches), for a hardware-counter pass; prints the kernel's description")
     ap.add_argument("--sorted", type=int, default=-1,
                     help="1: run the implicit GEMM over row-sorted maps (conv_mode 1); 0: unsorted; "
                          "-1: the default of this benchmark")
@@ -79,6 +82,16 @@ def kmap_bytes_subm(n, n_pad, cap, kvol):
 def kmap_bytes_down(n, n_out, n_out_pad, cap, cand, kvol):
     return (16.0 * n + 16.0 * cand + 12.0 * cap + 12.0 * n_out + 16.0 * n_out + 12.0 * cand
             + 4.0 * kvol * n_out_pad)
+
+
+# HBM bytes per launch of the roofline kernel from hardware counters (FETCH_SIZE and
+# WRITE_SIZE passes of `rocprofv3 --pmc ... -- python bench.py --pmc-target`, each scaled
+# by what the same counter reads for the 256 MiB copy of that run), keyed by the kernel
+# description this script prints.  None when the kernel that dominates has not been
+# measured that way.
+PMC_TRAFFIC_BYTES = {
+    "igemm k(3, 3, 3) s(1, 1, 1) 256->256 level(8, 8, 8) n_out=8045 nnz=52857": 105601226,
+}
 
 
 def roofline_of(flops, nbytes, ms):
@@ -169,7 +182,7 @@ def network_layers(model, inp):
     return records, out
 
 
-def dominant_layer_roofline(ts, F, records, caches):
+def dominant_layer_roofline(ts, F, records, caches, pmc_target=False):
     """Group the network's conv launches by (level, geometry, channels), time each
     group's kernel alone with HIP events on the launch stream, and report the roofline
     of the group with the largest total time."""
@@ -189,17 +202,30 @@ def dominant_layer_roofline(ts, F, records, caches):
         omap = km["out_in_map_t"] if transposed else km["out_in_map"]
         x = torch.randn(r["n_in"], cin, device="cuda", dtype=torch.float16)
         w = r["mod"].kernel.detach()
-        ms = event_ms(lambda: backend.conv_forward_implicit_gemm_cuda(x, w, omap, r["n_out"], cout),
-                      iters=30, warm=5)
+        run = (lambda x=x, w=w, omap=omap, n_out=r["n_out"], cout=cout:
+               backend.conv_forward_implicit_gemm_cuda(x, w, omap, n_out, cout))
+        ms = event_ms(run, iters=30, warm=5)
         total = ms * len(rs)
         if best is None or total > best["total_ms"]:
             kvol = ks[0] * ks[1] * ks[2]
             nnz = int((omap[:r["n_out"]] >= 0).sum().item())
             flops, nbytes = conv_work(r["n_in"], r["n_out"], omap.shape[0], nnz, kvol, cin, cout, 2)
             best = {"total_ms": total, "ms": ms, "launches": len(rs), "flops": flops, "bytes": nbytes,
+                    "run": run,
                     "desc": f"igemm k{ks} s{stride} {'T ' if transposed else ''}{cin}->{cout} "
                             f"level{level} n_out={r['n_out']} nnz={nnz}"}
+    if pmc_target:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        for _ in range(5):
+            best["run"]()
+        torch.cuda.synchronize()
+        return {"kernel": best["desc"]}
     roof = roofline_of(best["flops"], best["bytes"], best["ms"])
+    roof["traffic"] = PMC_TRAFFIC_BYTES.get(best["desc"])
     roof["kernel"] = best["desc"]
     roof["launch_ms"] = round(best["ms"], 5)
     roof["launches_per_step"] = best["launches"]
@@ -291,6 +317,13 @@ def main():
             step()
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) * 1e3 / steps
+
+    if args.pmc_target:
+        with torch.no_grad():
+            inp = ts.SparseTensor(feats, coords)
+            records, _ = network_layers(model, inp)
+            print(json.dumps(dominant_layer_roofline(ts, F, records, inp._caches, pmc_target=True)))
+        return
 
     ms_per_step = timed(model, args.steps, args.warmup)
     ms_unfused = timed(unfused, max(args.steps // 2, 1), 2)
