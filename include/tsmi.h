@@ -227,6 +227,12 @@ int64_t tsmi_conv_workspace_elems(int64_t n_tile_rows, int64_t n_out, int kvol, 
 /* Y[i,:] = sum_k [m = map[i,k] >= 0] X[m,:] W[k] (+ bias) for i < n_out; every
  * output row is written.  `map` has at least n_out rows.  `workspace` (float
  * [workspace_elems], may be NULL) enables the offset split described above.
+ * `tile_counters` (int32 [n_tile_counters], may be NULL) lets the workgroup that
+ * finishes a tile's last partial sum add them up itself instead of a second
+ * launch: the array must be all zero on entry and is all zero again when the
+ * launch completes, so one zero-filled array can serve every call on a stream
+ * (calls that overlap on the GPU must not share it); 4096 entries cover every
+ * problem that is split.
  * Epilogue, shared by every convolution entry point: y = act(sum + bias +
  * residual), with bias [cout] and residual [n_out, cout] of the I/O type (either
  * may be NULL) and act = max(., 0) when relu != 0 — the bias add of
@@ -237,12 +243,14 @@ int64_t tsmi_conv_workspace_elems(int64_t n_tile_rows, int64_t n_out, int kvol, 
 int tsmi_conv_implicit_gemm(tsmi_stream_t s, const void *x, const void *w_packed,
                             const int32_t *map, int64_t n_map_rows, int64_t n_out, int kvol,
                             int cin, int cout, int dtype, const void *bias, const void *residual,
-                            int relu, float *workspace, int64_t workspace_elems, void *y);
+                            int relu, float *workspace, int64_t workspace_elems,
+                            int32_t *tile_counters, int64_t n_tile_counters, void *y);
 
 /* Same sum over a row-sorted map: tile row r of split s reads
  * reorder_map[r, s*L..] and adds into output row reorder_loc[s, r].
  * `workspace` (tsmi_conv_workspace_elems floats; required for split > 1) receives
- * the per-split fp32 sums, which are then added into y.  reduced_mask may be NULL
+ * the per-split fp32 sums, which are then added into y; tile_counters as above
+ * (used when split == 1).  reduced_mask may be NULL
  * (the kernel derives its skipping from the map itself).  Replaces
  * conv_forward_implicit_gemm_sorted_cuda
  * (convolution/convolution_forward_implicit_gemm_sorted_cuda.cu:1755-2230). */
@@ -251,7 +259,8 @@ int tsmi_conv_implicit_gemm_sorted(tsmi_stream_t s, const void *x, const void *w
                                    const int32_t *reorder_loc, int64_t n_pad, int64_t n_out,
                                    int kvol, int split, int cin, int cout, int dtype,
                                    const void *bias, const void *residual, int relu,
-                                   float *workspace, int64_t workspace_elems, void *y);
+                                   float *workspace, int64_t workspace_elems,
+                                   int32_t *tile_counters, int64_t n_tile_counters, void *y);
 
 /* Fetch-on-demand: one launch over 128-padded pair lists gathers X rows, multiplies
  * by W[k] and writes partial[qnbaddrs[k] + p, :] (fp32 for TSMI_F32, else the I/O

@@ -44,7 +44,7 @@ def _f32(t):
 
 
 CHANNELS = [(32, 32), (64, 64), (128, 128), (4, 32), (5, 16), (16, 16), (96, 96), (128, 96),
-            (24, 40), (32, 19), (7, 3), (192, 256)]
+            (24, 40), (32, 19), (7, 3), (192, 256), (96, 160), (64, 128), (256, 130)]
 
 
 @pytest.mark.parametrize("cin,cout", CHANNELS)
@@ -285,3 +285,38 @@ def test_fuse_inference_matches_unfused_unet(mods):
         # and in half precision, against the fp32 network
         got16 = copy.deepcopy(fused).half()(ts.SparseTensor(x.half(), coords))
         assert rel_rms(_f32(got16[-1].feats), _f32(ref[-1].feats)) < 3e-2
+
+
+@pytest.mark.parametrize("cin,cout", [(64, 64), (128, 128), (96, 160), (256, 256)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_offset_split_sums_in_kernel_equal_second_launch(mods, cin, cout, dtype):
+    """Small maps split the kernel offsets over several workgroups.  With tile counters
+    the last workgroup of a tile adds the partial sums; without, a second launch does.
+    Both add in split order, so the results are bit-identical; the counters are left
+    zero, and a second call on the same counters gives the same result."""
+    _, backend, _, F = mods
+    rng = np.random.default_rng(cin + cout)
+    coords = random_coords(rng, 4000, (24, 24, 16))
+    n = len(coords)
+    kmap = F.build_kernel_map(dev(coords), n, 3, 1, 1, mode="hashmap_on_the_fly")
+    omap = kmap["out_in_map"]
+    x, w = _case(rng, n, cin, cout, 27, dtype)
+    wp = backend.pack_weights(w)
+    code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype]
+    C, ptr = backend._C, backend._ptr
+    ws_elems = C.tsmi_conv_workspace_elems(n, n, 27, 1, cin, cout, code, 0)
+    assert ws_elems > 0  # this size is split
+    ws = torch.empty(ws_elems, dtype=torch.float32, device="cuda")
+    counters = torch.zeros(4096, dtype=torch.int32, device="cuda")
+    bias = torch.from_numpy(rng.standard_normal(cout).astype(np.float32)).to("cuda", dtype)
+    outs = []
+    for cnt in (None, counters, counters):
+        y = torch.full((n, cout), float("nan"), dtype=dtype, device="cuda")
+        backend._check(C.tsmi_conv_implicit_gemm(backend._stream(), ptr(x), ptr(wp), ptr(omap), omap.shape[0],
+                                                 n, 27, cin, cout, code, ptr(bias), None, 1, ptr(ws),
+                                                 ws_elems, ptr(cnt), 4096, ptr(y)))
+        outs.append(y)
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[1], outs[2])
+    assert int(counters.abs().sum().item()) == 0
+    want = np.maximum(oracle.conv_implicit_gemm(_f32(x), _f32(w), omap.cpu().numpy(), n) + _f32(bias), 0)
+    assert rel_rms(_f32(outs[1]), want) < TOL[dtype]

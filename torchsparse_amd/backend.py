@@ -57,9 +57,10 @@ def _load():
         "tsmi_build_masks": [_vp, _vp, _i64, _vp, _i32, _i64, _i64, _vp, _vp],
         "tsmi_pack_weights": [_vp, _vp, _vp, _i32, _i32, _i32, _i32],
         "tsmi_conv_implicit_gemm": [_vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _i32, _i32, _vp, _vp,
-                                    _i32, _vp, _i64, _vp],
+                                    _i32, _vp, _i64, _vp, _i64, _vp],
         "tsmi_conv_implicit_gemm_sorted": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32,
-                                           _i32, _i32, _i32, _vp, _vp, _i32, _vp, _i64, _vp],
+                                           _i32, _i32, _i32, _vp, _vp, _i32, _vp, _i64, _vp, _i64,
+                                           _vp],
         "tsmi_conv_fetch_on_demand": [_vp, _vp, _vp, _vp, _i64, _vp, _vp, _i64, _vp, _i64, _i32,
                                       _i32, _i32, _i32, _i32, _i32, _vp, _vp, _i32, _vp, _vp],
         "tsmi_gs_gather": [_vp, _vp, _vp, _i64, _i32, _i32, _i32, _vp],
@@ -457,6 +458,20 @@ def _epilogue_args(bias, residual, x, n_out, cout):
     return _ptr(bias), _ptr(residual)
 
 
+_TILE_COUNTERS = {}
+_N_TILE_COUNTERS = 4096
+
+
+def _tile_counters(device):
+    """Zero-filled int32 array shared by the split convolutions of one stream (each
+    launch leaves it zero again)."""
+    key = (device.index, _stream())
+    t = _TILE_COUNTERS.get(key)
+    if t is None:
+        t = _TILE_COUNTERS[key] = torch.zeros(_N_TILE_COUNTERS, dtype=torch.int32, device=device)
+    return t
+
+
 def conv_forward_implicit_gemm_cuda(in_feats, kernel, out_in_map, num_out_feats, num_out_channels,
                                     allow_tf32=False, allow_fp16=True, bias=None, residual=None,
                                     relu=False) -> torch.Tensor:
@@ -476,7 +491,9 @@ def conv_forward_implicit_gemm_cuda(in_feats, kernel, out_in_map, num_out_feats,
     pb, pr = _epilogue_args(bias, residual, x, num_out_feats, cout)
     _check(_C.tsmi_conv_implicit_gemm(_stream(), _ptr(x), _ptr(wp), _ptr(out_in_map),
                                       out_in_map.shape[0], num_out_feats, kvol, cin, cout, code,
-                                      pb, pr, int(relu), _ptr(ws), ws_elems, _ptr(y)))
+                                      pb, pr, int(relu), _ptr(ws), ws_elems,
+                                      _ptr(_tile_counters(x.device)) if ws is not None else None,
+                                      _N_TILE_COUNTERS, _ptr(y)))
     return y
 
 
@@ -499,7 +516,9 @@ def conv_forward_implicit_gemm_sorted_cuda(in_feats, kernel, reorder_out_in_map,
     _check(_C.tsmi_conv_implicit_gemm_sorted(_stream(), _ptr(x), _ptr(wp), _ptr(reorder_out_in_map),
                                              _ptr(reduced_mask), _ptr(reorder_loc), n_pad,
                                              num_out_feats, kvol, split, cin, cout, code,
-                                             pb, pr, int(relu), _ptr(ws), ws_elems, _ptr(y)))
+                                             pb, pr, int(relu), _ptr(ws), ws_elems,
+                                      _ptr(_tile_counters(x.device)) if ws is not None else None,
+                                      _N_TILE_COUNTERS, _ptr(y)))
     return y
 
 

@@ -51,7 +51,8 @@ extern "C" int tsmi_conv_implicit_gemm(tsmi_stream_t s, const void *x, const voi
                                        const int32_t *map, int64_t n_map_rows, int64_t n_out,
                                        int kvol, int cin, int cout, int dtype, const void *bias,
                                        const void *residual, int relu, float *workspace,
-                                       int64_t workspace_elems, void *y) {
+                                       int64_t workspace_elems, int32_t *tile_counters,
+                                       int64_t n_tile_counters, void *y) {
   const ConvOps *ops = ops_for(dtype);
   if (int e = check_shapes("conv_implicit_gemm", ops, kvol, cin, cout)) return e;
   TSMI_REQUIRE(n_out >= 0 && n_map_rows >= n_out, "conv_implicit_gemm: map has %lld rows, need %lld",
@@ -61,7 +62,8 @@ extern "C" int tsmi_conv_implicit_gemm(tsmi_stream_t s, const void *x, const voi
   TSMI_REQUIRE(aligned16(x) && aligned16(w_packed) && aligned16(y),
                "conv_implicit_gemm: x, w_packed and y must be 16-byte aligned");
   return ops->igemm((hipStream_t)s, x, w_packed, map, n_map_rows, n_out, n_out, kvol, cin, cout,
-                    bias, residual, relu, y, nullptr, 0, 1, workspace, workspace_elems);
+                    bias, residual, relu, y, nullptr, 0, 1, workspace, workspace_elems,
+                    tile_counters, tile_counters ? n_tile_counters : 0);
 }
 
 extern "C" int tsmi_conv_implicit_gemm_sorted(tsmi_stream_t s, const void *x, const void *w_packed,
@@ -71,6 +73,7 @@ extern "C" int tsmi_conv_implicit_gemm_sorted(tsmi_stream_t s, const void *x, co
                                               int64_t n_out, int kvol, int split, int cin, int cout,
                                               int dtype, const void *bias, const void *residual,
                                               int relu, float *workspace, int64_t workspace_elems,
+                                              int32_t *tile_counters, int64_t n_tile_counters,
                                               void *y) {
   (void)reduced_mask;  // tile skipping is derived from the staged map itself
   const ConvOps *ops = ops_for(dtype);
@@ -86,7 +89,8 @@ extern "C" int tsmi_conv_implicit_gemm_sorted(tsmi_stream_t s, const void *x, co
   TSMI_REQUIRE(aligned16(x) && aligned16(w_packed) && aligned16(y),
                "conv_implicit_gemm_sorted: x, w_packed and y must be 16-byte aligned");
   return ops->igemm((hipStream_t)s, x, w_packed, reorder_map, n_pad, n_pad, n_out, kvol, cin, cout,
-                    bias, residual, relu, y, reorder_loc, n_pad, split, workspace, workspace_elems);
+                    bias, residual, relu, y, reorder_loc, n_pad, split, workspace, workspace_elems,
+                    tile_counters, tile_counters ? n_tile_counters : 0);
 }
 
 extern "C" int tsmi_conv_fetch_on_demand(tsmi_stream_t s, const void *x, const void *w_packed,

@@ -33,6 +33,8 @@ struct TraitsBF16 {
 #define TSMI_TRAITS TraitsBF16
 #define TSMI_SUFFIX bf16
 #include "conv_igemm.inc"
+#include "conv_tile.inc"
+#include "conv_plan.inc"
 #include "conv_igemm_tail.inc"
 
 namespace tsmi {

@@ -30,6 +30,8 @@ struct TraitsF16 {
 #define TSMI_TRAITS TraitsF16
 #define TSMI_SUFFIX f16
 #include "conv_igemm.inc"
+#include "conv_tile.inc"
+#include "conv_plan.inc"
 #include "conv_igemm_tail.inc"
 
 namespace tsmi {

@@ -33,6 +33,8 @@ struct TraitsF32 {
 #define TSMI_TRAITS TraitsF32
 #define TSMI_SUFFIX f32
 #include "conv_igemm.inc"
+#include "conv_tile.inc"
+#include "conv_plan.inc"
 #include "conv_igemm_tail.inc"
 
 namespace tsmi {

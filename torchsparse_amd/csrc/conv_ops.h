@@ -20,7 +20,8 @@ struct ConvOps {
   int (*igemm)(hipStream_t s, const void *x, const void *wp, const int32_t *map,
                int64_t n_map_rows, int64_t n_tile_rows, int64_t n_out, int kvol, int cin, int cout,
                const void *bias, const void *residual, int relu, void *y, const int32_t *row_out,
-               int64_t row_out_stride, int split, float *partial, int64_t partial_elems);
+               int64_t row_out_stride, int split, float *partial, int64_t partial_elems,
+               int32_t *counters, int64_t n_counters);
   // out[nbaddrs[k] + p, :] = X[rows[nbaddrs[k] + p], :] W[k] over 128-padded pair lists
   int (*pairs)(hipStream_t s, const void *x, const void *wp, const int32_t *rows,
                const int32_t *nbaddrs, const int32_t *qnbaddrs, int64_t qnnz, int kvol, int cin,
