@@ -1,0 +1,161 @@
+"""The benchmark configurations at their full sizes.
+
+The 20k-voxel fp32 layer is small enough for the CPU oracle to check every output.
+The detection backbone (two merged multi-sweep samples) and the ~1M-voxel 256->256
+layer are checked through properties that do not need a full CPU run: map symmetry,
+sortedness and uniqueness of generated coordinates, batch independence, linearity,
+and oracle values on a random sample of output rows."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import rel_rms
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def mods():
+    import torchsparse_amd as ts
+    from torchsparse_amd import backend
+    from torchsparse_amd import nn as spnn
+    from torchsparse_amd.nn import functional as F
+    from torchsparse_amd.utils import synthetic
+    return ts, backend, spnn, F, synthetic
+
+
+def _rows_expected(x, w, omap_rows):
+    """sum_k X[map[i,k]] W[k] for the given map rows, float64 accumulation."""
+    out = np.zeros((omap_rows.shape[0], w.shape[2]), dtype=np.float64)
+    for k in range(w.shape[0]):
+        m = omap_rows[:, k]
+        ok = m >= 0
+        if ok.any():
+            out[ok] += x[m[ok]].astype(np.float64) @ w[k].astype(np.float64)
+    return out
+
+
+def test_single_layer_20k_voxels_fp32_matches_oracle(mods):
+    ts, backend, spnn, F, synthetic = mods
+    coords = synthetic.uniform_voxels(20000, extent=128, seed=0)
+    rng = np.random.default_rng(0)
+    feats = rng.standard_normal((20000, 32)).astype(np.float32)
+    torch.manual_seed(0)
+    layer = spnn.Conv3d(32, 32, 3).cuda()
+    x = ts.SparseTensor(torch.from_numpy(feats).cuda(), torch.from_numpy(coords).cuda())
+    for flow in (F.Dataflow.ImplicitGEMM, F.Dataflow.GatherScatter, F.Dataflow.FetchOnDemand):
+        cfg = F.conv_config.get_default_conv_config()
+        cfg.dataflow = flow
+        xi = ts.SparseTensor(x.feats, x.coords)
+        y = F.conv3d(xi, layer.kernel, kernel_size=3, padding=1, config=cfg)
+        want_map = oracle.kmap_subm(coords, (3, 3, 3))
+        key = ((1, 1, 1), (3, 3, 3), (1, 1, 1), (1, 1, 1))
+        if flow == F.Dataflow.ImplicitGEMM:
+            got_map = xi._caches.kmaps[key]["out_in_map"].cpu().numpy()
+            np.testing.assert_array_equal(got_map[:20000], want_map[:20000])
+            assert (got_map[20000:] == -1).all() and got_map.shape[0] == 20096
+        want = oracle.conv_implicit_gemm(feats, layer.kernel.detach().cpu().numpy(), want_map, 20000)
+        assert rel_rms(y.feats.detach().cpu().numpy(), want) < 1e-4, flow
+        assert torch.equal(y.coords, x.coords)
+
+
+def test_detection_backbone_batch_of_two(mods):
+    ts, backend, spnn, F, synthetic = mods
+    from torchsparse_amd.backbones import VoxelResBackBone8x
+    coords_np, spatial_range = synthetic.multisweep_voxels(seed=2)
+    n = coords_np.shape[0]
+    assert coords_np[:, 0].max() == 1 and n > 100000
+    torch.manual_seed(1)
+    net = VoxelResBackBone8x(in_channels=5).cuda().half().eval()
+    feats = torch.randn(n, 5, device="cuda", dtype=torch.float16)
+    coords = torch.from_numpy(coords_np).cuda()
+    with torch.no_grad():
+        both = net(ts.SparseTensor(feats, coords, spatial_range=spatial_range))
+        singles = []
+        for b in (0, 1):
+            sel = coords[:, 0] == b
+            c = coords[sel].clone()
+            c[:, 0] = 0
+            singles.append(net(ts.SparseTensor(feats[sel], c, spatial_range=(1,) + tuple(spatial_range[1:]))))
+    for name, out in both.items():
+        oc = out.coords.cpu().numpy()
+        # generated coordinates: unique, ascending (b, x, y, z) for the strided levels
+        assert len(np.unique(oc, axis=0)) == len(oc)
+        if name != "x_conv1":
+            key = ((oc[:, 0].astype(np.int64) << 54) | (oc[:, 1].astype(np.int64) << 36)
+                   | (oc[:, 2].astype(np.int64) << 18) | oc[:, 3].astype(np.int64))
+            assert (np.diff(key) > 0).all(), name
+        # batch independence: sample b of the batched run == the run on sample b alone
+        for b in (0, 1):
+            sel = out.coords[:, 0] == b
+            got_c = out.coords[sel].clone()
+            got_c[:, 0] = 0
+            assert torch.equal(got_c, singles[b][name].coords), name
+            got, want = out.feats[sel].float().cpu().numpy(), singles[b][name].feats.float().cpu().numpy()
+            # same sums; tile shapes and offset splits (so fp16 roundings of the
+            # intermediate activations) differ between the two problem sizes
+            assert rel_rms(got, want) < 1e-2, (name, b)
+    # one strided map of the batched input against the oracle, exactly
+    kmap = F.build_kernel_map(coords, n, 3, 2, 1, mode="hashmap_on_the_fly",
+                              spatial_range=spatial_range)
+    strided = (spatial_range[0],) + tuple((v + 2 - 2 - 1) // 2 + 1 for v in spatial_range[1:])
+    assert tuple(kmap["spatial_range"]) == strided
+    want_map, want_coords = oracle.kmap_downsample(coords_np, (3, 3, 3), (2, 2, 2), (1, 1, 1),
+                                                   spatial_range=strided)
+    np.testing.assert_array_equal(kmap["coords"].cpu().numpy(), want_coords)
+    got = kmap["out_in_map"].cpu().numpy()
+    np.testing.assert_array_equal(got[:len(want_coords)], want_map[:len(want_coords)])
+
+
+def test_million_voxel_256_channel_layer(mods):
+    ts, backend, spnn, F, synthetic = mods
+    coords_np = synthetic.sphere_shell_voxels(seed=3)
+    n = coords_np.shape[0]
+    assert n > 900000
+    coords = torch.from_numpy(coords_np).cuda()
+    kmap = F.build_kernel_map(coords, n, 3, 1, 1, mode="hashmap_on_the_fly")
+    omap = kmap["out_in_map"]
+    assert omap.shape == ((n + 127) // 128 * 128, 27)
+    m = omap[:n]
+    # map properties: centre is the identity, and j is i's neighbour at offset k iff i is
+    # j's neighbour at the mirrored offset 26-k
+    assert torch.equal(m[:, 13], torch.arange(n, device="cuda", dtype=torch.int32))
+    for k in (0, 5, 12):
+        i = torch.nonzero(m[:, k] >= 0).squeeze(1)
+        j = m[i, k].long()
+        assert torch.equal(m[j, 26 - k].long(), i)
+    assert (omap[n:] == -1).all()
+    # a sample of rows against a dictionary of the coordinates
+    rng = np.random.default_rng(5)
+    rows = rng.choice(n, 3000, replace=False)
+    lut = {tuple(c): i for i, c in enumerate(coords_np.tolist())}
+    offs = oracle.kernel_offsets((3, 3, 3))
+    got_rows = m[torch.from_numpy(rows).cuda()].cpu().numpy()
+    for r, g in zip(rows[:300], got_rows[:300]):
+        b, x, y, z = coords_np[r]
+        want = [lut.get((b, x + o[0], y + o[1], z + o[2]), -1) for o in offs]
+        assert g.tolist() == want
+
+    torch.manual_seed(2)
+    x1 = torch.randn(n, 256, device="cuda", dtype=torch.float16)
+    w = (torch.rand(27, 256, 256, device="cuda") * 2 - 1).mul_(1 / np.sqrt(256 * 27)).half()
+    y1 = backend.conv_forward_implicit_gemm_cuda(x1, w, omap, n, 256)
+    # sampled rows against a float64 evaluation of the definition
+    want = _rows_expected(x1.float().cpu().numpy(), w.float().cpu().numpy(), got_rows)
+    got = y1[torch.from_numpy(rows).cuda()].float().cpu().numpy()
+    assert rel_rms(got, want) < 1e-2
+    # linearity in the features (power-of-two scale: exact in fp16)
+    x2 = torch.randn(n, 256, device="cuda", dtype=torch.float16)
+    y2 = backend.conv_forward_implicit_gemm_cuda(x2, w, omap, n, 256)
+    y12 = backend.conv_forward_implicit_gemm_cuda((2 * x1 + x2), w, omap, n, 256)
+    lin = 2 * y1.float() + y2.float()
+    assert rel_rms(y12.float().cpu().numpy(), lin.cpu().numpy()) < 1e-2
+    # the three dataflows agree at this size
+    cfg_rows = torch.from_numpy(rows).cuda()
+    for flow in (F.Dataflow.FetchOnDemand, F.Dataflow.GatherScatter):
+        cfg = F.conv_config.get_default_conv_config()
+        cfg.dataflow = flow
+        xi = ts.SparseTensor(x1, coords)
+        y = F.conv3d(xi, w, kernel_size=3, padding=1, config=cfg).feats
+        assert rel_rms(y[cfg_rows].float().cpu().numpy(), want) < 1e-2, flow
