@@ -31,6 +31,7 @@ struct TraitsF16 {
 #define TSMI_SUFFIX f16
 #include "conv_igemm.inc"
 #include "conv_tile.inc"
+#include "conv_igemm2.inc"
 #include "conv_plan.inc"
 #include "conv_igemm_tail.inc"
 

@@ -34,6 +34,7 @@ struct TraitsF32 {
 #define TSMI_SUFFIX f32
 #include "conv_igemm.inc"
 #include "conv_tile.inc"
+#include "conv_igemm2.inc"
 #include "conv_plan.inc"
 #include "conv_igemm_tail.inc"
 
