@@ -91,8 +91,10 @@ int tsmi_kmap_query(tsmi_stream_t s, const int64_t *keys, const int32_t *vals, i
                     int32_t *out_in_map);
 
 /* Per-column maximum of coords -> out_max int32[4] (device).  n may be 0 (result 0).
+ * clear_first = 0 when out_max already holds zeros (saves the fill launch).
  * Replaces coords.max(0).values (hashmap_on_the_fly.py:33). */
-int tsmi_coords_max(tsmi_stream_t s, const int32_t *coords, int64_t n, int32_t *out_max);
+int tsmi_coords_max(tsmi_stream_t s, const int32_t *coords, int64_t n, int32_t *out_max,
+                    int clear_first);
 
 /* Candidate output coordinates of a strided convolution, de-duplicated by inserting
  * them, packed as (b<<54 | x<<36 | y<<18 | z), into the (empty) OUTPUT table
@@ -116,14 +118,13 @@ int tsmi_downsample_candidates(tsmi_stream_t s, const int32_t *in_coords, int64_
                                int64_t cap, int32_t *counters);
 
 /* Gather the non-empty slots of a table: stored_keys_out[0..count) = the stored keys
- * (key + 1) in slot order, *count_out = their number (device int32).  Scratch:
- * tsmi_sort_temp_bytes(cap).  Together with tsmi_sort_keys this is the de-duplicated,
- * sorted candidate list torch::_unique returns (others/sparsemapping_cuda.cu:478);
- * a stream compaction replaces the reference's one-atomic-per-candidate append
+ * (key + 1) in arbitrary order, *count_out (device int32, zero on entry) += their
+ * number.  Together with tsmi_sort_keys this is the de-duplicated, sorted candidate
+ * list torch::_unique returns (others/sparsemapping_cuda.cu:478); a compaction with
+ * one atomic per workgroup replaces the reference's one-atomic-per-candidate append
  * (others/sparsemapping_cuda.cu:103-105). */
 int tsmi_hashtable_compact_keys(tsmi_stream_t s, const int64_t *keys, int64_t cap,
-                                int64_t *stored_keys_out, int32_t *count_out, void *temp,
-                                int64_t temp_bytes);
+                                int64_t *stored_keys_out, int32_t *count_out);
 
 /* Bytes of scratch tsmi_sort_keys / tsmi_argsort_desc need for n items. */
 int64_t tsmi_sort_temp_bytes(int64_t n);

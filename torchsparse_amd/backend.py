@@ -41,9 +41,9 @@ def _load():
         "tsmi_hashtable_insert_keys": [_vp, _vp, _vp, _i64, _vp, _i64, _vp],
         "tsmi_hashtable_lookup_keys": [_vp, _vp, _vp, _i64, _vp, _i64, _vp],
         "tsmi_kmap_query": [_vp, _vp, _vp, _i64, _vp, _i64, _i64, _I3, _I3, _I3, _vp],
-        "tsmi_coords_max": [_vp, _vp, _i64, _vp],
+        "tsmi_coords_max": [_vp, _vp, _i64, _vp, _i32],
         "tsmi_downsample_candidates": [_vp, _vp, _i64, _I3, _I3, _I3, _vp, _vp, _i32, _vp, _i64, _vp],
-        "tsmi_hashtable_compact_keys": [_vp, _vp, _i64, _vp, _vp, _vp, _i64],
+        "tsmi_hashtable_compact_keys": [_vp, _vp, _i64, _vp, _vp],
         "tsmi_sort_keys": [_vp, _vp, _vp, _i64, _i32, _vp, _i64],
         "tsmi_downsample_finalize": [_vp, _vp, _i64, _vp, _vp, _i64, _vp],
         "tsmi_transpose_map": [_vp, _vp, _i64, _i32, _vp, _i64],
@@ -225,7 +225,7 @@ def coords_max(coords: torch.Tensor) -> torch.Tensor:
     """Device int32[4] per-column maximum (no host synchronisation)."""
     coords = _need(coords, torch.int32, "coords")
     out = torch.empty(4, dtype=torch.int32, device=coords.device)
-    _check(_C.tsmi_coords_max(_stream(), _ptr(coords), coords.shape[0], _ptr(out)))
+    _check(_C.tsmi_coords_max(_stream(), _ptr(coords), coords.shape[0], _ptr(out), 1))
     return out
 
 
@@ -254,7 +254,8 @@ def downsample_coords(coords: torch.Tensor, kernel_sizes, stride, padding, coord
         if coords_max_host is not None:
             host_max = _I3(*[int(v) for v in coords_max_host])
         else:
-            in_max = coords_max(coords)
+            in_max = counters[4:8]  # still zero: the maximum lands here without a fill launch
+            _check(_C.tsmi_coords_max(_stream(), _ptr(coords), n, _ptr(in_max), 0))
     s = _stream()
     _check(_C.tsmi_downsample_candidates(s, _ptr(coords), n, _I3(*ks), _I3(*st), _I3(*pd), host_max,
                                          _ptr(in_max), mode, _ptr(table.keys), cap, _ptr(counters)))
@@ -262,8 +263,7 @@ def downsample_coords(coords: torch.Tensor, kernel_sizes, stride, padding, coord
     temp_bytes = _C.tsmi_sort_temp_bytes(cap)
     scratch = torch.empty(2 * cap + temp_bytes // 8 + 1, dtype=torch.int64, device=dev)
     uniq, sorted_keys, temp = scratch[:cap], scratch[cap:2 * cap], scratch[2 * cap:]
-    _check(_C.tsmi_hashtable_compact_keys(s, _ptr(table.keys), cap, _ptr(uniq), _ptr(counters),
-                                          _ptr(temp), temp_bytes))
+    _check(_C.tsmi_hashtable_compact_keys(s, _ptr(table.keys), cap, _ptr(uniq), _ptr(counters)))
     n_out, overflow = counters[:2].tolist()
     if overflow:
         raise ValueError(

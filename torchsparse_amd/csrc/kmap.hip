@@ -189,6 +189,34 @@ __global__ void downsample_candidates_kernel(const int4 *in_coords, int64_t n_in
   (void)fresh;
 }
 
+// Occupied slots of a table, gathered in arbitrary order: one atomic per workgroup
+// reserves the output range (a counter bumped once per wavefront or per key would
+// serialise on its one address).
+__global__ __launch_bounds__(kBlock) void compact_keys_kernel(const unsigned long long *keys,
+                                                              int64_t cap, unsigned long long *out,
+                                                              int32_t *count) {
+  __shared__ int wave_base[kBlock / 64];
+  __shared__ int block_base;
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  const unsigned long long k = i < cap ? keys[i] : 0ULL;
+  const unsigned long long b = __ballot(k != 0ULL);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (lane == 0) wave_base[wave] = __popcll(b);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int total = 0;
+    for (int w = 0; w < kBlock / 64; ++w) {
+      const int c = wave_base[w];
+      wave_base[w] = total;
+      total += c;
+    }
+    block_base = total ? atomicAdd(count, total) : 0;
+  }
+  __syncthreads();
+  if (k != 0ULL)
+    out[block_base + wave_base[wave] + __popcll(b & ((1ULL << lane) - 1ULL))] = k;
+}
+
 __global__ void downsample_finalize_kernel(const unsigned long long *sorted, int64_t n_out,
                                            TableView t, int4 *out_coords) {
   int64_t r = (int64_t)blockIdx.x * kBlock + threadIdx.x;
@@ -485,10 +513,11 @@ extern "C" int tsmi_kmap_query(tsmi_stream_t s, const int64_t *keys, const int32
 }
 
 extern "C" int tsmi_coords_max(tsmi_stream_t s, const int32_t *coords, int64_t n,
-                               int32_t *out_max) {
+                               int32_t *out_max, int clear_first) {
   TSMI_REQUIRE(out_max && n >= 0 && (n == 0 || coords), "coords_max: bad arguments");
-  hipLaunchKernelGGL(fill_kernel<int32_t>, dim3(1), dim3(kBlock), 0, (hipStream_t)s, out_max,
-                     (int64_t)4, 0);
+  if (clear_first)
+    hipLaunchKernelGGL(fill_kernel<int32_t>, dim3(1), dim3(kBlock), 0, (hipStream_t)s, out_max,
+                       (int64_t)4, 0);
   if (n > 0) {
     TSMI_GRID_CHECK(n);
     hipLaunchKernelGGL(coords_max_kernel, grid_for(n), dim3(kBlock), 0, (hipStream_t)s,
@@ -524,6 +553,17 @@ extern "C" int tsmi_downsample_candidates(tsmi_stream_t s, const int32_t *in_coo
                      (hipStream_t)s, (const int4 *)in_coords, n_in, total, g, hm, in_max_dev, mode,
                      t, counters);
   return check_launch("tsmi_downsample_candidates");
+}
+
+extern "C" int tsmi_hashtable_compact_keys(tsmi_stream_t s, const int64_t *keys, int64_t cap,
+                                           int64_t *stored_keys_out, int32_t *count_out) {
+  TSMI_REQUIRE(keys && stored_keys_out && count_out && cap >= 1 && cap < (int64_t(1) << 31),
+               "hashtable_compact_keys: bad arguments");
+  TSMI_GRID_CHECK(cap);
+  hipLaunchKernelGGL(compact_keys_kernel, grid_for(cap), dim3(kBlock), 0, (hipStream_t)s,
+                     (const unsigned long long *)keys, cap, (unsigned long long *)stored_keys_out,
+                     count_out);
+  return check_launch("tsmi_hashtable_compact_keys");
 }
 
 extern "C" int tsmi_downsample_finalize(tsmi_stream_t s, const int64_t *sorted_keys, int64_t n_out,

@@ -4,7 +4,6 @@
 #include <cstring>
 
 #include <rocprim/device/device_radix_sort.hpp>
-#include <rocprim/device/device_select.hpp>
 #include <rocprim/iterator/counting_iterator.hpp>
 
 #include "common.h"
@@ -13,9 +12,6 @@ using namespace tsmi;
 
 namespace {
 constexpr int64_t kAlign = 256;
-struct NonZero {
-  __device__ bool operator()(const unsigned long long &v) const { return v != 0ULL; }
-};
 }
 
 extern "C" int64_t tsmi_sort_temp_bytes(int64_t n) {
@@ -32,35 +28,8 @@ extern "C" int64_t tsmi_sort_temp_bytes(int64_t n) {
     fail(TSMI_ERR_HIP, "sort_temp_bytes: size query failed");
     return -1;
   }
-  size_t c = 0;
-  hipError_t e3 = rocprim::select(nullptr, c, (const unsigned long long *)nullptr,
-                                  (unsigned long long *)nullptr, (unsigned int *)nullptr, (size_t)n,
-                                  NonZero(), (hipStream_t)0);
-  if (e3 != hipSuccess) {
-    fail(TSMI_ERR_HIP, "sort_temp_bytes: size query failed");
-    return -1;
-  }
   int64_t m = (int64_t)(a > b ? a : b);
-  if ((int64_t)c > m) m = (int64_t)c;
   return (m + kAlign - 1) / kAlign * kAlign + kAlign;
-}
-
-extern "C" int tsmi_hashtable_compact_keys(tsmi_stream_t s, const int64_t *keys, int64_t cap,
-                                           int64_t *stored_keys_out, int32_t *count_out, void *temp,
-                                           int64_t temp_bytes) {
-  TSMI_REQUIRE(keys && stored_keys_out && count_out && temp && cap >= 1 && cap < (int64_t(1) << 31),
-               "hashtable_compact_keys: bad arguments");
-  size_t need = 0;
-  (void)rocprim::select(nullptr, need, (const unsigned long long *)keys,
-                        (unsigned long long *)stored_keys_out, (unsigned int *)count_out, (size_t)cap,
-                        NonZero(), (hipStream_t)s);
-  TSMI_REQUIRE((int64_t)need <= temp_bytes, "hashtable_compact_keys: scratch too small (%lld < %lld)",
-               (long long)temp_bytes, (long long)need);
-  hipError_t e = rocprim::select(temp, need, (const unsigned long long *)keys,
-                                 (unsigned long long *)stored_keys_out, (unsigned int *)count_out,
-                                 (size_t)cap, NonZero(), (hipStream_t)s);
-  if (e != hipSuccess) return fail(TSMI_ERR_HIP, "hashtable_compact_keys: %s", hipGetErrorString(e));
-  return check_launch("tsmi_hashtable_compact_keys");
 }
 
 extern "C" int tsmi_sort_keys(tsmi_stream_t s, const int64_t *keys_in, int64_t *keys_out, int64_t n,
