@@ -246,9 +246,10 @@ def cpu_baseline(records, level_coords):
     import oracle
     cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
     rng = np.random.default_rng(0)
-    t_map = t_conv = 0.0
+    t_map = t_conv = t_ref = 0.0
     pair_cache = {}
     n_layers = 0
+    ref = oracle.ref_module()  # the reference's own CPU convolution, compiled in place
     for r in records:
         if r["ks"] == (1, 1, 1):
             continue
@@ -271,8 +272,21 @@ def cpu_baseline(records, level_coords):
         t0 = time.perf_counter()
         oracle.conv_gather_scatter(x, w, nb, sz, r["n_out"], transpose=transposed, variant=1)
         t_conv += time.perf_counter() - t0
+        if ref is not None:
+            n_y = r["n_out"]
+            y = torch.zeros(n_y, r["cout"])
+            tx, tw, tnb, tsz = torch.from_numpy(x), torch.from_numpy(w), torch.from_numpy(nb), torch.from_numpy(sz)
+            t0 = time.perf_counter()
+            ref.conv_forward_gather_scatter_cpu(tx, y, tw, tnb, tsz, transposed)
+            t_ref += time.perf_counter() - t0
         n_layers += 1
-    return {"value": round((t_map + t_conv) * 1e3, 1), "unit": "ms", "cores": cores, "kind": "port",
+    extra = {}
+    if ref is not None:
+        extra = {"reference_conv_ms": round(t_ref * 1e3, 1),
+                 "reference_conv": "conv_forward_gather_scatter_cpu of the reference (its own sources, "
+                                   "compiled) over the same layers, torch threads = "
+                                   f"{torch.get_num_threads()}"}
+    return {**extra, "value": round((t_map + t_conv) * 1e3, 1), "unit": "ms", "cores": cores, "kind": "port",
             "sample": f"{n_layers} sparse conv layers (fp32) + {len(pair_cache)} kernel maps of one "
                       f"MinkUNet forward on the same scan; BN/ReLU/concat/1x1x1 layers excluded; "
                       f"maps {t_map * 1e3:.0f} ms, convs {t_conv * 1e3:.0f} ms",

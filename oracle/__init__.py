@@ -33,6 +33,10 @@ the checks live in ``tests/test_oracle_*.py``):
                            reduces to X @ W
   conv_gather_scatter      the compiled reference CPU conv (oracle/_ref) on golden
                            vectors in tests/golden/; float64 closed form
+  conv_backward_*          the compiled reference CPU backward (oracle/_ref) on golden
+                           vectors in tests/golden/; torch autograd through the
+                           dense nn.Conv3d equivalent; finite differences of the
+                           oracle's own forward
   hash_cpu /               golden value hash_cpu([[0,1,2,3]]) = 321218472033932309
   kernel_hash_cpu          and vectors from the compiled reference (tests/golden/)
   hash_query_cpu           python dict; third-party google::dense_hash_map is not
@@ -258,6 +262,28 @@ def conv_gather_scatter(x, w, nbmaps, nbsizes, n_out, transpose=False, variant=1
                                   _p(nbmaps, _i32p), _p(nbsizes, _i32p), _p(y, _f32p), n_out,
                                   int(bool(transpose)), int(variant))
     return y
+
+
+def conv_backward_gather_scatter(x, w, nbmaps, nbsizes, dy, transpose=False):
+    """(dx, dw) of conv_gather_scatter with respect to x and w."""
+    x, w, nbmaps, nbsizes, dy = _f32(x), _f32(w), _i32(nbmaps), _i32(nbsizes), _f32(dy)
+    kvol, cin, cout = w.shape
+    dx, dw = np.empty_like(x), np.empty_like(w)
+    lib().tso_conv_backward_gather_scatter(_p(x, _f32p), x.shape[0], cin, _p(w, _f32p), kvol, cout,
+                                           _p(nbmaps, _i32p), _p(nbsizes, _i32p), _p(dy, _f32p),
+                                           _p(dx, _f32p), _p(dw, _f32p), int(bool(transpose)))
+    return dx, dw
+
+
+def conv_backward_implicit_gemm(x, w, out_in_map, dy):
+    """(dx, dw) of conv_implicit_gemm over the first len(dy) rows of the forward map."""
+    x, w, m, dy = _f32(x), _f32(w), _i32(out_in_map), _f32(dy)
+    kvol, cin, cout = w.shape
+    dx, dw = np.empty_like(x), np.empty_like(w)
+    lib().tso_conv_backward_implicit_gemm(_p(x, _f32p), x.shape[0], cin, _p(w, _f32p), kvol, cout,
+                                          _p(m, _i32p), dy.shape[0], _p(dy, _f32p), _p(dx, _f32p),
+                                          _p(dw, _f32p))
+    return dx, dw
 
 
 def hash_cpu(rows):

@@ -557,6 +557,83 @@ TSO_EXPORT int tso_conv_gather_scatter(const float *x, int n_in, int cin,
   return 0;
 }
 
+/* Backward of the gather-scatter convolution, pair lists in (in, out) columns:
+ *   dX[in] += dY[out] W[k]^T,   dW[k] = sum_pairs X[in]^T dY[out]
+ * for every pair of every offset (no centre shortcut: `flag` is false in the
+ * reference).  transpose swaps the roles of the two columns.  Accumulates in
+ * double.  Follows conv_backward_gather_scatter_cpu
+ * (convolution/convolution_gather_scatter_cpu.cpp:111-188). */
+TSO_EXPORT void tso_conv_backward_gather_scatter(
+    const float *x, int n_in, int cin, const float *w, int kvol, int cout,
+    const int *nbmaps, const int *nbsizes, const float *dy, float *dx, float *dw,
+    int transpose) {
+  double *dxa = (double *)calloc((size_t)n_in * cin, sizeof(double));
+  double *dwa = (double *)calloc((size_t)kvol * cin * cout, sizeof(double));
+  int64_t cur = 0;
+  for (int k = 0; k < kvol; k++) {
+    int nk = nbsizes[k];
+    const int *pairs = nbmaps + cur;
+    const float *wk = w + (int64_t)k * cin * cout;
+    double *dwk = dwa + (int64_t)k * cin * cout;
+    for (int p = 0; p < nk; p++) {
+      int in = pairs[2 * p + transpose];
+      int out = pairs[2 * p + 1 - transpose];
+      if (in < 0 || out < 0) continue;
+      const float *g = dy + (int64_t)out * cout;
+      const float *xr = x + (int64_t)in * cin;
+      double *dxr = dxa + (int64_t)in * cin;
+      for (int ci = 0; ci < cin; ci++) {
+        double a = 0.0, xv = xr[ci];
+        for (int c = 0; c < cout; c++) {
+          a += (double)g[c] * wk[(int64_t)ci * cout + c];
+          dwk[(int64_t)ci * cout + c] += xv * g[c];
+        }
+        dxr[ci] += a;
+      }
+    }
+    cur += 2 * (int64_t)nk;
+  }
+  for (int64_t i = 0; i < (int64_t)n_in * cin; i++) dx[i] = (float)dxa[i];
+  for (int64_t i = 0; i < (int64_t)kvol * cin * cout; i++) dw[i] = (float)dwa[i];
+  free(dxa);
+  free(dwa);
+}
+
+/* The same gradients from the forward map: for map[i,k] = m >= 0,
+ *   dX[m] += dY[i] W[k]^T,   dW[k] += X[m]^T dY[i].
+ * This is what the reference's dgrad (the forward kernel over out_in_map_bwd with
+ * W[k]^T) and wgrad kernels compute (nn/functional/conv/func/implicit_gemm.py:129-190). */
+TSO_EXPORT void tso_conv_backward_implicit_gemm(const float *x, int n_in, int cin,
+                                                const float *w, int kvol, int cout,
+                                                const int *map, int n_out,
+                                                const float *dy, float *dx, float *dw) {
+  double *dxa = (double *)calloc((size_t)n_in * cin, sizeof(double));
+  double *dwa = (double *)calloc((size_t)kvol * cin * cout, sizeof(double));
+  for (int i = 0; i < n_out; i++) {
+    const float *g = dy + (int64_t)i * cout;
+    for (int k = 0; k < kvol; k++) {
+      int m = map[(int64_t)i * kvol + k];
+      if (m < 0) continue;
+      const float *wk = w + (int64_t)k * cin * cout;
+      double *dwk = dwa + (int64_t)k * cin * cout;
+      const float *xr = x + (int64_t)m * cin;
+      double *dxr = dxa + (int64_t)m * cin;
+      for (int ci = 0; ci < cin; ci++) {
+        double a = 0.0, xv = xr[ci];
+        for (int c = 0; c < cout; c++) {
+          a += (double)g[c] * wk[(int64_t)ci * cout + c];
+          dwk[(int64_t)ci * cout + c] += xv * g[c];
+        }
+        dxr[ci] += a;
+      }
+    }
+  }
+  for (int64_t i = 0; i < (int64_t)n_in * cin; i++) dx[i] = (float)dxa[i];
+  for (int64_t i = 0; i < (int64_t)kvol * cin * cout; i++) dw[i] = (float)dwa[i];
+  free(dxa);
+  free(dwa);
+}
+
 /* ---------------------------------------- CPU map recipe of the CPU backend */
 
 /* 64-bit FNV-1a over the four int32 fields of a row, then the 60-bit fold.

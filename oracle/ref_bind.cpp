@@ -8,6 +8,7 @@
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("conv_forward_gather_scatter_cpu", &conv_forward_gather_scatter_cpu);
+  m.def("conv_backward_gather_scatter_cpu", &conv_backward_gather_scatter_cpu);
   m.def("hash_cpu", &hash_cpu);
   m.def("kernel_hash_cpu", &kernel_hash_cpu);
 }

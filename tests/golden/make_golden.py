@@ -38,6 +38,7 @@ def main():
         "down3": (oracle.kmap_downsample(coords, 3, 2, 1)[0], None, False, 5, 7),
     }
     out["coords"] = coords
+    bwd = {}
     for name, (omap, n_out, transpose, cin, cout) in cases.items():
         if n_out is None:
             n_out = int((omap >= 0).any(1).sum())
@@ -58,7 +59,17 @@ def main():
         out[name + "_w"] = w
         out[name + "_y"] = y.numpy()
         out[name + "_transpose"] = np.array(transpose)
+        # backward of the same case
+        dy = rng.standard_normal((n_y, cout)).astype(np.float32)
+        dx, dw = torch.zeros(n_x, cin), torch.zeros(kvol, cin, cout)
+        ref.conv_backward_gather_scatter_cpu(torch.from_numpy(x), dx, torch.from_numpy(dy),
+                                             torch.from_numpy(w), dw, torch.from_numpy(nbmaps),
+                                             torch.from_numpy(nbsizes), transpose)
+        bwd[name + "_dy"] = dy
+        bwd[name + "_dx"] = dx.numpy()
+        bwd[name + "_dw"] = dw.numpy()
     np.savez_compressed(os.path.join(HERE, "conv_gs_cpu.npz"), **out)
+    np.savez_compressed(os.path.join(HERE, "conv_gs_bwd_cpu.npz"), **bwd)
 
     rows = rng.integers(-50, 3000, (64, 4)).astype(np.int32)
     rows[0] = [0, 1, 2, 3]

@@ -153,3 +153,84 @@ def test_closed_form_float64():
     w = rng.uniform(-0.1, 0.1, (27, 24, 40)).astype(np.float32)
     y = oracle.conv_implicit_gemm(x, w, omap, 3000)
     assert rel_rms(y, conv_closed_form(x, w, omap, 3000)) < 1e-6
+
+
+# ------------------------------------------------------------------ backward
+
+@pytest.mark.parametrize("name", ["subm3", "down2", "up2", "down3"])
+def test_backward_gather_scatter_matches_reference_golden(name):
+    """conv_backward_gather_scatter_cpu of the compiled reference
+    (convolution_gather_scatter_cpu.cpp:111-188) on the golden cases."""
+    g = np.load(os.path.join(GOLD, "conv_gs_cpu.npz"))
+    b = np.load(os.path.join(GOLD, "conv_gs_bwd_cpu.npz"))
+    dx, dw = oracle.conv_backward_gather_scatter(g[name + "_x"], g[name + "_w"], g[name + "_nbmaps"],
+                                                 g[name + "_nbsizes"], b[name + "_dy"],
+                                                 bool(g[name + "_transpose"]))
+    assert rel_rms(dx, b[name + "_dx"]) < 1e-5  # the reference sums in fp32
+    assert rel_rms(dw, b[name + "_dw"]) < 1e-5  # the reference sums in fp32
+
+
+@pytest.mark.parametrize("name", ["subm3", "down2", "down3"])
+def test_backward_from_map_equals_backward_from_pairs(name):
+    g = np.load(os.path.join(GOLD, "conv_gs_cpu.npz"))
+    b = np.load(os.path.join(GOLD, "conv_gs_bwd_cpu.npz"))
+    dx, dw = oracle.conv_backward_implicit_gemm(g[name + "_x"], g[name + "_w"], g[name + "_map"],
+                                                b[name + "_dy"])
+    assert rel_rms(dx, b[name + "_dx"]) < 1e-5  # the reference sums in fp32
+    assert rel_rms(dw, b[name + "_dw"]) < 1e-5  # the reference sums in fp32
+
+
+@pytest.mark.parametrize("k,s", [(3, 1), (2, 2), (3, 2)])
+def test_backward_equals_autograd_of_dense_conv(k, s):
+    """Gradients of the dense nn.functional.conv3d equivalent, restricted to the active
+    voxels (the reference's own test method, tests/python/test_single_layer_conv.py)."""
+    rng = np.random.default_rng(5)
+    shape, IC, OC = (6, 5, 4), 6, 5
+    coords = random_coords(rng, 30, shape)
+    feats = rng.uniform(-1, 1, (30, IC)).astype(np.float32)
+    filters = rng.uniform(-1, 1, (k, k, k, IC, OC)).astype(np.float32)
+    w = filters.reshape(-1, IC, OC)
+    pad = (k - 1) // 2 if k % 2 == 1 else 0
+    if s == 1:
+        omap, ocoords = oracle.kmap_subm(coords, k, coords_max=[0] + [v - 1 for v in shape]), coords
+    else:
+        sr = (1,) + tuple((shape[a] + 2 * pad - (k - 1) - 1) // s + 1 for a in range(3))
+        omap, ocoords = oracle.kmap_downsample(coords, k, s, pad, spatial_range=sr)
+    dy = rng.standard_normal((len(ocoords), OC)).astype(np.float32)
+    dx, dw = oracle.conv_backward_implicit_gemm(feats, w, omap, dy)
+
+    dense = torch.zeros(1, IC, *shape, dtype=torch.float64)
+    for c, f in zip(coords, feats):
+        dense[0, :, c[1], c[2], c[3]] = torch.from_numpy(f.astype(np.float64))
+    dense.requires_grad_(True)
+    f_t = torch.from_numpy(filters.astype(np.float64)).requires_grad_(True)
+    if k % 2 == 1:
+        weight, xin = f_t.permute(4, 3, 2, 1, 0), dense
+    else:
+        weight, xin = f_t.permute(4, 3, 0, 1, 2), torch.nn.functional.pad(dense, (0, k - 1) * 3)
+    out = torch.nn.functional.conv3d(xin, weight, stride=s, padding=pad)
+    gout = torch.zeros_like(out)
+    for c, g in zip(ocoords, dy):
+        gout[0, :, c[1], c[2], c[3]] = torch.from_numpy(g.astype(np.float64))
+    out.backward(gout)
+    want_dx = np.stack([dense.grad[0, :, c[1], c[2], c[3]].numpy() for c in coords])
+    want_dw = f_t.grad.numpy().reshape(-1, IC, OC)
+    assert rel_rms(dx, want_dx) < 1e-5
+    assert rel_rms(dw, want_dw) < 1e-5
+
+
+def test_backward_is_the_derivative_of_the_oracle_forward():
+    rng = np.random.default_rng(6)
+    coords = random_coords(rng, 40, (5, 5, 5))
+    omap = oracle.kmap_subm(coords, 3)
+    x = rng.standard_normal((40, 3)).astype(np.float32)
+    w = rng.standard_normal((27, 3, 4)).astype(np.float32)
+    dy = rng.standard_normal((40, 4)).astype(np.float32)
+    dx, dw = oracle.conv_backward_implicit_gemm(x, w, omap, dy)
+    # the forward is bilinear: <dy, conv(x + e, w)> - <dy, conv(x, w)> = <dx, e> exactly
+    e = rng.standard_normal(x.shape).astype(np.float32)
+    lhs = (dy * (oracle.conv_implicit_gemm(x + e, w, omap, 40) - oracle.conv_implicit_gemm(x, w, omap, 40))).sum()
+    assert abs(lhs - (dx * e).sum()) < 1e-3 * max(1.0, abs(lhs))
+    ew = rng.standard_normal(w.shape).astype(np.float32)
+    lhs = (dy * (oracle.conv_implicit_gemm(x, w + ew, omap, 40) - oracle.conv_implicit_gemm(x, w, omap, 40))).sum()
+    assert abs(lhs - (dw * ew).sum()) < 1e-3 * max(1.0, abs(lhs))
