@@ -263,6 +263,22 @@ int tsmi_conv_implicit_gemm_sorted(tsmi_stream_t s, const void *x, const void *w
                                    float *workspace, int64_t workspace_elems,
                                    int32_t *tile_counters, int64_t n_tile_counters, void *y);
 
+/* Weight gradient: dw[k][c][n] = sum_i [m = map_bwd[i,k] >= 0] x[i][c] * dy[m][n], with
+ * map_bwd int32 [n_map_rows >= n_in, K_vol] the transposed kernel map (tsmi_transpose_map
+ * of the forward map: input row, offset -> output row), dy [n_out, cout] and dw
+ * [K_vol, cin, cout] of the I/O type, fp32 accumulation.  `workspace` holds
+ * tsmi_conv_wgrad_workspace_elems floats (per-split partial sums, added by a second
+ * launch).  The input gradient needs no entry point of its own: it is
+ * tsmi_conv_implicit_gemm over map_bwd with the weights transposed per offset
+ * (nn/functional/conv/func/implicit_gemm.py:171-180).  Replaces
+ * conv_backward_wgrad_implicit_gemm_cuda
+ * (convolution/convolution_backward_wgrad_implicit_gemm_cuda.cu:1614-2042), which
+ * returns the same sums as [K_vol*cout, cin]. */
+int64_t tsmi_conv_wgrad_workspace_elems(int64_t n_in, int kvol, int cin, int cout, int dtype);
+int tsmi_conv_wgrad(tsmi_stream_t s, const void *x, const void *dy, const int32_t *map_bwd,
+                    int64_t n_map_rows, int64_t n_in, int kvol, int cin, int cout, int dtype,
+                    float *workspace, int64_t workspace_elems, void *dw);
+
 /* Fetch-on-demand: one launch over 128-padded pair lists gathers X rows, multiplies
  * by W[k] and writes partial[qnbaddrs[k] + p, :] (fp32 for TSMI_F32, else the I/O
  * type); a second launch sums the partials of each output row through output_mask

@@ -1,0 +1,129 @@
+"""GPU parity of the convolution backward (input and weight gradients) against the CPU
+oracle.  Tolerances relative to the RMS of the expected gradient: 1e-4 fp32, 1e-2 fp16,
+3e-2 bf16 (fp32 accumulation; the oracle gets the inputs already rounded to the I/O type)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import random_coords, rel_rms
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float32: 1e-4, torch.float16: 1e-2, torch.bfloat16: 3e-2}
+
+
+@pytest.fixture(scope="module")
+def mods():
+    import torchsparse_amd as ts
+    from torchsparse_amd import backend
+    from torchsparse_amd import nn as spnn
+    from torchsparse_amd.nn import functional as F
+    return ts, backend, spnn, F
+
+
+def dev(a, dtype=torch.int32):
+    return torch.from_numpy(np.ascontiguousarray(a)).to("cuda", dtype)
+
+
+def _f32(t):
+    return t.detach().float().cpu().numpy()
+
+
+@pytest.mark.parametrize("cin,cout", [(32, 32), (64, 96), (96, 64), (128, 128), (16, 40), (5, 7), (4, 32), (200, 72)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32, torch.bfloat16])
+def test_wgrad_and_dgrad_kernels_match_oracle(mods, cin, cout, dtype):
+    _, backend, _, F = mods
+    rng = np.random.default_rng(cin * 100 + cout)
+    coords = random_coords(rng, 1800, (22, 20, 12))
+    n = len(coords)
+    kmap = F.build_kernel_map(dev(coords), n, 3, 1, 1, mode="hashmap_on_the_fly")
+    omap = kmap["out_in_map"]
+    x = torch.from_numpy(rng.standard_normal((n, cin)).astype(np.float32)).to("cuda", dtype)
+    w = torch.from_numpy(rng.uniform(-0.1, 0.1, (27, cin, cout)).astype(np.float32)).to("cuda", dtype)
+    dy = torch.from_numpy(rng.standard_normal((n, cout)).astype(np.float32)).to("cuda", dtype)
+    map_bwd = backend.convert_transposed_out_in_map(omap, (n + 127) // 128 * 128, n)
+    dw = backend.conv_backward_wgrad_implicit_gemm_cuda(dy, x, map_bwd, n)
+    dx = backend.conv_forward_implicit_gemm_cuda(dy, w.transpose(1, 2).contiguous(), map_bwd, n, cin)
+    want_dx, want_dw = oracle.conv_backward_implicit_gemm(_f32(x), _f32(w), omap.cpu().numpy(), _f32(dy))
+    assert dw.shape == (27, cin, cout) and dw.dtype == dtype
+    assert rel_rms(_f32(dw), want_dw) < TOL[dtype]
+    assert rel_rms(_f32(dx), want_dx) < TOL[dtype]
+
+
+@pytest.mark.parametrize("n", [1, 31, 32, 33, 500, 5000])
+def test_wgrad_ragged_row_counts(mods, n):
+    _, backend, _, F = mods
+    rng = np.random.default_rng(n)
+    coords = random_coords(rng, n, (30, 30, 10))
+    n = len(coords)
+    kmap = F.build_kernel_map(dev(coords), n, 3, 1, 1, mode="hashmap_on_the_fly")
+    omap = kmap["out_in_map"]
+    x = torch.from_numpy(rng.standard_normal((n, 24)).astype(np.float32)).cuda()
+    dy = torch.from_numpy(rng.standard_normal((n, 40)).astype(np.float32)).cuda()
+    w = np.zeros((27, 24, 40), np.float32)
+    map_bwd = backend.convert_transposed_out_in_map(omap, (n + 127) // 128 * 128, n)
+    dw = backend.conv_backward_wgrad_implicit_gemm_cuda(dy, x, map_bwd, n)
+    _, want_dw = oracle.conv_backward_implicit_gemm(_f32(x), w, omap.cpu().numpy(), _f32(dy))
+    assert rel_rms(_f32(dw), want_dw) < 1e-4
+
+
+@pytest.mark.parametrize("geom", [(3, 1, 1), (2, 2, 0), (3, 2, 1), (2, 1, 0)])
+@pytest.mark.parametrize("flow", ["ImplicitGEMM", "GatherScatter", "FetchOnDemand"])
+def test_autograd_through_conv3d_matches_oracle(mods, geom, flow):
+    """loss = sum(conv(x) * g): x.grad and kernel.grad for every dataflow and geometry,
+    including the bias gradient."""
+    ts, backend, spnn, F = mods
+    k, s, pad = geom
+    rng = np.random.default_rng(k * 10 + s)
+    coords = random_coords(rng, 900, (16, 14, 10))
+    n = len(coords)
+    cin, cout = 16, 24
+    x = torch.from_numpy(rng.standard_normal((n, cin)).astype(np.float32)).cuda().requires_grad_(True)
+    torch.manual_seed(k)
+    layer = spnn.Conv3d(cin, cout, k, stride=s, padding=pad, bias=True).cuda()
+    cfg = F.conv_config.get_default_conv_config()
+    cfg.dataflow = getattr(F.Dataflow, flow)
+    layer._config = cfg
+    inp = ts.SparseTensor(x, dev(coords))
+    out = F.conv3d(inp, layer.kernel, kernel_size=k, bias=layer.bias, stride=s, padding=pad, config=cfg)
+    g = torch.from_numpy(rng.standard_normal(tuple(out.feats.shape)).astype(np.float32)).cuda()
+    (out.feats * g).sum().backward()
+    if s == 1:
+        omap = oracle.kmap_subm(coords, k)
+    else:
+        omap, _ = oracle.kmap_downsample(coords, k, s, pad)
+    want_dx, want_dw = oracle.conv_backward_implicit_gemm(_f32(x), _f32(layer.kernel), omap, _f32(g))
+    assert rel_rms(_f32(x.grad), want_dx) < 1e-4
+    assert rel_rms(_f32(layer.kernel.grad), want_dw) < 1e-4
+    assert rel_rms(_f32(layer.bias.grad), _f32(g).sum(0)) < 1e-4
+
+
+def test_autograd_through_transposed_conv_and_relu_residual(mods):
+    ts, backend, spnn, F = mods
+    rng = np.random.default_rng(11)
+    coords = random_coords(rng, 1200, (20, 18, 10))
+    n = len(coords)
+    torch.manual_seed(0)
+    down = spnn.Conv3d(8, 12, 2, stride=2).cuda()
+    up = spnn.Conv3d(12, 6, 2, stride=2, transposed=True).cuda()
+    x = torch.from_numpy(rng.standard_normal((n, 8)).astype(np.float32)).cuda().requires_grad_(True)
+    res = torch.from_numpy(rng.standard_normal((n, 6)).astype(np.float32)).cuda().requires_grad_(True)
+    inp = ts.SparseTensor(x, dev(coords))
+    mid = down(inp)
+    out = F.conv3d(mid, up.kernel, kernel_size=2, stride=2, transposed=True, residual=res, activation="relu")
+    g = torch.from_numpy(rng.standard_normal((n, 6)).astype(np.float32)).cuda()
+    (out.feats * g).sum().backward()
+    # oracle: chain rule by hand
+    omap, ocoords = oracle.kmap_downsample(coords, 2, 2, 0)
+    n_mid = len(ocoords)
+    mid_np = oracle.conv_implicit_gemm(_f32(x), _f32(down.kernel), omap, n_mid)
+    tmap = oracle.transpose_map(omap[:n_mid], n)
+    pre = oracle.conv_implicit_gemm(mid_np, _f32(up.kernel), tmap, n) + _f32(res)
+    gpre = _f32(g) * (pre > 0)
+    dmid, dw_up = oracle.conv_backward_implicit_gemm(mid_np, _f32(up.kernel), tmap, gpre)
+    dx, dw_down = oracle.conv_backward_implicit_gemm(_f32(x), _f32(down.kernel), omap, dmid)
+    assert rel_rms(_f32(res.grad), gpre) < 1e-4
+    assert rel_rms(_f32(up.kernel.grad), dw_up) < 1e-4
+    assert rel_rms(_f32(down.kernel.grad), dw_down) < 1e-4
+    assert rel_rms(_f32(x.grad), dx) < 1e-4

@@ -34,6 +34,8 @@ def _load():
     lib.tsmi_packed_weight_elems.restype = _i64
     lib.tsmi_packed_weight_elems.argtypes = [_i32, _i32, _i32]
     lib.tsmi_conv_workspace_elems.restype = _i64
+    lib.tsmi_conv_wgrad_workspace_elems.restype = _i64
+    lib.tsmi_conv_wgrad_workspace_elems.argtypes = [_i64, _i32, _i32, _i32, _i32]
     lib.tsmi_conv_workspace_elems.argtypes = [_i64, _i64, _i32, _i32, _i32, _i32, _i32, _i32]
     sig = {
         "tsmi_hashtable_clear": [_vp, _vp, _vp, _i64],
@@ -61,6 +63,7 @@ def _load():
         "tsmi_conv_implicit_gemm_sorted": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32,
                                            _i32, _i32, _i32, _vp, _vp, _i32, _vp, _i64, _vp, _i64,
                                            _vp],
+        "tsmi_conv_wgrad": [_vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _i32, _i32, _vp, _i64, _vp],
         "tsmi_conv_fetch_on_demand": [_vp, _vp, _vp, _vp, _i64, _vp, _vp, _i64, _vp, _i64, _i32,
                                       _i32, _i32, _i32, _i32, _i32, _vp, _vp, _i32, _vp, _vp],
         "tsmi_gs_gather": [_vp, _vp, _vp, _i64, _i32, _i32, _i32, _vp],
@@ -520,6 +523,30 @@ def conv_forward_implicit_gemm_sorted_cuda(in_feats, kernel, reorder_out_in_map,
                                       _ptr(_tile_counters(x.device)) if ws is not None else None,
                                       _N_TILE_COUNTERS, _ptr(y)))
     return y
+
+
+def conv_backward_wgrad_implicit_gemm_cuda(grad_out: torch.Tensor, in_feats: torch.Tensor,
+                                           out_in_map_bwd: torch.Tensor, num_in_feats: int,
+                                           split_k_iters: int = 32, allow_tf32=False,
+                                           allow_fp16=True) -> torch.Tensor:
+    """Weight gradient [K_vol, Cin, Cout] of the I/O type —
+    convolution/convolution_backward_wgrad_implicit_gemm_cuda.cu:1614-2042, which returns
+    the same sums laid out [K_vol*Cout, Cin].  out_in_map_bwd maps (input row, offset) to
+    the output row; split_k_iters is accepted and ignored (the row split is chosen by the
+    library)."""
+    if in_feats.dtype != grad_out.dtype:
+        raise ValueError("in_feats and grad_out must have the same dtype")
+    x = _need(in_feats, in_feats.dtype, "in_feats")
+    dy = _need(grad_out, grad_out.dtype, "grad_out")
+    m = _need(out_in_map_bwd, torch.int32, "out_in_map_bwd")
+    kvol, cin, cout = m.shape[1], x.shape[1], dy.shape[1]
+    code = _dtype_code(x)
+    dw = torch.empty((kvol, cin, cout), dtype=x.dtype, device=x.device)
+    ws_elems = _C.tsmi_conv_wgrad_workspace_elems(num_in_feats, kvol, cin, cout, code)
+    ws = torch.empty(max(ws_elems, 1), dtype=torch.float32, device=x.device)
+    _check(_C.tsmi_conv_wgrad(_stream(), _ptr(x), _ptr(dy), _ptr(m), m.shape[0], num_in_feats, kvol,
+                              cin, cout, code, _ptr(ws), ws_elems, _ptr(dw)))
+    return dw
 
 
 def conv_forward_fetch_on_demand_cuda(in_feats, kernel, nbmaps, sum_nnz, nbaddrs, qnbaddrs,

@@ -93,6 +93,28 @@ extern "C" int tsmi_conv_implicit_gemm_sorted(tsmi_stream_t s, const void *x, co
                     tile_counters, tile_counters ? n_tile_counters : 0);
 }
 
+extern "C" int64_t tsmi_conv_wgrad_workspace_elems(int64_t n_in, int kvol, int cin, int cout,
+                                                   int dtype) {
+  const ConvOps *ops = ops_for(dtype);
+  if (!ops || n_in < 0 || kvol < 1 || cin < 1 || cout < 1) return 0;
+  return ops->wgrad_workspace(n_in, kvol, cin, cout);
+}
+
+extern "C" int tsmi_conv_wgrad(tsmi_stream_t s, const void *x, const void *dy,
+                               const int32_t *map_bwd, int64_t n_map_rows, int64_t n_in, int kvol,
+                               int cin, int cout, int dtype, float *workspace,
+                               int64_t workspace_elems, void *dw) {
+  const ConvOps *ops = ops_for(dtype);
+  if (int e = check_shapes("conv_wgrad", ops, kvol, cin, cout)) return e;
+  TSMI_REQUIRE(n_in >= 0 && n_map_rows >= n_in, "conv_wgrad: map has %lld rows, need %lld",
+               (long long)n_map_rows, (long long)n_in);
+  TSMI_REQUIRE(dw && workspace, "conv_wgrad: null output or workspace");
+  TSMI_REQUIRE(n_in == 0 || (x && dy && map_bwd), "conv_wgrad: null pointer");
+  TSMI_REQUIRE(aligned16(x) && aligned16(dy), "conv_wgrad: x and dy must be 16-byte aligned");
+  return ops->wgrad((hipStream_t)s, x, dy, map_bwd, n_in, kvol, cin, cout, workspace,
+                    workspace_elems, dw);
+}
+
 extern "C" int tsmi_conv_fetch_on_demand(tsmi_stream_t s, const void *x, const void *w_packed,
                                          const int32_t *nbmaps_planar, int64_t nnz,
                                          const int32_t *nbaddrs, const int32_t *qnbaddrs,

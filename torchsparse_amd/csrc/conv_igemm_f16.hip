@@ -33,6 +33,7 @@ struct TraitsF16 {
 #include "conv_tile.inc"
 #include "conv_igemm2.inc"
 #include "conv_plan.inc"
+#include "conv_wgrad.inc"
 #include "conv_igemm_tail.inc"
 
 namespace tsmi {

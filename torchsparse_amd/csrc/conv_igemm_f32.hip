@@ -36,6 +36,7 @@ struct TraitsF32 {
 #include "conv_tile.inc"
 #include "conv_igemm2.inc"
 #include "conv_plan.inc"
+#include "conv_wgrad.inc"
 #include "conv_igemm_tail.inc"
 
 namespace tsmi {

@@ -33,6 +33,10 @@ struct ConvOps {
                  const void *residual, int relu, void *y);
   int (*gather)(hipStream_t s, const void *x, const int32_t *pairs, int64_t nnz, int cin, int col,
                 void *buffer);
+  // dW[k] = sum over input rows i of X[i]^T dY[map_bwd[i,k]]
+  int64_t (*wgrad_workspace)(int64_t n_in, int kvol, int cin, int cout);
+  int (*wgrad)(hipStream_t s, const void *x, const void *dy, const int32_t *map_bwd, int64_t n_in,
+               int kvol, int cin, int cout, float *partial, int64_t partial_elems, void *dw);
 };
 
 const ConvOps &conv_ops_f16();

@@ -1,0 +1,84 @@
+"""Backward of the sparse convolution, shared by the three dataflows.
+
+    dX[m]  += dY[i] W[k]^T          (input gradient)
+    dW[k]  += X[m]^T dY[i]          for every map entry  map[i, k] = m >= 0
+
+The input gradient is the forward implicit-GEMM kernel over the transposed map with
+the weights transposed per offset; the weight gradient has a kernel of its own
+(tsmi_conv_wgrad).  Both follow the reference's func/implicit_gemm.py:108-190 (unsorted
+branch); the gather-scatter and fetch-on-demand dataflows get the same gradients from
+the same maps (the reference computes theirs with conv_backward_gather_scatter_cuda,
+func/gather_scatter.py:104-160 — same sums)."""
+from typing import Callable, Dict
+
+import torch
+
+from torchsparse_amd import backend
+from torchsparse_amd.utils import make_divisible
+
+__all__ = ["SparseConvFunction", "backward_map"]
+
+
+def backward_map(kmap: Dict, transposed: bool) -> torch.Tensor:
+    """(input row, offset) -> output row of the convolution, int32 [ceil128(N_in), K_vol].
+    For a transposed convolution that is the strided map itself; otherwise the transposed
+    map, built once and kept under ``out_in_map_bwd`` (build_kmap.py:191-194)."""
+    if transposed:
+        return kmap["out_in_map"]
+    if kmap.get("out_in_map_bwd") is None:
+        n_in, n_out = kmap["sizes"]
+        kmap["out_in_map_bwd"] = backend.convert_transposed_out_in_map(
+            kmap["out_in_map"], make_divisible(n_in, 128), n_out)
+    return kmap["out_in_map_bwd"]
+
+
+class SparseConvFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, input: torch.Tensor, weight: torch.Tensor, kmap: Dict, config: Dict,
+                transposed: bool, forward_impl: Callable) -> torch.Tensor:
+        out = forward_impl(input, weight, kmap, config, transposed, None, None, False)
+        ctx.save_for_backward(input, weight)
+        ctx.kmap, ctx.transposed = kmap, transposed
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_output: torch.Tensor):
+        input, weight = ctx.saved_tensors
+        kmap, transposed = ctx.kmap, ctx.transposed
+        from .implicit_gemm import _coerce
+        x, w = _coerce(input.detach(), weight.detach())
+        if w.dim() == 2:
+            w = w.unsqueeze(0)
+        dy = grad_output.contiguous()
+        if dy.dtype != x.dtype:
+            dy = dy.to(x.dtype)
+        map_bwd = backward_map(kmap, transposed)
+        sizes = kmap["sizes"]
+        n_in = sizes[1] if transposed else sizes[0]
+        grad_input = grad_weight = None
+        if ctx.needs_input_grad[0]:
+            grad_input = backend.conv_forward_implicit_gemm_cuda(
+                dy, w.transpose(1, 2).contiguous(), map_bwd, n_in, w.shape[1])
+            if grad_input.dtype != input.dtype:
+                grad_input = grad_input.to(input.dtype)
+        if ctx.needs_input_grad[1]:
+            grad_weight = backend.conv_backward_wgrad_implicit_gemm_cuda(dy, x, map_bwd, n_in)
+            grad_weight = grad_weight.reshape(weight.shape)
+            if grad_weight.dtype != weight.dtype:
+                grad_weight = grad_weight.to(weight.dtype)
+        return grad_input, grad_weight, None, None, None, None
+
+
+def differentiable(forward_impl: Callable):
+    """Wrap a dataflow's forward: with autograd active the convolution goes through
+    SparseConvFunction and bias / residual / ReLU are applied by autograd-aware ops."""
+    def apply(input, weight, kmap, config, transposed=False, bias=None, residual=None, relu=False):
+        if torch.is_grad_enabled() and (input.requires_grad or weight.requires_grad):
+            out = SparseConvFunction.apply(input, weight, kmap, config, transposed, forward_impl)
+            if bias is not None:
+                out = out + bias.to(out.dtype)
+            if residual is not None:
+                out = out + residual.to(out.dtype)
+            return torch.relu(out) if relu else out
+        return forward_impl(input, weight, kmap, config, transposed, bias, residual, relu)
+    return apply

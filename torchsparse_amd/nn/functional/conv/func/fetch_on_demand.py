@@ -6,6 +6,8 @@ from torchsparse_amd import backend, backends
 from .gather_scatter import _center_offset
 from .implicit_gemm import _coerce
 
+from .autograd import differentiable  # noqa: E402
+
 __all__ = ["FetchOnDemandConvolutionFuntion"]
 
 
@@ -16,9 +18,9 @@ class FetchOnDemandConvolutionFuntion:
     read for compatibility; all offsets always run in one launch."""
 
     @staticmethod
-    def apply(input: torch.Tensor, weight: torch.Tensor, kmap: Dict, config: Dict,
-              transposed: bool = False, bias: Optional[torch.Tensor] = None,
-              residual: Optional[torch.Tensor] = None, relu: bool = False) -> torch.Tensor:
+    def _forward(input: torch.Tensor, weight: torch.Tensor, kmap: Dict, config: Dict,
+                 transposed: bool = False, bias: Optional[torch.Tensor] = None,
+                 residual: Optional[torch.Tensor] = None, relu: bool = False) -> torch.Tensor:
         sizes = kmap["sizes"]
         out_dtype = weight.dtype
         input, weight = _coerce(input, weight)
@@ -35,3 +37,6 @@ class FetchOnDemandConvolutionFuntion:
             row_mask=kmap["input_mask"] if transposed else kmap["output_mask"],
             center_k=_center_offset(kmap, kvol), bias=bias, residual=residual, relu=relu)
         return out if out.dtype == out_dtype else out.to(out_dtype)
+
+
+FetchOnDemandConvolutionFuntion.apply = staticmethod(differentiable(FetchOnDemandConvolutionFuntion._forward))

@@ -5,6 +5,8 @@ import torch
 from torchsparse_amd import backend
 from .implicit_gemm import _coerce
 
+from .autograd import differentiable  # noqa: E402
+
 __all__ = ["GatherScatterConvolutionFuntion"]
 
 
@@ -20,9 +22,9 @@ class GatherScatterConvolutionFuntion:
     config for compatibility; they never change the result."""
 
     @staticmethod
-    def apply(input: torch.Tensor, weight: torch.Tensor, kmap: Dict, config: Dict,
-              transposed: bool = False, bias: Optional[torch.Tensor] = None,
-              residual: Optional[torch.Tensor] = None, relu: bool = False) -> torch.Tensor:
+    def _forward(input: torch.Tensor, weight: torch.Tensor, kmap: Dict, config: Dict,
+                 transposed: bool = False, bias: Optional[torch.Tensor] = None,
+                 residual: Optional[torch.Tensor] = None, relu: bool = False) -> torch.Tensor:
         sizes = kmap["sizes"]
         out_dtype = weight.dtype
         input, weight = _coerce(input, weight)
@@ -41,3 +43,6 @@ class GatherScatterConvolutionFuntion:
             qsum_nnz=None if kmap.get("qmapsize") is None else int(kmap["qmapsize"]),
             center_k=_center_offset(kmap, kvol), bias=bias, residual=residual, relu=relu)
         return out if out.dtype == out_dtype else out.to(out_dtype)
+
+
+GatherScatterConvolutionFuntion.apply = staticmethod(differentiable(GatherScatterConvolutionFuntion._forward))

@@ -4,6 +4,8 @@ import torch
 
 from torchsparse_amd import backend, backends
 
+from .autograd import differentiable  # noqa: E402
+
 __all__ = ["ImplicitGEMMConvolutionFuntion"]
 
 
@@ -19,14 +21,13 @@ def _coerce(input: torch.Tensor, weight: torch.Tensor):
 
 
 class ImplicitGEMMConvolutionFuntion:
-    """Forward of the implicit-GEMM dataflow (the reference's
-    func/implicit_gemm.py:15-106).  Forward only: this build has no backward kernels,
-    so the result carries no autograd history."""
+    """The implicit-GEMM dataflow (the reference's func/implicit_gemm.py:15-190);
+    ``apply`` is differentiable (func/autograd.py)."""
 
     @staticmethod
-    def apply(input: torch.Tensor, weight: torch.Tensor, kmap: Dict, config: Dict,
-              transposed: bool = False, bias: Optional[torch.Tensor] = None,
-              residual: Optional[torch.Tensor] = None, relu: bool = False) -> torch.Tensor:
+    def _forward(input: torch.Tensor, weight: torch.Tensor, kmap: Dict, config: Dict,
+                 transposed: bool = False, bias: Optional[torch.Tensor] = None,
+                 residual: Optional[torch.Tensor] = None, relu: bool = False) -> torch.Tensor:
         sizes = kmap["sizes"]
         sfx = "_t" if transposed else ""
         num_out_feats = sizes[0] if transposed else sizes[1]
@@ -46,3 +47,6 @@ class ImplicitGEMMConvolutionFuntion:
                 kmap["reorder_loc" + sfx], num_out_feats, weight.shape[-1],
                 backends.allow_tf32, backends.allow_fp16, bias=bias, residual=residual, relu=relu)
         return out if out.dtype == out_dtype else out.to(out_dtype)
+
+
+ImplicitGEMMConvolutionFuntion.apply = staticmethod(differentiable(ImplicitGEMMConvolutionFuntion._forward))
