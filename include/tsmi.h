@@ -279,6 +279,34 @@ int tsmi_conv_wgrad(tsmi_stream_t s, const void *x, const void *dy, const int32_
                     int64_t n_map_rows, int64_t n_in, int kvol, int cin, int cout, int dtype,
                     float *workspace, int64_t workspace_elems, void *dw);
 
+/* Weight gradient over pair lists.  tsmi_wgrad_pairs_build turns a kernel map (int32
+ * [n_rows, K_vol], -1 = none) into per-offset lists of (map value, row) pairs ordered by
+ * row: offset k's list starts at entry 32 * seg_steps[k] of `pairs` and is padded with
+ * (-1, -1) to a multiple of 32 entries; seg_steps int32[K_vol + 1] counts those blocks of
+ * 32, nbsizes int32[K_vol] the pairs themselves.  `pairs` holds
+ * tsmi_wgrad_pairs_capacity(n_rows, K_vol) entries of two int32 (only the part the lists
+ * need is written), block_counts is scratch of K_vol * ceil(n_rows / 256) int32.  Nothing
+ * is read back to the host.  K_vol <= 511.
+ *
+ * tsmi_conv_wgrad_pairs: dw[k][c][n] = sum over offset k's pairs of x[a][c] * dy[b][n],
+ * a = pair[x_col], b = pair[1 - x_col] (x_col 0: the map values index x, as in a forward
+ * map out_in_map[out, k] = in; x_col 1: the rows index x, as for a transposed
+ * convolution over the same map).  Only rows that take part in an offset are read.  cin
+ * and cout must be multiples of 16 bytes of elements (other widths: tsmi_conv_wgrad).
+ * `workspace` holds tsmi_conv_wgrad_pairs_workspace_elems floats; pair_cap is the
+ * capacity `pairs` was built with.  Same sums as conv_backward_gather_scatter_cuda's
+ * grad_kernel (convolution/convolution_gather_scatter_cuda.cu:815-915) and as
+ * conv_backward_wgrad_implicit_gemm_cuda, accumulated in fp32. */
+int64_t tsmi_wgrad_pairs_capacity(int64_t n_rows, int kvol);
+int tsmi_wgrad_pairs_build(tsmi_stream_t s, const int32_t *map, int64_t n_rows, int kvol,
+                           int32_t *block_counts, int32_t *nbsizes, int32_t *pairs,
+                           int32_t *seg_steps);
+int64_t tsmi_conv_wgrad_pairs_workspace_elems(int64_t pair_cap, int kvol, int cin, int cout,
+                                              int dtype);
+int tsmi_conv_wgrad_pairs(tsmi_stream_t s, const void *x, const void *dy, const int32_t *pairs,
+                          const int32_t *seg_steps, int64_t pair_cap, int x_col, int kvol, int cin,
+                          int cout, int dtype, float *workspace, int64_t workspace_elems, void *dw);
+
 /* Fetch-on-demand: one launch over 128-padded pair lists gathers X rows, multiplies
  * by W[k] and writes partial[qnbaddrs[k] + p, :] (fp32 for TSMI_F32, else the I/O
  * type); a second launch sums the partials of each output row through output_mask

@@ -68,6 +68,97 @@ def test_wgrad_ragged_row_counts(mods, n):
     assert rel_rms(_f32(dw), want_dw) < 1e-4
 
 
+def _expected_pair_lists(omap, n_rows):
+    """Per offset: (map value, row) for every row with an entry, ascending rows, padded
+    with (-1, -1) to a multiple of 32."""
+    pairs, seg = [], [0]
+    for k in range(omap.shape[1]):
+        rows = np.nonzero(omap[:n_rows, k] >= 0)[0]
+        blk = np.full(((len(rows) + 31) // 32 * 32, 2), -1, np.int32)
+        blk[:len(rows), 0] = omap[rows, k]
+        blk[:len(rows), 1] = rows
+        pairs.append(blk)
+        seg.append(seg[-1] + len(blk) // 32)
+    return np.concatenate(pairs), np.array(seg, np.int32)
+
+
+@pytest.mark.parametrize("n,geom", [(1, (3, 1, 1)), (33, (3, 1, 1)), (700, (3, 1, 1)), (5000, (3, 1, 1)),
+                                    (3000, (2, 2, 0)), (3000, (3, 2, 1)), (400, (5, 1, 2))])
+def test_wgrad_pair_lists_are_exact(mods, n, geom):
+    _, backend, _, F = mods
+    rng = np.random.default_rng(n + geom[0])
+    coords = random_coords(rng, n, (30, 30, 10))
+    kmap = F.build_kernel_map(dev(coords), len(coords), *geom, mode="hashmap_on_the_fly")
+    n_out = kmap["sizes"][1]
+    omap = kmap["out_in_map"].cpu().numpy()
+    got = backend.wgrad_pair_lists(kmap["out_in_map"], n_out)
+    want_pairs, want_seg = _expected_pair_lists(omap, n_out)
+    np.testing.assert_array_equal(got["seg_steps"].cpu().numpy(), want_seg)
+    np.testing.assert_array_equal(got["nbsizes"].cpu().numpy(), (omap[:n_out] >= 0).sum(0))
+    np.testing.assert_array_equal(got["pairs"].cpu().numpy()[:len(want_pairs)], want_pairs)
+    assert got["pairs"].shape[0] >= len(want_pairs)
+
+
+@pytest.mark.parametrize("cin,cout", [(32, 32), (64, 96), (96, 64), (128, 128), (16, 40), (8, 8), (200, 72),
+                                      (256, 160), (384, 32)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32, torch.bfloat16])
+def test_wgrad_over_pair_lists_matches_oracle(mods, cin, cout, dtype):
+    _, backend, _, F = mods
+    rng = np.random.default_rng(cin * 100 + cout)
+    coords = random_coords(rng, 1800, (22, 20, 12))
+    n = len(coords)
+    kmap = F.build_kernel_map(dev(coords), n, 3, 1, 1, mode="hashmap_on_the_fly")
+    omap = kmap["out_in_map"]
+    x = torch.from_numpy(rng.standard_normal((n, cin)).astype(np.float32)).to("cuda", dtype)
+    dy = torch.from_numpy(rng.standard_normal((n, cout)).astype(np.float32)).to("cuda", dtype)
+    lists = backend.wgrad_pair_lists(omap, n)
+    assert backend.wgrad_pairs_supported(x, dy)
+    dw = backend.conv_backward_wgrad_pairs_cuda(dy, x, lists, 0)
+    w = np.zeros((27, cin, cout), np.float32)
+    _, want_dw = oracle.conv_backward_implicit_gemm(_f32(x), w, omap.cpu().numpy(), _f32(dy))
+    assert dw.shape == (27, cin, cout) and dw.dtype == dtype
+    assert rel_rms(_f32(dw), want_dw) < TOL[dtype]
+    # the same lists with the roles of the two columns exchanged: the transposed gradient
+    dw_t = backend.conv_backward_wgrad_pairs_cuda(x, dy, lists, 1)
+    assert rel_rms(_f32(dw_t), want_dw.transpose(0, 2, 1)) < TOL[dtype]
+    # and the same sums as the map form, run twice: bit-identical results
+    again = backend.conv_backward_wgrad_pairs_cuda(dy, x, lists, 0)
+    assert torch.equal(dw, again)
+
+
+@pytest.mark.parametrize("n,geom", [(1, (3, 1, 1)), (31, (3, 1, 1)), (257, (3, 1, 1)), (9000, (3, 1, 1)),
+                                    (4000, (2, 2, 0)), (300, (5, 1, 2))])
+def test_wgrad_over_pair_lists_row_counts_and_geometries(mods, n, geom):
+    """Few rows (ranges without work), strided maps (n_in != n_out), a 125-offset kernel."""
+    _, backend, _, F = mods
+    rng = np.random.default_rng(n)
+    coords = random_coords(rng, n, (30, 30, 10))
+    n_in = len(coords)
+    kmap = F.build_kernel_map(dev(coords), n_in, *geom, mode="hashmap_on_the_fly")
+    n_out = kmap["sizes"][1]
+    omap = kmap["out_in_map"]
+    x = torch.from_numpy(rng.standard_normal((n_in, 24)).astype(np.float32)).cuda()
+    dy = torch.from_numpy(rng.standard_normal((n_out, 40)).astype(np.float32)).cuda()
+    dw = backend.conv_backward_wgrad_pairs_cuda(dy, x, backend.wgrad_pair_lists(omap, n_out), 0)
+    w = np.zeros((omap.shape[1], 24, 40), np.float32)
+    _, want_dw = oracle.conv_backward_implicit_gemm(_f32(x), w, omap.cpu().numpy()[:n_out], _f32(dy))
+    assert rel_rms(_f32(dw), want_dw) < 1e-4
+
+
+def test_wgrad_over_pair_lists_rejects_odd_widths(mods):
+    _, backend, _, F = mods
+    rng = np.random.default_rng(0)
+    coords = random_coords(rng, 200, (10, 10, 10))
+    n = len(coords)
+    kmap = F.build_kernel_map(dev(coords), n, 3, 1, 1, mode="hashmap_on_the_fly")
+    lists = backend.wgrad_pair_lists(kmap["out_in_map"], n)
+    x = torch.randn(n, 5, device="cuda", dtype=torch.float16)
+    dy = torch.randn(n, 16, device="cuda", dtype=torch.float16)
+    assert not backend.wgrad_pairs_supported(x, dy)
+    with pytest.raises(ValueError, match="multiples of"):
+        backend.conv_backward_wgrad_pairs_cuda(dy, x, lists, 0)
+
+
 @pytest.mark.parametrize("geom", [(3, 1, 1), (2, 2, 0), (3, 2, 1), (2, 1, 0)])
 @pytest.mark.parametrize("flow", ["ImplicitGEMM", "GatherScatter", "FetchOnDemand"])
 def test_autograd_through_conv3d_matches_oracle(mods, geom, flow):

@@ -37,6 +37,10 @@ def _load():
     lib.tsmi_conv_wgrad_workspace_elems.restype = _i64
     lib.tsmi_conv_wgrad_workspace_elems.argtypes = [_i64, _i32, _i32, _i32, _i32]
     lib.tsmi_conv_workspace_elems.argtypes = [_i64, _i64, _i32, _i32, _i32, _i32, _i32, _i32]
+    lib.tsmi_wgrad_pairs_capacity.restype = _i64
+    lib.tsmi_wgrad_pairs_capacity.argtypes = [_i64, _i32]
+    lib.tsmi_conv_wgrad_pairs_workspace_elems.restype = _i64
+    lib.tsmi_conv_wgrad_pairs_workspace_elems.argtypes = [_i64, _i32, _i32, _i32, _i32]
     sig = {
         "tsmi_hashtable_clear": [_vp, _vp, _vp, _i64],
         "tsmi_hashtable_insert_coords": [_vp, _vp, _vp, _i64, _vp, _i64, _vp],
@@ -64,6 +68,9 @@ def _load():
                                            _i32, _i32, _i32, _vp, _vp, _i32, _vp, _i64, _vp, _i64,
                                            _vp],
         "tsmi_conv_wgrad": [_vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _i32, _i32, _vp, _i64, _vp],
+        "tsmi_wgrad_pairs_build": [_vp, _vp, _i64, _i32, _vp, _vp, _vp, _vp],
+        "tsmi_conv_wgrad_pairs": [_vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _i32, _vp,
+                                  _i64, _vp],
         "tsmi_conv_fetch_on_demand": [_vp, _vp, _vp, _vp, _i64, _vp, _vp, _i64, _vp, _i64, _i32,
                                       _i32, _i32, _i32, _i32, _i32, _vp, _vp, _i32, _vp, _vp],
         "tsmi_gs_gather": [_vp, _vp, _vp, _i64, _i32, _i32, _i32, _vp],
@@ -546,6 +553,56 @@ def conv_backward_wgrad_implicit_gemm_cuda(grad_out: torch.Tensor, in_feats: tor
     ws = torch.empty(max(ws_elems, 1), dtype=torch.float32, device=x.device)
     _check(_C.tsmi_conv_wgrad(_stream(), _ptr(x), _ptr(dy), _ptr(m), m.shape[0], num_in_feats, kvol,
                               cin, cout, code, _ptr(ws), ws_elems, _ptr(dw)))
+    return dw
+
+
+def wgrad_pair_lists(out_in_map: torch.Tensor, n_rows: int) -> dict:
+    """Per-offset (map value, row) pair lists of a kernel map, padded to blocks of 32, for
+    conv_backward_wgrad_pairs_cuda.  No host read-back: `pairs` is sized for a full map and
+    only the part the lists need is written.  Returns dict(pairs int32 [cap, 2], seg_steps
+    int32 [K_vol+1] (first 32-pair block of each offset), nbsizes int32 [K_vol])."""
+    m = _need(out_in_map, torch.int32, "out_in_map")
+    if n_rows > m.shape[0]:
+        raise ValueError(f"map has {m.shape[0]} rows, need {n_rows}")
+    kvol, dev = m.shape[1], m.device
+    cap = _C.tsmi_wgrad_pairs_capacity(n_rows, kvol)
+    pairs = torch.empty((max(cap, 1), 2), dtype=torch.int32, device=dev)
+    block_counts = torch.empty(kvol * max((n_rows + 255) // 256, 1), dtype=torch.int32, device=dev)
+    nbsizes = torch.empty(kvol, dtype=torch.int32, device=dev)
+    seg_steps = torch.empty(kvol + 1, dtype=torch.int32, device=dev)
+    _check(_C.tsmi_wgrad_pairs_build(_stream(), _ptr(m), n_rows, kvol, _ptr(block_counts),
+                                     _ptr(nbsizes), _ptr(pairs), _ptr(seg_steps)))
+    return dict(pairs=pairs, seg_steps=seg_steps, nbsizes=nbsizes, cap=cap)
+
+
+def wgrad_pairs_supported(in_feats: torch.Tensor, grad_out: torch.Tensor) -> bool:
+    """The pair-list weight gradient moves 16-byte pieces of rows: both channel counts
+    must be multiples of 16 bytes of elements."""
+    per = 16 // in_feats.element_size()
+    return in_feats.shape[1] % per == 0 and grad_out.shape[1] % per == 0
+
+
+def conv_backward_wgrad_pairs_cuda(grad_out: torch.Tensor, in_feats: torch.Tensor, pair_lists: dict,
+                                   x_col: int = 0) -> torch.Tensor:
+    """Weight gradient [K_vol, Cin, Cout] of the I/O type from the pair lists of
+    wgrad_pair_lists: dW[k] = sum over offset k's pairs of in_feats[pair[x_col]]^T
+    grad_out[pair[1 - x_col]].  The sums of conv_backward_gather_scatter_cuda's grad_kernel
+    (convolution/convolution_gather_scatter_cuda.cu:815-915), reading only rows that take
+    part in an offset."""
+    if in_feats.dtype != grad_out.dtype:
+        raise ValueError("in_feats and grad_out must have the same dtype")
+    x = _need(in_feats, in_feats.dtype, "in_feats")
+    dy = _need(grad_out, grad_out.dtype, "grad_out")
+    pairs = _need(pair_lists["pairs"], torch.int32, "pairs")
+    seg_steps = _need(pair_lists["seg_steps"], torch.int32, "seg_steps")
+    kvol, cin, cout = seg_steps.numel() - 1, x.shape[1], dy.shape[1]
+    code = _dtype_code(x)
+    cap = int(pair_lists["cap"])
+    dw = torch.empty((kvol, cin, cout), dtype=x.dtype, device=x.device)
+    ws_elems = _C.tsmi_conv_wgrad_pairs_workspace_elems(cap, kvol, cin, cout, code)
+    ws = torch.empty(max(ws_elems, 1), dtype=torch.float32, device=x.device)
+    _check(_C.tsmi_conv_wgrad_pairs(_stream(), _ptr(x), _ptr(dy), _ptr(pairs), _ptr(seg_steps), cap,
+                                    int(x_col), kvol, cin, cout, code, _ptr(ws), ws_elems, _ptr(dw)))
     return dw
 
 

@@ -27,6 +27,11 @@ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 // an int64 element count through this helper and refuses anything larger.
 inline bool grid_fits(int64_t blocks) { return blocks >= 0 && blocks < (int64_t(1) << 31); }
 
+// Weight-gradient pair lists: pairs per reduction step (each offset's list is padded to a
+// multiple of it) and the largest kernel volume the kernels keep a segment table for.
+constexpr int kWgradPairStep = 32;
+constexpr int kWgradMaxKvol = 511;
+
 }  // namespace tsmi
 
 #define TSMI_REQUIRE(cond, ...)                                            \

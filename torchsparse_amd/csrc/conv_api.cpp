@@ -115,6 +115,29 @@ extern "C" int tsmi_conv_wgrad(tsmi_stream_t s, const void *x, const void *dy,
                     workspace_elems, dw);
 }
 
+extern "C" int64_t tsmi_conv_wgrad_pairs_workspace_elems(int64_t pair_cap, int kvol, int cin,
+                                                         int cout, int dtype) {
+  const ConvOps *ops = ops_for(dtype);
+  if (!ops || pair_cap < 0 || kvol < 1 || cin < 1 || cout < 1) return 0;
+  return ops->wgrad_pairs_workspace(pair_cap, kvol, cin, cout);
+}
+
+extern "C" int tsmi_conv_wgrad_pairs(tsmi_stream_t s, const void *x, const void *dy,
+                                     const int32_t *pairs, const int32_t *seg_steps,
+                                     int64_t pair_cap, int x_col, int kvol, int cin, int cout,
+                                     int dtype, float *workspace, int64_t workspace_elems,
+                                     void *dw) {
+  const ConvOps *ops = ops_for(dtype);
+  if (int e = check_shapes("conv_wgrad_pairs", ops, kvol, cin, cout)) return e;
+  TSMI_REQUIRE(pair_cap >= 0 && (x_col == 0 || x_col == 1), "conv_wgrad_pairs: bad arguments");
+  TSMI_REQUIRE(dw && workspace && seg_steps, "conv_wgrad_pairs: null output, workspace or seg_steps");
+  TSMI_REQUIRE(pair_cap == 0 || (x && dy && pairs), "conv_wgrad_pairs: null pointer");
+  TSMI_REQUIRE(aligned16(x) && aligned16(dy) && ((uintptr_t)pairs & 7) == 0,
+               "conv_wgrad_pairs: x and dy must be 16-byte aligned, pairs 8-byte aligned");
+  return ops->wgrad_pairs((hipStream_t)s, x, dy, pairs, seg_steps, pair_cap, x_col, kvol, cin, cout,
+                          workspace, workspace_elems, dw);
+}
+
 extern "C" int tsmi_conv_fetch_on_demand(tsmi_stream_t s, const void *x, const void *w_packed,
                                          const int32_t *nbmaps_planar, int64_t nnz,
                                          const int32_t *nbaddrs, const int32_t *qnbaddrs,

@@ -37,6 +37,7 @@ struct TraitsBF16 {
 #include "conv_igemm2.inc"
 #include "conv_plan.inc"
 #include "conv_wgrad.inc"
+#include "conv_wgrad_pairs.inc"
 #include "conv_igemm_tail.inc"
 
 namespace tsmi {

@@ -37,6 +37,11 @@ struct ConvOps {
   int64_t (*wgrad_workspace)(int64_t n_in, int kvol, int cin, int cout);
   int (*wgrad)(hipStream_t s, const void *x, const void *dy, const int32_t *map_bwd, int64_t n_in,
                int kvol, int cin, int cout, float *partial, int64_t partial_elems, void *dw);
+  // the same sums over padded pair lists (tsmi_wgrad_pairs_build); pairs[:, x_col] indexes x
+  int64_t (*wgrad_pairs_workspace)(int64_t pair_cap, int kvol, int cin, int cout);
+  int (*wgrad_pairs)(hipStream_t s, const void *x, const void *dy, const int32_t *pairs,
+                     const int32_t *seg_steps, int64_t pair_cap, int x_col, int kvol, int cin,
+                     int cout, float *partial, int64_t partial_elems, void *dw);
 };
 
 const ConvOps &conv_ops_f16();

@@ -372,6 +372,61 @@ __global__ void pair_fill_kernel(const int32_t *map, int64_t n_rows, int kvol, i
   }
 }
 
+// Pair lists for the weight gradient: offset k's pairs (map value, row), ordered by row,
+// start at entry seg_steps[k] * kWgradPairStep and are padded with (-1, -1) up to the next
+// multiple of kWgradPairStep, so that a block of kWgradPairStep consecutive entries never
+// mixes two offsets.  `offsets` is the exclusive scan of the per-(offset, block) counts.
+__global__ void wgrad_pair_fill_kernel(const int32_t *map, int64_t n_rows, int kvol, int64_t nblk,
+                                       const int32_t *offsets, const int32_t *nbsizes,
+                                       int32_t *pairs, int32_t *seg_steps) {
+  __shared__ int wave_cnt[kBlock / 64];
+  __shared__ int seg[kWgradMaxKvol + 1];
+  for (int k = threadIdx.x; k < kvol; k += kBlock) seg[k + 1] = nbsizes[k];
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0;
+    for (int k = 0; k < kvol; ++k) {
+      const int c = seg[k + 1];
+      seg[k] = run;
+      run += (c + kWgradPairStep - 1) / kWgradPairStep;
+    }
+    seg[kvol] = run;
+  }
+  __syncthreads();
+  if (blockIdx.x == 0) {
+    for (int k = threadIdx.x; k <= kvol; k += kBlock) seg_steps[k] = seg[k];
+    // the padding entries behind each list
+    for (int k = 0; k < kvol; ++k) {
+      const int64_t end = (int64_t)seg[k] * kWgradPairStep + nbsizes[k];
+      const int64_t stop = (int64_t)seg[k + 1] * kWgradPairStep;
+      const int64_t pos = end + threadIdx.x;
+      if (pos < stop) {
+        pairs[2 * pos] = -1;
+        pairs[2 * pos + 1] = -1;
+      }
+    }
+  }
+  int64_t row = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  for (int k = 0; k < kvol; ++k) {
+    int32_t v = row < n_rows ? map[row * kvol + k] : -1;
+    bool valid = v != -1;
+    unsigned long long b = __ballot(valid);
+    if (lane == 0) wave_cnt[wave] = __popcll(b);
+    __syncthreads();
+    int before = 0;
+    for (int w = 0; w < wave; ++w) before += wave_cnt[w];
+    if (valid) {
+      int rank = before + __popcll(b & ((1ULL << lane) - 1ULL));
+      int64_t pos = (int64_t)seg[k] * kWgradPairStep +
+                    (offsets[(int64_t)k * nblk + blockIdx.x] - offsets[(int64_t)k * nblk]) + rank;
+      pairs[2 * pos] = v;
+      pairs[2 * pos + 1] = (int32_t)row;
+    }
+    __syncthreads();
+  }
+}
+
 // One thread per pair: offset by binary search over the exclusive scan, position
 // inside the offset's list by subtraction.
 __global__ void masks_from_pairs_kernel(const int32_t *pairs, int64_t nnz, const int32_t *nbaddrs,
@@ -690,6 +745,33 @@ extern "C" int tsmi_pair_lists_fill(tsmi_stream_t s, const int32_t *map, int64_t
                        n_in, n_out, input_mask, output_mask, skip_k);
   }
   return check_launch("tsmi_pair_lists_fill");
+}
+
+extern "C" int64_t tsmi_wgrad_pairs_capacity(int64_t n_rows, int kvol) {
+  if (n_rows < 0 || kvol < 1) return 0;
+  return n_rows * kvol + (int64_t)kvol * (kWgradPairStep - 1);
+}
+
+extern "C" int tsmi_wgrad_pairs_build(tsmi_stream_t s, const int32_t *map, int64_t n_rows, int kvol,
+                                      int32_t *block_counts, int32_t *nbsizes, int32_t *pairs,
+                                      int32_t *seg_steps) {
+  TSMI_REQUIRE(kvol >= 1 && kvol <= kWgradMaxKvol && n_rows >= 0,
+               "wgrad_pairs_build: bad sizes (kernel volume %d, at most %d)", kvol, kWgradMaxKvol);
+  TSMI_REQUIRE(nbsizes && seg_steps, "wgrad_pairs_build: null pointer");
+  TSMI_REQUIRE(n_rows * kvol < (int64_t(1) << 31), "wgrad_pairs_build: too many map entries");
+  if (n_rows == 0) {
+    hipLaunchKernelGGL(fill_kernel<int32_t>, grid_for(kvol + 1), dim3(kBlock), 0, (hipStream_t)s,
+                       seg_steps, (int64_t)kvol + 1, 0);
+    hipLaunchKernelGGL(fill_kernel<int32_t>, grid_for(kvol), dim3(kBlock), 0, (hipStream_t)s,
+                       nbsizes, (int64_t)kvol, 0);
+    return check_launch("tsmi_wgrad_pairs_build");
+  }
+  if (int e = tsmi_pair_lists_count(s, map, n_rows, kvol, block_counts, nbsizes)) return e;
+  TSMI_REQUIRE(pairs, "wgrad_pairs_build: null pairs");
+  int64_t nblk = ceil_div(n_rows, kBlock);
+  hipLaunchKernelGGL(wgrad_pair_fill_kernel, dim3((unsigned)nblk), dim3(kBlock), 0, (hipStream_t)s,
+                     map, n_rows, kvol, nblk, block_counts, nbsizes, pairs, seg_steps);
+  return check_launch("tsmi_wgrad_pairs_build");
 }
 
 extern "C" int tsmi_exclusive_scan_quantified(tsmi_stream_t s, int kvol, const int32_t *nbsizes,

@@ -4,7 +4,9 @@
     dW[k]  += X[m]^T dY[i]          for every map entry  map[i, k] = m >= 0
 
 The input gradient is the forward implicit-GEMM kernel over the transposed map with
-the weights transposed per offset; the weight gradient has a kernel of its own
+the weights transposed per offset.  The weight gradient runs over per-offset pair lists
+derived from the map (tsmi_conv_wgrad_pairs: only rows that take part in an offset are
+read); channel counts that are not a multiple of 16 bytes use the map form
 (tsmi_conv_wgrad).  Both follow the reference's func/implicit_gemm.py:108-190 (unsorted
 branch); the gather-scatter and fetch-on-demand dataflows get the same gradients from
 the same maps (the reference computes theirs with conv_backward_gather_scatter_cuda,
@@ -16,7 +18,7 @@ import torch
 from torchsparse_amd import backend
 from torchsparse_amd.utils import make_divisible
 
-__all__ = ["SparseConvFunction", "backward_map"]
+__all__ = ["SparseConvFunction", "backward_map", "wgrad_pairs"]
 
 
 def backward_map(kmap: Dict, transposed: bool) -> torch.Tensor:
@@ -26,10 +28,21 @@ def backward_map(kmap: Dict, transposed: bool) -> torch.Tensor:
     if transposed:
         return kmap["out_in_map"]
     if kmap.get("out_in_map_bwd") is None:
-        n_in, n_out = kmap["sizes"]
-        kmap["out_in_map_bwd"] = backend.convert_transposed_out_in_map(
-            kmap["out_in_map"], make_divisible(n_in, 128), n_out)
+        if kmap.get("out_in_map_t") is not None:  # a transposed convolution already built it
+            kmap["out_in_map_bwd"] = kmap["out_in_map_t"]
+        else:
+            n_in, n_out = kmap["sizes"]
+            kmap["out_in_map_bwd"] = backend.convert_transposed_out_in_map(
+                kmap["out_in_map"], make_divisible(n_in, 128), n_out)
     return kmap["out_in_map_bwd"]
+
+
+def wgrad_pairs(kmap: Dict) -> Dict:
+    """Per-offset (input row, output row) pair lists of the strided / submanifold map, built
+    once per map and shared by every convolution (transposed ones included) that uses it."""
+    if kmap.get("wgrad_pairs") is None:
+        kmap["wgrad_pairs"] = backend.wgrad_pair_lists(kmap["out_in_map"], kmap["sizes"][1])
+    return kmap["wgrad_pairs"]
 
 
 class SparseConvFunction(torch.autograd.Function):
@@ -52,17 +65,23 @@ class SparseConvFunction(torch.autograd.Function):
         dy = grad_output.contiguous()
         if dy.dtype != x.dtype:
             dy = dy.to(x.dtype)
-        map_bwd = backward_map(kmap, transposed)
         sizes = kmap["sizes"]
         n_in = sizes[1] if transposed else sizes[0]
         grad_input = grad_weight = None
         if ctx.needs_input_grad[0]:
             grad_input = backend.conv_forward_implicit_gemm_cuda(
-                dy, w.transpose(1, 2).contiguous(), map_bwd, n_in, w.shape[1])
+                dy, w.transpose(1, 2).contiguous(), backward_map(kmap, transposed), n_in, w.shape[1])
             if grad_input.dtype != input.dtype:
                 grad_input = grad_input.to(input.dtype)
         if ctx.needs_input_grad[1]:
-            grad_weight = backend.conv_backward_wgrad_implicit_gemm_cuda(dy, x, map_bwd, n_in)
+            if backend.wgrad_pairs_supported(x, dy):
+                # the map's values index the strided convolution's input: x for a plain
+                # convolution (column 0), dy for a transposed one
+                grad_weight = backend.conv_backward_wgrad_pairs_cuda(
+                    dy, x, wgrad_pairs(kmap), 1 if transposed else 0)
+            else:
+                grad_weight = backend.conv_backward_wgrad_implicit_gemm_cuda(
+                    dy, x, backward_map(kmap, transposed), n_in)
             grad_weight = grad_weight.reshape(weight.shape)
             if grad_weight.dtype != weight.dtype:
                 grad_weight = grad_weight.to(weight.dtype)
