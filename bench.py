@@ -1,6 +1,6 @@
 """Benchmark of the sparse-convolution forward hot path on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-layers]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-layers] [--no-backward]
 
 One step = one MinkUNet (SparseResUNet42 + 19-class linear head) forward in fp16 on a
 synthetic 64-beam LiDAR scan (~90k voxels, 4 input channels), starting from a fresh
@@ -17,6 +17,8 @@ Also measured (same JSON line):
                 alone with HIP events on the launch stream
   cpu_baseline  the CPU oracle (a C restatement of the reference's CPU backend) running
                 the network's sparse convolutions and kernel maps on the host cores
+  backward      input- and weight-gradient kernels of the sweep's submanifold layers, the
+                pair-list build the weight gradient needs, one training step of the network
 """
 import argparse
 import json
@@ -42,6 +44,7 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-layers", action="store_true", help="skip the single-layer sweep")
     ap.add_argument("--no-roofline", action="store_true", help="skip the per-kernel roofline timing")
+    ap.add_argument("--no-backward", action="store_true", help="skip the backward (training) figures")
     ap.add_argument("--pmc-target", default=None, metavar="KERNEL",
                     help="run only a 256 MiB device copy (5 launches) and one conv kernel (5 launches) "
                          "for a hardware-counter pass; KERNEL is the description a normal run prints "
@@ -162,6 +165,51 @@ def layer_sweep(ts, spnn, F, backend, coords_dev, n):
                     "eff_TFLOPs": round(flops / conv_ms / 1e9, 2),
                     "min_bytes_GBps": round(nbytes / conv_ms / 1e6, 1)})
         del y
+    return out
+
+
+def backward_sweep(ts, spnn, F, backend, coords_dev, n, feats):
+    """Backward of the sweep's submanifold layers on the same scan (fp16, HIP events): input
+    gradient (the forward kernel over the transposed map), weight gradient over pair lists,
+    the build of those lists; and one training step (forward + backward, batch-norm in
+    training mode) of the whole network."""
+    from torchsparse_amd.backbones import SparseResUNet42
+    km = F.build_kernel_map(coords_dev, n, 3, 1, 1, mode="hashmap_on_the_fly")
+    omap = km["out_in_map"]
+    nnz = int((omap[:n] >= 0).sum().item())
+    map_bwd = backend.convert_transposed_out_in_map(omap, omap.shape[0], n)
+    lists = backend.wgrad_pair_lists(omap, n)
+    out = {"pair_lists_ms": round(event_ms(lambda: backend.wgrad_pair_lists(omap, n), iters=10), 4),
+           "transposed_map_ms": round(event_ms(
+               lambda: backend.convert_transposed_out_in_map(omap, omap.shape[0], n), iters=10), 4),
+           "layers": []}
+    for c in (32, 64, 96, 128):
+        x = torch.randn(n, c, device="cuda", dtype=torch.float16)
+        dy = torch.randn(n, c, device="cuda", dtype=torch.float16)
+        wt = torch.randn(27, c, c, device="cuda", dtype=torch.float16) * 0.05
+        dgrad = event_ms(lambda: backend.conv_forward_implicit_gemm_cuda(dy, wt, map_bwd, n, c), iters=20)
+        wgrad = event_ms(lambda: backend.conv_backward_wgrad_pairs_cuda(dy, x, lists, 0), iters=20)
+        flops = 2.0 * nnz * c * c
+        # bytes the weight gradient has to move: every pair's two rows once, the pair list, dW
+        wbytes = nnz * (2 * c * 2 + 8) + 27 * c * c * 2
+        out["layers"].append({"layer": f"subm_k3_{c}_{c}", "nnz": nnz,
+                              "dgrad_ms": round(dgrad, 4), "dgrad_eff_TFLOPs": round(flops / dgrad / 1e9, 2),
+                              "wgrad_ms": round(wgrad, 4), "wgrad_eff_TFLOPs": round(flops / wgrad / 1e9, 2),
+                              "wgrad_gathered_GBps": round(wbytes / wgrad / 1e6, 1)})
+    net = SparseResUNet42(in_channels=4).cuda().half().train()
+
+    def step():
+        net.zero_grad(set_to_none=True)
+        y = net(ts.SparseTensor(feats, coords_dev))[-1].feats
+        y.float().square().mean().backward()
+    for _ in range(3):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(10):
+        step()
+    torch.cuda.synchronize()
+    out["train_step_ms"] = round((time.perf_counter() - t0) * 100, 4)
     return out
 
 
@@ -354,6 +402,7 @@ def main():
         roof = None if args.no_roofline else dominant_layer_roofline(ts, F, records, inp._caches)
         level_coords = {lvl: c[0].cpu().numpy() for lvl, c in inp._caches.cmaps.items()}
         layers = None if args.no_layers else layer_sweep(ts, spnn, F, backend, coords, n)
+    backward = None if args.no_backward else backward_sweep(ts, spnn, F, backend, coords, n, feats)
     cpu = None if args.no_cpu else cpu_baseline(records, level_coords)
 
     result = {
@@ -367,7 +416,7 @@ def main():
                    "voxels": n, "warm_map_ms_per_step": round(warm_ms, 4),
                    "unfused_ms_per_step": round(ms_unfused, 4),
                    "conv_mode": F.get_conv_mode().value},
-        "roofline": roof, "cpu_baseline": cpu, "layers": layers,
+        "roofline": roof, "cpu_baseline": cpu, "layers": layers, "backward": backward,
     }
     print(json.dumps(result))
 
