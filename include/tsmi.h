@@ -296,8 +296,14 @@ int tsmi_conv_wgrad(tsmi_stream_t s, const void *x, const void *dy, const int32_
  * `workspace` holds tsmi_conv_wgrad_pairs_workspace_elems floats; pair_cap is the
  * capacity `pairs` was built with.  Same sums as conv_backward_gather_scatter_cuda's
  * grad_kernel (convolution/convolution_gather_scatter_cuda.cu:815-915) and as
- * conv_backward_wgrad_implicit_gemm_cuda, accumulated in fp32. */
+ * conv_backward_wgrad_implicit_gemm_cuda, accumulated in fp32.
+ *
+ * tsmi_wgrad_pairs_pad makes the same padded lists from pair lists that already exist
+ * (nbmaps_inter int32[nnz,2], offset k's nbsizes[k] pairs one after the other, as the
+ * gather-scatter dataflow holds them); `pairs` then needs nnz + 31 * K_vol entries. */
 int64_t tsmi_wgrad_pairs_capacity(int64_t n_rows, int kvol);
+int tsmi_wgrad_pairs_pad(tsmi_stream_t s, const int32_t *nbmaps_inter, int64_t nnz,
+                         const int32_t *nbsizes, int kvol, int32_t *pairs, int32_t *seg_steps);
 int tsmi_wgrad_pairs_build(tsmi_stream_t s, const int32_t *map, int64_t n_rows, int kvol,
                            int32_t *block_counts, int32_t *nbsizes, int32_t *pairs,
                            int32_t *seg_steps);

@@ -159,6 +159,64 @@ def test_wgrad_over_pair_lists_rejects_odd_widths(mods):
         backend.conv_backward_wgrad_pairs_cuda(dy, x, lists, 0)
 
 
+@pytest.mark.parametrize("geom", [(3, 1, 1), (2, 2, 0), (3, 2, 1)])
+@pytest.mark.parametrize("transpose", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_backward_over_gather_scatter_pair_lists(mods, geom, transpose, dtype):
+    """conv_backward_gather_scatter_cuda fills both gradients in place from the dataflow's
+    own pair lists; the oracle's pair-list backward is the reference CPU kernel's restatement."""
+    _, backend, _, F = mods
+    rng = np.random.default_rng(sum(geom) + transpose)
+    coords = random_coords(rng, 1500, (20, 18, 12))
+    n_in = len(coords)
+    kmap = F.build_kernel_map(dev(coords), n_in, *geom, mode="hashmap_on_the_fly",
+                              dataflow=F.Dataflow.GatherScatter)
+    n_out = kmap["sizes"][1]
+    kvol, cin, cout = kmap["out_in_map"].shape[1], 24, 40
+    n_x, n_y = (n_out, n_in) if transpose else (n_in, n_out)
+    x = torch.from_numpy(rng.standard_normal((n_x, cin)).astype(np.float32)).to("cuda", dtype)
+    dy = torch.from_numpy(rng.standard_normal((n_y, cout)).astype(np.float32)).to("cuda", dtype)
+    w = torch.from_numpy(rng.uniform(-0.1, 0.1, (kvol, cin, cout)).astype(np.float32)).to("cuda", dtype)
+    nbmaps = kmap["nbmaps"].int()
+    dx, dw = torch.empty(0, device="cuda", dtype=dtype), torch.empty(0, device="cuda", dtype=dtype)
+    backend.conv_backward_gather_scatter_cuda(x, dx, dy, w, dw, nbmaps, kmap["nbsizes"].cpu(), transpose)
+    want_dx, want_dw = oracle.conv_backward_gather_scatter(
+        _f32(x), _f32(w), nbmaps.cpu().numpy(), kmap["nbsizes"].cpu().numpy(), _f32(dy), transpose)
+    assert dx.shape == x.shape and dw.shape == w.shape
+    assert rel_rms(_f32(dx), want_dx) < TOL[dtype]
+    assert rel_rms(_f32(dw), want_dw) < TOL[dtype]
+
+
+@pytest.mark.parametrize("ifsort", [False, True])
+def test_training_kernel_map_holds_the_backward_products(mods, ifsort):
+    _, backend, _, F = mods
+    rng = np.random.default_rng(3)
+    coords = random_coords(rng, 2500, (20, 18, 12))
+    n_in = len(coords)
+    kmap = F.build_kernel_map(dev(coords), n_in, 3, 2, 1, mode="hashmap_on_the_fly", training=True,
+                              ifsort=ifsort, split_mask_num=1, split_mask_num_bwd=3)
+    n_out = kmap["sizes"][1]
+    omap = kmap["out_in_map"].cpu().numpy()
+    bwd = kmap["out_in_map_bwd"].cpu().numpy()
+    assert bwd.shape == ((n_in + 127) // 128 * 128, 27)
+    want = np.full_like(bwd, -1)
+    rows, ks = np.nonzero(omap[:n_out] >= 0)
+    want[omap[rows, ks], ks] = rows
+    np.testing.assert_array_equal(bwd, want)
+    if not ifsort:
+        assert kmap["reorder_out_in_map_bwd"] is None
+        return
+    loc = kmap["reorder_loc_bwd"].cpu().numpy()
+    assert loc.shape == (3, bwd.shape[0])
+    for s in range(3):
+        assert sorted(loc[s].tolist()) == list(range(bwd.shape[0]))
+    ro = kmap["reorder_out_in_map_bwd"].cpu().numpy()
+    for s in range(3):
+        np.testing.assert_array_equal(ro[:, s * 9:(s + 1) * 9], bwd[loc[s]][:, s * 9:(s + 1) * 9])
+    assert kmap["reduced_sorted_mask_bwd_wgrad"].shape == (3, (bwd.shape[0] - 1) // 64 + 1)
+    assert kmap["reduced_sorted_mask_bwd_dgrad"].shape == (3, (bwd.shape[0] - 1) // 128 + 1)
+
+
 @pytest.mark.parametrize("geom", [(3, 1, 1), (2, 2, 0), (3, 2, 1), (2, 1, 0)])
 @pytest.mark.parametrize("flow", ["ImplicitGEMM", "GatherScatter", "FetchOnDemand"])
 def test_autograd_through_conv3d_matches_oracle(mods, geom, flow):

@@ -69,6 +69,7 @@ def _load():
                                            _vp],
         "tsmi_conv_wgrad": [_vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _i32, _i32, _vp, _i64, _vp],
         "tsmi_wgrad_pairs_build": [_vp, _vp, _i64, _i32, _vp, _vp, _vp, _vp],
+        "tsmi_wgrad_pairs_pad": [_vp, _vp, _i64, _vp, _i32, _vp, _vp],
         "tsmi_conv_wgrad_pairs": [_vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _i32, _vp,
                                   _i64, _vp],
         "tsmi_conv_fetch_on_demand": [_vp, _vp, _vp, _vp, _i64, _vp, _vp, _i64, _vp, _i64, _i32,
@@ -575,6 +576,21 @@ def wgrad_pair_lists(out_in_map: torch.Tensor, n_rows: int) -> dict:
     return dict(pairs=pairs, seg_steps=seg_steps, nbsizes=nbsizes, cap=cap)
 
 
+def wgrad_pair_lists_from_nbmaps(nbmaps: torch.Tensor, nbsizes: torch.Tensor) -> dict:
+    """The padded lists of wgrad_pair_lists from the gather-scatter dataflow's own pair
+    lists: nbmaps int32 [nnz, 2] rows (in, out) ordered by offset, nbsizes [K_vol]."""
+    nbmaps = _need(nbmaps, torch.int32, "nbmaps")
+    dev = nbmaps.device
+    sizes = nbsizes.to(device=dev, dtype=torch.int32).contiguous()
+    kvol, nnz = sizes.numel(), nbmaps.shape[0]
+    cap = nnz + 31 * kvol
+    pairs = torch.empty((max(cap, 1), 2), dtype=torch.int32, device=dev)
+    seg_steps = torch.empty(kvol + 1, dtype=torch.int32, device=dev)
+    _check(_C.tsmi_wgrad_pairs_pad(_stream(), _ptr(nbmaps), nnz, _ptr(sizes), kvol, _ptr(pairs),
+                                   _ptr(seg_steps)))
+    return dict(pairs=pairs, seg_steps=seg_steps, nbsizes=sizes, cap=cap)
+
+
 def wgrad_pairs_supported(in_feats: torch.Tensor, grad_out: torch.Tensor) -> bool:
     """The pair-list weight gradient moves 16-byte pieces of rows: both channel counts
     must be multiples of 16 bytes of elements."""
@@ -604,6 +620,39 @@ def conv_backward_wgrad_pairs_cuda(grad_out: torch.Tensor, in_feats: torch.Tenso
     _check(_C.tsmi_conv_wgrad_pairs(_stream(), _ptr(x), _ptr(dy), _ptr(pairs), _ptr(seg_steps), cap,
                                     int(x_col), kvol, cin, cout, code, _ptr(ws), ws_elems, _ptr(dw)))
     return dw
+
+
+def conv_backward_gather_scatter_cuda(in_feat: torch.Tensor, grad_in_feat: torch.Tensor,
+                                      grad_out_feat: torch.Tensor, kernel: torch.Tensor,
+                                      grad_kernel: torch.Tensor, neighbor_map: torch.Tensor,
+                                      neighbor_offset: torch.Tensor, transpose: bool) -> None:
+    """convolution/convolution_gather_scatter_cuda.cu:815-915: fills grad_in_feat (shape of
+    in_feat) and grad_kernel (shape of kernel) in place from the pair lists neighbor_map
+    int32 [nnz, 2] rows (in, out) and their per-offset sizes neighbor_offset.
+
+    grad_in  = the forward dataflow over the same lists with the two columns exchanged and
+               the weights transposed per offset (sums through the masks, no atomics);
+    grad_w   = the pair-list weight-gradient kernel (the map form's sums for channel counts
+               that are not a multiple of 16 bytes are not reachable from pair lists:
+               those raise)."""
+    x = _need(in_feat, in_feat.dtype, "in_feat")
+    dy = _need(grad_out_feat, x.dtype, "grad_out_feat")
+    nbmaps = _need(neighbor_map, torch.int32, "neighbor_map")
+    w = kernel if kernel.dim() == 3 else kernel.unsqueeze(0)
+    kvol = w.shape[0]
+    if not transpose:
+        n_in, n_out = x.shape[0], dy.shape[0]   # sizes of the pair columns (in, out)
+    else:
+        n_in, n_out = dy.shape[0], x.shape[0]
+    sizes = neighbor_offset.to(device=x.device, dtype=torch.int32)
+    imask, omask = build_mask_from_kmap(n_in, n_out, nbmaps, sizes)
+    center = kvol // 2 if (n_in == n_out and kvol % 2 == 1) else -1
+    dx = conv_forward_gather_scatter_cuda(dy, w.transpose(1, 2).contiguous(), nbmaps, sizes, imask, omask,
+                                          x.shape[0], transpose=not transpose, center_k=center)
+    lists = wgrad_pair_lists_from_nbmaps(nbmaps, sizes)
+    dw = conv_backward_wgrad_pairs_cuda(dy, x, lists, 1 if transpose else 0)
+    grad_in_feat.resize_(x.shape).copy_(dx)
+    grad_kernel.resize_(kernel.shape).copy_(dw.reshape(kernel.shape))
 
 
 def conv_forward_fetch_on_demand_cuda(in_feats, kernel, nbmaps, sum_nnz, nbaddrs, qnbaddrs,

@@ -427,6 +427,49 @@ __global__ void wgrad_pair_fill_kernel(const int32_t *map, int64_t n_rows, int k
   }
 }
 
+// Padded copy of existing interleaved pair lists (offset k's nbsizes[k] pairs follow each
+// other without gaps): the layout wgrad_pair_fill_kernel writes.  One thread per entry of
+// the padded array; `limit` bounds the entries a launch may touch.
+__global__ void wgrad_pair_pad_kernel(const int32_t *nbmaps, int64_t nnz, const int32_t *nbsizes,
+                                      int kvol, int64_t limit, int32_t *pairs,
+                                      int32_t *seg_steps) {
+  __shared__ int seg[kWgradMaxKvol + 1];   // padded start of each list, in steps
+  __shared__ int src[kWgradMaxKvol + 1];   // start of each list in nbmaps
+  for (int k = threadIdx.x; k < kvol; k += kBlock) seg[k + 1] = nbsizes[k];
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0, raw = 0;
+    for (int k = 0; k < kvol; ++k) {
+      const int c = seg[k + 1];
+      seg[k] = run;
+      src[k] = raw;
+      run += (c + kWgradPairStep - 1) / kWgradPairStep;
+      raw += c;
+    }
+    seg[kvol] = run;
+    src[kvol] = raw;
+  }
+  __syncthreads();
+  if (blockIdx.x == 0)
+    for (int k = threadIdx.x; k <= kvol; k += kBlock) seg_steps[k] = seg[k];
+  const int64_t pos = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (pos >= limit || pos >= (int64_t)seg[kvol] * kWgradPairStep) return;
+  const int step = (int)(pos / kWgradPairStep);
+  int lo = 0, hi = kvol;  // largest k with seg[k] <= step
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (seg[mid] <= step) lo = mid; else hi = mid;
+  }
+  const int64_t j = pos - (int64_t)seg[lo] * kWgradPairStep;
+  int32_t a = -1, b = -1;
+  if (j < src[lo + 1] - src[lo] && src[lo] + j < nnz) {
+    a = nbmaps[2 * (src[lo] + j)];
+    b = nbmaps[2 * (src[lo] + j) + 1];
+  }
+  pairs[2 * pos] = a;
+  pairs[2 * pos + 1] = b;
+}
+
 // One thread per pair: offset by binary search over the exclusive scan, position
 // inside the offset's list by subtraction.
 __global__ void masks_from_pairs_kernel(const int32_t *pairs, int64_t nnz, const int32_t *nbaddrs,
@@ -772,6 +815,20 @@ extern "C" int tsmi_wgrad_pairs_build(tsmi_stream_t s, const int32_t *map, int64
   hipLaunchKernelGGL(wgrad_pair_fill_kernel, dim3((unsigned)nblk), dim3(kBlock), 0, (hipStream_t)s,
                      map, n_rows, kvol, nblk, block_counts, nbsizes, pairs, seg_steps);
   return check_launch("tsmi_wgrad_pairs_build");
+}
+
+extern "C" int tsmi_wgrad_pairs_pad(tsmi_stream_t s, const int32_t *nbmaps_inter, int64_t nnz,
+                                    const int32_t *nbsizes, int kvol, int32_t *pairs,
+                                    int32_t *seg_steps) {
+  TSMI_REQUIRE(kvol >= 1 && kvol <= kWgradMaxKvol && nnz >= 0,
+               "wgrad_pairs_pad: bad sizes (kernel volume %d, at most %d)", kvol, kWgradMaxKvol);
+  TSMI_REQUIRE(nbsizes && seg_steps && pairs, "wgrad_pairs_pad: null pointer");
+  TSMI_REQUIRE(nnz == 0 || nbmaps_inter, "wgrad_pairs_pad: null pair list");
+  const int64_t limit = nnz + (int64_t)kvol * (kWgradPairStep - 1);
+  TSMI_GRID_CHECK(limit);
+  hipLaunchKernelGGL(wgrad_pair_pad_kernel, grid_for(std::max<int64_t>(limit, 1)), dim3(kBlock), 0,
+                     (hipStream_t)s, nbmaps_inter, nnz, nbsizes, kvol, limit, pairs, seg_steps);
+  return check_launch("tsmi_wgrad_pairs_pad");
 }
 
 extern "C" int tsmi_exclusive_scan_quantified(tsmi_stream_t s, int kvol, const int32_t *nbsizes,

@@ -23,6 +23,7 @@ from ..conv_config import Dataflow
 __all__ = ["build_kernel_map", "transpose_kernel_map"]
 
 cta_M = 128  # row padding of every map and tile size of the reduced masks
+cta_M_wgrad = 64  # reduce tile of the sorted weight-gradient mask (build_kmap.py:16)
 
 
 def _empty_kmap(hashmap_keys, hashmap_vals, spatial_range) -> Dict:
@@ -55,6 +56,24 @@ def _sort_products(kmap: Dict, out_in_map: torch.Tensor, valid_n: int, split_mas
     kmap["reduced_sorted_mask" + suffix] = backend.reduce_bitmask_cuda(sorted_mask, cta_M)
     kmap["reorder_loc" + suffix] = reorder_loc
     kmap["sorted_mask" + suffix] = sorted_mask
+
+
+def _backward_products(kmap: Dict, ifsort: bool, split_mask_num_bwd: int) -> None:
+    """Training-time products (build_kmap.py:191-220): the transposed map the input gradient
+    runs over and, for sorted mode, its sort products with the reference's two reduce tiles
+    (64 rows for the weight gradient, 128 for the input gradient).  The backward here runs
+    unsorted, so the sort products are built only when ``ifsort`` asks for them."""
+    n_in, n_out = kmap["sizes"]
+    bwd = backend.convert_transposed_out_in_map(kmap["out_in_map"], make_divisible(n_in, cta_M), n_out)
+    kmap["out_in_map_bwd"] = bwd
+    if not ifsort:
+        return
+    bitmask = backend.derive_bitmask_from_out_in_map(bwd, split_mask_num_bwd, n_in)
+    sorted_mask, reorder_loc = backend.sort_bitmask_descending(bitmask)
+    kmap["reorder_out_in_map_bwd"] = backend.reorder_out_in_map_cuda(bwd, reorder_loc)
+    kmap["reduced_sorted_mask_bwd_wgrad"] = backend.reduce_bitmask_cuda(sorted_mask, cta_M_wgrad)
+    kmap["reduced_sorted_mask_bwd_dgrad"] = backend.reduce_bitmask_cuda(sorted_mask, cta_M)
+    kmap["reorder_loc_bwd"] = reorder_loc
 
 
 def _pair_products(kmap: Dict, dataflow: Dataflow) -> None:
@@ -146,6 +165,8 @@ def build_kernel_map(_coords: torch.Tensor, input_node_num: int,
     if dataflow == Dataflow.ImplicitGEMM:
         if ifsort:
             _sort_products(kmap, out_in_map, kmap["sizes"][1], split_mask_num)
+        if training:
+            _backward_products(kmap, ifsort, split_mask_num_bwd)
     else:
         _pair_products(kmap, dataflow)
     return kmap
