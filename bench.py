@@ -1,6 +1,6 @@
 """Benchmark of the sparse-convolution forward hot path on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-layers] [--no-backward]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-layers] [--no-backward] [--no-tune]
 
 One step = one MinkUNet (SparseResUNet42 + 19-class linear head) forward in fp16 on a
 synthetic 64-beam LiDAR scan (~90k voxels, 4 input channels), starting from a fresh
@@ -17,6 +17,8 @@ Also measured (same JSON line):
                 alone with HIP events on the launch stream
   cpu_baseline  the CPU oracle (a C restatement of the reference's CPU backend) running
                 the network's sparse convolutions and kernel maps on the host cores
+  tuned         utils.tune.tune over the three dataflows and the sorted variants, and the
+                step time of the tuned network beside the default configuration's
   backward      input- and weight-gradient kernels of the sweep's submanifold layers, the
                 pair-list build the weight gradient needs, one training step of the network
 """
@@ -45,6 +47,7 @@ def parse():
     ap.add_argument("--no-layers", action="store_true", help="skip the single-layer sweep")
     ap.add_argument("--no-roofline", action="store_true", help="skip the per-kernel roofline timing")
     ap.add_argument("--no-backward", action="store_true", help="skip the backward (training) figures")
+    ap.add_argument("--no-tune", action="store_true", help="skip the per-group tuner run")
     ap.add_argument("--pmc-target", default=None, metavar="KERNEL",
                     help="run only a 256 MiB device copy (5 launches) and one conv kernel (5 launches) "
                          "for a hardware-counter pass; KERNEL is the description a normal run prints "
@@ -403,6 +406,23 @@ def main():
         level_coords = {lvl: c[0].cpu().numpy() for lvl, c in inp._caches.cmaps.items()}
         layers = None if args.no_layers else layer_sweep(ts, spnn, F, backend, coords, n)
     backward = None if args.no_backward else backward_sweep(ts, spnn, F, backend, coords, n, feats)
+    tuned = None
+    if not args.no_tune:
+        # the per-group tuner over all three dataflows and the sorted variants, then the same
+        # timed loop on the tuned copy of the network
+        import tempfile
+        from torchsparse_amd.utils.tune import tune
+        tuned_model = copy.deepcopy(model)
+        with tempfile.TemporaryDirectory() as tmp:
+            chosen = tune(tuned_model, [ts.SparseTensor(feats, coords) for _ in range(3)], n_samples=3,
+                          save_dir=tmp, tune_tag="bench", verbose=False, skip_warning=True,
+                          dataflow_range=[F.Dataflow.ImplicitGEMM, F.Dataflow.FetchOnDemand,
+                                          F.Dataflow.GatherScatter])
+        tuned = {"ms_per_step": round(timed(tuned_model, args.steps, args.warmup), 4),
+                 "default_ms_per_step": round(timed(model, args.steps, args.warmup), 4),
+                 "groups": [{"level": g[0], "kernel": g[1], "stride": g[2],
+                             "dataflow": c["dataflow"].name, "ifsort": c["ifsort"],
+                             "split_mask_num": c["split_mask_num"]} for g, c in chosen.items()]}
     cpu = None if args.no_cpu else cpu_baseline(records, level_coords)
 
     result = {
@@ -417,6 +437,7 @@ def main():
                    "unfused_ms_per_step": round(ms_unfused, 4),
                    "conv_mode": F.get_conv_mode().value},
         "roofline": roof, "cpu_baseline": cpu, "layers": layers, "backward": backward,
+        "tuned": tuned,
     }
     print(json.dumps(result))
 
