@@ -1,6 +1,6 @@
 """Benchmark of the sparse-convolution forward hot path on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-layers] [--no-backward] [--no-tune]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-layers] [--no-backward] [--no-tune] [--no-pointops]
 
 One step = one MinkUNet (SparseResUNet42 + 19-class linear head) forward in fp16 on a
 synthetic 64-beam LiDAR scan (~90k voxels, 4 input channels), starting from a fresh
@@ -19,6 +19,8 @@ Also measured (same JSON line):
                 the network's sparse convolutions and kernel maps on the host cores
   tuned         utils.tune.tune over the three dataflows and the sorted variants, and the
                 step time of the tuned network beside the default configuration's
+  pointops      the point-voxel operators (hash, query, count, voxelize, devoxelize) on a
+                synthetic 1M-point cloud: ms and GB/s of the bytes each has to touch
   backward      input- and weight-gradient kernels of the sweep's submanifold layers, the
                 pair-list build the weight gradient needs, one training step of the network
 """
@@ -48,6 +50,7 @@ def parse():
     ap.add_argument("--no-roofline", action="store_true", help="skip the per-kernel roofline timing")
     ap.add_argument("--no-backward", action="store_true", help="skip the backward (training) figures")
     ap.add_argument("--no-tune", action="store_true", help="skip the per-group tuner run")
+    ap.add_argument("--no-pointops", action="store_true", help="skip the point-voxel operator sweep")
     ap.add_argument("--pmc-target", default=None, metavar="KERNEL",
                     help="run only a 256 MiB device copy (5 launches) and one conv kernel (5 launches) "
                          "for a hardware-counter pass; KERNEL is the description a normal run prints "
@@ -214,6 +217,50 @@ def backward_sweep(ts, spnn, F, backend, coords_dev, n, feats):
     torch.cuda.synchronize()
     out["train_step_ms"] = round((time.perf_counter() - t0) * 100, 4)
     return out
+
+
+def pointops_sweep(F):
+    """The point-voxel operators on a synthetic cloud (1M points in ~200k voxels, 64 channels,
+    fp16): HIP-event time and the rate at which the bytes each op has to touch move."""
+    n, c, b = 1_000_000, 64, 2
+    g = torch.Generator(device="cuda").manual_seed(0)
+    pts = torch.rand(n, 3, device="cuda", generator=g) * torch.tensor([160.0, 160.0, 8.0], device="cuda")
+    pc = torch.cat([torch.zeros(n, 1, device="cuda", dtype=torch.int32), pts.floor().int()], 1).contiguous()
+    offsets = torch.tensor([[dx, dy, dz] for dx in (0, 1) for dy in (0, 1) for dz in (0, 1)],
+                           device="cuda", dtype=torch.int32)
+    pc_hash = F.sphash(pc)
+    vox_hash = torch.unique(pc_hash)
+    n_vox = vox_hash.numel()
+    idx = F.sphashquery(pc_hash, vox_hash).int()
+    counts = F.spcount(idx, n_vox)
+    corner = F.sphashquery(F.sphash(pc, offsets).t().contiguous(), vox_hash).int().contiguous()
+    w = F.calc_ti_weights(pts, corner, scale=1)
+    feats = torch.randn(n, c, device="cuda", dtype=torch.float16)
+    vfeat = torch.randn(n_vox, c, device="cuda", dtype=torch.float16)
+    from torchsparse_amd import backend
+    rows = []
+
+    def add(name, fn, nbytes):
+        ms = event_ms(fn, iters=20)
+        rows.append({"op": name, "ms": round(ms, 4), "GBps": round(nbytes / ms / 1e6, 1)})
+
+    add("sphash", lambda: F.sphash(pc), 24 * n)
+    add("sphash_8_offsets", lambda: F.sphash(pc, offsets), 16 * n + 64 * n)
+    add("sphashquery", lambda: F.sphashquery(pc_hash, vox_hash), 12 * backend.hash_capacity(n_vox) * 2 + 8 * n_vox + 12 * n)
+    add("spcount", lambda: F.spcount(idx, n_vox), 4 * n + 8 * n_vox)
+    def regroup(t, groups):
+        t._tsmi_groups = None
+        backend.group_by_index(t, groups)
+
+    add("group_points_by_voxel", lambda: regroup(idx, n_vox), 2 * 8 * n * 2 + 4 * n_vox)
+    add("group_corners_by_voxel", lambda: regroup(corner, n_vox), 2 * 8 * 8 * n * 2 + 4 * n_vox)
+    add("spvoxelize", lambda: backend.voxelize_forward_cuda(feats, idx, counts), n * (c * b + 4) + n_vox * c * b)
+    add("spvoxelize_backward", lambda: backend.voxelize_backward_cuda(vfeat, idx, counts, n),
+        n * (c * b + 4) + n_vox * c * b)
+    add("spdevoxelize", lambda: backend.devoxelize_forward_cuda(vfeat, corner, w), n * (c * b + 64) + n_vox * c * b)
+    add("spdevoxelize_backward", lambda: backend.devoxelize_backward_cuda(feats, corner, w, n_vox),
+        n * (c * b + 64) + n_vox * c * b)
+    return {"points": n, "voxels": n_vox, "channels": c, "dtype": "f16", "ops": rows}
 
 
 def network_layers(model, inp):
@@ -406,6 +453,7 @@ def main():
         level_coords = {lvl: c[0].cpu().numpy() for lvl, c in inp._caches.cmaps.items()}
         layers = None if args.no_layers else layer_sweep(ts, spnn, F, backend, coords, n)
     backward = None if args.no_backward else backward_sweep(ts, spnn, F, backend, coords, n, feats)
+    pointops = None if args.no_pointops else pointops_sweep(F)
     tuned = None
     if not args.no_tune:
         # the per-group tuner over all three dataflows and the sorted variants, then the same
@@ -437,7 +485,7 @@ def main():
                    "unfused_ms_per_step": round(ms_unfused, 4),
                    "conv_mode": F.get_conv_mode().value},
         "roofline": roof, "cpu_baseline": cpu, "layers": layers, "backward": backward,
-        "tuned": tuned,
+        "tuned": tuned, "pointops": pointops,
     }
     print(json.dumps(result))
 

@@ -352,6 +352,74 @@ int tsmi_gs_scatter(tsmi_stream_t s, const void *out_buffer, const int32_t *nbad
                     const int32_t *row_mask, int64_t n_out, int kvol, int cout, int dtype,
                     int center_k, const void *bias, const void *residual, int relu, void *y);
 
+/* ------------------------------------------------------ point-voxel operators
+ * Row tensors are [rows, c] of dtype TSMI_F32 / TSMI_F16 / TSMI_BF16, sums run in fp32.
+ * Rows are moved 16 bytes per thread when c is a multiple of 16 bytes of elements and the
+ * tensors are 16-byte aligned, element by element otherwise. */
+
+/* out[i] = 64-bit FNV-1a hash of the four int32 fields of coords[i] (no 60-bit fold).
+ * Replaces hash_cuda (hash/hash_cuda.cu:9-22,64-70). */
+int tsmi_hash_coords(tsmi_stream_t s, const int32_t *coords, int64_t n, int64_t *out);
+
+/* out[k*n + i] = hash of (coords[i,0], coords[i,1:4] + offsets[k]); offsets int32[kvol,3] on
+ * the device, out int64[kvol,n].  Replaces kernel_hash_cuda (hash/hash_cuda.cu:26-57,72-83). */
+int tsmi_kernel_hash(tsmi_stream_t s, const int32_t *coords, int64_t n, const int32_t *offsets,
+                     int kvol, int64_t *out);
+
+/* out[v] = number of i with idx[i] == v for v in [0, num); other indices are skipped.  `out`
+ * is cleared here.  Replaces count_cuda (others/count_cuda.cu:10-31). */
+int tsmi_count(tsmi_stream_t s, const int32_t *idx, int64_t n, int32_t *out, int num);
+
+/* Grouping of an index array, the preparation of the two row sums below: `order` int32[m]
+ * receives the positions e of idx with 0 <= idx[e] < n_groups sorted by (idx[e], e) — only the
+ * first starts[n_groups] entries are meaningful — and starts int32[n_groups + 1] the beginning of
+ * every group's run.  `temp` holds tsmi_group_temp_bytes(m) bytes.  A radix sort over the bits
+ * n_groups needs plus one binary search per group; no host read-back.  No counterpart in the
+ * reference, which adds with atomicAdd instead. */
+int64_t tsmi_group_temp_bytes(int64_t m);
+int tsmi_group_by_index(tsmi_stream_t s, const int32_t *idx, int64_t m, int64_t n_groups, void *temp,
+                        int64_t temp_bytes, int32_t *order, int32_t *starts);
+
+/* out[v,:] = (sum of feats[i,:] over the points i of voxel v) / counts[v], zero when counts[v]
+ * is 0; (order, starts) = tsmi_group_by_index of the points' voxel indices idx int32[n] with
+ * n_groups = n1, so points with an index outside [0, n1) add nothing.  The points of a voxel
+ * are added in ascending order: results do not vary from run to run.
+ * Replaces voxelize_forward_cuda (voxelize/voxelize_cuda.cu:42-60,82-100). */
+int tsmi_voxelize_forward(tsmi_stream_t s, const void *feats, const int32_t *counts,
+                          const int32_t *order, const int32_t *starts, int64_t n, int c, int64_t n1,
+                          int dtype, void *out);
+
+/* bottom_grad[i,:] = top_grad[idx[i],:] / counts[idx[i]] (zero for skipped points).
+ * Replaces voxelize_backward_cuda (voxelize/voxelize_cuda.cu:62-80,102-120), without its
+ * atomics: every output row has one writer. */
+int tsmi_voxelize_backward(tsmi_stream_t s, const void *top_grad, const int32_t *idx,
+                           const int32_t *counts, int64_t n, int c, int64_t n1, int dtype,
+                           void *bottom_grad);
+
+/* out[i,:] = sum_k weight[i,k] * feat[indices[i,k],:] over the 8 corners, indices int32[n,8]
+ * (negative = absent), weight fp32 [n,8], feat [n_vox, c].
+ * Replaces devoxelize_forward_cuda (devoxelize/devoxelize_cuda.cu:11-33,62-79); the weights are
+ * always fp32 here. */
+int tsmi_devoxelize_forward(tsmi_stream_t s, const void *feat, const int32_t *indices,
+                            const float *weight, int64_t n, int64_t n_vox, int c, int dtype,
+                            void *out);
+
+/* bottom_grad[v,:] = sum over (i,k) with indices[i,k] == v of weight[i,k] * top_grad[i,:];
+ * (order, starts) = tsmi_group_by_index of the flattened indices int32[8n] with n_groups = n_vox.
+ * Replaces devoxelize_backward_cuda (devoxelize/devoxelize_cuda.cu:37-58,83-98). */
+int tsmi_devoxelize_backward(tsmi_stream_t s, const void *top_grad, const float *weight,
+                             const int32_t *order, const int32_t *starts, int64_t n, int64_t n_vox,
+                             int c, int dtype, void *bottom_grad);
+
+/* dense[b,x,y,z,:] = feats[i,:] for coords[i] = (b,x,y,z) inside spatial_range (HOST int32[4],
+ * extents B,X,Y,Z); the caller clears `dense` first.  The backward copies the other way
+ * (rows outside the range receive zeros).
+ * Replace to_dense_forward_cuda / to_dense_backward_cuda (voxelize/voxelize_cuda.cu:10-40,122-141). */
+int tsmi_to_dense_forward(tsmi_stream_t s, const void *feats, const int32_t *coords, int64_t n, int c,
+                          const int32_t *spatial_range, int dtype, void *dense);
+int tsmi_to_dense_backward(tsmi_stream_t s, const void *top_grad, const int32_t *coords, int64_t n,
+                           int c, const int32_t *spatial_range, int dtype, void *bottom_grad);
+
 #pragma GCC visibility pop
 #ifdef __cplusplus
 }

@@ -39,6 +39,19 @@ the checks live in ``tests/test_oracle_*.py``):
                            oracle's own forward
   hash_cpu /               golden value hash_cpu([[0,1,2,3]]) = 321218472033932309
   kernel_hash_cpu          and vectors from the compiled reference (tests/golden/)
+  hash_gpu /               hash_cpu's golden vectors: folding hash_gpu's value to 60 bits
+  kernel_hash_gpu          must give them (hash_cuda.cu only drops the fold); kernel_hash
+                           = hash of the shifted rows
+  count                    compiled reference count_cpu (golden), numpy bincount
+  voxelize_forward /       compiled reference voxelize_{forward,backward}_cpu (golden);
+  voxelize_backward        numpy add.at closed form; backward = adjoint of forward
+  devoxelize_forward       compiled reference devoxelize_forward_cpu (golden); einsum
+  devoxelize_backward      adjoint identity <devox(f), g> = <f, devox_bwd(g)> with the
+                           pinned forward, and a scatter-add closed form.  The reference's
+                           CPU backward is defective (indexes the gradient by voxel) and
+                           is deliberately not used as evidence
+  to_dense_forward /       numpy fancy indexing; backward(forward(x)) == x
+  to_dense_backward
   hash_query_cpu           python dict; third-party google::dense_hash_map is not
                            vendored by the reference and no reference test covers
                            it: parity unpinned beyond "exact-match dictionary"
@@ -328,3 +341,78 @@ def kmap_cpu_backend(coords, kernel_size):
     k_idx, out_idx = np.nonzero(res != -1)
     nbmaps = np.stack([res[k_idx, out_idx], out_idx], 1).astype(np.int32)
     return nbmaps, nbsizes
+
+
+# ---------------------------------------------------------------- point-voxel operators
+
+
+def hash_gpu(rows):
+    rows = _i32(rows)
+    out = np.empty(rows.shape[0], np.int64)
+    lib().tso_hash_gpu(_p(rows, _i32p), ctypes.c_int64(rows.shape[0]), _p(out, _i64p))
+    return out
+
+
+def kernel_hash_gpu(rows, offsets):
+    rows, offsets = _i32(rows), _i32(offsets)
+    out = np.empty((offsets.shape[0], rows.shape[0]), np.int64)
+    lib().tso_kernel_hash_gpu(_p(rows, _i32p), ctypes.c_int64(rows.shape[0]), _p(offsets, _i32p),
+                              offsets.shape[0], _p(out, _i64p))
+    return out
+
+
+def count(idx, s):
+    idx = _i32(idx)
+    out = np.empty(int(s), np.int32)
+    lib().tso_count(_p(idx, _i32p), ctypes.c_int64(idx.shape[0]), int(s), _p(out, _i32p))
+    return out
+
+
+def voxelize_forward(feats, idx, counts):
+    feats, idx, counts = _f32(feats), _i32(idx), _i32(counts)
+    out = np.empty((counts.shape[0], feats.shape[1]), np.float32)
+    lib().tso_voxelize_forward(_p(feats, _f32p), ctypes.c_int64(feats.shape[0]), feats.shape[1],
+                               _p(idx, _i32p), _p(counts, _i32p), ctypes.c_int64(counts.shape[0]),
+                               _p(out, _f32p))
+    return out
+
+
+def voxelize_backward(top, idx, counts, n):
+    top, idx, counts = _f32(top), _i32(idx), _i32(counts)
+    out = np.empty((int(n), top.shape[1]), np.float32)
+    lib().tso_voxelize_backward(_p(top, _f32p), _p(idx, _i32p), _p(counts, _i32p), ctypes.c_int64(int(n)),
+                                top.shape[1], ctypes.c_int64(counts.shape[0]), _p(out, _f32p))
+    return out
+
+
+def devoxelize_forward(feat, indices, weight):
+    feat, indices, weight = _f32(feat), _i32(indices), _f32(weight)
+    out = np.empty((indices.shape[0], feat.shape[1]), np.float32)
+    lib().tso_devoxelize_forward(_p(feat, _f32p), feat.shape[1], _p(indices, _i32p), _p(weight, _f32p),
+                                 ctypes.c_int64(indices.shape[0]), _p(out, _f32p))
+    return out
+
+
+def devoxelize_backward(top, indices, weight, n_vox):
+    top, indices, weight = _f32(top), _i32(indices), _f32(weight)
+    out = np.empty((int(n_vox), top.shape[1]), np.float32)
+    lib().tso_devoxelize_backward(_p(top, _f32p), _p(indices, _i32p), _p(weight, _f32p),
+                                  ctypes.c_int64(indices.shape[0]), ctypes.c_int64(int(n_vox)),
+                                  top.shape[1], _p(out, _f32p))
+    return out
+
+
+def to_dense_forward(feats, coords, spatial_range):
+    feats, coords, rng = _f32(feats), _i32(coords), _i32(spatial_range)
+    out = np.empty(tuple(int(v) for v in rng) + (feats.shape[1],), np.float32)
+    lib().tso_to_dense_forward(_p(feats, _f32p), _p(coords, _i32p), ctypes.c_int64(feats.shape[0]),
+                               feats.shape[1], _p(rng, _i32p), _p(out, _f32p))
+    return out
+
+
+def to_dense_backward(top, coords, spatial_range):
+    top, coords, rng = _f32(top), _i32(coords), _i32(spatial_range)
+    out = np.empty((coords.shape[0], top.shape[-1]), np.float32)
+    lib().tso_to_dense_backward(_p(top, _f32p), _p(coords, _i32p), ctypes.c_int64(coords.shape[0]),
+                                top.shape[-1], _p(rng, _i32p), _p(out, _f32p))
+    return out

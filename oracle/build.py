@@ -25,8 +25,8 @@ def build_oracle(verbose: bool = False) -> str:
 
 
 def build_ref(verbose: bool = False):
-    """Compile convolution_gather_scatter_cpu.cpp + hash_cpu.cpp of the reference
-    behind oracle/ref_bind.cpp.  Returns the path of the built module or None
+    """Compile the reference's CPU sources (gather-scatter convolution, hash, count,
+    voxelize, devoxelize) behind oracle/ref_bind.cpp.  Returns the path of the built module or None
     when the reference tree is absent."""
     if not os.path.isdir(REFERENCE_BACKEND):
         return None
@@ -40,6 +40,9 @@ def build_ref(verbose: bool = False):
             os.path.join(HERE, "ref_bind.cpp"),
             os.path.join(REFERENCE_BACKEND, "convolution", "convolution_gather_scatter_cpu.cpp"),
             os.path.join(REFERENCE_BACKEND, "hash", "hash_cpu.cpp"),
+            os.path.join(REFERENCE_BACKEND, "others", "count_cpu.cpp"),
+            os.path.join(REFERENCE_BACKEND, "voxelize", "voxelize_cpu.cpp"),
+            os.path.join(REFERENCE_BACKEND, "devoxelize", "devoxelize_cpu.cpp"),
         ],
         extra_include_paths=[REFERENCE_BACKEND],
         extra_cflags=["-O3", "-fopenmp"],

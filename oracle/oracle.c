@@ -704,3 +704,126 @@ TSO_EXPORT void tso_hash_query_cpu(const int64_t *hash_query, int64_t n_query,
   free(tk);
   free(tv);
 }
+
+/* ------------------------------------------------ point-voxel operators */
+
+/* The GPU hash of a coordinate row: 64-bit FNV-1a over its four int32 fields, WITHOUT the
+ * 60-bit fold of the CPU version.  Follows backend/hash/hash_cuda.cu:9-22 (the fold is
+ * commented out there). */
+static uint64_t fnv_row_nofold(const int *row) {
+  uint64_t h = 14695981039346656037ULL;
+  for (int j = 0; j < 4; j++) {
+    h ^= (unsigned int)row[j];
+    h *= 1099511628211ULL;
+  }
+  return h;
+}
+
+TSO_EXPORT void tso_hash_gpu(const int *data, int64_t n, int64_t *out) {
+  for (int64_t i = 0; i < n; i++) out[i] = (int64_t)fnv_row_nofold(data + 4 * i);
+}
+
+/* out[k*n+i] = hash(data[i,0], data[i,1:4] + offsets[k]): the offsets move the three
+ * spatial fields, the batch field in column 0 stays.  Follows hash_cuda.cu:26-52. */
+TSO_EXPORT void tso_kernel_hash_gpu(const int *data, int64_t n, const int *offsets, int kvol,
+                                    int64_t *out) {
+  for (int k = 0; k < kvol; k++)
+    for (int64_t i = 0; i < n; i++) {
+      int row[4];
+      row[0] = data[4 * i];
+      for (int j = 1; j < 4; j++) row[j] = data[4 * i + j] + offsets[3 * k + j - 1];
+      out[(int64_t)k * n + i] = (int64_t)fnv_row_nofold(row);
+    }
+}
+
+/* out[v] = number of i with idx[i] == v; negative indices are skipped.
+ * Follows backend/others/count_cpu.cpp:7-23 (count_cuda.cu:10-17 is the same sum). */
+TSO_EXPORT void tso_count(const int *idx, int64_t n, int s, int *out) {
+  memset(out, 0, sizeof(int) * (size_t)s);
+  for (int64_t i = 0; i < n; i++)
+    if (idx[i] >= 0 && idx[i] < s) out[idx[i]]++;
+}
+
+/* out[v,:] = sum over points i with idx[i] == v of feats[i,:] / counts[v].  Points whose
+ * index is outside [0, n1) or whose voxel has count 0 contribute nothing.
+ * Follows backend/voxelize/voxelize_cpu.cpp:7-25 with the index guard of
+ * voxelize_cuda.cu:55-57; accumulation in double. */
+TSO_EXPORT void tso_voxelize_forward(const float *feats, int64_t n, int c, const int *idx,
+                                     const int *counts, int64_t n1, float *out) {
+  double *acc = (double *)calloc((size_t)(n1 * c > 0 ? n1 * c : 1), sizeof(double));
+  for (int64_t i = 0; i < n; i++) {
+    const int pos = idx[i];
+    if (pos < 0 || pos >= n1 || counts[pos] == 0) continue;
+    for (int j = 0; j < c; j++) acc[(int64_t)pos * c + j] += (double)feats[i * c + j] / (double)counts[pos];
+  }
+  for (int64_t i = 0; i < n1 * c; i++) out[i] = (float)acc[i];
+  free(acc);
+}
+
+/* bottom[i,:] = top[idx[i],:] / counts[idx[i]] (0 for skipped points).
+ * Follows voxelize_cpu.cpp:27-43. */
+TSO_EXPORT void tso_voxelize_backward(const float *top, const int *idx, const int *counts,
+                                      int64_t n, int c, int64_t n1, float *bottom) {
+  for (int64_t i = 0; i < n; i++) {
+    const int pos = idx[i];
+    const int ok = !(pos < 0 || pos >= n1 || counts[pos] == 0);
+    for (int j = 0; j < c; j++)
+      bottom[i * c + j] = ok ? (float)((double)top[(int64_t)pos * c + j] / (double)counts[pos]) : 0.f;
+  }
+}
+
+/* out[i,:] = sum_k weight[i,k] * feat[indices[i,k],:] over the 8 corner voxels, negative
+ * index = absent corner.  Follows backend/devoxelize/devoxelize_cpu.cpp:10-32. */
+TSO_EXPORT void tso_devoxelize_forward(const float *feat, int c, const int *indices,
+                                       const float *weight, int64_t n, float *out) {
+  for (int64_t i = 0; i < n; i++)
+    for (int j = 0; j < c; j++) {
+      double acc = 0.0;
+      for (int k = 0; k < 8; k++) {
+        const int v = indices[8 * i + k];
+        if (v >= 0) acc += (double)weight[8 * i + k] * (double)feat[(int64_t)v * c + j];
+      }
+      out[i * c + j] = (float)acc;
+    }
+}
+
+/* bottom[v,:] = sum over (i,k) with indices[i,k] == v of weight[i,k] * top[i,:]: the adjoint
+ * of the forward.  Follows backend/devoxelize/devoxelize_cuda.cu:37-58.  (The CPU file's
+ * backward, devoxelize_cpu.cpp:36-59, reads top_grad at the VOXEL index and writes through
+ * negative indices; it is not the adjoint and is not followed.) */
+TSO_EXPORT void tso_devoxelize_backward(const float *top, const int *indices, const float *weight,
+                                        int64_t n, int64_t n_vox, int c, float *bottom) {
+  double *acc = (double *)calloc((size_t)(n_vox * c > 0 ? n_vox * c : 1), sizeof(double));
+  for (int64_t i = 0; i < n; i++)
+    for (int k = 0; k < 8; k++) {
+      const int v = indices[8 * i + k];
+      if (v < 0 || v >= n_vox) continue;
+      for (int j = 0; j < c; j++)
+        acc[(int64_t)v * c + j] += (double)weight[8 * i + k] * (double)top[i * c + j];
+    }
+  for (int64_t i = 0; i < n_vox * c; i++) bottom[i] = (float)acc[i];
+  free(acc);
+}
+
+/* dense[b,x,y,z,:] = feats[i,:] for coords[i] = (b,x,y,z); `dense` is zero elsewhere.
+ * Follows backend/voxelize/voxelize_cuda.cu:10-24 (to_dense_forward_kernel). */
+TSO_EXPORT void tso_to_dense_forward(const float *feats, const int *coords, int64_t n, int c,
+                                     const int *range, float *dense) {
+  const int64_t cells = (int64_t)range[0] * range[1] * range[2] * range[3];
+  memset(dense, 0, sizeof(float) * (size_t)(cells * c));
+  for (int64_t i = 0; i < n; i++) {
+    const int *q = coords + 4 * i;
+    const int64_t pos = (((int64_t)q[0] * range[1] + q[1]) * range[2] + q[2]) * range[3] + q[3];
+    memcpy(dense + pos * c, feats + i * c, sizeof(float) * (size_t)c);
+  }
+}
+
+/* bottom[i,:] = top[b,x,y,z,:].  Follows voxelize_cuda.cu:26-40. */
+TSO_EXPORT void tso_to_dense_backward(const float *top, const int *coords, int64_t n, int c,
+                                      const int *range, float *bottom) {
+  for (int64_t i = 0; i < n; i++) {
+    const int *q = coords + 4 * i;
+    const int64_t pos = (((int64_t)q[0] * range[1] + q[1]) * range[2] + q[2]) * range[3] + q[3];
+    memcpy(bottom + i * c, top + pos * c, sizeof(float) * (size_t)c);
+  }
+}

@@ -9,6 +9,9 @@ compiled reference produced for them; no reference source text is stored.
                     on submanifold k=3, strided k=2/s=2, its transposed use, and
                     strided k=3/s=2 pair lists
   hash_cpu.npz      hash_cpu / kernel_hash_cpu (backend/hash/hash_cpu.cpp:43-59)
+  pointops_cpu.npz  count_cpu (others/count_cpu.cpp:7-23), voxelize_forward_cpu /
+                    voxelize_backward_cpu (voxelize/voxelize_cpu.cpp:7-43),
+                    devoxelize_forward_cpu (devoxelize/devoxelize_cpu.cpp:10-32)
 """
 import os
 import sys
@@ -78,6 +81,26 @@ def main():
     kh = ref.kernel_hash_cpu(torch.from_numpy(rows), torch.from_numpy(offs)).numpy()
     np.savez_compressed(os.path.join(HERE, "hash_cpu.npz"), rows=rows, offsets=offs, hash=h,
                         kernel_hash=kh)
+    # point-voxel operators: 300 points falling into 90 voxels (some empty), 5 channels
+    n_pts, n_vox, ch = 300, 90, 5
+    idx = rng.integers(0, 80, n_pts).astype(np.int32)        # voxels 80..89 stay empty
+    idx[rng.integers(0, n_pts, 20)] = -1                     # points outside every voxel
+    counts = ref.count_cpu(torch.from_numpy(idx), n_vox).numpy()
+    valid = idx >= 0                                          # the CPU kernels do not guard the index
+    pts = rng.standard_normal((n_pts, ch)).astype(np.float32)
+    vox = ref.voxelize_forward_cpu(torch.from_numpy(pts[valid]), torch.from_numpy(idx[valid]),
+                                   torch.from_numpy(counts)).numpy()
+    top = rng.standard_normal((n_vox, ch)).astype(np.float32)
+    vox_bwd = ref.voxelize_backward_cpu(torch.from_numpy(top), torch.from_numpy(idx[valid]),
+                                        torch.from_numpy(counts), int(valid.sum())).numpy()
+    corner = rng.integers(-1, n_vox, (n_pts, 8)).astype(np.int32)
+    wts = rng.uniform(0, 1, (n_pts, 8)).astype(np.float32)
+    vfeat = rng.standard_normal((n_vox, ch)).astype(np.float32)
+    devox = ref.devoxelize_forward_cpu(torch.from_numpy(vfeat), torch.from_numpy(corner),
+                                       torch.from_numpy(wts)).numpy()
+    np.savez_compressed(os.path.join(HERE, "pointops_cpu.npz"), idx=idx, n_vox=np.array(n_vox),
+                        counts=counts, pts=pts, vox=vox, top=top, vox_bwd=vox_bwd, corner=corner,
+                        wts=wts, vfeat=vfeat, devox=devox)
     print("written", os.listdir(HERE))
 
 

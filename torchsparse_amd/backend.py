@@ -20,6 +20,7 @@ _DTYPE_CODE = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
 
 _vp, _i64, _i32, _f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
 _I3 = ctypes.c_int32 * 3
+_I4 = ctypes.c_int32 * 4
 
 
 def _load():
@@ -37,6 +38,8 @@ def _load():
     lib.tsmi_conv_wgrad_workspace_elems.restype = _i64
     lib.tsmi_conv_wgrad_workspace_elems.argtypes = [_i64, _i32, _i32, _i32, _i32]
     lib.tsmi_conv_workspace_elems.argtypes = [_i64, _i64, _i32, _i32, _i32, _i32, _i32, _i32]
+    lib.tsmi_group_temp_bytes.restype = _i64
+    lib.tsmi_group_temp_bytes.argtypes = [_i64]
     lib.tsmi_wgrad_pairs_capacity.restype = _i64
     lib.tsmi_wgrad_pairs_capacity.argtypes = [_i64, _i32]
     lib.tsmi_conv_wgrad_pairs_workspace_elems.restype = _i64
@@ -74,6 +77,16 @@ def _load():
                                   _i64, _vp],
         "tsmi_conv_fetch_on_demand": [_vp, _vp, _vp, _vp, _i64, _vp, _vp, _i64, _vp, _i64, _i32,
                                       _i32, _i32, _i32, _i32, _i32, _vp, _vp, _i32, _vp, _vp],
+        "tsmi_hash_coords": [_vp, _vp, _i64, _vp],
+        "tsmi_kernel_hash": [_vp, _vp, _i64, _vp, _i32, _vp],
+        "tsmi_count": [_vp, _vp, _i64, _vp, _i32],
+        "tsmi_group_by_index": [_vp, _vp, _i64, _i64, _vp, _i64, _vp, _vp],
+        "tsmi_voxelize_forward": [_vp, _vp, _vp, _vp, _vp, _i64, _i32, _i64, _i32, _vp],
+        "tsmi_voxelize_backward": [_vp, _vp, _vp, _vp, _i64, _i32, _i64, _i32, _vp],
+        "tsmi_devoxelize_forward": [_vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _vp],
+        "tsmi_devoxelize_backward": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _vp],
+        "tsmi_to_dense_forward": [_vp, _vp, _vp, _i64, _i32, _I4, _i32, _vp],
+        "tsmi_to_dense_backward": [_vp, _vp, _vp, _i64, _i32, _I4, _i32, _vp],
         "tsmi_gs_gather": [_vp, _vp, _vp, _i64, _i32, _i32, _i32, _vp],
         "tsmi_gs_gemm": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _i32, _i32, _vp],
         "tsmi_gs_scatter": [_vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _vp, _vp, _i32, _vp],
@@ -712,3 +725,126 @@ def conv_forward_gather_scatter_cuda(in_feats, kernel, nbmaps, nbsizes, input_ma
     _check(_C.tsmi_gs_scatter(s, _ptr(products), _ptr(nbaddrs), _ptr(row_mask), output_size, kvol,
                               cout, code, center_k, pb, pr, int(relu), _ptr(y)))
     return y
+
+
+# ------------------------------------------------------------ point-voxel operators
+
+
+def hash_cuda(coords: torch.Tensor) -> torch.Tensor:
+    """hash/hash_cuda.cu:64-70: int64 [N] FNV-1a hashes of int32 [N,4] rows."""
+    coords = _need(coords, torch.int32, "coords")
+    out = torch.empty(coords.shape[0], dtype=torch.int64, device=coords.device)
+    _check(_C.tsmi_hash_coords(_stream(), _ptr(coords), coords.shape[0], _ptr(out)))
+    return out
+
+
+def kernel_hash_cuda(coords: torch.Tensor, kernel_offset: torch.Tensor) -> torch.Tensor:
+    """hash/hash_cuda.cu:72-83: int64 [K,N] hashes of the rows shifted by each offset."""
+    coords = _need(coords, torch.int32, "coords")
+    offsets = _need(kernel_offset, torch.int32, "kernel_offset")
+    out = torch.empty((offsets.shape[0], coords.shape[0]), dtype=torch.int64, device=coords.device)
+    _check(_C.tsmi_kernel_hash(_stream(), _ptr(coords), coords.shape[0], _ptr(offsets),
+                               offsets.shape[0], _ptr(out)))
+    return out
+
+
+def count_cuda(idx: torch.Tensor, num: int) -> torch.Tensor:
+    """others/count_cuda.cu:24-31: int32 [num] occurrences of each index (negatives skipped)."""
+    idx = _need(idx, torch.int32, "idx")
+    out = torch.empty(int(num), dtype=torch.int32, device=idx.device)
+    _check(_C.tsmi_count(_stream(), _ptr(idx), idx.numel(), _ptr(out), int(num)))
+    return out
+
+
+def group_by_index(idx: torch.Tensor, n_groups: int):
+    """(order, starts) of an int32 index tensor: the positions of the entries with a value in
+    [0, n_groups) sorted by (value, position), and the start of every value's run.  Kept on
+    the tensor (and rebuilt when it is modified in place): a network voxelizes and
+    devoxelizes through the same indices many times."""
+    idx = _need(idx, torch.int32, "idx")
+    cached = getattr(idx, "_tsmi_groups", None)
+    if cached is not None and cached[0] == (idx._version, int(n_groups)):
+        return cached[1], cached[2]
+    m, dev = idx.numel(), idx.device
+    temp_bytes = _C.tsmi_group_temp_bytes(m)
+    temp = torch.empty(max(temp_bytes, 1), dtype=torch.uint8, device=dev)
+    order = torch.empty(max(m, 1), dtype=torch.int32, device=dev)
+    starts = torch.empty(int(n_groups) + 1, dtype=torch.int32, device=dev)
+    _check(_C.tsmi_group_by_index(_stream(), _ptr(idx), m, int(n_groups), _ptr(temp), temp_bytes,
+                                  _ptr(order), _ptr(starts)))
+    idx._tsmi_groups = ((idx._version, int(n_groups)), order, starts)
+    return order, starts
+
+
+def voxelize_forward_cuda(inputs: torch.Tensor, idx: torch.Tensor, counts: torch.Tensor) -> torch.Tensor:
+    """voxelize/voxelize_cuda.cu:82-100: [N1, C] means of the points of each voxel."""
+    x = _need(inputs, inputs.dtype, "inputs")
+    idx, counts = _need(idx, torch.int32, "idx"), _need(counts, torch.int32, "counts")
+    n, c, n1 = x.shape[0], x.shape[1], counts.shape[0]
+    if idx.numel() != n:
+        raise ValueError(f"idx has {idx.numel()} entries for {n} points")
+    order, starts = group_by_index(idx, n1)
+    out = torch.empty((n1, c), dtype=x.dtype, device=x.device)
+    _check(_C.tsmi_voxelize_forward(_stream(), _ptr(x), _ptr(counts), _ptr(order), _ptr(starts), n, c,
+                                    n1, _dtype_code(x), _ptr(out)))
+    return out
+
+
+def voxelize_backward_cuda(top_grad: torch.Tensor, idx: torch.Tensor, counts: torch.Tensor,
+                           n: int) -> torch.Tensor:
+    """voxelize/voxelize_cuda.cu:102-120."""
+    g = _need(top_grad, top_grad.dtype, "top_grad")
+    idx, counts = _need(idx, torch.int32, "idx"), _need(counts, torch.int32, "counts")
+    out = torch.empty((int(n), g.shape[1]), dtype=g.dtype, device=g.device)
+    _check(_C.tsmi_voxelize_backward(_stream(), _ptr(g), _ptr(idx), _ptr(counts), int(n), g.shape[1],
+                                     counts.shape[0], _dtype_code(g), _ptr(out)))
+    return out
+
+
+def devoxelize_forward_cuda(feat: torch.Tensor, indices: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """devoxelize/devoxelize_cuda.cu:62-79: [N, C] interpolations from 8 corner voxels
+    (indices int32 [N,8], weight [N,8]; the weights are used in fp32)."""
+    f = _need(feat, feat.dtype, "feat")
+    indices = _need(indices, torch.int32, "indices")
+    w = _need(weight.float(), torch.float32, "weight")
+    n = indices.shape[0]
+    out = torch.empty((n, f.shape[1]), dtype=f.dtype, device=f.device)
+    _check(_C.tsmi_devoxelize_forward(_stream(), _ptr(f), _ptr(indices), _ptr(w), n, f.shape[0],
+                                      f.shape[1], _dtype_code(f), _ptr(out)))
+    return out
+
+
+def devoxelize_backward_cuda(top_grad: torch.Tensor, indices: torch.Tensor, weight: torch.Tensor,
+                             n: int) -> torch.Tensor:
+    """devoxelize/devoxelize_cuda.cu:83-98: [n, C] gradient with respect to the voxel features."""
+    g = _need(top_grad, top_grad.dtype, "top_grad")
+    indices = _need(indices, torch.int32, "indices")
+    w = _need(weight.float(), torch.float32, "weight")
+    if indices.shape[0] != g.shape[0] or w.numel() != indices.numel():
+        raise ValueError("top_grad, indices and weight disagree on the number of points")
+    order, starts = group_by_index(indices, int(n))
+    out = torch.empty((int(n), g.shape[1]), dtype=g.dtype, device=g.device)
+    _check(_C.tsmi_devoxelize_backward(_stream(), _ptr(g), _ptr(w), _ptr(order), _ptr(starts),
+                                       indices.shape[0], int(n), g.shape[1], _dtype_code(g), _ptr(out)))
+    return out
+
+
+def to_dense_forward_cuda(inputs: torch.Tensor, idx: torch.Tensor, spatial_range, outputs: torch.Tensor) -> None:
+    """voxelize/voxelize_cuda.cu:122-131: outputs [B,X,Y,Z,C] (already zero) receives the rows."""
+    x = _need(inputs, inputs.dtype, "inputs")
+    idx = _need(idx, torch.int32, "idx")
+    out = _need(outputs, x.dtype, "outputs")
+    rng = [int(v) for v in (spatial_range.tolist() if torch.is_tensor(spatial_range) else spatial_range)]
+    _check(_C.tsmi_to_dense_forward(_stream(), _ptr(x), _ptr(idx), x.shape[0], x.shape[1], _I4(*rng),
+                                    _dtype_code(x), _ptr(out)))
+
+
+def to_dense_backward_cuda(top_grad: torch.Tensor, idx: torch.Tensor, spatial_range,
+                           bottom_grad: torch.Tensor) -> None:
+    """voxelize/voxelize_cuda.cu:133-141."""
+    g = _need(top_grad, top_grad.dtype, "top_grad")
+    idx = _need(idx, torch.int32, "idx")
+    out = _need(bottom_grad, g.dtype, "bottom_grad")
+    rng = [int(v) for v in (spatial_range.tolist() if torch.is_tensor(spatial_range) else spatial_range)]
+    _check(_C.tsmi_to_dense_backward(_stream(), _ptr(g), _ptr(idx), out.shape[0], out.shape[1], _I4(*rng),
+                                     _dtype_code(g), _ptr(out)))

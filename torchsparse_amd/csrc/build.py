@@ -18,6 +18,7 @@ SOURCES = [
     "common.cpp",
     "kmap.hip",
     "sort.hip",
+    "pointops.hip",
     "conv_api.cpp",
     "conv_igemm_f16.hip",
     "conv_igemm_bf16.hip",

@@ -8,7 +8,8 @@ from .utils import make_ntuple
 from .utils.tensor_cache import (TensorCache, TensorCacheMode, get_global_tensor_cache,
                                  get_tensor_cache_mode, set_global_tensor_cache)
 
-__all__ = ["SparseTensor", "get_allow_negative_coordinates", "set_allow_negative_coordinates"]
+__all__ = ["SparseTensor", "PointTensor", "get_allow_negative_coordinates",
+           "set_allow_negative_coordinates"]
 
 _allow_negative_coordinates = False
 
@@ -89,11 +90,34 @@ class SparseTensor:
     def dense(self) -> torch.Tensor:
         """[B, X, Y, Z, C] dense tensor (needs spatial_range)."""
         assert self.spatial_range is not None
-        c = self.coords.long()
-        out = torch.zeros(*self.spatial_range, self.feats.shape[1], dtype=self.feats.dtype,
-                          device=self.feats.device)
-        out[c[:, 0], c[:, 1], c[:, 2], c[:, 3]] = self.feats
-        return out
+        from .utils.to_dense import to_dense
+        return to_dense(self.feats, self.coords, self.spatial_range)
 
     def __add__(self, other: "SparseTensor") -> "SparseTensor":
         return self._like(self.feats + other.feats)
+
+
+class PointTensor:
+    """Features [N, C] at floating-point positions [N, 4], with the per-stride voxel indices
+    and interpolation weights point-voxel networks cache on it
+    (the reference's torchsparse/tensor.py:116-140)."""
+
+    def __init__(self, feats, coords, idx_query=None, weights=None):
+        self.F = feats
+        self.C = coords
+        self.idx_query = idx_query if idx_query is not None else {}
+        self.weights = weights if weights is not None else {}
+        self.additional_features = {"idx_query": {}, "counts": {}}
+
+    def cuda(self):
+        self.F, self.C = self.F.cuda(), self.C.cuda()
+        return self
+
+    def detach(self):
+        self.F, self.C = self.F.detach(), self.C.detach()
+        return self
+
+    def to(self, device, non_blocking: bool = True):
+        self.F = self.F.to(device, non_blocking=non_blocking)
+        self.C = self.C.to(device, non_blocking=non_blocking)
+        return self
