@@ -14,7 +14,7 @@
  * replaces.  Paths are relative to the reference's torchsparse/backend/.
  *
  * Shared conventions
- *   coords       int32 [N,4] rows (b, x, y, z); 0 <= x,y,z < 2^18, 0 <= b < 512
+ *   coords       int32 [N,4] rows (b, x, y, z); -2^17 <= x,y,z < 2^17, 0 <= b < 512
  *   out_in_map   int32 [N_pad, K_vol], -1 = no neighbour, N_pad = ceil128(N_out)
  *   kernel index odd K_vol: x is the fastest digit; even K_vol: z is the fastest
  *   hash table   two caller-owned arrays keys int64[cap], vals int32[cap];
@@ -90,32 +90,35 @@ int tsmi_kmap_query(tsmi_stream_t s, const int64_t *keys, const int32_t *vals, i
                     const int32_t ks[3], const int32_t stride[3], const int32_t pad[3],
                     int32_t *out_in_map);
 
-/* Per-column maximum of coords -> out_max int32[4] (device).  n may be 0 (result 0).
+/* Per-column maximum of non-negative coords -> out_max int32[4] (device).  n may be 0 (result 0).
  * clear_first = 0 when out_max already holds zeros (saves the fill launch).
  * Replaces coords.max(0).values (hashmap_on_the_fly.py:33). */
 int tsmi_coords_max(tsmi_stream_t s, const int32_t *coords, int64_t n, int32_t *out_max,
                     int clear_first);
 
 /* Candidate output coordinates of a strided convolution, de-duplicated by inserting
- * them, packed as (b<<54 | x<<36 | y<<18 | z), into the (empty) OUTPUT table
+ * them, packed as (b<<54 | x'<<36 | y'<<18 | z') with x' = x + 2^17, into the (empty) OUTPUT table
  * (keys, cap); vals are not touched.  counters[1] (device int32[2], zero on entry) is
  * set to 1 if the table overflowed.
  *   mode 0: o = (in + pad + digit - (ks-1)) / stride where divisible and
- *           0 <= o <= out_max per axis — downsample_grid_kmap_stage1_specialized_fast
+ *           out_min <= o <= out_max per axis — downsample_grid_kmap_stage1_specialized_fast
  *           (others/sparsemapping_cuda.cu:60-107) and get_output_coords_kernel
  *           (others/downsample_cuda.cu:62-141).  When ks == stride and pad == 0 every
  *           input has exactly one candidate, floor(in / stride), and one thread per
  *           input is launched instead of one per (input, offset).
  *   mode 1: o = floor(in / stride), unbounded — spdownsample for stride in {1, ks}
  *           or "minkowski" mode (nn/functional/conv/kmap/downsample.py:30-37).
- * The bound is out_max_host[3] when in_max_dev is NULL, otherwise it is derived on
- * the device as (in_max_dev[1+a] + 2*pad - (ks-1)) / stride
- * (hashmap_on_the_fly.py:33-37). */
+ * The upper bound is out_max_host[3] when in_max_dev is NULL, otherwise it is derived on
+ * the device as floor((in_max_dev[1+a] + 2*pad - (ks-1)) / stride)
+ * (hashmap_on_the_fly.py:33-37).  The lower bound is 0 when in_min_dev is NULL; with
+ * in_min_dev (device int32[4], the per-column minima of the input coordinates: negative
+ * coordinates allowed) it is (in_min_dev[1+a] - 2*pad + (ks-1)) / stride rounded toward zero
+ * (hashmap_on_the_fly.py:39-43), and in_max_dev must then hold the true maxima. */
 int tsmi_downsample_candidates(tsmi_stream_t s, const int32_t *in_coords, int64_t n_in,
                                const int32_t ks[3], const int32_t stride[3],
                                const int32_t pad[3], const int32_t out_max_host[3],
-                               const int32_t *in_max_dev, int mode, int64_t *keys,
-                               int64_t cap, int32_t *counters);
+                               const int32_t *in_max_dev, const int32_t *in_min_dev, int mode,
+                               int64_t *keys, int64_t cap, int32_t *counters);
 
 /* Gather the non-empty slots of a table: stored_keys_out[0..count) = the stored keys
  * (key + 1) in arbitrary order, *count_out (device int32, zero on entry) += their

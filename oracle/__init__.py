@@ -141,9 +141,11 @@ def kmap_subm(coords, kernel_size, coords_min=None, coords_max=None):
     return out
 
 
-def downsample_bounds(coords, kernel_size, stride, padding, spatial_range=None):
+def downsample_bounds(coords, kernel_size, stride, padding, spatial_range=None, allow_negative=False):
     """coords_min / coords_max of the OUTPUT grid, as kmap/func/hashmap_on_the_fly.py:27-45
-    computes them (spatial_range here is the already-strided one of build_kmap.py:65-72)."""
+    computes them (spatial_range here is the already-strided one of build_kmap.py:65-72).
+    With allow_negative the minimum is (min - 2 pad + (ks-1)) / stride, a true division
+    stored into an int tensor, i.e. rounded toward zero (:39-43)."""
     ks, st, pd = _triple(kernel_size), _triple(stride), _triple(padding)
     if spatial_range is not None:
         cmax = _i32([x - 1 for x in spatial_range])
@@ -151,15 +153,19 @@ def downsample_bounds(coords, kernel_size, stride, padding, spatial_range=None):
         cmax = _i32(coords).max(0).astype(np.int64)
         cmax[1:] = (cmax[1:] + 2 * pd - (ks - 1)) // st
         cmax = _i32(cmax)
+    if allow_negative:
+        cmin = _i32(coords).min(0).astype(np.int64)
+        cmin[1:] = np.trunc((cmin[1:] - 2 * pd + (ks - 1)) / st).astype(np.int64)
+        return _i32(cmin), cmax
     return _i32([0, 0, 0, 0]), cmax
 
 
-def kmap_downsample(coords, kernel_size, stride, padding, spatial_range=None):
+def kmap_downsample(coords, kernel_size, stride, padding, spatial_range=None, allow_negative=False):
     """Returns (out_in_map [ceil128(N_out),K_vol], out_coords [N_out,4])."""
     coords = _i32(coords)
     n = coords.shape[0]
     ks, st, pd = _triple(kernel_size), _triple(stride), _triple(padding)
-    cmin, cmax = downsample_bounds(coords, ks, st, pd, spatial_range)
+    cmin, cmax = downsample_bounds(coords, ks, st, pd, spatial_range, allow_negative)
     kvol = int(np.prod(ks))
     buf = np.empty((max(n * kvol, 1), 4), np.int32)
     n_out = lib().tso_downsample_coords(_p(coords, _i32p), n, _p(cmin, _i32p), _p(cmax, _i32p),

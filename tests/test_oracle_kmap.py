@@ -207,3 +207,47 @@ def test_cpu_backend_recipe_equals_exact_map():
     want_nb, want_sz = oracle.pair_lists(oracle.kmap_subm(coords, 3))
     np.testing.assert_array_equal(sz, want_sz)
     np.testing.assert_array_equal(nb, want_nb)
+
+
+def test_negative_lower_bound_follows_the_torch_expression():
+    """hashmap_on_the_fly.py:39-43 stores a true division into an int tensor; the oracle's
+    bound must round the same way (toward zero), checked by evaluating that expression."""
+    import torch
+    rng = np.random.default_rng(11)
+    for _ in range(20):
+        coords = rng.integers(-40, 40, (50, 4)).astype(np.int32)
+        ks = rng.integers(1, 5, 3)
+        st = rng.integers(1, 4, 3)
+        pd = rng.integers(0, 3, 3)
+        cmin_t = torch.from_numpy(coords).min(0).values
+        cmin_t[1:] = torch.div(cmin_t[1:] - 2 * torch.from_numpy(pd) + (torch.from_numpy(ks) - 1),
+                               torch.from_numpy(st))
+        got, _ = oracle.downsample_bounds(coords, ks, st, pd, allow_negative=True)
+        np.testing.assert_array_equal(got, cmin_t.numpy())
+    # with the flag off the bound is zero and negative candidates are dropped
+    got, _ = oracle.downsample_bounds(coords, ks, st, pd)
+    assert got.tolist() == [0, 0, 0, 0]
+
+
+def test_strided_outputs_at_negative_coordinates_are_the_valid_candidates():
+    """Brute force over every (input, offset): the output set with allow_negative is exactly
+    the candidates inside [coords_min, coords_max]."""
+    rng = np.random.default_rng(12)
+    coords = np.unique(rng.integers(-9, 9, (120, 4)).astype(np.int32), axis=0)
+    coords[:, 0] = np.abs(coords[:, 0]) % 2
+    coords = np.unique(coords, axis=0)
+    for ks, st, pd in [(2, 2, 0), (3, 2, 1), (3, 1, 1), (2, 3, 0)]:
+        cmin, cmax = oracle.downsample_bounds(coords, ks, st, pd, allow_negative=True)
+        want = set()
+        for b, x, y, z in coords.tolist():
+            for dx in range(ks):
+                for dy in range(ks):
+                    for dz in range(ks):
+                        num = (x + pd - dx, y + pd - dy, z + pd - dz)
+                        if any(v % st for v in num):
+                            continue
+                        o = tuple(v // st for v in num)
+                        if all(cmin[a + 1] <= o[a] <= cmax[a + 1] for a in range(3)):
+                            want.add((b,) + o)
+        _, out = oracle.kmap_downsample(coords, ks, st, pd, allow_negative=True)
+        assert [tuple(r) for r in out.tolist()] == sorted(want)

@@ -51,7 +51,7 @@ def _load():
         "tsmi_hashtable_lookup_keys": [_vp, _vp, _vp, _i64, _vp, _i64, _vp],
         "tsmi_kmap_query": [_vp, _vp, _vp, _i64, _vp, _i64, _i64, _I3, _I3, _I3, _vp],
         "tsmi_coords_max": [_vp, _vp, _i64, _vp, _i32],
-        "tsmi_downsample_candidates": [_vp, _vp, _i64, _I3, _I3, _I3, _vp, _vp, _i32, _vp, _i64, _vp],
+        "tsmi_downsample_candidates": [_vp, _vp, _i64, _I3, _I3, _I3, _vp, _vp, _vp, _i32, _vp, _i64, _vp],
         "tsmi_hashtable_compact_keys": [_vp, _vp, _i64, _vp, _vp],
         "tsmi_sort_keys": [_vp, _vp, _vp, _i64, _i32, _vp, _i64],
         "tsmi_downsample_finalize": [_vp, _vp, _i64, _vp, _vp, _i64, _vp],
@@ -254,11 +254,12 @@ def coords_max(coords: torch.Tensor) -> torch.Tensor:
 
 
 def downsample_coords(coords: torch.Tensor, kernel_sizes, stride, padding, coords_max_host=None,
-                      mode: int = 0, rsv_ratio: float = 2.0):
+                      mode: int = 0, rsv_ratio: float = 2.0, allow_negative: bool = False):
     """Output coordinates of a strided convolution in ascending (b,x,y,z) order and
     the hash table that indexes them.  Returns (out_coords, GPUHashTable).
     One host read-back (the number of outputs) — the reference has two
-    (others/sparsemapping_cuda.cu:477-479)."""
+    (others/sparsemapping_cuda.cu:477-479).  With ``allow_negative`` the outputs are bounded
+    below by the reference's coords_min (hashmap_on_the_fly.py:39-43) instead of 0."""
     coords = _need(coords, torch.int32, "coords")
     ks, st, pd = _triple(kernel_sizes), _triple(stride), _triple(padding)
     n = coords.shape[0]
@@ -272,17 +273,22 @@ def downsample_coords(coords: torch.Tensor, kernel_sizes, stride, padding, coord
     cap = hash_capacity(n * min(fan, 2), rsv_ratio)
     table = GPUHashTable(cap, device=dev)
     counters = table.counters  # zero on a fresh table
-    in_max = None
+    in_max = in_min = None
     host_max = None
     if mode == 0:
         if coords_max_host is not None:
             host_max = _I3(*[int(v) for v in coords_max_host])
+        elif allow_negative and n > 0:
+            in_max = coords.max(0).values.contiguous()  # the true maxima, possibly negative
         else:
             in_max = counters[4:8]  # still zero: the maximum lands here without a fill launch
             _check(_C.tsmi_coords_max(_stream(), _ptr(coords), n, _ptr(in_max), 0))
+        if allow_negative and n > 0:
+            in_min = coords.min(0).values.contiguous()
     s = _stream()
     _check(_C.tsmi_downsample_candidates(s, _ptr(coords), n, _I3(*ks), _I3(*st), _I3(*pd), host_max,
-                                         _ptr(in_max), mode, _ptr(table.keys), cap, _ptr(counters)))
+                                         _ptr(in_max), _ptr(in_min), mode, _ptr(table.keys), cap,
+                                         _ptr(counters)))
     # unique keys = the occupied slots of the table: compact, read the count back, sort
     temp_bytes = _C.tsmi_sort_temp_bytes(cap)
     scratch = torch.empty(2 * cap + temp_bytes // 8 + 1, dtype=torch.int64, device=dev)

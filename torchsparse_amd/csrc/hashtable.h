@@ -12,8 +12,9 @@
 
 namespace tsmi {
 
-constexpr int kCoordBits = 18;            // x, y, z each in [0, 2^18)
+constexpr int kCoordBits = 18;            // x, y, z each in [-2^17, 2^17): packed with a bias
 constexpr int kCoordLimit = 1 << kCoordBits;
+constexpr int kCoordBias = 1 << (kCoordBits - 1);
 constexpr int kBatchLimit = 512;          // keeps key + 1 positive in int64
 
 struct TableView {
@@ -24,21 +25,24 @@ struct TableView {
 };
 
 __device__ __forceinline__ bool coords_packable(int b, int x, int y, int z) {
-  return (unsigned)x < (unsigned)kCoordLimit && (unsigned)y < (unsigned)kCoordLimit &&
-         (unsigned)z < (unsigned)kCoordLimit && (unsigned)b < (unsigned)kBatchLimit;
+  return (unsigned)(x + kCoordBias) < (unsigned)kCoordLimit &&
+         (unsigned)(y + kCoordBias) < (unsigned)kCoordLimit &&
+         (unsigned)(z + kCoordBias) < (unsigned)kCoordLimit && (unsigned)b < (unsigned)kBatchLimit;
 }
 
 __device__ __forceinline__ unsigned long long pack_coords(int b, int x, int y, int z) {
+  // the bias keeps ascending key order = ascending (b, x, y, z) order for negative values too
   return ((unsigned long long)(unsigned)b << (3 * kCoordBits)) |
-         ((unsigned long long)(unsigned)x << (2 * kCoordBits)) |
-         ((unsigned long long)(unsigned)y << kCoordBits) | (unsigned long long)(unsigned)z;
+         ((unsigned long long)(unsigned)(x + kCoordBias) << (2 * kCoordBits)) |
+         ((unsigned long long)(unsigned)(y + kCoordBias) << kCoordBits) |
+         (unsigned long long)(unsigned)(z + kCoordBias);
 }
 
 __device__ __forceinline__ void unpack_coords(unsigned long long key, int *c) {
   const unsigned mask = kCoordLimit - 1;
-  c[3] = (int)(key & mask);
-  c[2] = (int)((key >> kCoordBits) & mask);
-  c[1] = (int)((key >> (2 * kCoordBits)) & mask);
+  c[3] = (int)(key & mask) - kCoordBias;
+  c[2] = (int)((key >> kCoordBits) & mask) - kCoordBias;
+  c[1] = (int)((key >> (2 * kCoordBits)) & mask) - kCoordBias;
   c[0] = (int)(key >> (3 * kCoordBits));
 }
 

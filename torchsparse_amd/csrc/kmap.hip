@@ -125,10 +125,27 @@ __global__ void coords_max_kernel(const int4 *coords, int64_t n, int32_t *out_ma
   }
 }
 
+__device__ __forceinline__ int floor_div(int a, int b) {
+  int q = a / b;
+  return (a % b != 0 && ((a < 0) != (b < 0))) ? q - 1 : q;
+}
+
+// Output range of axis a: upper bound from the host or floor((max + 2 pad - (ks-1)) / stride)
+// of the largest input coordinate; lower bound 0, or, when negative coordinates are allowed
+// (in_min_dev given), (min - 2 pad + (ks-1)) / stride rounded toward zero.
+__device__ __forceinline__ void output_range(const Geom &g, int a, int3 out_max_host,
+                                             const int32_t *in_max_dev, const int32_t *in_min_dev,
+                                             int *lo, int *hi) {
+  *hi = in_max_dev ? floor_div(in_max_dev[1 + a] + 2 * g.pad[a] - (g.ks[a] - 1), g.stride[a])
+                   : (a == 0 ? out_max_host.x : (a == 1 ? out_max_host.y : out_max_host.z));
+  *lo = in_min_dev ? (in_min_dev[1 + a] - 2 * g.pad[a] + (g.ks[a] - 1)) / g.stride[a] : 0;
+}
+
 // mode 0: thread per (input, offset); modes 1 and 2: thread per input.
 __global__ void downsample_candidates_kernel(const int4 *in_coords, int64_t n_in, int64_t total,
                                              Geom g, int3 out_max_host, const int32_t *in_max_dev,
-                                             int mode, TableView t, int32_t *counters) {
+                                             const int32_t *in_min_dev, int mode, TableView t,
+                                             int32_t *counters) {
   int64_t tid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (tid >= total) return;
   int b, x, y, z;
@@ -146,10 +163,9 @@ __global__ void downsample_candidates_kernel(const int4 *in_coords, int64_t n_in
       if (v[a] % g.stride[a] != 0 && v[a] < 0) --q;
       o[a] = q;
       if (mode == 2) {
-        int hi = in_max_dev
-                     ? (in_max_dev[1 + a] + 2 * g.pad[a] - (g.ks[a] - 1)) / g.stride[a]
-                     : (a == 0 ? out_max_host.x : (a == 1 ? out_max_host.y : out_max_host.z));
-        if (o[a] < 0 || o[a] > hi) return;
+        int lo, hi;
+        output_range(g, a, out_max_host, in_max_dev, in_min_dev, &lo, &hi);
+        if (o[a] < lo || o[a] > hi) return;
       }
     }
     x = o[0];
@@ -169,10 +185,9 @@ __global__ void downsample_candidates_kernel(const int4 *in_coords, int64_t n_in
       int num = v[a] + g.pad[a] + d[a] - (g.ks[a] - 1);
       if (num % g.stride[a] != 0) return;
       o[a] = num / g.stride[a];
-      int hi = in_max_dev
-                   ? (in_max_dev[1 + a] + 2 * g.pad[a] - (g.ks[a] - 1)) / g.stride[a]
-                   : (a == 0 ? out_max_host.x : (a == 1 ? out_max_host.y : out_max_host.z));
-      if (o[a] < 0 || o[a] > hi) return;
+      int lo, hi;
+      output_range(g, a, out_max_host, in_max_dev, in_min_dev, &lo, &hi);
+      if (o[a] < lo || o[a] > hi) return;
     }
     x = o[0];
     y = o[1];
@@ -627,8 +642,9 @@ extern "C" int tsmi_coords_max(tsmi_stream_t s, const int32_t *coords, int64_t n
 extern "C" int tsmi_downsample_candidates(tsmi_stream_t s, const int32_t *in_coords, int64_t n_in,
                                           const int32_t ks[3], const int32_t stride[3],
                                           const int32_t pad[3], const int32_t out_max_host[3],
-                                          const int32_t *in_max_dev, int mode, int64_t *keys,
-                                          int64_t cap, int32_t *counters) {
+                                          const int32_t *in_max_dev, const int32_t *in_min_dev,
+                                          int mode, int64_t *keys, int64_t cap,
+                                          int32_t *counters) {
   TableView t;
   Geom g;
   static int32_t dummy_vals;  // the de-duplication pass never touches vals
@@ -648,8 +664,8 @@ extern "C" int tsmi_downsample_candidates(tsmi_stream_t s, const int32_t *in_coo
   int3 hm = make_int3(0, 0, 0);
   if (out_max_host) hm = make_int3(out_max_host[0], out_max_host[1], out_max_host[2]);
   hipLaunchKernelGGL(downsample_candidates_kernel, grid_for(total), dim3(kBlock), 0,
-                     (hipStream_t)s, (const int4 *)in_coords, n_in, total, g, hm, in_max_dev, mode,
-                     t, counters);
+                     (hipStream_t)s, (const int4 *)in_coords, n_in, total, g, hm, in_max_dev,
+                     in_min_dev, mode, t, counters);
   return check_launch("tsmi_downsample_candidates");
 }
 

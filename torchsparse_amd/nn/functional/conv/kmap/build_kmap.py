@@ -143,8 +143,10 @@ def build_kernel_map(_coords: torch.Tensor, input_node_num: int,
         out_table = in_table
     elif mode == "hashmap_on_the_fly":
         host_max = None if new_range is None else tuple(x - 1 for x in new_range[1:])
-        out_coords, out_table = backend.downsample_coords(coords, kernel_size, stride, padding,
-                                                          host_max, 0, backends.hash_rsv_ratio)
+        from torchsparse_amd.tensor import get_allow_negative_coordinates
+        out_coords, out_table = backend.downsample_coords(
+            coords, kernel_size, stride, padding, host_max, 0, backends.hash_rsv_ratio,
+            allow_negative=get_allow_negative_coordinates())
         pad_eff = padding
     else:  # "hashmap": coordinates first, then a padding-free centred lookup
         from .downsample import spdownsample

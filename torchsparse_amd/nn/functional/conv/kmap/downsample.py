@@ -27,5 +27,7 @@ def spdownsample(_coords: torch.Tensor, stride: Union[int, Tuple[int, ...]] = 2,
         out, table = backend.downsample_coords(coords, kernel_size, stride, padding, None, mode=1)
     else:
         host_max = None if spatial_range is None else tuple(x - 1 for x in spatial_range[1:])
-        out, table = backend.downsample_coords(coords, kernel_size, stride, padding, host_max, mode=0)
+        from torchsparse_amd.tensor import get_allow_negative_coordinates
+        out, table = backend.downsample_coords(coords, kernel_size, stride, padding, host_max, mode=0,
+                                               allow_negative=get_allow_negative_coordinates())
     return (out, table) if return_table else out

@@ -19,11 +19,11 @@ def get_allow_negative_coordinates() -> bool:
 
 
 def set_allow_negative_coordinates(flag: bool) -> None:
-    """Negative coordinates are not supported by the packed hash keys of this build."""
+    """Let strided convolutions produce outputs at negative coordinates (tensor.py:24-26):
+    the lower bound of the output range becomes the reference's coords_min instead of 0.
+    Submanifold maps and the hash tables accept coordinates in [-2^17, 2^17) either way."""
     global _allow_negative_coordinates
-    if flag:
-        raise NotImplementedError("negative voxel coordinates are not supported")
-    _allow_negative_coordinates = False
+    _allow_negative_coordinates = bool(flag)
 
 
 class SparseTensor:
