@@ -108,6 +108,9 @@ int tsmi_coords_max(tsmi_stream_t s, const int32_t *coords, int64_t n, int32_t *
  *           input is launched instead of one per (input, offset).
  *   mode 1: o = floor(in / stride), unbounded — spdownsample for stride in {1, ks}
  *           or "minkowski" mode (nn/functional/conv/kmap/downsample.py:30-37).
+ *   mode 3: o = clamp(in * stride + digit - (ks-1)/2, 0, out_max_host) for every offset —
+ *           the output coordinates of a generative transposed convolution
+ *           (nn/functional/conv/kmap/upsample.py:12-41).
  * The upper bound is out_max_host[3] when in_max_dev is NULL, otherwise it is derived on
  * the device as floor((in_max_dev[1+a] + 2*pad - (ks-1)) / stride)
  * (hashmap_on_the_fly.py:33-37).  The lower bound is 0 when in_min_dev is NULL; with

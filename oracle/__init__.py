@@ -21,6 +21,10 @@ the checks live in ``tests/test_oracle_*.py``):
                            k in {2,3,5} x s in {1,2,3}
   spdownsample_floor /     numpy unique(axis=0); dense nn.Conv3d equivalence
   lookup_coords
+  upsample_generative_     numpy restatement of the torch recipe; with lookup_coords (pinned
+  coords / kmap_generative above) the convolution over the map equals a dense
+                           torch conv_transpose3d with the flipped kernel (odd kernels,
+                           inputs away from the clamped border)
   transpose_map            exact inverse relation, checked by brute force;
                            torch.nn.ConvTranspose3d equivalence (k == s)
   derive_bitmask /         closed-form definitions re-derived with numpy bit ops on
@@ -198,6 +202,33 @@ def lookup_coords(in_coords, out_coords, kernel_size, stride):
                             out_coords.shape[0], _p(ks, _i32p), _p(st, _i32p), n_pad,
                             _p(omap, _i32p))
     return omap
+
+
+def upsample_generative_coords(coords, kernel_size, stride, spatial_range):
+    """unique(clamp(coords * stride + offset, 0, range - 1)) over all kernel offsets, ascending
+    (b,x,y,z) — nn/functional/conv/kmap/upsample.py:12-41 (torch.unique(dim=0) sorts rows)."""
+    coords = _i32(coords)
+    ks, st = _triple(kernel_size), _triple(stride)
+    offs = kernel_offsets(ks)
+    c = coords.astype(np.int64)
+    c[:, 1:] *= st
+    cand = np.repeat(c[:, None, :], offs.shape[0], axis=1)
+    cand[:, :, 1:] += offs[None]
+    for a in range(1, 4):
+        np.clip(cand[:, :, a], 0, int(spatial_range[a]) - 1, out=cand[:, :, a])
+    return np.unique(cand.reshape(-1, 4), axis=0).astype(np.int32)
+
+
+def kmap_generative(coords, kernel_size, stride, spatial_range):
+    """(out_in_map, out_coords) of a generative transposed convolution —
+    kmap/func/hashmap.py:24-83: the table holds coords * stride, the outputs are looked up
+    with stride 1 (lookup_coords)."""
+    coords = _i32(coords)
+    st = _triple(stride)
+    out_coords = upsample_generative_coords(coords, kernel_size, stride, spatial_range)
+    scaled = coords.copy()
+    scaled[:, 1:] *= st
+    return lookup_coords(scaled, out_coords, kernel_size, 1), out_coords
 
 
 def transpose_map(out_in_map, n_in):

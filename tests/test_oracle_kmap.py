@@ -251,3 +251,42 @@ def test_strided_outputs_at_negative_coordinates_are_the_valid_candidates():
                             want.add((b,) + o)
         _, out = oracle.kmap_downsample(coords, ks, st, pd, allow_negative=True)
         assert [tuple(r) for r in out.tolist()] == sorted(want)
+
+
+@pytest.mark.parametrize("ks,st", [(3, 2), (3, 1), (3, 3), (5, 2)])
+def test_generative_map_equals_dense_transposed_convolution(ks, st):
+    """y[o] = sum_k x[i] W[k] with i*s = o + offset_k is conv_transpose3d with the kernel
+    flipped and padding (ks-1)/2; inputs are kept away from the border so that the clamp of
+    the generated coordinates does not act."""
+    import torch
+    rng = np.random.default_rng(ks * 10 + st)
+    ext = 6
+    cells = np.stack(np.unravel_index(rng.choice(ext ** 3, 40, replace=False), (ext,) * 3), 1)
+    coords = np.concatenate([np.zeros((40, 1), np.int32), cells.astype(np.int32) + 2], 1)
+    big = (ext + 4) * st + ks
+    omap, out_coords = oracle.kmap_generative(coords, ks, st, (1, big, big, big))
+    cin, cout = 3, 4
+    x = rng.standard_normal((40, cin)).astype(np.float32)
+    w = rng.standard_normal((ks ** 3, cin, cout)).astype(np.float32)
+    y = oracle.conv_implicit_gemm(x, w, omap, len(out_coords))
+    dense = torch.zeros(1, cin, ext + 4, ext + 4, ext + 4, dtype=torch.float64)
+    dense[0, :, coords[:, 1], coords[:, 2], coords[:, 3]] = torch.from_numpy(x.T).double()
+    # weight k applies to offset (dx,dy,dz), x fastest; conv_transpose3d wants [cin, cout, kx, ky, kz]
+    wt = torch.from_numpy(w).double().reshape(ks, ks, ks, cin, cout).permute(3, 4, 2, 1, 0)
+    wt = torch.flip(wt, dims=(2, 3, 4))
+    full = torch.nn.functional.conv_transpose3d(dense, wt, stride=st, padding=(ks - 1) // 2)[0]
+    got = np.zeros(tuple(full.shape[1:]) + (cout,))
+    got[out_coords[:, 1], out_coords[:, 2], out_coords[:, 3]] = y
+    np.testing.assert_allclose(got, full.permute(1, 2, 3, 0).numpy(), rtol=1e-4, atol=1e-4)
+
+
+def test_generative_coordinates_are_clamped_and_unique():
+    coords = np.array([[0, 0, 0, 0], [0, 3, 3, 3], [1, 3, 0, 1]], np.int32)
+    out = oracle.upsample_generative_coords(coords, 3, 2, (2, 6, 6, 6))
+    assert out[:, 1:].min() == 0 and out[:, 1:].max() == 5
+    assert len(np.unique(out, axis=0)) == len(out)
+    key = ((out[:, 0].astype(np.int64) * 8 + out[:, 1]) * 8 + out[:, 2]) * 8 + out[:, 3]
+    assert (np.diff(key) > 0).all()
+    # voxel (0,0,0): offsets -1..1 around 0 clamp to {0,1}^3 -> 8 cells of batch 0 near the origin
+    near = out[(out[:, 0] == 0) & (out[:, 1:] <= 1).all(1)]
+    assert len(near) == 8

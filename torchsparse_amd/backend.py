@@ -270,12 +270,17 @@ def downsample_coords(coords: torch.Tensor, kernel_sizes, stride, padding, coord
     if mode == 0:
         for k, s in zip(ks, st):
             fan *= -(-k // s)
-    cap = hash_capacity(n * min(fan, 2), rsv_ratio)
+    if mode == 3:  # generative upsampling: up to one output per (input, offset)
+        cap = hash_capacity(n * ks[0] * ks[1] * ks[2], rsv_ratio)
+    else:
+        cap = hash_capacity(n * min(fan, 2), rsv_ratio)
     table = GPUHashTable(cap, device=dev)
     counters = table.counters  # zero on a fresh table
     in_max = in_min = None
     host_max = None
-    if mode == 0:
+    if mode == 3:
+        host_max = _I3(*[int(v) for v in coords_max_host])
+    elif mode == 0:
         if coords_max_host is not None:
             host_max = _I3(*[int(v) for v in coords_max_host])
         elif allow_negative and n > 0:

@@ -141,7 +141,8 @@ __device__ __forceinline__ void output_range(const Geom &g, int a, int3 out_max_
   *lo = in_min_dev ? (in_min_dev[1 + a] - 2 * g.pad[a] + (g.ks[a] - 1)) / g.stride[a] : 0;
 }
 
-// mode 0: thread per (input, offset); modes 1 and 2: thread per input.
+// mode 0: thread per (input, offset); modes 1 and 2: thread per input; mode 3 (generative
+// upsampling): thread per (input, offset), o = clamp(in * stride + digit - (ks-1)/2, 0, max).
 __global__ void downsample_candidates_kernel(const int4 *in_coords, int64_t n_in, int64_t total,
                                              Geom g, int3 out_max_host, const int32_t *in_max_dev,
                                              const int32_t *in_min_dev, int mode, TableView t,
@@ -149,7 +150,24 @@ __global__ void downsample_candidates_kernel(const int4 *in_coords, int64_t n_in
   int64_t tid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (tid >= total) return;
   int b, x, y, z;
-  if (mode != 0) {
+  if (mode == 3) {
+    int64_t i = tid / g.kvol;
+    int k = (int)(tid - i * g.kvol);
+    int4 c = in_coords[i];
+    b = c.x;
+    int d[3];
+    decode_digits(k, g, d);
+    int v[3] = {c.y, c.z, c.w};
+    int o[3];
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+      const int hi = a == 0 ? out_max_host.x : (a == 1 ? out_max_host.y : out_max_host.z);
+      o[a] = min(max(v[a] * g.stride[a] + d[a] - (g.ks[a] - 1) / 2, 0), hi);
+    }
+    x = o[0];
+    y = o[1];
+    z = o[2];
+  } else if (mode != 0) {
     // one candidate per input: o = floor(in / stride).  mode 1 keeps it unbounded; mode 2
     // is the strided-convolution rule specialised to kernel size == stride, zero padding
     // (o*s <= in < o*s + k has exactly one solution), bounded like mode 0.
@@ -650,7 +668,8 @@ extern "C" int tsmi_downsample_candidates(tsmi_stream_t s, const int32_t *in_coo
   static int32_t dummy_vals;  // the de-duplication pass never touches vals
   if (int e = make_table(&t, keys, &dummy_vals, cap)) return e;
   if (int e = make_geom(&g, ks, stride, pad)) return e;
-  TSMI_REQUIRE(mode == 0 || mode == 1, "downsample_candidates: mode must be 0 or 1");
+  TSMI_REQUIRE(mode == 0 || mode == 1 || mode == 3, "downsample_candidates: mode must be 0, 1 or 3");
+  TSMI_REQUIRE(mode != 3 || out_max_host, "downsample_candidates: mode 3 needs out_max_host");
   // kernel size == stride and zero padding: every input has exactly one candidate
   if (mode == 0 && ks[0] == stride[0] && ks[1] == stride[1] && ks[2] == stride[2] &&
       pad[0] == 0 && pad[1] == 0 && pad[2] == 0)
@@ -659,7 +678,7 @@ extern "C" int tsmi_downsample_candidates(tsmi_stream_t s, const int32_t *in_coo
   TSMI_REQUIRE(counters, "downsample_candidates: null counters");
   TSMI_REQUIRE(mode == 1 || in_max_dev || out_max_host, "downsample_candidates: no output bound");
   if (n_in == 0) return TSMI_OK;
-  int64_t total = mode != 0 ? n_in : n_in * g.kvol;
+  int64_t total = (mode == 1 || mode == 2) ? n_in : n_in * g.kvol;
   TSMI_GRID_CHECK(total);
   int3 hm = make_int3(0, 0, 0);
   if (out_max_host) hm = make_int3(out_max_host[0], out_max_host[1], out_max_host[2]);

@@ -93,9 +93,22 @@ def conv3d(input: SparseTensor, weight: torch.Tensor,
             caches.hashmaps.setdefault(out_stride, kmap["out_hashmap"])
         out_feats = conv_fn.apply(feats, weight, kmap, config, False, bias, residual, relu)
         output = SparseTensor._make(out_feats, kmap["coords"], out_stride, kmap["spatial_range"], caches)
+    elif generative:
+        # generative transposed convolution (conv.py:162-204): outputs are created around
+        # every input; the map is never cached and the caches of coarser levels are dropped
+        fine_stride = tuple(input.stride[a] // stride[a] for a in range(3))
+        kmap = build_kernel_map(
+            coords, feats.shape[0], kernel_size, stride, padding, None, None,
+            input.spatial_range, config["kmap_mode"], dataflow,
+            downsample_mode=config["downsample_mode"], training=training,
+            ifsort=config["ifsort"], generative=True, split_mask_num=config["split_mask_num"])
+        out_feats = conv_fn.apply(feats, weight, kmap, config, False, bias, residual, relu)
+        caches.cmaps[fine_stride] = (kmap["coords"], kmap.get("spatial_range"))
+        caches.kmaps = dict()
+        caches.hashmaps = dict()
+        output = SparseTensor._make(out_feats, kmap["coords"], fine_stride, kmap.get("spatial_range"),
+                                    caches)
     else:
-        if generative:
-            raise NotImplementedError("generative transposed convolution is not part of this build")
         fine_stride = tuple(input.stride[a] // stride[a] for a in range(3))
         kmap = caches.kmaps.get((fine_stride, kernel_size, stride, dilation))
         kmap = transpose_kernel_map(kmap, config["ifsort"], training=training,

@@ -76,6 +76,36 @@ def _backward_products(kmap: Dict, ifsort: bool, split_mask_num_bwd: int) -> Non
     kmap["reorder_loc_bwd"] = reorder_loc
 
 
+def _generative_kmap(kmap: Dict, coords: torch.Tensor, input_node_num: int, kernel_size, stride,
+                     padding, new_range, dataflow, ifsort: bool, split_mask_num: int) -> Dict:
+    """Map of a generative transposed convolution (kmap/func/hashmap.py:24-83): the outputs are
+    generated around the inputs scaled by the stride (kmap/upsample.py), the table indexes the
+    scaled inputs, and out_in_map[o, k] = the input whose scaled coordinate is o + offset k
+    (a stride-1 centred look-up).  The output range is the reference's: the STRIDED range of
+    build_kmap.py:65-74, also for this upsampling map."""
+    from .upsample import spupsample_generative
+    out_coords, out_table = spupsample_generative(coords, stride, kernel_size, padding, new_range,
+                                                  return_table=True)
+    scaled = coords.clone()
+    scaled[:, 1:] *= torch.tensor(stride, dtype=coords.dtype, device=coords.device)
+    in_table = backend.GPUHashTable(backend.hash_capacity(coords.shape[0], backends.hash_rsv_ratio),
+                                    device=coords.device)
+    in_table.insert_bxyz(scaled)
+    pad = tuple((k - 1) // 2 for k in kernel_size)
+    kmap["out_in_map"] = in_table.query_bxyz(out_coords, kernel_size, (1, 1, 1), pad)
+    kmap["coords"] = out_coords
+    kmap["sizes"] = (input_node_num, out_coords.shape[0])
+    kmap["in_hashmap"] = (in_table.keys, in_table.vals)
+    kmap["out_hashmap"] = (out_table.keys, out_table.vals)
+    kmap["hashmap_keys"], kmap["hashmap_vals"] = in_table.keys, in_table.vals
+    if dataflow == Dataflow.ImplicitGEMM:
+        if ifsort:
+            _sort_products(kmap, kmap["out_in_map"], kmap["sizes"][1], split_mask_num)
+    else:
+        _pair_products(kmap, dataflow)
+    return kmap
+
+
 def _pair_products(kmap: Dict, dataflow: Dataflow) -> None:
     """Pair lists, masks and scans for the GatherScatter / FetchOnDemand dataflows
     (kmap/func/hashmap_on_the_fly.py:112-207).  Both dataflows get the masks and the
@@ -109,8 +139,6 @@ def build_kernel_map(_coords: torch.Tensor, input_node_num: int,
 
     ``hashmap_keys`` / ``hashmap_vals`` — when given — are a table that already
     indexes the INPUT coordinates ``_coords`` (it is reused instead of rebuilt)."""
-    if generative:
-        raise NotImplementedError("generative transposed convolution is not part of this build")
     if mode not in ("hashmap_on_the_fly", "hashmap"):
         if mode == "grid":
             raise AssertionError("grid mode is temporarily deprecated.")
@@ -120,9 +148,16 @@ def build_kernel_map(_coords: torch.Tensor, input_node_num: int,
     assert backends.hash_rsv_ratio >= 2, (
         f"hash_rsv_ratio should be no less than 2, now {backends.hash_rsv_ratio}.")
 
+    if generative and mode == "hashmap_on_the_fly":
+        raise ValueError(f"Unsupported kmap_mode: {mode} for generative convolution "
+                         "(please switch to kmap_mode=hashmap).")
+
     kernel_size, stride, padding = (make_ntuple(v, ndim=3) for v in (kernel_size, stride, padding))
     new_range = _strided_range(spatial_range, kernel_size, stride, padding)
     kmap = _empty_kmap(hashmap_keys, hashmap_vals, new_range)
+    if generative:
+        return _generative_kmap(kmap, _coords.contiguous(), input_node_num, kernel_size, stride,
+                                padding, new_range, dataflow, ifsort, split_mask_num)
     subm = all(s == 1 for s in stride)
     coords = _coords.contiguous()
     n_in = coords.shape[0]
