@@ -100,7 +100,7 @@ def kmap_bytes_down(n, n_out, n_out_pad, cap, cand, kvol):
 # description this script prints.  None when the kernel that dominates has not been
 # measured that way.
 PMC_TRAFFIC_BYTES = {
-    "igemm k(3, 3, 3) s(1, 1, 1) 96->96 level(1, 1, 1) n_out=89834 nnz=505724": 81452037,
+    "igemm k(3, 3, 3) s(1, 1, 1) 96->96 level(1, 1, 1) n_out=89834 nnz=505724": 81538296,
 }
 
 
@@ -344,9 +344,10 @@ def cpu_baseline(records, level_coords):
     import oracle
     cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
     rng = np.random.default_rng(0)
-    t_map = t_conv = t_ref = 0.0
+    t_map = t_conv = t_ref = t_conv_same = 0.0
     pair_cache = {}
-    n_layers = 0
+    n_layers = n_ref_layers = 0
+    ref_budget_s = 15.0  # the compiled reference convolution is slow: stop timing it after this
     ref = oracle.ref_module()  # the reference's own CPU convolution, compiled in place
     for r in records:
         if r["ks"] == (1, 1, 1):
@@ -369,21 +370,26 @@ def cpu_baseline(records, level_coords):
         w = rng.standard_normal((len(sz), r["cin"], r["cout"])).astype(np.float32)
         t0 = time.perf_counter()
         oracle.conv_gather_scatter(x, w, nb, sz, r["n_out"], transpose=transposed, variant=1)
-        t_conv += time.perf_counter() - t0
-        if ref is not None:
+        dt = time.perf_counter() - t0
+        t_conv += dt
+        if ref is not None and t_ref < ref_budget_s:
             n_y = r["n_out"]
             y = torch.zeros(n_y, r["cout"])
             tx, tw, tnb, tsz = torch.from_numpy(x), torch.from_numpy(w), torch.from_numpy(nb), torch.from_numpy(sz)
             t0 = time.perf_counter()
             ref.conv_forward_gather_scatter_cpu(tx, y, tw, tnb, tsz, transposed)
             t_ref += time.perf_counter() - t0
+            t_conv_same += dt
+            n_ref_layers += 1
         n_layers += 1
     extra = {}
     if ref is not None:
         extra = {"reference_conv_ms": round(t_ref * 1e3, 1),
                  "reference_conv": "conv_forward_gather_scatter_cpu of the reference (its own sources, "
-                                   "compiled) over the same layers, torch threads = "
-                                   f"{torch.get_num_threads()}"}
+                                   f"compiled) over the first {n_ref_layers} of the layers (stopped "
+                                   f"after {ref_budget_s:.0f} s), torch threads = "
+                                   f"{torch.get_num_threads()}; the port takes "
+                                   f"{t_conv_same * 1e3:.0f} ms on those layers"}
     return {**extra, "value": round((t_map + t_conv) * 1e3, 1), "unit": "ms", "cores": cores, "kind": "port",
             "sample": f"{n_layers} sparse conv layers (fp32) + {len(pair_cache)} kernel maps of one "
                       f"MinkUNet forward on the same scan; BN/ReLU/concat/1x1x1 layers excluded; "
