@@ -231,9 +231,9 @@ def pointops_sweep(F):
     pc_hash = F.sphash(pc)
     vox_hash = torch.unique(pc_hash)
     n_vox = vox_hash.numel()
-    idx = F.sphashquery(pc_hash, vox_hash).int()
+    idx = F.sphashquery(pc_hash, vox_hash)
     counts = F.spcount(idx, n_vox)
-    corner = F.sphashquery(F.sphash(pc, offsets).t().contiguous(), vox_hash).int().contiguous()
+    corner = F.sphashquery(F.sphash(pc, offsets).t().contiguous(), vox_hash)
     w = F.calc_ti_weights(pts, corner, scale=1)
     feats = torch.randn(n, c, device="cuda", dtype=torch.float16)
     vfeat = torch.randn(n_vox, c, device="cuda", dtype=torch.float16)

@@ -58,7 +58,7 @@ def test_sphashquery_finds_rows_and_reports_missing(mods):
     got = F.sphashquery(q_hash, ref_hash).cpu().numpy()
     lut = {tuple(c): i for i, c in enumerate(coords.tolist())}
     want = np.array([[lut.get(tuple(r), -1) for r in q] for q in queries.tolist()])
-    assert got.shape == (700, 3) and got.dtype == np.int64
+    assert got.shape == (700, 3) and got.dtype == np.int32
     np.testing.assert_array_equal(got, want)
     assert (got[::7, 0] == -1).all()
 
@@ -186,7 +186,7 @@ def test_point_voxel_round_trip(mods):
     sparse_hash = torch.unique(pc_hash)
     idx_query = F.sphashquery(pc_hash, sparse_hash)
     assert (idx_query >= 0).all()
-    counts = F.spcount(idx_query.int(), len(sparse_hash))
+    counts = F.spcount(idx_query, len(sparse_hash))
     assert int(counts.sum()) == len(pts)
     feats = dev(rng.standard_normal((len(pts), 16)).astype(np.float32))
     vox = F.spvoxelize(feats, idx_query, counts)
@@ -196,7 +196,7 @@ def test_point_voxel_round_trip(mods):
     ones = torch.ones(len(pts), 4, device="cuda")
     v1 = F.spvoxelize(ones, idx_query, counts)
     corner = torch.full((len(pts), 8), -1, device="cuda", dtype=torch.int32)
-    corner[:, 0] = idx_query.int()
+    corner[:, 0] = idx_query
     w = torch.zeros(len(pts), 8, device="cuda")
     w[:, 0] = 1
     back = F.spdevoxelize(v1, corner, w)
