@@ -151,6 +151,24 @@ def test_million_voxel_256_channel_layer(mods):
     y12 = backend.conv_forward_implicit_gemm_cuda((2 * x1 + x2), w, omap, n, 256)
     lin = 2 * y1.float() + y2.float()
     assert rel_rms(y12.float().cpu().numpy(), lin.cpu().numpy()) < 1e-2
+    # weight gradient at this size: the pair-list kernel against an fp32 GEMM of the gathered
+    # rows (hipBLASLt through torch: an independent implementation) for a few offsets, and
+    # the input gradient's adjoint identity <conv(x), g> = <x, dgrad(g)>
+    g1 = torch.randn(n, 256, device="cuda", dtype=torch.float16)
+    lists = backend.wgrad_pair_lists(omap, n)
+    dw = backend.conv_backward_wgrad_pairs_cuda(g1, x1, lists, 0)
+    assert dw.shape == (27, 256, 256)
+    for k in (0, 13, 22):
+        out_rows = torch.nonzero(m[:, k] >= 0).squeeze(1)
+        in_rows = m[out_rows, k].long()
+        want_k = x1[in_rows].float().t() @ g1[out_rows].float()
+        assert rel_rms(dw[k].float().cpu().numpy(), want_k.cpu().numpy()) < 1e-2, k
+    assert torch.equal(dw, backend.conv_backward_wgrad_pairs_cuda(g1, x1, lists, 0))
+    map_bwd = backend.convert_transposed_out_in_map(omap, omap.shape[0], n)
+    dx = backend.conv_forward_implicit_gemm_cuda(g1, w.transpose(1, 2).contiguous(), map_bwd, n, 256)
+    lhs = (y1.float() * g1.float()).sum().item()
+    rhs = (x1.float() * dx.float()).sum().item()
+    assert abs(lhs - rhs) < 2e-2 * max(abs(lhs), (y1.float().norm() * g1.float().norm()).item() * 1e-2)
     # the three dataflows agree at this size
     cfg_rows = torch.from_numpy(rows).cuda()
     for flow in (F.Dataflow.FetchOnDemand, F.Dataflow.GatherScatter):

@@ -615,11 +615,12 @@ def wgrad_pair_lists_from_nbmaps(nbmaps: torch.Tensor, nbsizes: torch.Tensor) ->
     return dict(pairs=pairs, seg_steps=seg_steps, nbsizes=sizes, cap=cap)
 
 
-def wgrad_pairs_supported(in_feats: torch.Tensor, grad_out: torch.Tensor) -> bool:
+def wgrad_pairs_supported(in_feats: torch.Tensor, grad_out: torch.Tensor, kernel_volume: int = 1) -> bool:
     """The pair-list weight gradient moves 16-byte pieces of rows: both channel counts
-    must be multiples of 16 bytes of elements."""
+    must be multiples of 16 bytes of elements; its segment table holds 511 offsets."""
     per = 16 // in_feats.element_size()
-    return in_feats.shape[1] % per == 0 and grad_out.shape[1] % per == 0
+    return (in_feats.shape[1] % per == 0 and grad_out.shape[1] % per == 0
+            and kernel_volume <= 511)
 
 
 def conv_backward_wgrad_pairs_cuda(grad_out: torch.Tensor, in_feats: torch.Tensor, pair_lists: dict,

@@ -74,7 +74,7 @@ class SparseConvFunction(torch.autograd.Function):
             if grad_input.dtype != input.dtype:
                 grad_input = grad_input.to(input.dtype)
         if ctx.needs_input_grad[1]:
-            if backend.wgrad_pairs_supported(x, dy):
+            if backend.wgrad_pairs_supported(x, dy, w.shape[0]):
                 # the map's values index the strided convolution's input: x for a plain
                 # convolution (column 0), dy for a transposed one
                 grad_weight = backend.conv_backward_wgrad_pairs_cuda(
