@@ -179,8 +179,8 @@ int tsmi_reduce_bitmask(tsmi_stream_t s, const int32_t *sorted_mask, int split,
 
 /* Pair lists, phase 1: per-offset counts.  nbsizes int32[K_vol] := number of
  * rows < n_rows with map[row,k] != -1; block_counts int32[K_vol * nblk] is
- * scratch for phase 2, nblk = ceil(n_rows / 256).  Replaces torch.sum(results
- * != -1, dim=1) (hashmap_on_the_fly.py:139,186). */
+ * scratch for phase 2, nblk = ceil(n_rows / 256).  K_vol <= 512.  Replaces
+ * torch.sum(results != -1, dim=1) (hashmap_on_the_fly.py:139,186). */
 int tsmi_pair_lists_count(tsmi_stream_t s, const int32_t *map, int64_t n_rows, int kvol,
                           int32_t *block_counts, int32_t *nbsizes);
 
@@ -192,11 +192,12 @@ int tsmi_pair_lists_count(tsmi_stream_t s, const int32_t *map, int64_t n_rows, i
  *     pair inside offset k's list (pre-filled with -1 here); the centre offset of
  *     an odd-volume map with n_in == n_out is skipped — build_mask_from_kmap
  *     (others/sparsemapping_cuda.cu:235-256,510-548).
- * nnz is the sum of nbsizes (the caller read it back to size the arrays). */
+ * nbsizes is phase 1's (device); nnz is its sum (the caller read it back to size the
+ * arrays). */
 int tsmi_pair_lists_fill(tsmi_stream_t s, const int32_t *map, int64_t n_rows, int kvol,
-                         int32_t *block_counts, int64_t nnz, int32_t *nbmaps_inter,
-                         int32_t *nbmaps_planar, int64_t n_in, int64_t n_out,
-                         int32_t *input_mask, int32_t *output_mask);
+                         int32_t *block_counts, const int32_t *nbsizes, int64_t nnz,
+                         int32_t *nbmaps_inter, int32_t *nbmaps_planar, int64_t n_in,
+                         int64_t n_out, int32_t *input_mask, int32_t *output_mask);
 
 /* input_mask / output_mask (see tsmi_pair_lists_fill) from an existing interleaved
  * pair list and nbaddrs = exclusive scan of its per-offset sizes.  Replaces

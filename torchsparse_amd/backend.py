@@ -61,7 +61,7 @@ def _load():
         "tsmi_reorder_map": [_vp, _vp, _vp, _i64, _i32, _i32, _vp],
         "tsmi_reduce_bitmask": [_vp, _vp, _i32, _i64, _i32, _vp],
         "tsmi_pair_lists_count": [_vp, _vp, _i64, _i32, _vp, _vp],
-        "tsmi_pair_lists_fill": [_vp, _vp, _i64, _i32, _vp, _i64, _vp, _vp, _i64, _i64, _vp, _vp],
+        "tsmi_pair_lists_fill": [_vp, _vp, _i64, _i32, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _vp, _vp],
         "tsmi_exclusive_scan_quantified": [_vp, _i32, _vp, _i32, _vp, _vp],
         "tsmi_build_masks": [_vp, _vp, _i64, _vp, _i32, _i64, _i64, _vp, _vp],
         "tsmi_pack_weights": [_vp, _vp, _vp, _i32, _i32, _i32, _i32],
@@ -411,8 +411,9 @@ def pair_lists(out_in_map: torch.Tensor, n_in: int, n_out: int, want_inter=True,
     planar = torch.empty((2, nnz), dtype=torch.int32, device=dev) if want_planar else None
     imask = torch.empty(kvol * n_in, dtype=torch.int32, device=dev) if want_masks else None
     omask = torch.empty(kvol * n_out, dtype=torch.int32, device=dev) if want_masks else None
-    _check(_C.tsmi_pair_lists_fill(_stream(), _ptr(out_in_map), n_out, kvol, _ptr(block_counts), nnz,
-                                   _ptr(inter), _ptr(planar), n_in, n_out, _ptr(imask), _ptr(omask)))
+    _check(_C.tsmi_pair_lists_fill(_stream(), _ptr(out_in_map), n_out, kvol, _ptr(block_counts),
+                                   _ptr(nbsizes), nnz, _ptr(inter), _ptr(planar), n_in, n_out,
+                                   _ptr(imask), _ptr(omask)))
     return dict(nbmaps_inter=inter, nbmaps_planar=planar, nbsizes=nbsizes, input_mask=imask,
                 output_mask=omask, nnz=nnz)
 

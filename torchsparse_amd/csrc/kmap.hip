@@ -316,148 +316,189 @@ __global__ void reduce_bitmask_kernel(const int32_t *mask, int split, int64_t n_
 
 // ---- pair lists: per-block counts, in-place scan, ordered fill ---------------
 
-__global__ void pair_count_kernel(const int32_t *map, int64_t n_rows, int kvol, int64_t nblk,
-                                  int32_t *block_counts) {
-  __shared__ int wave_cnt[kBlock / 64];
-  int64_t row = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  for (int k = 0; k < kvol; ++k) {
-    bool valid = row < n_rows && map[row * kvol + k] != -1;
-    unsigned long long b = __ballot(valid);
-    if (lane == 0) wave_cnt[wave] = __popcll(b);
-    __syncthreads();
-    if (threadIdx.x == 0)
-      block_counts[(int64_t)k * nblk + blockIdx.x] =
-          wave_cnt[0] + wave_cnt[1] + wave_cnt[2] + wave_cnt[3];
-    __syncthreads();
+// Pair lists, shared structure of the kernels below: a block owns 256 consecutive map rows
+// (one per thread) and walks the offsets in chunks of kPairChunk.  The chunk's part of the
+// block's rows is staged in LDS with coalesced loads (for K_vol <= 32 the block's whole span
+// of the map, contiguous) — a thread walking its own row straight from memory makes every
+// wavefront load touch 54 cache lines, and with a few dozen wavefronts per CU those lines
+// do not survive in the L1 until the next offset (measured: 340 GB/s of map).  Per offset a
+// wavefront then ballots "row has an entry" out of LDS (row stride odd: no bank conflicts).
+constexpr int kPairMaxKvol = 512;  // offsets the per-block start table holds
+constexpr int kPairChunk = 32;     // offsets staged at a time
+constexpr int kPairStride = kPairChunk + 1;
+
+// tile[r * kPairStride + j] = map[row0 + r][k0 + j] for r < 256, j < kc (-1 past the end)
+__device__ __forceinline__ void pair_stage_rows(const int32_t *map, int64_t row0, int64_t n_rows,
+                                                int kvol, int k0, int kc, int32_t *tile) {
+  const float inv = 1.0f / (float)kc;
+  for (int idx = threadIdx.x; idx < kBlock * kc; idx += kBlock) {
+    const int r = (int)(((float)idx + 0.5f) * inv);  // idx / kc, exact for idx < 2^20
+    const int j = idx - r * kc;
+    const int64_t row = row0 + r;
+    tile[r * kPairStride + j] = row < n_rows ? map[row * kvol + k0 + j] : -1;
   }
 }
 
-// Single block: exclusive scan of `n` counts in place; nbsizes[k] from the scan.
-__global__ void pair_scan_kernel(int32_t *counts, int64_t n, int kvol, int64_t nblk,
-                                 int32_t *nbsizes) {
+__global__ __launch_bounds__(kBlock) void pair_count_kernel(const int32_t *map, int64_t n_rows,
+                                                            int kvol, int64_t nblk,
+                                                            int32_t *block_counts) {
+  __shared__ int32_t tile[kBlock * kPairStride];
+  __shared__ int wave_cnt[kBlock / 64][kPairChunk];
+  const int64_t row0 = (int64_t)blockIdx.x * kBlock;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  for (int k0 = 0; k0 < kvol; k0 += kPairChunk) {
+    const int kc = min(kPairChunk, kvol - k0);
+    pair_stage_rows(map, row0, n_rows, kvol, k0, kc, tile);
+    __syncthreads();
+    int my = 0;  // lane j keeps the count of offset k0 + j
+    for (int j = 0; j < kc; ++j) {
+      const int c = __popcll(__ballot(tile[threadIdx.x * kPairStride + j] != -1));
+      if (lane == j) my = c;
+    }
+    if (lane < kc) wave_cnt[wave][lane] = my;
+    __syncthreads();
+    if (threadIdx.x < kc)
+      block_counts[(int64_t)(k0 + threadIdx.x) * nblk + blockIdx.x] =
+          wave_cnt[0][threadIdx.x] + wave_cnt[1][threadIdx.x] + wave_cnt[2][threadIdx.x] +
+          wave_cnt[3][threadIdx.x];
+  }
+}
+
+// Block k: exclusive scan of offset k's per-block counts in place (positions relative to the
+// start of the offset's list); nbsizes[k] = their sum.
+__global__ __launch_bounds__(1024) void pair_scan_kernel(int32_t *counts, int kvol, int64_t nblk,
+                                                         int32_t *nbsizes) {
   __shared__ int part[1024];
-  __shared__ int total_s;
   const int t = threadIdx.x;
-  int64_t chunk = (n + 1023) / 1024;
-  int64_t begin = min((int64_t)t * chunk, n), end = min(begin + chunk, n);
+  int32_t *mine = counts + (int64_t)blockIdx.x * nblk;
+  const int64_t chunk = (nblk + 1023) / 1024;
+  const int64_t begin = min((int64_t)t * chunk, nblk), end = min(begin + chunk, nblk);
   int sum = 0;
-  for (int64_t i = begin; i < end; ++i) sum += counts[i];
+  for (int64_t i = begin; i < end; ++i) sum += mine[i];
   part[t] = sum;
   __syncthreads();
-  // Hillis-Steele inclusive scan over 1024 partial sums
-  for (int off = 1; off < 1024; off <<= 1) {
-    int v = t >= off ? part[t - off] : 0;
+  for (int off = 1; off < 1024; off <<= 1) {  // Hillis-Steele inclusive scan of the partial sums
+    const int v = t >= off ? part[t - off] : 0;
     __syncthreads();
     part[t] += v;
     __syncthreads();
   }
   int run = part[t] - sum;
-  if (t == 1023) total_s = part[t];
   for (int64_t i = begin; i < end; ++i) {
-    int c = counts[i];
-    counts[i] = run;
+    const int c = mine[i];
+    mine[i] = run;
     run += c;
   }
+  if (t == 1023) nbsizes[blockIdx.x] = part[t];
+}
+
+// start[k] = first position of offset k's list: the sum of the earlier offsets' sizes, each
+// rounded up to a multiple of `quantum` entries first.
+__device__ __forceinline__ void pair_list_starts(const int32_t *nbsizes, int kvol, int quantum,
+                                                 int *start) {
+  for (int k = threadIdx.x; k < kvol; k += kBlock) start[k + 1] = nbsizes[k];
   __syncthreads();
-  for (int k = t; k < kvol; k += 1024) {
-    int start = counts[(int64_t)k * nblk];
-    int stop = k + 1 < kvol ? counts[(int64_t)(k + 1) * nblk] : total_s;
-    nbsizes[k] = stop - start;
+  if (threadIdx.x == 0) {
+    int run = 0;
+    for (int k = 0; k < kvol; ++k) {
+      const int c = start[k + 1];
+      start[k] = run;
+      run += (c + quantum - 1) / quantum * quantum;
+    }
+    start[kvol] = run;
+  }
+  __syncthreads();
+}
+
+// Rank of every entry of the staged chunk inside its (block, offset) run, by two ballot
+// passes around one barrier; `emit(k, value, row, position inside the offset's list)` is
+// called for every entry.
+template <typename Emit>
+__device__ __forceinline__ void pair_for_each(const int32_t *map, int64_t n_rows, int kvol,
+                                              int64_t nblk, const int32_t *offsets, int32_t *tile,
+                                              int (*wave_cnt)[kPairChunk], Emit emit) {
+  const int64_t row0 = (int64_t)blockIdx.x * kBlock;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  for (int k0 = 0; k0 < kvol; k0 += kPairChunk) {
+    const int kc = min(kPairChunk, kvol - k0);
+    __syncthreads();  // the previous chunk's tile and counts are no longer read
+    pair_stage_rows(map, row0, n_rows, kvol, k0, kc, tile);
+    __syncthreads();
+    int my = 0;
+    for (int j = 0; j < kc; ++j) {
+      const int c = __popcll(__ballot(tile[threadIdx.x * kPairStride + j] != -1));
+      if (lane == j) my = c;
+    }
+    if (lane < kc) wave_cnt[wave][lane] = my;
+    __syncthreads();
+    for (int j = 0; j < kc; ++j) {
+      const int32_t v = tile[threadIdx.x * kPairStride + j];
+      const unsigned long long b = __ballot(v != -1);
+      if (v == -1) continue;
+      int before = 0;
+      for (int w = 0; w < wave; ++w) before += wave_cnt[w][j];
+      const int in_list = offsets[(int64_t)(k0 + j) * nblk + blockIdx.x] + before +
+                          __popcll(b & ((1ULL << lane) - 1ULL));
+      emit(k0 + j, v, (int32_t)(row0 + threadIdx.x), in_list);
+    }
   }
 }
 
-__global__ void pair_fill_kernel(const int32_t *map, int64_t n_rows, int kvol, int64_t nblk,
-                                 const int32_t *offsets, int64_t nnz, int32_t *inter,
-                                 int32_t *planar, int64_t n_in, int64_t n_out, int32_t *input_mask,
-                                 int32_t *output_mask, int skip_k) {
-  __shared__ int wave_cnt[kBlock / 64];
-  int64_t row = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  for (int k = 0; k < kvol; ++k) {
-    int32_t in = row < n_rows ? map[row * kvol + k] : -1;
-    bool valid = in != -1;
-    unsigned long long b = __ballot(valid);
-    if (lane == 0) wave_cnt[wave] = __popcll(b);
-    __syncthreads();
-    int before = 0;
-    for (int w = 0; w < wave; ++w) before += wave_cnt[w];
-    if (valid) {
-      int rank = before + __popcll(b & ((1ULL << lane) - 1ULL));
-      int64_t pos = (int64_t)offsets[(int64_t)k * nblk + blockIdx.x] + rank;
-      if (pos < nnz) {
-        if (inter) {
-          inter[2 * pos] = in;
-          inter[2 * pos + 1] = (int32_t)row;
-        }
-        if (planar) {
-          planar[pos] = in;
-          planar[nnz + pos] = (int32_t)row;
-        }
-        if (k != skip_k) {
-          int32_t p = (int32_t)(pos - offsets[(int64_t)k * nblk]);
-          if (input_mask && in >= 0 && in < n_in) input_mask[(int64_t)k * n_in + in] = p;
-          if (output_mask && row < n_out) output_mask[(int64_t)k * n_out + row] = p;
-        }
-      }
-    }
-    __syncthreads();
-  }
+__global__ __launch_bounds__(kBlock) void pair_fill_kernel(
+    const int32_t *map, int64_t n_rows, int kvol, int64_t nblk, const int32_t *offsets,
+    const int32_t *nbsizes, int64_t nnz, int32_t *inter, int32_t *planar, int64_t n_in, int64_t n_out,
+    int32_t *input_mask, int32_t *output_mask, int skip_k) {
+  __shared__ int32_t tile[kBlock * kPairStride];
+  __shared__ int wave_cnt[kBlock / 64][kPairChunk];
+  __shared__ int start[kPairMaxKvol + 1];
+  pair_list_starts(nbsizes, kvol, 1, start);
+  pair_for_each(map, n_rows, kvol, nblk, offsets, tile, wave_cnt,
+                [&](int k, int32_t in, int32_t row, int in_list) {
+                  const int64_t pos = (int64_t)start[k] + in_list;
+                  if (pos >= nnz) return;
+                  if (inter) {
+                    inter[2 * pos] = in;
+                    inter[2 * pos + 1] = row;
+                  }
+                  if (planar) {
+                    planar[pos] = in;
+                    planar[nnz + pos] = row;
+                  }
+                  if (k != skip_k) {
+                    if (input_mask && in >= 0 && in < n_in) input_mask[(int64_t)k * n_in + in] = in_list;
+                    if (output_mask && row < n_out) output_mask[(int64_t)k * n_out + row] = in_list;
+                  }
+                });
 }
 
 // Pair lists for the weight gradient: offset k's pairs (map value, row), ordered by row,
 // start at entry seg_steps[k] * kWgradPairStep and are padded with (-1, -1) up to the next
 // multiple of kWgradPairStep, so that a block of kWgradPairStep consecutive entries never
-// mixes two offsets.  `offsets` is the exclusive scan of the per-(offset, block) counts.
-__global__ void wgrad_pair_fill_kernel(const int32_t *map, int64_t n_rows, int kvol, int64_t nblk,
-                                       const int32_t *offsets, const int32_t *nbsizes,
-                                       int32_t *pairs, int32_t *seg_steps) {
-  __shared__ int wave_cnt[kBlock / 64];
-  __shared__ int seg[kWgradMaxKvol + 1];
-  for (int k = threadIdx.x; k < kvol; k += kBlock) seg[k + 1] = nbsizes[k];
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    int run = 0;
-    for (int k = 0; k < kvol; ++k) {
-      const int c = seg[k + 1];
-      seg[k] = run;
-      run += (c + kWgradPairStep - 1) / kWgradPairStep;
-    }
-    seg[kvol] = run;
-  }
-  __syncthreads();
+// mixes two offsets.  `offsets` holds each block's first position inside its offset's list.
+__global__ __launch_bounds__(kBlock) void wgrad_pair_fill_kernel(
+    const int32_t *map, int64_t n_rows, int kvol, int64_t nblk, const int32_t *offsets,
+    const int32_t *nbsizes, int32_t *pairs, int32_t *seg_steps) {
+  __shared__ int32_t tile[kBlock * kPairStride];
+  __shared__ int wave_cnt[kBlock / 64][kPairChunk];
+  __shared__ int start[kPairMaxKvol + 1];
+  pair_list_starts(nbsizes, kvol, kWgradPairStep, start);
   if (blockIdx.x == 0) {
-    for (int k = threadIdx.x; k <= kvol; k += kBlock) seg_steps[k] = seg[k];
+    for (int k = threadIdx.x; k <= kvol; k += kBlock) seg_steps[k] = start[k] / kWgradPairStep;
     // the padding entries behind each list
     for (int k = 0; k < kvol; ++k) {
-      const int64_t end = (int64_t)seg[k] * kWgradPairStep + nbsizes[k];
-      const int64_t stop = (int64_t)seg[k + 1] * kWgradPairStep;
-      const int64_t pos = end + threadIdx.x;
-      if (pos < stop) {
+      const int64_t pos = (int64_t)start[k] + nbsizes[k] + threadIdx.x;
+      if (pos < start[k + 1]) {
         pairs[2 * pos] = -1;
         pairs[2 * pos + 1] = -1;
       }
     }
   }
-  int64_t row = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  for (int k = 0; k < kvol; ++k) {
-    int32_t v = row < n_rows ? map[row * kvol + k] : -1;
-    bool valid = v != -1;
-    unsigned long long b = __ballot(valid);
-    if (lane == 0) wave_cnt[wave] = __popcll(b);
-    __syncthreads();
-    int before = 0;
-    for (int w = 0; w < wave; ++w) before += wave_cnt[w];
-    if (valid) {
-      int rank = before + __popcll(b & ((1ULL << lane) - 1ULL));
-      int64_t pos = (int64_t)seg[k] * kWgradPairStep +
-                    (offsets[(int64_t)k * nblk + blockIdx.x] - offsets[(int64_t)k * nblk]) + rank;
-      pairs[2 * pos] = v;
-      pairs[2 * pos + 1] = (int32_t)row;
-    }
-    __syncthreads();
-  }
+  pair_for_each(map, n_rows, kvol, nblk, offsets, tile, wave_cnt,
+                [&](int k, int32_t v, int32_t row, int in_list) {
+                  const int64_t pos = (int64_t)start[k] + in_list;
+                  pairs[2 * pos] = v;
+                  pairs[2 * pos + 1] = row;
+                });
 }
 
 // Padded copy of existing interleaved pair lists (offset k's nbsizes[k] pairs follow each
@@ -781,7 +822,8 @@ extern "C" int tsmi_reduce_bitmask(tsmi_stream_t s, const int32_t *sorted_mask, 
 
 extern "C" int tsmi_pair_lists_count(tsmi_stream_t s, const int32_t *map, int64_t n_rows, int kvol,
                                      int32_t *block_counts, int32_t *nbsizes) {
-  TSMI_REQUIRE(kvol >= 1 && n_rows >= 0 && nbsizes, "pair_lists_count: bad arguments");
+  TSMI_REQUIRE(kvol >= 1 && kvol <= kPairMaxKvol && n_rows >= 0 && nbsizes,
+               "pair_lists_count: bad arguments (kernel volume %d, at most %d)", kvol, kPairMaxKvol);
   int64_t nblk = ceil_div(n_rows, kBlock);
   if (n_rows == 0) {
     hipLaunchKernelGGL(fill_kernel<int32_t>, grid_for(kvol), dim3(kBlock), 0, (hipStream_t)s,
@@ -792,16 +834,16 @@ extern "C" int tsmi_pair_lists_count(tsmi_stream_t s, const int32_t *map, int64_
   TSMI_REQUIRE(grid_fits(nblk), "pair_lists_count: too many rows");
   hipLaunchKernelGGL(pair_count_kernel, dim3((unsigned)nblk), dim3(kBlock), 0, (hipStream_t)s, map,
                      n_rows, kvol, nblk, block_counts);
-  hipLaunchKernelGGL(pair_scan_kernel, dim3(1), dim3(1024), 0, (hipStream_t)s, block_counts,
-                     nblk * kvol, kvol, nblk, nbsizes);
+  hipLaunchKernelGGL(pair_scan_kernel, dim3(kvol), dim3(1024), 0, (hipStream_t)s, block_counts, kvol,
+                     nblk, nbsizes);
   return check_launch("tsmi_pair_lists_count");
 }
 
 extern "C" int tsmi_pair_lists_fill(tsmi_stream_t s, const int32_t *map, int64_t n_rows, int kvol,
-                                    int32_t *block_counts, int64_t nnz, int32_t *nbmaps_inter,
-                                    int32_t *nbmaps_planar, int64_t n_in, int64_t n_out,
-                                    int32_t *input_mask, int32_t *output_mask) {
-  TSMI_REQUIRE(kvol >= 1 && n_rows >= 0 && nnz >= 0 && n_in >= 0 && n_out >= 0,
+                                    int32_t *block_counts, const int32_t *nbsizes, int64_t nnz,
+                                    int32_t *nbmaps_inter, int32_t *nbmaps_planar, int64_t n_in,
+                                    int64_t n_out, int32_t *input_mask, int32_t *output_mask) {
+  TSMI_REQUIRE(kvol >= 1 && kvol <= kPairMaxKvol && n_rows >= 0 && nnz >= 0 && n_in >= 0 && n_out >= 0,
                "pair_lists_fill: bad sizes");
   if (input_mask && n_in > 0) {
     TSMI_GRID_CHECK(n_in * kvol);
@@ -814,13 +856,13 @@ extern "C" int tsmi_pair_lists_fill(tsmi_stream_t s, const int32_t *map, int64_t
                        (hipStream_t)s, output_mask, n_out * kvol, -1);
   }
   if (n_rows > 0 && nnz > 0) {
-    TSMI_REQUIRE(map && block_counts, "pair_lists_fill: null pointer");
+    TSMI_REQUIRE(map && block_counts && nbsizes, "pair_lists_fill: null pointer");
     int64_t nblk = ceil_div(n_rows, kBlock);
     TSMI_REQUIRE(grid_fits(nblk), "pair_lists_fill: too many rows");
     int skip_k = (n_in == n_out && kvol % 2 == 1) ? kvol / 2 : -1;
     hipLaunchKernelGGL(pair_fill_kernel, dim3((unsigned)nblk), dim3(kBlock), 0, (hipStream_t)s,
-                       map, n_rows, kvol, nblk, block_counts, nnz, nbmaps_inter, nbmaps_planar,
-                       n_in, n_out, input_mask, output_mask, skip_k);
+                       map, n_rows, kvol, nblk, block_counts, nbsizes, nnz, nbmaps_inter,
+                       nbmaps_planar, n_in, n_out, input_mask, output_mask, skip_k);
   }
   return check_launch("tsmi_pair_lists_fill");
 }
