@@ -273,23 +273,6 @@ __global__ void transpose_map_kernel(const int32_t *map, int64_t total, int kvol
   map_t[(int64_t)in * kvol + k] = (int32_t)out;
 }
 
-__global__ void derive_bitmask_kernel(const int32_t *map, int64_t n_pad, int kvol, int split,
-                                      int len, int64_t valid_n, int32_t *bitmask) {
-  int64_t tid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (tid >= n_pad * split) return;
-  int s = (int)(tid / n_pad);
-  int64_t r = tid - (int64_t)s * n_pad;
-  int32_t result = -1;
-  if (r < valid_n) {
-    int begin = s * len;
-    int l = min(len, kvol - begin);
-    uint32_t m = 0;
-    const int32_t *row = map + r * kvol + begin;
-    for (int i = 0; i < l; ++i) m |= (uint32_t)(row[i] >= 0) << i;
-    result = (int32_t)m;
-  }
-  bitmask[tid] = result;
-}
 
 __global__ void reorder_map_kernel(const int32_t *map, const int32_t *loc, int64_t n_pad, int kvol,
                                    int len, int32_t *out) {
@@ -337,6 +320,28 @@ __device__ __forceinline__ void pair_stage_rows(const int32_t *map, int64_t row0
     const int64_t row = row0 + r;
     tile[r * kPairStride + j] = row < n_rows ? map[row * kvol + k0 + j] : -1;
   }
+}
+
+// bitmask[s][r] bit i = row r has an entry at offset s*len + i (-1 for rows >= valid_n).  A
+// block stages the split's offsets of its 256 rows through LDS like the pair-list kernels.
+__global__ __launch_bounds__(kBlock) void derive_bitmask_kernel(const int32_t *map, int64_t n_pad,
+                                                                int kvol, int split, int len,
+                                                                int64_t valid_n, int32_t *bitmask) {
+  __shared__ int32_t tile[kBlock * kPairStride];
+  const int s = blockIdx.y;
+  const int64_t row0 = (int64_t)blockIdx.x * kBlock, r = row0 + threadIdx.x;
+  const int begin = s * len;
+  const int l = min(len, kvol - begin);
+  pair_stage_rows(map, row0, valid_n, kvol, begin, l, tile);
+  __syncthreads();
+  if (r >= n_pad) return;
+  int32_t result = -1;
+  if (r < valid_n) {
+    uint32_t m = 0;
+    for (int i = 0; i < l; ++i) m |= (uint32_t)(tile[threadIdx.x * kPairStride + i] >= 0) << i;
+    result = (int32_t)m;
+  }
+  bitmask[(int64_t)s * n_pad + r] = result;
 }
 
 __global__ __launch_bounds__(kBlock) void pair_count_kernel(const int32_t *map, int64_t n_rows,
@@ -787,9 +792,9 @@ extern "C" int tsmi_derive_bitmask(tsmi_stream_t s, const int32_t *map, int64_t 
   int64_t total = n_pad * split;
   if (total == 0) return TSMI_OK;
   TSMI_REQUIRE(map && bitmask, "derive_bitmask: null pointer");
-  TSMI_GRID_CHECK(total);
-  hipLaunchKernelGGL(derive_bitmask_kernel, grid_for(total), dim3(kBlock), 0, (hipStream_t)s, map,
-                     n_pad, kvol, split, len, valid_n, bitmask);
+  TSMI_GRID_CHECK(n_pad);
+  hipLaunchKernelGGL(derive_bitmask_kernel, dim3(grid_for(n_pad).x, split), dim3(kBlock), 0,
+                     (hipStream_t)s, map, n_pad, kvol, split, len, valid_n, bitmask);
   return check_launch("tsmi_derive_bitmask");
 }
 
