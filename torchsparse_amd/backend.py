@@ -517,6 +517,11 @@ def conv_forward_implicit_gemm_cuda(in_feats, kernel, out_in_map, num_out_feats,
     x, wp, (kvol, cin, cout) = _conv_common(in_feats, kernel)
     if cout != num_out_channels:
         raise ValueError("num_out_channels does not match the kernel")
+    return _implicit_gemm(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias, residual, relu)
+
+
+def _implicit_gemm(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias=None, residual=None,
+                   relu=False) -> torch.Tensor:
     y = torch.empty((num_out_feats, cout), dtype=x.dtype, device=x.device)
     code = _dtype_code(x)
     ws, ws_elems = None, 0
@@ -531,6 +536,25 @@ def conv_forward_implicit_gemm_cuda(in_feats, kernel, out_in_map, num_out_feats,
                                       _ptr(_tile_counters(x.device)) if ws is not None else None,
                                       _N_TILE_COUNTERS, _ptr(y)))
     return y
+
+
+def conv_dgrad_implicit_gemm_cuda(grad_out, kernel, in_out_map, num_in_feats) -> torch.Tensor:
+    """Input gradient dX[m] = sum_k dY[map[m, k]] W[k]^T: the forward kernel over the
+    (input row, offset) -> output row map with the weights transposed per offset
+    (the reference's func/implicit_gemm.py:124-141).  The packed layout of W[k]^T is
+    [Cin padded, Cout padded] row-major, which is W[k] itself when neither channel count
+    needs padding: then the kernel tensor is passed as it is."""
+    w = kernel if kernel.dim() == 3 else kernel.unsqueeze(0)
+    kvol, cin, cout = w.shape
+    if w.is_contiguous() and _C.tsmi_packed_weight_elems(kvol, cout, cin) == w.numel():
+        if grad_out.dtype != w.dtype:
+            raise ValueError(f"feature dtype {grad_out.dtype} and kernel dtype {w.dtype} differ")
+        if grad_out.shape[1] != cout:
+            raise ValueError("Input feature size and kernel size mismatch")
+        dy = grad_out if grad_out.is_contiguous() else grad_out.contiguous()
+        return _implicit_gemm(dy, w.detach(), kvol, cout, cin, in_out_map, num_in_feats)
+    return conv_forward_implicit_gemm_cuda(grad_out, w.transpose(1, 2).contiguous(), in_out_map,
+                                           num_in_feats, cin)
 
 
 def conv_forward_implicit_gemm_sorted_cuda(in_feats, kernel, reorder_out_in_map, reduced_mask,

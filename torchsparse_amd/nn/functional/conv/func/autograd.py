@@ -69,8 +69,8 @@ class SparseConvFunction(torch.autograd.Function):
         n_in = sizes[1] if transposed else sizes[0]
         grad_input = grad_weight = None
         if ctx.needs_input_grad[0]:
-            grad_input = backend.conv_forward_implicit_gemm_cuda(
-                dy, w.transpose(1, 2).contiguous(), backward_map(kmap, transposed), n_in, w.shape[1])
+            grad_input = backend.conv_dgrad_implicit_gemm_cuda(
+                dy, w, backward_map(kmap, transposed), n_in)
             if grad_input.dtype != input.dtype:
                 grad_input = grad_input.to(input.dtype)
         if ctx.needs_input_grad[1]:
