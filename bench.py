@@ -342,11 +342,12 @@ def cpu_baseline(records, level_coords):
     """The oracle's CPU convolution (gather -> GEMM -> scatter, fp32, threads over rows)
     and kernel-map builders over the network's sparse conv layers and maps, once."""
     import oracle
-    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    cores = oracle.set_threads(int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
     rng = np.random.default_rng(0)
     t_map = t_conv = t_ref = t_conv_same = 0.0
     pair_cache = {}
     n_layers = n_ref_layers = 0
+    timed_layers = []
     ref_budget_s = 15.0  # the compiled reference convolution is slow: stop timing it after this
     ref = oracle.ref_module()  # the reference's own CPU convolution, compiled in place
     for r in records:
@@ -372,6 +373,7 @@ def cpu_baseline(records, level_coords):
         oracle.conv_gather_scatter(x, w, nb, sz, r["n_out"], transpose=transposed, variant=1)
         dt = time.perf_counter() - t0
         t_conv += dt
+        timed_layers.append((dict(r, key=key), dt))
         if ref is not None and t_ref < ref_budget_s:
             n_y = r["n_out"]
             y = torch.zeros(n_y, r["cout"])
@@ -390,7 +392,37 @@ def cpu_baseline(records, level_coords):
                                    f"after {ref_budget_s:.0f} s), torch threads = "
                                    f"{torch.get_num_threads()}; the port takes "
                                    f"{t_conv_same * 1e3:.0f} ms on those layers"}
+    # the same convolutions with the reference's own threading (a parallel region per row over
+    # the channel loop) and on one thread, each on a bounded prefix of the layers
+    for name, variant, threads in (("faithful_threading", 0, cores), ("one_thread", 1, 1)):
+        oracle.set_threads(threads)
+        t_v = t_same = 0.0
+        n_v = 0
+        for r, dt in timed_layers:
+            if t_v > 5.0:
+                break
+            nb, sz = pair_cache[r["key"]]
+            x = rng.standard_normal((r["n_in"], r["cin"])).astype(np.float32)
+            w = rng.standard_normal((len(sz), r["cin"], r["cout"])).astype(np.float32)
+            t0 = time.perf_counter()
+            oracle.conv_gather_scatter(x, w, nb, sz, r["n_out"], transpose=r["transposed"], variant=variant)
+            t_v += time.perf_counter() - t0
+            t_same += dt
+            n_v += 1
+        extra[name] = {"conv_ms": round(t_v * 1e3, 1), "layers": n_v, "threads": threads,
+                       "row_parallel_ms_same_layers": round(t_same * 1e3, 1)}
+    oracle.set_threads(cores)
+    model = ""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
     return {**extra, "value": round((t_map + t_conv) * 1e3, 1), "unit": "ms", "cores": cores, "kind": "port",
+            "cpu_model": model, "host_cpus": os.cpu_count(),
             "sample": f"{n_layers} sparse conv layers (fp32) + {len(pair_cache)} kernel maps of one "
                       f"MinkUNet forward on the same scan; BN/ReLU/concat/1x1x1 layers excluded; "
                       f"maps {t_map * 1e3:.0f} ms, convs {t_conv * 1e3:.0f} ms",

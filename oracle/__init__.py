@@ -302,6 +302,11 @@ def conv_implicit_gemm(x, w, out_in_map, n_out):
     return y
 
 
+def set_threads(n: int = 0) -> int:
+    """Set (n > 0) and return the OpenMP thread count of the C restatement; timing only."""
+    return int(lib().tso_set_threads(int(n)))
+
+
 def conv_gather_scatter(x, w, nbmaps, nbsizes, n_out, transpose=False, variant=1):
     x, w, nbmaps, nbsizes = _f32(x), _f32(w), _i32(nbmaps), _i32(nbsizes)
     kvol, cin, cout = w.shape

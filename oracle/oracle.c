@@ -19,8 +19,24 @@
 #include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
 
 #define TSO_EXPORT __attribute__((visibility("default")))
+
+/* Thread count of the parallel loops below (timing only; results do not depend on it).
+ * Returns the count now in force. */
+TSO_EXPORT int tso_set_threads(int n) {
+#ifdef _OPENMP
+  if (n > 0) omp_set_num_threads(n);
+  return omp_get_max_threads();
+#else
+  (void)n;
+  return 1;
+#endif
+}
 
 /* ------------------------------------------------------------------ helpers */
 
