@@ -276,3 +276,52 @@ def test_autograd_through_transposed_conv_and_relu_residual(mods):
     assert rel_rms(_f32(up.kernel.grad), dw_up) < 1e-4
     assert rel_rms(_f32(down.kernel.grad), dw_down) < 1e-4
     assert rel_rms(_f32(x.grad), dx) < 1e-4
+
+
+@pytest.mark.parametrize("geom", [(3, 1, 1), (2, 2, 0), (3, 2, 1)])
+@pytest.mark.parametrize("splits", [(1, 1), (3, 2)])
+@pytest.mark.parametrize("cin,cout", [(16, 24), (32, 64)])
+def test_sorted_configuration_runs_the_input_gradient_over_sorted_products(mods, geom, splits, cin, cout,
+                                                                           monkeypatch):
+    """ifsort: the input gradient goes through the mask-sorted transposed map (both the packed
+    and the as-stored weight forms) and equals the oracle's; a transposed convolution uses
+    the strided map's forward sort products."""
+    ts, backend, spnn, F = mods
+    k, s, pad = geom
+    calls = []
+    real = backend.conv_dgrad_implicit_gemm_sorted_cuda
+    monkeypatch.setattr(backend, "conv_dgrad_implicit_gemm_sorted_cuda",
+                        lambda *a, **kw: (calls.append(a[2].shape), real(*a, **kw))[1])
+    rng = np.random.default_rng(k * 7 + s)
+    coords = random_coords(rng, 1500, (18, 14, 12))
+    n = len(coords)
+    cfg = F.conv_config.get_default_conv_config()
+    cfg.ifsort, cfg.split_mask_num, cfg.split_mask_num_bwd = True, splits[0], splits[1]
+    torch.manual_seed(k)
+    layer = spnn.Conv3d(cin, cout, k, stride=s, padding=pad).cuda()
+    x = torch.from_numpy(rng.standard_normal((n, cin)).astype(np.float32)).cuda().requires_grad_(True)
+    out = F.conv3d(ts.SparseTensor(x, dev(coords)), layer.kernel, kernel_size=k, stride=s, padding=pad,
+                   config=cfg, training=True)
+    g = torch.from_numpy(rng.standard_normal(tuple(out.feats.shape)).astype(np.float32)).cuda()
+    if s == 1:
+        omap = oracle.kmap_subm(coords, k)
+        (out.feats * g).sum().backward()
+        want_dx, want_dw = oracle.conv_backward_implicit_gemm(_f32(x), _f32(layer.kernel), omap, _f32(g))
+        assert len(calls) == 1
+    else:
+        # strided convolution followed by its transposed twin on the same (sorted) map
+        up = spnn.Conv3d(cout, cin, k, stride=s, transposed=True).cuda()
+        back = F.conv3d(out, up.kernel, kernel_size=k, stride=s, padding=pad, transposed=True, config=cfg,
+                        training=True)
+        g = torch.from_numpy(rng.standard_normal((n, cin)).astype(np.float32)).cuda()
+        (back.feats * g).sum().backward()
+        omap, ocoords = oracle.kmap_downsample(coords, k, s, pad)
+        n_mid = len(ocoords)
+        mid = oracle.conv_implicit_gemm(_f32(x), _f32(layer.kernel), omap, n_mid)
+        tmap = oracle.transpose_map(omap[:n_mid], n)
+        dmid, dw_up = oracle.conv_backward_implicit_gemm(mid, _f32(up.kernel), tmap, _f32(g))
+        want_dx, want_dw = oracle.conv_backward_implicit_gemm(_f32(x), _f32(layer.kernel), omap, dmid)
+        assert rel_rms(_f32(up.kernel.grad), dw_up) < 1e-4
+        assert len(calls) == 2
+    assert rel_rms(_f32(x.grad), want_dx) < 1e-4
+    assert rel_rms(_f32(layer.kernel.grad), want_dw) < 1e-4

@@ -563,6 +563,12 @@ def conv_forward_implicit_gemm_sorted_cuda(in_feats, kernel, reorder_out_in_map,
                                            residual=None, relu=False) -> torch.Tensor:
     """convolution/convolution_forward_implicit_gemm_sorted_cuda.cu:1755-2230."""
     x, wp, (kvol, cin, cout) = _conv_common(in_feats, kernel)
+    return _implicit_gemm_sorted(x, wp, kvol, cin, cout, reorder_out_in_map, reduced_mask, reorder_loc,
+                                 num_out_feats, bias, residual, relu)
+
+
+def _implicit_gemm_sorted(x, wp, kvol, cin, cout, reorder_out_in_map, reduced_mask, reorder_loc,
+                          num_out_feats, bias=None, residual=None, relu=False) -> torch.Tensor:
     split = reorder_loc.shape[0]
     n_pad = reorder_out_in_map.shape[0]
     y = torch.empty((num_out_feats, cout), dtype=x.dtype, device=x.device)
@@ -577,9 +583,28 @@ def conv_forward_implicit_gemm_sorted_cuda(in_feats, kernel, reorder_out_in_map,
                                              _ptr(reduced_mask), _ptr(reorder_loc), n_pad,
                                              num_out_feats, kvol, split, cin, cout, code,
                                              pb, pr, int(relu), _ptr(ws), ws_elems,
-                                      _ptr(_tile_counters(x.device)) if ws is not None else None,
-                                      _N_TILE_COUNTERS, _ptr(y)))
+                                             _ptr(_tile_counters(x.device)) if ws is not None else None,
+                                             _N_TILE_COUNTERS, _ptr(y)))
     return y
+
+
+def conv_dgrad_implicit_gemm_sorted_cuda(grad_out, kernel, reorder_in_out_map, reduced_mask,
+                                         reorder_loc, num_in_feats) -> torch.Tensor:
+    """conv_dgrad_implicit_gemm_cuda over the mask-sorted (input row, offset) -> output row map:
+    the input gradient of the reference's sorted branch (func/implicit_gemm.py:130-141)."""
+    w = kernel if kernel.dim() == 3 else kernel.unsqueeze(0)
+    kvol, cin, cout = w.shape
+    if w.is_contiguous() and _C.tsmi_packed_weight_elems(kvol, cout, cin) == w.numel():
+        if grad_out.dtype != w.dtype:
+            raise ValueError(f"feature dtype {grad_out.dtype} and kernel dtype {w.dtype} differ")
+        if grad_out.shape[1] != cout:
+            raise ValueError("Input feature size and kernel size mismatch")
+        dy = grad_out if grad_out.is_contiguous() else grad_out.contiguous()
+        return _implicit_gemm_sorted(dy, w.detach(), kvol, cout, cin, reorder_in_out_map, reduced_mask,
+                                     reorder_loc, num_in_feats)
+    return conv_forward_implicit_gemm_sorted_cuda(grad_out, w.transpose(1, 2).contiguous(),
+                                                  reorder_in_out_map, reduced_mask, reorder_loc,
+                                                  num_in_feats, cin)
 
 
 def conv_backward_wgrad_implicit_gemm_cuda(grad_out: torch.Tensor, in_feats: torch.Tensor,

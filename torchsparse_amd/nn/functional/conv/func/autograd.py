@@ -4,7 +4,9 @@
     dW[k]  += X[m]^T dY[i]          for every map entry  map[i, k] = m >= 0
 
 The input gradient is the forward implicit-GEMM kernel over the transposed map with
-the weights transposed per offset.  The weight gradient runs over per-offset pair lists
+the weights transposed per offset; a sorted configuration (``ifsort``) whose map carries
+the backward sort products runs it over the mask-sorted transposed map, as the
+reference's sorted branch does.  The weight gradient runs over per-offset pair lists
 derived from the map (tsmi_conv_wgrad_pairs: only rows that take part in an offset are
 read); channel counts that are not a multiple of 16 bytes use the map form
 (tsmi_conv_wgrad).  Both follow the reference's func/implicit_gemm.py:108-190 (unsorted
@@ -18,7 +20,7 @@ import torch
 from torchsparse_amd import backend
 from torchsparse_amd.utils import make_divisible
 
-__all__ = ["SparseConvFunction", "backward_map", "wgrad_pairs"]
+__all__ = ["SparseConvFunction", "backward_map", "backward_sort_products", "wgrad_pairs"]
 
 
 def backward_map(kmap: Dict, transposed: bool) -> torch.Tensor:
@@ -37,6 +39,17 @@ def backward_map(kmap: Dict, transposed: bool) -> torch.Tensor:
     return kmap["out_in_map_bwd"]
 
 
+def backward_sort_products(kmap: Dict, transposed: bool):
+    """(mask-sorted backward map, its reduced masks for 128-row tiles, row order) when the map
+    was built with them, else None.  A plain convolution's are the ``*_bwd`` products of a
+    training-time sorted map (build_kmap.py:195-220); a transposed convolution runs its
+    input gradient over the strided map itself, whose products are the forward ones."""
+    names = (("reorder_out_in_map", "reduced_sorted_mask", "reorder_loc") if transposed else
+             ("reorder_out_in_map_bwd", "reduced_sorted_mask_bwd_dgrad", "reorder_loc_bwd"))
+    products = tuple(kmap.get(n) for n in names)
+    return None if any(p is None for p in products) else products
+
+
 def wgrad_pairs(kmap: Dict) -> Dict:
     """Per-offset (input row, output row) pair lists of the strided / submanifold map, built
     once per map and shared by every convolution (transposed ones included) that uses it."""
@@ -52,6 +65,7 @@ class SparseConvFunction(torch.autograd.Function):
         out = forward_impl(input, weight, kmap, config, transposed, None, None, False)
         ctx.save_for_backward(input, weight)
         ctx.kmap, ctx.transposed = kmap, transposed
+        ctx.ifsort = bool(config.get("ifsort", False)) if config is not None else False
         return out
 
     @staticmethod
@@ -69,8 +83,12 @@ class SparseConvFunction(torch.autograd.Function):
         n_in = sizes[1] if transposed else sizes[0]
         grad_input = grad_weight = None
         if ctx.needs_input_grad[0]:
-            grad_input = backend.conv_dgrad_implicit_gemm_cuda(
-                dy, w, backward_map(kmap, transposed), n_in)
+            products = backward_sort_products(kmap, transposed) if ctx.ifsort else None
+            if products is not None:
+                grad_input = backend.conv_dgrad_implicit_gemm_sorted_cuda(dy, w, *products, n_in)
+            else:
+                grad_input = backend.conv_dgrad_implicit_gemm_cuda(
+                    dy, w, backward_map(kmap, transposed), n_in)
             if grad_input.dtype != input.dtype:
                 grad_input = grad_input.to(input.dtype)
         if ctx.needs_input_grad[1]:

@@ -61,8 +61,9 @@ def _sort_products(kmap: Dict, out_in_map: torch.Tensor, valid_n: int, split_mas
 def _backward_products(kmap: Dict, ifsort: bool, split_mask_num_bwd: int) -> None:
     """Training-time products (build_kmap.py:191-220): the transposed map the input gradient
     runs over and, for sorted mode, its sort products with the reference's two reduce tiles
-    (64 rows for the weight gradient, 128 for the input gradient).  The backward here runs
-    unsorted, so the sort products are built only when ``ifsort`` asks for them."""
+    (64 rows for the weight gradient, 128 for the input gradient).  The input gradient of a
+    sorted configuration runs over them; the weight gradient works from pair lists and
+    needs none."""
     n_in, n_out = kmap["sizes"]
     bwd = backend.convert_transposed_out_in_map(kmap["out_in_map"], make_divisible(n_in, cta_M), n_out)
     kmap["out_in_map_bwd"] = bwd
