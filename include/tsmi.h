@@ -90,6 +90,16 @@ int tsmi_kmap_query(tsmi_stream_t s, const int64_t *keys, const int32_t *vals, i
                     const int32_t ks[3], const int32_t stride[3], const int32_t pad[3],
                     int32_t *out_in_map);
 
+/* The same map for the submanifold case of an odd kernel (every ks[a] odd, stride 1,
+ * pad = (ks-1)/2) when `coords` are the table's own rows (row i inserted with value i, as
+ * tsmi_hashtable_insert_coords does): map[i,k] = j <=> map[j,K_vol-1-k] = i, so half of the
+ * offsets are probed and each hit is stored twice.  Fills the map with -1 first (n_pad
+ * rows).  Identical output to tsmi_kmap_query for coordinates without duplicates
+ * (others/sparsemapping_cuda.cu:144-231 probes all K_vol offsets). */
+int tsmi_kmap_query_subm(tsmi_stream_t s, const int64_t *keys, const int32_t *vals, int64_t cap,
+                         const int32_t *coords, int64_t n, int64_t n_pad, const int32_t ks[3],
+                         int32_t *out_in_map);
+
 /* Per-column maximum of non-negative coords -> out_max int32[4] (device).  n may be 0 (result 0).
  * clear_first = 0 when out_max already holds zeros (saves the fill launch).
  * Replaces coords.max(0).values (hashmap_on_the_fly.py:33). */

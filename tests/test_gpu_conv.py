@@ -74,6 +74,32 @@ def test_implicit_gemm_ragged_row_counts(mods, n):
     assert rel_rms(_f32(y), want) < 1e-2
 
 
+@pytest.mark.parametrize("cin,cout", [(1, 16), (3, 20), (4, 32), (5, 16), (8, 64), (8, 8), (6, 48), (4, 96)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("n,ks", [(1, 3), (127, 3), (129, 3), (3000, 3), (900, 2), (700, (3, 1, 3)), (500, 5)])
+def test_few_input_channels_all_row_counts_and_kernels(mods, cin, cout, dtype, n, ks):
+    """Layers of at most 8 input channels (16-bit types, up to 64 output channels, kernel
+    volumes up to 64) run the densely packed kernel; wider outputs and 5^3 kernels the general
+    one.  Bias, residual and ReLU included; compared with the oracle and, for the epilogue,
+    with the same sums formed by torch."""
+    _, backend, _, F = mods
+    rng = np.random.default_rng(cin * 100 + cout + n)
+    coords = random_coords(rng, n, (20, 18, 12))
+    stride = 1
+    kmap = F.build_kernel_map(dev(coords), n, ks, stride, 0, mode="hashmap_on_the_fly")
+    omap = kmap["out_in_map"]
+    x, w = _case(rng, n, cin, cout, omap.shape[1], dtype)
+    y = backend.conv_forward_implicit_gemm_cuda(x, w, omap, n, cout)
+    want = oracle.conv_implicit_gemm(_f32(x), _f32(w), omap.cpu().numpy(), n)
+    assert y.shape == (n, cout) and y.dtype == dtype
+    assert rel_rms(_f32(y), want) < TOL[dtype]
+    bias = torch.from_numpy(rng.standard_normal(cout).astype(np.float32)).to("cuda", dtype)
+    res = torch.from_numpy(rng.standard_normal((n, cout)).astype(np.float32)).to("cuda", dtype)
+    y2 = backend.conv_forward_implicit_gemm_cuda(x, w, omap, n, cout, bias=bias, residual=res, relu=True)
+    want2 = np.maximum(want + _f32(bias) + _f32(res), 0)
+    assert rel_rms(_f32(y2), want2) < TOL[dtype]
+
+
 @pytest.mark.parametrize("geom", [(3, 1, 1), (2, 2, 0), (3, 2, 1), (5, 1, 2), (2, 1, 0)])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 def test_all_dataflows_agree_with_oracle(mods, geom, dtype):
@@ -285,6 +311,38 @@ def test_fuse_inference_matches_unfused_unet(mods):
         # and in half precision, against the fp32 network
         got16 = copy.deepcopy(fused).half()(ts.SparseTensor(x.half(), coords))
         assert rel_rms(_f32(got16[-1].feats), _f32(ref[-1].feats)) < 3e-2
+
+
+def test_fuse_inference_matches_unfused_detection_backbone(mods):
+    """The detection backbone's basic blocks (two biased convolutions, identity shortcut)
+    fold the same way: every stage output of the fused network equals the unfused one's."""
+    ts, _, _, F = mods
+    from torchsparse_amd.backbones import VoxelResBackBone8x
+    from torchsparse_amd.backbones.detection import SparseBasicBlock
+    from torchsparse_amd.nn.utils import fuse_inference
+    import copy
+    torch.manual_seed(2)
+    rng = np.random.default_rng(12)
+    coords = dev(random_coords(rng, 7000, (33, 48, 48)))
+    x = torch.randn(7000, 5, device="cuda")
+    model = VoxelResBackBone8x(in_channels=5).cuda().eval()
+    for m in model.modules():
+        if isinstance(m, torch.nn.BatchNorm1d):
+            m.running_mean.normal_(0, 0.3)
+            m.running_var.uniform_(0.5, 1.5)
+            m.weight.data.uniform_(0.5, 1.5)
+            m.bias.data.normal_(0, 0.2)
+    fused = fuse_inference(copy.deepcopy(model))
+    blocks = [m for m in fused.modules() if isinstance(m, SparseBasicBlock)]
+    assert len(blocks) == 8 and all(b._fused_tail for b in blocks)
+    assert not any(isinstance(m, torch.nn.BatchNorm1d) for m in fused.modules())
+    with torch.no_grad():
+        ref = model(ts.SparseTensor(x, coords, spatial_range=(1, 33, 48, 48)))
+        got = fused(ts.SparseTensor(x, coords, spatial_range=(1, 33, 48, 48)))
+    assert set(ref) == set(got)
+    for name in ref:
+        assert torch.equal(ref[name].coords, got[name].coords), name
+        assert rel_rms(_f32(got[name].feats), _f32(ref[name].feats)) < 1e-3, name
 
 
 @pytest.mark.parametrize("cin,cout", [(64, 64), (128, 128), (96, 160), (256, 256)])

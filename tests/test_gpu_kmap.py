@@ -228,3 +228,36 @@ def test_medium_scan_maps_and_invariants():
     want_map, want_coords = oracle.kmap_downsample(coords, 3, 2, 1)
     np.testing.assert_array_equal(k3["coords"].cpu().numpy(), want_coords)
     np.testing.assert_array_equal(k3["out_in_map"].cpu().numpy(), want_map)
+
+
+@pytest.mark.parametrize("ks", [(3, 3, 3), (5, 5, 5), (3, 1, 1), (1, 3, 5), (1, 1, 1)])
+@pytest.mark.parametrize("n,shape", [(0, (4, 4, 4)), (1, (4, 4, 4)), (129, (6, 6, 5)), (5000, (30, 28, 12))])
+def test_mirrored_subm_query_equals_the_full_query(ks, n, shape):
+    """tsmi_kmap_query_subm (half of the offsets probed, hits stored twice) against
+    tsmi_kmap_query (every offset probed): identical maps, pad rows included; coordinates at the
+    edge of the packable range (negative ones too) and several batches."""
+    rng = np.random.default_rng(sum(ks) + n)
+    coords = random_coords(rng, n, shape, batch=2) if n else np.zeros((0, 4), np.int32)
+    if n > 100:
+        coords = coords.copy()
+        coords[: n // 2, 1:] -= np.array(shape, np.int32) // 2          # negative coordinates
+        coords[:8, 1] = (1 << 17) - 1 - np.arange(8)                    # largest packable x
+        coords[8:16, 3] = -(1 << 17) + np.arange(8)                     # smallest packable z
+        coords = np.unique(coords, axis=0)
+    table = backend.GPUHashTable(backend.hash_capacity(max(len(coords), 1), 2), device="cuda")
+    c = dev(coords)
+    table.insert_bxyz(c)
+    pad = tuple((k - 1) // 2 for k in ks)
+    full = table.query_bxyz(c, ks, (1, 1, 1), pad)
+    mirrored = table.query_subm_bxyz(c, ks)
+    assert mirrored.shape == full.shape and mirrored.dtype == torch.int32
+    assert torch.equal(mirrored, full)
+    if len(coords):
+        shifted = coords.copy()  # the map does not change under translation; the oracle ravels from 0
+        shifted[:, 1:] -= coords[:, 1:].min(0)
+        want = oracle.kmap_subm(shifted, ks)
+        np.testing.assert_array_equal(mirrored.cpu().numpy()[:len(coords)], want[:len(coords)])
+    with pytest.raises(ValueError):
+        backend._check(backend._C.tsmi_kmap_query_subm(
+            None, backend._ptr(table.keys), backend._ptr(table.vals), table.capacity, backend._ptr(c),
+            len(coords), len(coords), backend._I3(2, 3, 3), backend._ptr(full)))

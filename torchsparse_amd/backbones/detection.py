@@ -24,6 +24,10 @@ class SparseBasicBlock(nn.Module):
         self.bn2 = spnn.BatchNorm(channels, eps=1e-3, momentum=0.01)
 
     def forward(self, x: SparseTensor) -> SparseTensor:
+        if getattr(self, "_fused_tail", False):
+            # after nn.utils.fuse_inference(): norms folded into the convolutions, ReLU and
+            # the shortcut add in their epilogues
+            return self.conv2(self.conv1(x), residual=x.feats)
         out = self.bn2(self.conv2(self.relu(self.bn1(self.conv1(x)))))
         return self.relu(out + x)
 

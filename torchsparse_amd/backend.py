@@ -50,6 +50,7 @@ def _load():
         "tsmi_hashtable_insert_keys": [_vp, _vp, _vp, _i64, _vp, _i64, _vp],
         "tsmi_hashtable_lookup_keys": [_vp, _vp, _vp, _i64, _vp, _i64, _vp],
         "tsmi_kmap_query": [_vp, _vp, _vp, _i64, _vp, _i64, _i64, _I3, _I3, _I3, _vp],
+        "tsmi_kmap_query_subm": [_vp, _vp, _vp, _i64, _vp, _i64, _i64, _I3, _vp],
         "tsmi_coords_max": [_vp, _vp, _i64, _vp, _i32],
         "tsmi_downsample_candidates": [_vp, _vp, _i64, _I3, _I3, _I3, _vp, _vp, _vp, _i32, _vp, _i64, _vp],
         "tsmi_hashtable_compact_keys": [_vp, _vp, _i64, _vp, _vp],
@@ -187,6 +188,21 @@ class GPUHashTable:
         _check(_C.tsmi_hashtable_insert_coords(_stream(), _ptr(self.keys), _ptr(self.vals),
                                                self.capacity, _ptr(coords), coords.shape[0], None))
 
+    def query_subm_bxyz(self, coords, kernel_size) -> torch.Tensor:
+        """Stride-1 map over the table's own coordinates (row i inserted with value i).  Odd
+        kernels probe half of the offsets and mirror the hits; even ones take the general
+        query with offsets 0..ks-1."""
+        ks = _triple(kernel_size)
+        if any(k % 2 == 0 for k in ks):
+            return self.query_bxyz(coords, ks, (1, 1, 1), _subm_pad(ks))
+        coords = _need(coords, torch.int32, "coords")
+        n = coords.shape[0]
+        n_pad = make_divisible(n, 128)
+        omap = torch.empty((n_pad, ks[0] * ks[1] * ks[2]), dtype=torch.int32, device=coords.device)
+        _check(_C.tsmi_kmap_query_subm(_stream(), _ptr(self.keys), _ptr(self.vals), self.capacity,
+                                       _ptr(coords), n, n_pad, _I3(*ks), _ptr(omap)))
+        return omap
+
     def query_bxyz(self, out_coords, kernel_size, stride, pad, n_pad=None) -> torch.Tensor:
         out_coords = _need(out_coords, torch.int32, "coords")
         ks, st, pd = _triple(kernel_size), _triple(stride), _triple(pad)
@@ -242,7 +258,7 @@ def build_kernel_map_subm_hashmap(table: GPUHashTable, coords, coords_min, coord
     ks = _triple(kernel_sizes)
     if to_insert:
         table.insert_bxyz(coords)
-    return [table.query_bxyz(coords, ks, (1, 1, 1), _subm_pad(ks))]
+    return [table.query_subm_bxyz(coords, ks)]
 
 
 def coords_max(coords: torch.Tensor) -> torch.Tensor:

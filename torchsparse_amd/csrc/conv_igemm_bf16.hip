@@ -32,7 +32,10 @@ struct TraitsBF16 {
 
 #define TSMI_TRAITS TraitsBF16
 #define TSMI_SUFFIX bf16
+// 16-bit types also get the densely packed kernel for layers of at most 8 input channels
+#define TSMI_SMALL_CIN 1
 #include "conv_igemm.inc"
+#include "conv_small_cin.inc"
 #include "conv_tile.inc"
 #include "conv_igemm2.inc"
 #include "conv_plan.inc"

@@ -39,6 +39,12 @@ __global__ void fill_kernel(T *p, int64_t n, T v) {
   if (i < n) p[i] = v;
 }
 
+// n4 int4 stores of one value (16-byte aligned p).
+__global__ void fill_i32x4_kernel(int4 *p, int64_t n4, int32_t v) {
+  int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i < n4) p[i] = make_int4(v, v, v, v);
+}
+
 __global__ void table_clear_kernel(unsigned long long *keys, int32_t *vals, int64_t cap) {
   int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (i < cap) {
@@ -103,6 +109,32 @@ __global__ void kmap_query_kernel(TableView t, const int4 *out_coords, int64_t n
     }
   }
   map[tid] = result;
+}
+
+// Submanifold map of a centred odd kernel at stride 1 over the table's own coordinates (row i
+// was inserted with value i + 1).  map[i, k] = j  <=>  map[j, K_vol-1-k] = i, so only the first
+// half of the offsets and the centre are probed; a hit also writes the mirrored entry.  The map
+// must hold -1 everywhere before the launch.  One thread per (row, offset <= K_vol/2).
+__global__ void kmap_query_subm_kernel(TableView t, const int4 *coords, int64_t n, int64_t total,
+                                       Geom g, int32_t *map) {
+  int64_t tid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (tid >= total) return;
+  const int half = g.kvol >> 1;
+  int64_t row = tid / (half + 1);
+  int k = (int)(tid - row * (half + 1));
+  int4 c = coords[row];
+  int d[3];
+  decode_digits(k, g, d);
+  int x = c.y - g.pad[0] + d[0];
+  int y = c.z - g.pad[1] + d[1];
+  int z = c.w - g.pad[2] + d[2];
+  if (!coords_packable(c.x, x, y, z)) return;
+  uint32_t slot = table_find(t, pack_coords(c.x, x, y, z));
+  if (slot == 0xFFFFFFFFu) return;
+  const int32_t j = t.vals[slot] - 1;
+  map[row * g.kvol + k] = j;
+  // a table that indexes other rows than `coords` must not send the mirrored store astray
+  if (k != half && (uint64_t)j < (uint64_t)n) map[(int64_t)j * g.kvol + (g.kvol - 1 - k)] = (int32_t)row;
 }
 
 __global__ void coords_max_kernel(const int4 *coords, int64_t n, int32_t *out_max) {
@@ -687,6 +719,37 @@ extern "C" int tsmi_kmap_query(tsmi_stream_t s, const int64_t *keys, const int32
   hipLaunchKernelGGL(kmap_query_kernel, grid_for(total), dim3(kBlock), 0, (hipStream_t)s, t,
                      (const int4 *)out_coords, n_out, total, g, out_in_map);
   return check_launch("tsmi_kmap_query");
+}
+
+extern "C" int tsmi_kmap_query_subm(tsmi_stream_t s, const int64_t *keys, const int32_t *vals,
+                                    int64_t cap, const int32_t *coords, int64_t n, int64_t n_pad,
+                                    const int32_t ks[3], int32_t *out_in_map) {
+  TableView t;
+  Geom g;
+  if (int e = make_table(&t, keys, vals, cap)) return e;
+  TSMI_REQUIRE(ks && ks[0] % 2 == 1 && ks[1] % 2 == 1 && ks[2] % 2 == 1,
+               "kmap_query_subm: every kernel size must be odd");
+  const int32_t one[3] = {1, 1, 1};
+  const int32_t pad[3] = {(ks[0] - 1) / 2, (ks[1] - 1) / 2, (ks[2] - 1) / 2};
+  if (int e = make_geom(&g, ks, one, pad)) return e;
+  TSMI_REQUIRE(n >= 0 && n_pad >= n, "kmap_query_subm: n_pad < n");
+  TSMI_REQUIRE(n == 0 || coords, "kmap_query_subm: null coords");
+  TSMI_REQUIRE(n <= cap, "kmap_query_subm: more rows than table slots");
+  const int64_t cells = n_pad * g.kvol;
+  if (cells == 0) return TSMI_OK;
+  TSMI_REQUIRE(out_in_map, "kmap_query_subm: null out_in_map");
+  TSMI_GRID_CHECK(cells);
+  if (cells % 4 == 0 && (uintptr_t)out_in_map % 16 == 0)
+    hipLaunchKernelGGL(fill_i32x4_kernel, grid_for(cells / 4), dim3(kBlock), 0, (hipStream_t)s,
+                       (int4 *)out_in_map, cells / 4, -1);
+  else
+    hipLaunchKernelGGL(fill_kernel<int32_t>, grid_for(cells), dim3(kBlock), 0, (hipStream_t)s,
+                       out_in_map, cells, -1);
+  const int64_t total = n * (g.kvol / 2 + 1);
+  if (total > 0)
+    hipLaunchKernelGGL(kmap_query_subm_kernel, grid_for(total), dim3(kBlock), 0, (hipStream_t)s, t,
+                       (const int4 *)coords, n, total, g, out_in_map);
+  return check_launch("tsmi_kmap_query_subm");
 }
 
 extern "C" int tsmi_coords_max(tsmi_stream_t s, const int32_t *coords, int64_t n,

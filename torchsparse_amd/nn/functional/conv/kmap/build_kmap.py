@@ -192,7 +192,10 @@ def build_kernel_map(_coords: torch.Tensor, input_node_num: int,
     if subm and mode == "hashmap":
         pad_eff = tuple((k - 1) // 2 for k in kernel_size)
 
-    out_in_map = in_table.query_bxyz(out_coords, kernel_size, stride, pad_eff)
+    if subm and all(k % 2 == 1 for k in kernel_size):
+        out_in_map = in_table.query_subm_bxyz(out_coords, kernel_size)  # centred in both modes
+    else:
+        out_in_map = in_table.query_bxyz(out_coords, kernel_size, stride, pad_eff)
     kmap["out_in_map"] = out_in_map
     kmap["coords"] = out_coords if not subm else _coords
     kmap["sizes"] = (input_node_num, out_coords.shape[0])

@@ -50,9 +50,11 @@ def _fuse_sequential(seq: nn.Sequential) -> None:
 
 def fuse_inference(model: nn.Module) -> nn.Module:
     """Fold every (Conv3d, eval BatchNorm[, ReLU]) run found inside nn.Sequential
-    containers of `model`, and fuse the tail of the residual blocks."""
+    containers of `model`, and fuse the tail of the residual blocks (the U-Net's
+    SparseResBlock and the detection backbone's SparseBasicBlock)."""
+    from ...backbones.detection import SparseBasicBlock
     from ...backbones.modules.blocks import SparseResBlock
-    from ..modules import Conv3d
+    from ..modules import BatchNorm, Conv3d
     for m in model.modules():
         if isinstance(m, nn.Sequential):
             _fuse_sequential(m)
@@ -62,5 +64,15 @@ def fuse_inference(model: nn.Module) -> nn.Module:
             if isinstance(last_conv, Conv3d) and isinstance(last_norm, nn.Identity) \
                     and last_conv.kernel.dim() == 3 and last_conv.activation is None:
                 last_conv.activation = "relu"  # relu(main(x) + shortcut(x)) in one epilogue
+                m._fused_tail = True
+    for m in model.modules():
+        if isinstance(m, SparseBasicBlock) and not getattr(m, "_fused_tail", False):
+            norms = (m.bn1, m.bn2)
+            if all(isinstance(b, BatchNorm) and not b.training and b.track_running_stats for b in norms) \
+                    and m.conv1.activation is None and m.conv2.activation is None:
+                _fold(m.conv1, m.bn1)
+                _fold(m.conv2, m.bn2)
+                m.bn1, m.bn2 = nn.Identity(), nn.Identity()
+                m.conv1.activation = m.conv2.activation = "relu"
                 m._fused_tail = True
     return model
