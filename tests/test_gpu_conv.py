@@ -236,6 +236,39 @@ def test_pointwise_and_module_init(mods):
     assert spnn.Conv3d(4, 4, (3, 1, 1), stride=(2, 1, 1), padding=0).padding == (0, 0, 0)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n,cin,cout", [(0, 16, 8), (1, 32, 64), (100, 32, 64), (4097, 128, 96), (3000, 384, 256),
+                                        (2500, 96, 19), (700, 5, 7)])
+def test_pointwise_convolution_without_autograd_runs_the_fused_kernel(mods, dtype, n, cin, cout, monkeypatch):
+    """Outside autograd a 1x1x1 convolution goes through the implicit-GEMM kernels over the
+    identity map with bias, residual and ReLU in the epilogue; same result as the fp32 product."""
+    ts, backend, spnn, F = mods
+    calls = []
+    real = backend.conv_pointwise_cuda
+    monkeypatch.setattr(backend, "conv_pointwise_cuda", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+    rng = np.random.default_rng(n + cin)
+    coords = dev(random_coords(rng, n, (20, 20, 12))) if n else torch.zeros((0, 4), dtype=torch.int32, device="cuda")
+    x = torch.from_numpy(rng.standard_normal((n, cin)).astype(np.float32)).to("cuda", dtype)
+    torch.manual_seed(cin)
+    layer = spnn.Conv3d(cin, cout, 1, bias=True).to("cuda", dtype)
+    layer.bias.data.normal_()
+    res = torch.from_numpy(rng.standard_normal((n, cout)).astype(np.float32)).to("cuda", dtype)
+    with torch.no_grad():
+        plain = layer(ts.SparseTensor(x, coords))
+        fused = F.conv3d(ts.SparseTensor(x, coords), layer.kernel, 1, bias=layer.bias, residual=res,
+                         activation="relu")
+    assert len(calls) == 2 and plain.feats.shape == (n, cout) and plain.feats.dtype == dtype
+    if n == 0:
+        return
+    want = x.float() @ layer.kernel.float() + layer.bias.float()
+    assert rel_rms(_f32(plain.feats), _f32(want)) < TOL[dtype]
+    assert rel_rms(_f32(fused.feats), _f32(torch.relu(want + res.float()))) < TOL[dtype]
+    # with autograd the product stays torch's, and its gradients flow
+    out = layer(ts.SparseTensor(x, coords))
+    assert len(calls) == 2 and out.feats.requires_grad
+    assert rel_rms(_f32(out.feats.detach()), _f32(want)) < TOL[dtype]
+
+
 def test_kmap_cache_and_errors(mods):
     ts, backend, spnn, F = mods
     rng = np.random.default_rng(5)

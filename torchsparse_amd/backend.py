@@ -554,6 +554,35 @@ def _implicit_gemm(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias=None,
     return y
 
 
+_IDENTITY_MAPS = {}
+
+
+def _identity_map(n: int, device) -> torch.Tensor:
+    """int32 [ceil128(n), 1]: row i -> i, pad rows -1 (the map of a 1x1x1 convolution).  The
+    few most recent sizes are kept."""
+    key = (device.index if device.index is not None else _cur_device(), n)
+    m = _IDENTITY_MAPS.get(key)
+    if m is None:
+        if len(_IDENTITY_MAPS) >= 16:
+            _IDENTITY_MAPS.pop(next(iter(_IDENTITY_MAPS)))
+        m = torch.full((make_divisible(n, 128), 1), -1, dtype=torch.int32, device=device)
+        m[:n, 0] = torch.arange(n, dtype=torch.int32, device=device)
+        _IDENTITY_MAPS[key] = m
+    return m
+
+
+def conv_pointwise_cuda(in_feats, kernel, bias=None, residual=None, relu=False) -> torch.Tensor:
+    """1x1x1 convolution act(X W + bias + residual) through the implicit-GEMM kernels over the
+    identity map: bias, residual add and ReLU stay in the kernel epilogue (the reference's
+    conv.py:65-75 calls torch.mm and adds the bias afterwards)."""
+    n = in_feats.shape[0]
+    w = kernel if kernel.dim() == 3 else kernel.unsqueeze(0)
+    if n == 0:
+        return torch.empty((0, w.shape[2]), dtype=in_feats.dtype, device=in_feats.device)
+    return conv_forward_implicit_gemm_cuda(in_feats, kernel, _identity_map(n, in_feats.device), n,
+                                           w.shape[2], bias=bias, residual=residual, relu=relu)
+
+
 def conv_dgrad_implicit_gemm_cuda(grad_out, kernel, in_out_map, num_in_feats) -> torch.Tensor:
     """Input gradient dX[m] = sum_k dY[map[m, k]] W[k]^T: the forward kernel over the
     (input row, offset) -> output row map with the weights transposed per offset

@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 
@@ -18,6 +19,21 @@ void clear_error();
 inline int check_launch(const char *what) {
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(TSMI_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+  return TSMI_OK;
+}
+
+// Raises a kernel's dynamic-LDS limit to `bytes`, once per device: the attribute belongs to
+// the device's copy of the code object.  `done` is the kernel's bit mask of configured devices.
+inline int raise_dynamic_lds(const void *kernel, int bytes, std::atomic<uint64_t> &done,
+                             const char *what) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(TSMI_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+  const uint64_t bit = uint64_t(1) << (dev & 63);
+  if (done.load(std::memory_order_relaxed) & bit) return TSMI_OK;
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e != hipSuccess) return fail(TSMI_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+  done.fetch_or(bit, std::memory_order_relaxed);
   return TSMI_OK;
 }
 

@@ -68,11 +68,20 @@ def conv3d(input: SparseTensor, weight: torch.Tensor,
         caches.cmaps[input.stride] = (coords, input.spatial_range)
 
     if kernel_size == (1, 1, 1) and stride == (1, 1, 1) and dilation == (1, 1, 1):
-        out_feats = feats.matmul(weight) if bias is None else torch.addmm(bias, feats, weight)
-        if residual is not None:
-            out_feats += residual
-        if relu:
-            out_feats = torch.relu_(out_feats)
+        needs_grad = torch.is_grad_enabled() and any(
+            t is not None and t.requires_grad for t in (feats, weight, bias, residual))
+        if feats.is_cuda and not needs_grad and feats.dtype == weight.dtype and weight.dim() == 2:
+            # the implicit-GEMM kernels over the identity map: bias, residual and ReLU fused
+            from torchsparse_amd import backend
+            out_feats = backend.conv_pointwise_cuda(
+                feats, weight, None if bias is None else bias.to(feats.dtype),
+                None if residual is None else residual.contiguous(), relu)
+        else:
+            out_feats = feats.matmul(weight) if bias is None else torch.addmm(bias, feats, weight)
+            if residual is not None:
+                out_feats += residual
+            if relu:
+                out_feats = torch.relu_(out_feats)
         output = SparseTensor._make(out_feats, coords, input.stride, input.spatial_range, caches)
     elif not transposed:
         key = (input.stride, kernel_size, stride, dilation)
