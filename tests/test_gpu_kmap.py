@@ -261,3 +261,22 @@ def test_mirrored_subm_query_equals_the_full_query(ks, n, shape):
         backend._check(backend._C.tsmi_kmap_query_subm(
             None, backend._ptr(table.keys), backend._ptr(table.vals), table.capacity, backend._ptr(c),
             len(coords), len(coords), backend._I3(2, 3, 3), backend._ptr(full)))
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 1000, 4096, 4097, 16384, 16385, 60000])
+def test_sort_keys_small_and_large(n):
+    """tsmi_sort_keys (device-wide radix sort of packed coordinate keys): ascending, exact,
+    repeated keys kept, input untouched."""
+    rng = np.random.default_rng(n)
+    keys = rng.integers(0, 1 << 62, n, dtype=np.int64)
+    if n > 10:
+        keys[: n // 4] = keys[n // 2: n // 2 + n // 4]  # duplicates
+    C = backend._C
+    d_in = torch.from_numpy(keys).cuda()
+    d_out = torch.empty_like(d_in)
+    temp_bytes = C.tsmi_sort_temp_bytes(n)
+    temp = torch.empty(temp_bytes, dtype=torch.uint8, device="cuda")
+    backend._check(C.tsmi_sort_keys(None, backend._ptr(d_in), backend._ptr(d_out), n, 63,
+                                    backend._ptr(temp), temp_bytes))
+    np.testing.assert_array_equal(d_out.cpu().numpy(), np.sort(keys))
+    assert torch.equal(d_in.cpu(), torch.from_numpy(keys))  # the input is left alone
