@@ -269,6 +269,30 @@ def test_pointwise_convolution_without_autograd_runs_the_fused_kernel(mods, dtyp
     assert rel_rms(_f32(out.feats.detach()), _f32(want)) < TOL[dtype]
 
 
+@pytest.mark.parametrize("flow", ["ImplicitGEMM", "GatherScatter", "FetchOnDemand"])
+@pytest.mark.parametrize("ifsort", [False, True])
+def test_strided_convolution_without_outputs(mods, flow, ifsort):
+    """A voxel at the origin has no output under kernel 3, stride 2, padding 0 (the output
+    range is empty): every dataflow, sorted or not, returns an empty tensor and the gradients
+    of an empty output are zero."""
+    ts, backend, spnn, F = mods
+    if ifsort and flow != "ImplicitGEMM":
+        pytest.skip("pair-list dataflows never sort")
+    cfg = F.conv_config.get_default_conv_config()
+    cfg.dataflow, cfg.ifsort, cfg.split_mask_num = getattr(F.Dataflow, flow), ifsort, 3
+    coords = torch.tensor([[0, 0, 0, 0], [1, 1, 0, 1]], dtype=torch.int32, device="cuda")
+    layer = spnn.Conv3d(8, 16, 3, stride=2, padding=0, bias=True, config=cfg).cuda().half()
+    x = torch.randn(2, 8, device="cuda", dtype=torch.float16)
+    with torch.no_grad():
+        out = layer(ts.SparseTensor(x, coords))
+    assert out.feats.shape == (0, 16) and out.coords.shape == (0, 4)
+    xg = x.clone().requires_grad_(True)
+    out = layer(ts.SparseTensor(xg, coords))
+    out.feats.sum().backward()
+    assert out.feats.shape == (0, 16)
+    assert float(xg.grad.abs().max()) == 0.0 and float(layer.kernel.grad.abs().max()) == 0.0
+
+
 def test_kmap_cache_and_errors(mods):
     ts, backend, spnn, F = mods
     rng = np.random.default_rng(5)

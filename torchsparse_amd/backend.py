@@ -402,7 +402,7 @@ def reduce_bitmask_cuda(sorted_mask: torch.Tensor, tile: int) -> torch.Tensor:
     """others/reduce_bitmask_cuda.cu:60-84."""
     sorted_mask = _need(sorted_mask, torch.int32, "bitmask")
     split, n_pad = sorted_mask.shape
-    rows = (n_pad - 1) // tile + 1
+    rows = (n_pad - 1) // tile + 1 if n_pad > 0 else 0
     out = torch.empty((split, rows), dtype=torch.int32, device=sorted_mask.device)
     _check(_C.tsmi_reduce_bitmask(_stream(), _ptr(sorted_mask), split, n_pad, tile, _ptr(out)))
     return out
@@ -591,6 +591,8 @@ def conv_dgrad_implicit_gemm_cuda(grad_out, kernel, in_out_map, num_in_feats) ->
     needs padding: then the kernel tensor is passed as it is."""
     w = kernel if kernel.dim() == 3 else kernel.unsqueeze(0)
     kvol, cin, cout = w.shape
+    if grad_out.shape[0] == 0:  # a convolution without outputs: nothing flows back
+        return torch.zeros((num_in_feats, cin), dtype=grad_out.dtype, device=grad_out.device)
     if w.is_contiguous() and _C.tsmi_packed_weight_elems(kvol, cout, cin) == w.numel():
         if grad_out.dtype != w.dtype:
             raise ValueError(f"feature dtype {grad_out.dtype} and kernel dtype {w.dtype} differ")
@@ -639,6 +641,8 @@ def conv_dgrad_implicit_gemm_sorted_cuda(grad_out, kernel, reorder_in_out_map, r
     the input gradient of the reference's sorted branch (func/implicit_gemm.py:130-141)."""
     w = kernel if kernel.dim() == 3 else kernel.unsqueeze(0)
     kvol, cin, cout = w.shape
+    if grad_out.shape[0] == 0:
+        return torch.zeros((num_in_feats, cin), dtype=grad_out.dtype, device=grad_out.device)
     if w.is_contiguous() and _C.tsmi_packed_weight_elems(kvol, cout, cin) == w.numel():
         if grad_out.dtype != w.dtype:
             raise ValueError(f"feature dtype {grad_out.dtype} and kernel dtype {w.dtype} differ")
@@ -732,6 +736,8 @@ def conv_backward_wgrad_pairs_cuda(grad_out: torch.Tensor, in_feats: torch.Tenso
     pairs = _need(pair_lists["pairs"], torch.int32, "pairs")
     seg_steps = _need(pair_lists["seg_steps"], torch.int32, "seg_steps")
     kvol, cin, cout = seg_steps.numel() - 1, x.shape[1], dy.shape[1]
+    if x.shape[0] == 0 or dy.shape[0] == 0:
+        return torch.zeros((kvol, cin, cout), dtype=x.dtype, device=x.device)
     code = _dtype_code(x)
     cap = int(pair_lists["cap"])
     dw = torch.empty((kvol, cin, cout), dtype=x.dtype, device=x.device)

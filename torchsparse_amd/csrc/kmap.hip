@@ -878,7 +878,8 @@ extern "C" int tsmi_reduce_bitmask(tsmi_stream_t s, const int32_t *sorted_mask, 
                                    int64_t n_pad, int tile, int32_t *reduced) {
   if (tile < 4 || tile % 4 != 0)
     return fail(TSMI_ERR_RUNTIME, "[Bitmask reduce] reduce tile size must be multiple of 4.");
-  TSMI_REQUIRE(split >= 1 && n_pad >= 1, "reduce_bitmask: bad sizes");
+  TSMI_REQUIRE(split >= 1 && n_pad >= 0, "reduce_bitmask: bad sizes");
+  if (n_pad == 0) return TSMI_OK;  // a map without rows has no tiles
   TSMI_REQUIRE(sorted_mask && reduced, "reduce_bitmask: null pointer");
   int64_t rows = (n_pad - 1) / tile + 1;
   int64_t total = rows * split;

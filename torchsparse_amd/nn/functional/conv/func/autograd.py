@@ -82,6 +82,9 @@ class SparseConvFunction(torch.autograd.Function):
         sizes = kmap["sizes"]
         n_in = sizes[1] if transposed else sizes[0]
         grad_input = grad_weight = None
+        if dy.shape[0] == 0 or x.shape[0] == 0:  # no outputs (or no inputs): nothing flows back
+            return (torch.zeros_like(input) if ctx.needs_input_grad[0] else None,
+                    torch.zeros_like(weight) if ctx.needs_input_grad[1] else None, None, None, None, None)
         if ctx.needs_input_grad[0]:
             products = backward_sort_products(kmap, transposed) if ctx.ifsort else None
             if products is not None:
