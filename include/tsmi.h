@@ -199,15 +199,18 @@ int tsmi_pair_lists_count(tsmi_stream_t s, const int32_t *map, int64_t n_rows, i
  *   nbmaps_inter int32[nnz,2] rows (in,out)     — GatherScatter layout (:141-143)
  *   nbmaps_planar int32[2,nnz] all in, then out — FetchOnDemand layout (:187-200)
  *   input_mask int32[K_vol*n_in], output_mask int32[K_vol*n_out]: position of the
- *     pair inside offset k's list (pre-filled with -1 here); the centre offset of
- *     an odd-volume map with n_in == n_out is skipped — build_mask_from_kmap
- *     (others/sparsemapping_cuda.cu:235-256,510-548).
+ *     pair inside offset k's list (pre-filled with -1 here).  Offset mask_skip_k is left
+ *     out of the masks: the identity offset of an odd-volume submanifold map, whose pair
+ *     list needs no look-up (-1: none).  -2 applies the reference's rule, the centre
+ *     offset whenever the volume is odd and n_in == n_out — build_mask_from_kmap
+ *     (others/sparsemapping_cuda.cu:235-256,510-548) — which also fires for a strided
+ *     map that happens to have as many outputs as inputs.
  * nbsizes is phase 1's (device); nnz is its sum (the caller read it back to size the
  * arrays). */
 int tsmi_pair_lists_fill(tsmi_stream_t s, const int32_t *map, int64_t n_rows, int kvol,
                          int32_t *block_counts, const int32_t *nbsizes, int64_t nnz,
                          int32_t *nbmaps_inter, int32_t *nbmaps_planar, int64_t n_in,
-                         int64_t n_out, int32_t *input_mask, int32_t *output_mask);
+                         int64_t n_out, int mask_skip_k, int32_t *input_mask, int32_t *output_mask);
 
 /* input_mask / output_mask (see tsmi_pair_lists_fill) from an existing interleaved
  * pair list and nbaddrs = exclusive scan of its per-offset sizes.  Replaces

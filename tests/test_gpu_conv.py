@@ -293,6 +293,31 @@ def test_strided_convolution_without_outputs(mods, flow, ifsort):
     assert float(xg.grad.abs().max()) == 0.0 and float(layer.kernel.grad.abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("flow", ["ImplicitGEMM", "GatherScatter", "FetchOnDemand"])
+@pytest.mark.parametrize("n", [1, 2])
+def test_strided_convolution_with_as_many_outputs_as_inputs(mods, flow, n):
+    """Kernel 3, stride 2, padding 1 on one or two voxels gives as many outputs as inputs, but
+    the centre offset is not the identity: the pair-list dataflows must not take the map for a
+    submanifold one (the reference tells by the sizes and odd volume alone)."""
+    ts, backend, spnn, F = mods
+    coords = np.array([[0, 2, 3, 1], [0, 2, 3, 2]][:n], np.int32)
+    cfg = F.conv_config.get_default_conv_config()
+    cfg.dataflow = getattr(F.Dataflow, flow)
+    torch.manual_seed(n)
+    layer = spnn.Conv3d(8, 16, 3, stride=2, padding=1, config=cfg).cuda()
+    x = torch.randn(n, 8, device="cuda", requires_grad=True)
+    out = layer(ts.SparseTensor(x, dev(coords)))
+    omap, ocoords = oracle.kmap_downsample(coords, 3, 2, 1)
+    assert len(ocoords) == n and np.array_equal(out.coords.cpu().numpy(), ocoords)
+    want = oracle.conv_implicit_gemm(_f32(x), _f32(layer.kernel), omap, n)
+    assert rel_rms(_f32(out.feats), want) < 1e-4
+    g = torch.randn_like(out.feats)
+    (out.feats * g).sum().backward()
+    want_dx, want_dw = oracle.conv_backward_implicit_gemm(_f32(x), _f32(layer.kernel), omap, _f32(g))
+    assert rel_rms(_f32(x.grad), want_dx) < 1e-4
+    assert rel_rms(_f32(layer.kernel.grad), want_dw) < 1e-4
+
+
 def test_kmap_cache_and_errors(mods):
     ts, backend, spnn, F = mods
     rng = np.random.default_rng(5)

@@ -62,7 +62,7 @@ def _load():
         "tsmi_reorder_map": [_vp, _vp, _vp, _i64, _i32, _i32, _vp],
         "tsmi_reduce_bitmask": [_vp, _vp, _i32, _i64, _i32, _vp],
         "tsmi_pair_lists_count": [_vp, _vp, _i64, _i32, _vp, _vp],
-        "tsmi_pair_lists_fill": [_vp, _vp, _i64, _i32, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _vp, _vp],
+        "tsmi_pair_lists_fill": [_vp, _vp, _i64, _i32, _vp, _vp, _i64, _vp, _vp, _i64, _i64, _i32, _vp, _vp],
         "tsmi_exclusive_scan_quantified": [_vp, _i32, _vp, _i32, _vp, _vp],
         "tsmi_build_masks": [_vp, _vp, _i64, _vp, _i32, _i64, _i64, _vp, _vp],
         "tsmi_pack_weights": [_vp, _vp, _vp, _i32, _i32, _i32, _i32],
@@ -409,11 +409,13 @@ def reduce_bitmask_cuda(sorted_mask: torch.Tensor, tile: int) -> torch.Tensor:
 
 
 def pair_lists(out_in_map: torch.Tensor, n_in: int, n_out: int, want_inter=True, want_planar=False,
-               want_masks=True):
+               want_masks=True, mask_skip_k: int = -2):
     """Pair lists of a map, ordered by (offset, output row): the products of
     kmap/func/hashmap_on_the_fly.py:138-151 and :185-205 in one pass.
     Returns dict(nbmaps_inter, nbmaps_planar, nbsizes, input_mask, output_mask, nnz).
-    One host read-back (nnz)."""
+    One host read-back (nnz).  ``mask_skip_k``: the offset the masks leave out (the identity
+    offset of an odd submanifold map), -1 for none, -2 for the reference's rule (the centre
+    offset whenever the volume is odd and n_in == n_out)."""
     out_in_map = _need(out_in_map, torch.int32, "out_in_map")
     dev = out_in_map.device
     kvol = out_in_map.shape[1]
@@ -429,7 +431,7 @@ def pair_lists(out_in_map: torch.Tensor, n_in: int, n_out: int, want_inter=True,
     omask = torch.empty(kvol * n_out, dtype=torch.int32, device=dev) if want_masks else None
     _check(_C.tsmi_pair_lists_fill(_stream(), _ptr(out_in_map), n_out, kvol, _ptr(block_counts),
                                    _ptr(nbsizes), nnz, _ptr(inter), _ptr(planar), n_in, n_out,
-                                   _ptr(imask), _ptr(omask)))
+                                   int(mask_skip_k), _ptr(imask), _ptr(omask)))
     return dict(nbmaps_inter=inter, nbmaps_planar=planar, nbsizes=nbsizes, input_mask=imask,
                 output_mask=omask, nnz=nnz)
 
@@ -772,6 +774,8 @@ def conv_backward_gather_scatter_cuda(in_feat: torch.Tensor, grad_in_feat: torch
         n_in, n_out = dy.shape[0], x.shape[0]
     sizes = neighbor_offset.to(device=x.device, dtype=torch.int32)
     imask, omask = build_mask_from_kmap(n_in, n_out, nbmaps, sizes)
+    # pair lists alone do not say whether the centre offset is the identity: masks and scatter
+    # both follow the reference's rule here (odd volume and as many outputs as inputs)
     center = kvol // 2 if (n_in == n_out and kvol % 2 == 1) else -1
     dx = conv_forward_gather_scatter_cuda(dy, w.transpose(1, 2).contiguous(), nbmaps, sizes, imask, omask,
                                           x.shape[0], transpose=not transpose, center_k=center)

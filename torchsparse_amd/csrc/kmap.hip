@@ -911,7 +911,9 @@ extern "C" int tsmi_pair_lists_count(tsmi_stream_t s, const int32_t *map, int64_
 extern "C" int tsmi_pair_lists_fill(tsmi_stream_t s, const int32_t *map, int64_t n_rows, int kvol,
                                     int32_t *block_counts, const int32_t *nbsizes, int64_t nnz,
                                     int32_t *nbmaps_inter, int32_t *nbmaps_planar, int64_t n_in,
-                                    int64_t n_out, int32_t *input_mask, int32_t *output_mask) {
+                                    int64_t n_out, int mask_skip_k, int32_t *input_mask,
+                                    int32_t *output_mask) {
+  TSMI_REQUIRE(mask_skip_k >= -2 && mask_skip_k < kvol, "pair_lists_fill: bad mask_skip_k %d", mask_skip_k);
   TSMI_REQUIRE(kvol >= 1 && kvol <= kPairMaxKvol && n_rows >= 0 && nnz >= 0 && n_in >= 0 && n_out >= 0,
                "pair_lists_fill: bad sizes");
   if (input_mask && n_in > 0) {
@@ -928,7 +930,8 @@ extern "C" int tsmi_pair_lists_fill(tsmi_stream_t s, const int32_t *map, int64_t
     TSMI_REQUIRE(map && block_counts && nbsizes, "pair_lists_fill: null pointer");
     int64_t nblk = ceil_div(n_rows, kBlock);
     TSMI_REQUIRE(grid_fits(nblk), "pair_lists_fill: too many rows");
-    int skip_k = (n_in == n_out && kvol % 2 == 1) ? kvol / 2 : -1;
+    int skip_k = mask_skip_k;
+    if (skip_k == -2) skip_k = (n_in == n_out && kvol % 2 == 1) ? kvol / 2 : -1;  // the reference's rule
     hipLaunchKernelGGL(pair_fill_kernel, dim3((unsigned)nblk), dim3(kBlock), 0, (hipStream_t)s,
                        map, n_rows, kvol, nblk, block_counts, nbsizes, nnz, nbmaps_inter,
                        nbmaps_planar, n_in, n_out, input_mask, output_mask, skip_k);

@@ -11,9 +11,11 @@ __all__ = ["GatherScatterConvolutionFuntion"]
 
 
 def _center_offset(kmap: Dict, kvol: int) -> int:
-    """Index of the identity offset the masks skip (odd-volume submanifold map), or -1."""
-    n_in, n_out = kmap["sizes"]
-    return kvol // 2 if (n_in == n_out and kvol % 2 == 1) else -1
+    """Index of the identity offset of an odd-volume submanifold map (its pairs are (i, i) in
+    row order, so the scatter needs no mask look-up for it), or -1.  Decided by the map's
+    geometry: a strided map can have as many outputs as inputs without being one (the
+    reference tells by the sizes, convolution_gather_scatter_cuda.cu:497-499)."""
+    return kvol // 2 if (kmap.get("subm", False) and kvol % 2 == 1) else -1
 
 
 class GatherScatterConvolutionFuntion:

@@ -113,8 +113,11 @@ def _pair_products(kmap: Dict, dataflow: Dataflow) -> None:
     scans here: they make the reduction over offsets atomic free."""
     n_in, n_out = kmap["sizes"]
     fod = dataflow == Dataflow.FetchOnDemand
-    prod = backend.pair_lists(kmap["out_in_map"], n_in, n_out, want_inter=not fod, want_planar=fod)
     kvol = kmap["out_in_map"].shape[1]
+    # the masks leave out the identity offset of an odd submanifold map, and only that
+    skip = kvol // 2 if (kmap.get("subm", False) and kvol % 2 == 1) else -1
+    prod = backend.pair_lists(kmap["out_in_map"], n_in, n_out, want_inter=not fod, want_planar=fod,
+                              mask_skip_k=skip)
     dev = kmap["out_in_map"].device
     nbaddrs = torch.empty(kvol + 1, dtype=torch.int32, device=dev)
     qnbaddrs = torch.empty(kvol + 1, dtype=torch.int32, device=dev)
@@ -197,6 +200,7 @@ def build_kernel_map(_coords: torch.Tensor, input_node_num: int,
     else:
         out_in_map = in_table.query_bxyz(out_coords, kernel_size, stride, pad_eff)
     kmap["out_in_map"] = out_in_map
+    kmap["subm"] = subm  # stride 1: outputs are the inputs, the centre offset is the identity
     kmap["coords"] = out_coords if not subm else _coords
     kmap["sizes"] = (input_node_num, out_coords.shape[0])
     kmap["out_hashmap"] = (out_table.keys, out_table.vals)
