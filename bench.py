@@ -116,6 +116,22 @@ def roofline_of(flops, nbytes, ms):
             "frac": ach / HBM_PEAK_GBS, "traffic": None}
 
 
+def achievable_peaks():
+    """What this GPU sustains on the two textbook kernels, beside the published peaks the
+    roofline is priced against: a 1 GiB device-to-device copy (bytes read + written per second)
+    and a large fp16 GEMM through torch (hipBLASLt), fp32 accumulation."""
+    a = torch.empty(256 * 1024 * 1024, dtype=torch.float32, device="cuda")
+    b = torch.empty_like(a)
+    t_copy = event_ms(lambda: b.copy_(a), iters=10)
+    del a, b
+    m = 8192
+    x = torch.randn(m, m, device="cuda", dtype=torch.float16)
+    y = torch.randn(m, m, device="cuda", dtype=torch.float16)
+    t_gemm = event_ms(lambda: torch.matmul(x, y), iters=10)
+    return {"device_copy_GBps": round(2 * 1024 ** 3 / (t_copy * 1e-3) / 1e9, 1),
+            "gemm_f16_8192_TFLOPs": round(2 * m ** 3 / (t_gemm * 1e-3) / 1e12, 1)}
+
+
 def layer_sweep(ts, spnn, F, backend, coords_dev, n):
     """The five single layers of the sweep, fp16."""
     out = []
@@ -335,6 +351,7 @@ def dominant_layer_roofline(ts, F, records, caches, pmc_target=None):
     roof["algorithmic_flops"] = best["flops"]
     roof["achieved"] = round(roof["achieved"], 2)
     roof["frac"] = round(roof["frac"], 4)
+    roof["measured_on_this_gpu"] = achievable_peaks()
     return roof
 
 
