@@ -330,7 +330,7 @@ def dominant_layer_roofline(ts, F, records, caches, pmc_target=None):
         if best is None or total > best["total_ms"]:
             flops, nbytes = conv_work(r["n_in"], r["n_out"], omap.shape[0], nnz, kvol, cin, cout, 2)
             best = {"total_ms": total, "ms": ms, "launches": len(rs), "flops": flops, "bytes": nbytes,
-                    "run": run,
+                    "run": run, "issued": 2.0 * omap.shape[0] * kvol * cin * cout,
                     "desc": desc}
     if pmc_target:
         src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda")
@@ -349,6 +349,10 @@ def dominant_layer_roofline(ts, F, records, caches, pmc_target=None):
     roof["launches_per_step"] = best["launches"]
     roof["algorithmic_bytes"] = best["bytes"]
     roof["algorithmic_flops"] = best["flops"]
+    # the dense work over the whole map (every (row, offset) pair multiplied): what the MFMA
+    # pipe would execute without any skipping
+    roof["dense_map_flops"] = best["issued"]
+    roof["dense_map_TFLOPs"] = round(best["issued"] / (best["ms"] * 1e-3) / 1e12, 1)
     roof["achieved"] = round(roof["achieved"], 2)
     roof["frac"] = round(roof["frac"], 4)
     roof["measured_on_this_gpu"] = achievable_peaks()
