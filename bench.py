@@ -521,7 +521,7 @@ def main():
         from torchsparse_amd.utils.tune import tune
         tuned_model = copy.deepcopy(model)
         with tempfile.TemporaryDirectory() as tmp:
-            chosen = tune(tuned_model, [ts.SparseTensor(feats, coords) for _ in range(3)], n_samples=3,
+            chosen = tune(tuned_model, [ts.SparseTensor(feats, coords) for _ in range(12)], n_samples=12,
                           save_dir=tmp, tune_tag="bench", verbose=False, skip_warning=True,
                           dataflow_range=[F.Dataflow.ImplicitGEMM, F.Dataflow.FetchOnDemand,
                                           F.Dataflow.GatherScatter])
