@@ -173,7 +173,7 @@ __device__ __forceinline__ void output_range(const Geom &g, int a, int3 out_max_
   *lo = in_min_dev ? (in_min_dev[1 + a] - 2 * g.pad[a] + (g.ks[a] - 1)) / g.stride[a] : 0;
 }
 
-// mode 0: thread per (input, offset); modes 1 and 2: thread per input; mode 3 (generative
+// mode 0: thread per (input, exactly dividing offset); modes 1 and 2: thread per input; mode 3 (generative
 // upsampling): thread per (input, offset), o = clamp(in * stride + digit - (ks-1)/2, 0, max).
 __global__ void downsample_candidates_kernel(const int4 *in_coords, int64_t n_in, int64_t total,
                                              Geom g, int3 out_max_host, const int32_t *in_max_dev,
@@ -222,19 +222,27 @@ __global__ void downsample_candidates_kernel(const int4 *in_coords, int64_t n_in
     y = o[1];
     z = o[2];
   } else {
-    int64_t i = tid / g.kvol;
-    int k = (int)(tid - i * g.kvol);
+    // o = (in + pad + d - (ks-1)) / stride for the digits d in [0, ks) that make the division
+    // exact: per axis d = r, r + stride, ... with r = (ks-1 - in - pad) mod stride, at most
+    // ceil(ks / stride) of them.  One thread per (input, combination of such digits).
+    const int f0 = (g.ks[0] + g.stride[0] - 1) / g.stride[0];
+    const int f1 = (g.ks[1] + g.stride[1] - 1) / g.stride[1];
+    const int f2 = (g.ks[2] + g.stride[2] - 1) / g.stride[2];
+    const int fan = f0 * f1 * f2;
+    int64_t i = tid / fan;
+    int j = (int)(tid - i * fan);
+    const int jj[3] = {j % f0, (j / f0) % f1, j / (f0 * f1)};
     int4 c = in_coords[i];
     b = c.x;
-    int d[3];
-    decode_digits(k, g, d);
     int v[3] = {c.y, c.z, c.w};
     int o[3];
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
-      int num = v[a] + g.pad[a] + d[a] - (g.ks[a] - 1);
-      if (num % g.stride[a] != 0) return;
-      o[a] = num / g.stride[a];
+      int r = (g.ks[a] - 1 - v[a] - g.pad[a]) % g.stride[a];
+      if (r < 0) r += g.stride[a];
+      const int d = r + jj[a] * g.stride[a];
+      if (d >= g.ks[a]) return;
+      o[a] = (v[a] + g.pad[a] + d - (g.ks[a] - 1)) / g.stride[a];  // exact
       int lo, hi;
       output_range(g, a, out_max_host, in_max_dev, in_min_dev, &lo, &hi);
       if (o[a] < lo || o[a] > hi) return;
@@ -787,7 +795,12 @@ extern "C" int tsmi_downsample_candidates(tsmi_stream_t s, const int32_t *in_coo
   TSMI_REQUIRE(counters, "downsample_candidates: null counters");
   TSMI_REQUIRE(mode == 1 || in_max_dev || out_max_host, "downsample_candidates: no output bound");
   if (n_in == 0) return TSMI_OK;
-  int64_t total = (mode == 1 || mode == 2) ? n_in : n_in * g.kvol;
+  int64_t per_input = g.kvol;  // mode 3: every offset
+  if (mode == 1 || mode == 2) per_input = 1;
+  if (mode == 0)  // the digits that divide exactly: at most ceil(ks / stride) per axis
+    per_input = (int64_t)((ks[0] + stride[0] - 1) / stride[0]) * ((ks[1] + stride[1] - 1) / stride[1]) *
+                ((ks[2] + stride[2] - 1) / stride[2]);
+  int64_t total = n_in * per_input;
   TSMI_GRID_CHECK(total);
   int3 hm = make_int3(0, 0, 0);
   if (out_max_host) hm = make_int3(out_max_host[0], out_max_host[1], out_max_host[2]);
