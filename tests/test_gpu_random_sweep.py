@@ -165,12 +165,10 @@ def test_kernel_maps_of_arbitrary_geometry(mods, seed):
         what = f"seed {seed} case {case}: n={n} b={batch} ks={ks} st={st} pd={pd} range={sr} neg={neg}"
         ts.tensor.set_allow_negative_coordinates(neg)
         try:
+            # geometries with more than two outputs per input on average overflow the first table
+            # and are built again with room for every candidate
             kmap = F.build_kernel_map(torch.from_numpy(c).cuda(), n, ks, st, pd, mode="hashmap_on_the_fly",
                                       spatial_range=sr)
-        except ValueError as e:
-            # more than two outputs per input on average: the table is too small, as in the reference
-            assert "capacity of hashtable" in str(e), what
-            continue
         finally:
             ts.tensor.set_allow_negative_coordinates(False)
         if subm:

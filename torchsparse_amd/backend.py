@@ -270,7 +270,8 @@ def coords_max(coords: torch.Tensor) -> torch.Tensor:
 
 
 def downsample_coords(coords: torch.Tensor, kernel_sizes, stride, padding, coords_max_host=None,
-                      mode: int = 0, rsv_ratio: float = 2.0, allow_negative: bool = False):
+                      mode: int = 0, rsv_ratio: float = 2.0, allow_negative: bool = False,
+                      _reserve_all: bool = False):
     """Output coordinates of a strided convolution in ascending (b,x,y,z) order and
     the hash table that indexes them.  Returns (out_coords, GPUHashTable).
     One host read-back (the number of outputs) — the reference has two
@@ -281,7 +282,8 @@ def downsample_coords(coords: torch.Tensor, kernel_sizes, stride, padding, coord
     n = coords.shape[0]
     dev = coords.device
     # a voxel has up to prod(ceil(ks/stride)) outputs; reserve for the ones a surface
-    # typically produces and report overflow like the reference does
+    # typically produces, and for all of them on a second attempt when that was too few (the
+    # reference sizes its table for two outputs per input and raises, hashmap_on_the_fly.py:56-58)
     fan = 1
     if mode == 0:
         for k, s in zip(ks, st):
@@ -289,7 +291,7 @@ def downsample_coords(coords: torch.Tensor, kernel_sizes, stride, padding, coord
     if mode == 3:  # generative upsampling: up to one output per (input, offset)
         cap = hash_capacity(n * ks[0] * ks[1] * ks[2], rsv_ratio)
     else:
-        cap = hash_capacity(n * min(fan, 2), rsv_ratio)
+        cap = hash_capacity(n * (fan if _reserve_all else min(fan, 2)), rsv_ratio)
     table = GPUHashTable(cap, device=dev)
     counters = table.counters  # zero on a fresh table
     in_max = in_min = None
@@ -316,6 +318,9 @@ def downsample_coords(coords: torch.Tensor, kernel_sizes, stride, padding, coord
     uniq, sorted_keys, temp = scratch[:cap], scratch[cap:2 * cap], scratch[2 * cap:]
     _check(_C.tsmi_hashtable_compact_keys(s, _ptr(table.keys), cap, _ptr(uniq), _ptr(counters)))
     n_out, overflow = counters[:2].tolist()
+    if overflow and mode == 0 and fan > 2 and not _reserve_all:
+        return downsample_coords(coords, kernel_sizes, stride, padding, coords_max_host, mode, rsv_ratio,
+                                 allow_negative, _reserve_all=True)
     if overflow:
         raise ValueError(
             "The capacity of hashtable is not sufficient. Please enlarge reserved space for "
