@@ -1,6 +1,6 @@
 """Benchmark of the sparse-convolution forward hot path on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-layers] [--no-backward] [--no-tune] [--no-pointops]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-layers] [--no-backward] [--no-tune] [--no-pointops] [--no-configs]
 
 One step = one MinkUNet (SparseResUNet42 + 19-class linear head) forward in fp16 on a
 synthetic 64-beam LiDAR scan (~90k voxels, 4 input channels), starting from a fresh
@@ -51,6 +51,8 @@ def parse():
     ap.add_argument("--no-backward", action="store_true", help="skip the backward (training) figures")
     ap.add_argument("--no-tune", action="store_true", help="skip the per-group tuner run")
     ap.add_argument("--no-pointops", action="store_true", help="skip the point-voxel operator sweep")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="skip the detection-backbone and 1M-voxel figures")
     ap.add_argument("--pmc-target", default=None, metavar="KERNEL",
                     help="run only a 256 MiB device copy (5 launches) and one conv kernel (5 launches) "
                          "for a hardware-counter pass; KERNEL is the description a normal run prints "
@@ -232,6 +234,51 @@ def backward_sweep(ts, spnn, F, backend, coords_dev, n, feats):
         step()
     torch.cuda.synchronize()
     out["train_step_ms"] = round((time.perf_counter() - t0) * 100, 4)
+    return out
+
+
+def other_configs(ts, spnn, F, backend):
+    """The two larger configurations of the benchmark set, as single figures: the detection
+    backbone (batch 2, merged sweeps, (41, 1440, 1440) grid, 5 input channels, fp16, inference form)
+    and one 256 -> 256 submanifold layer on ~1M voxels (sphere shells in 512^3), unsorted and sorted."""
+    from torchsparse_amd.backbones import VoxelResBackBone8x
+    from torchsparse_amd.nn.utils import fuse_inference
+    from torchsparse_amd.utils import synthetic
+    out = {}
+    coords_np, spatial_range = synthetic.multisweep_voxels(seed=2)
+    coords = torch.from_numpy(coords_np).cuda()
+    n = coords.shape[0]
+    feats = torch.randn(n, 5, device="cuda", dtype=torch.float16)
+    torch.manual_seed(1)
+    net = fuse_inference(VoxelResBackBone8x(in_channels=5).cuda().half().eval())
+    warm = ts.SparseTensor(feats, coords, spatial_range=spatial_range)
+
+    def run(x):
+        with torch.no_grad():
+            return net(x)
+    out["detection_backbone"] = {
+        "voxels": n, "batch": 2, "spatial_range": list(spatial_range),
+        "ms_maps_rebuilt": round(event_ms(lambda: run(ts.SparseTensor(feats, coords, spatial_range=spatial_range)),
+                                          iters=10), 4),
+        "ms_maps_cached": round(event_ms(lambda: run(warm), iters=10), 4)}
+    del net, warm, feats, coords
+    coords = torch.from_numpy(synthetic.sphere_shell_voxels(seed=3)).cuda()
+    n = coords.shape[0]
+    t_map = event_ms(lambda: F.build_kernel_map(coords, n, 3, 1, 1, mode="hashmap_on_the_fly"), iters=5)
+    t_map_sorted = event_ms(lambda: F.build_kernel_map(coords, n, 3, 1, 1, mode="hashmap_on_the_fly", ifsort=True),
+                            iters=5)
+    km = F.build_kernel_map(coords, n, 3, 1, 1, mode="hashmap_on_the_fly", ifsort=True)
+    nnz = int((km["out_in_map"][:n] >= 0).sum().item())
+    x = torch.randn(n, 256, device="cuda", dtype=torch.float16)
+    w = torch.randn(27, 256, 256, device="cuda", dtype=torch.float16) * 0.02
+    t = event_ms(lambda: backend.conv_forward_implicit_gemm_cuda(x, w, km["out_in_map"], n, 256), iters=5)
+    t_sorted = event_ms(lambda: backend.conv_forward_implicit_gemm_sorted_cuda(
+        x, w, km["reorder_out_in_map"], km["reduced_sorted_mask"], km["reorder_loc"], n, 256), iters=5)
+    flops = 2.0 * nnz * 256 * 256
+    out["subm_k3_256_256_1M"] = {
+        "voxels": n, "nnz": nnz, "kmap_ms": round(t_map, 4), "kmap_with_sort_products_ms": round(t_map_sorted, 4),
+        "conv_ms": round(t, 4), "eff_TFLOPs": round(flops / (t * 1e-3) / 1e12, 1),
+        "conv_sorted_ms": round(t_sorted, 4), "sorted_eff_TFLOPs": round(flops / (t_sorted * 1e-3) / 1e12, 1)}
     return out
 
 
@@ -513,6 +560,7 @@ def main():
         layers = None if args.no_layers else layer_sweep(ts, spnn, F, backend, coords, n)
     backward = None if args.no_backward else backward_sweep(ts, spnn, F, backend, coords, n, feats)
     pointops = None if args.no_pointops else pointops_sweep(F)
+    configs = None if args.no_configs else other_configs(ts, spnn, F, backend)
     tuned = None
     if not args.no_tune:
         # the per-group tuner over all three dataflows and the sorted variants, then the same
@@ -544,7 +592,7 @@ def main():
                    "unfused_ms_per_step": round(ms_unfused, 4),
                    "conv_mode": F.get_conv_mode().value},
         "roofline": roof, "cpu_baseline": cpu, "layers": layers, "backward": backward,
-        "tuned": tuned, "pointops": pointops,
+        "tuned": tuned, "pointops": pointops, "other_configs": configs,
     }
     print(json.dumps(result))
 
