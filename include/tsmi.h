@@ -158,6 +158,38 @@ int tsmi_downsample_finalize(tsmi_stream_t s, const int64_t *sorted_keys, int64_
                              const int64_t *keys, int32_t *vals, int64_t cap,
                              int32_t *out_coords);
 
+/* Output coordinates of a strided convolution through an occupancy bitmap of the output
+ * grid: the same result as tsmi_downsample_candidates (mode 0) + compact + sort + finalize
+ * when every coordinate is non-negative and the grid (batches x extents) has at most
+ * 32 * bitmap_words cells; no hash insertion of candidates and no sort.  Replaces
+ * downsample_cuda's candidate / unique passes (others/downsample_cuda.cu:147-190,
+ * others/sparsemapping_cuda.cu:429-507).
+ *
+ * tsmi_downsample_grid_count marks the bitmap (after clearing the part THIS call uses when
+ * clear_first is set, for callers that pass uninitialised scratch every time; otherwise the
+ * caller guarantees it is all zero) and counts its set bits:
+ * counters[0] = number of outputs, counters[2] = 1 when the grid does not fit (nothing is
+ * then marked and the caller takes the sorting path).  in_max_dev is the device int32[4]
+ * per-column maximum of in_coords (tsmi_coords_max); out_max_host, when given, bounds the
+ * three spatial axes instead.  bitmap int32[bitmap_words] (16-byte aligned, a multiple of
+ * 2048 words, at most 2^25) and chunk_counts int32[bitmap_words / 2048] are scratch that
+ * tsmi_downsample_grid_emit reads back: it writes out_coords int32[n_out,4] in ascending
+ * (b,x,y,z) order, inserts coordinate -> row + 1 into the EMPTY output table
+ * (keys, vals, cap; counters[1] = 1 if the table was too small) and leaves the bitmap
+ * all zero again, so that one bitmap can serve call after call without clear_first.
+ * in_max_host, when given, is a host copy of in_max_dev (read back with the counters): the
+ * extents are then computed on the host and only the chunks inside the grid are launched. */
+int tsmi_downsample_grid_count(tsmi_stream_t s, const int32_t *in_coords, int64_t n_in,
+                               const int32_t ks[3], const int32_t stride[3], const int32_t pad[3],
+                               const int32_t out_max_host[3], const int32_t *in_max_dev,
+                               int32_t *bitmap, int64_t bitmap_words, int clear_first,
+                               int32_t *chunk_counts, int32_t *counters);
+int tsmi_downsample_grid_emit(tsmi_stream_t s, const int32_t ks[3], const int32_t stride[3],
+                              const int32_t pad[3], const int32_t out_max_host[3],
+                              const int32_t *in_max_dev, const int32_t *in_max_host,
+                              int32_t *bitmap, int64_t bitmap_words, const int32_t *chunk_prefix, int64_t n_out, int64_t *keys,
+                              int32_t *vals, int64_t cap, int32_t *out_coords, int32_t *counters);
+
 /* map_t[in,k] = out for every map[out,k] = in >= 0, out < n_rows; map_t
  * [n_rows_t, K_vol] is filled with -1 first.  Replaces
  * convert_transposed_out_in_map (others/query_cuda.cu:9-15,50-54) plus the

@@ -53,7 +53,9 @@ DOWN_CASES = [(2, 2, 0), (3, 2, 1), (3, 3, 1), (5, 2, 2), (5, 3, 2), (2, 3, 0), 
 
 @pytest.mark.parametrize("ks,stride,pad", DOWN_CASES)
 @pytest.mark.parametrize("with_range", [False, True])
-def test_downsample_map_matches_oracle(ks, stride, pad, with_range):
+@pytest.mark.parametrize("through_grid", [True, False])
+def test_downsample_map_matches_oracle(ks, stride, pad, with_range, through_grid, monkeypatch):
+    monkeypatch.setattr(backend, "downsample_through_grid", through_grid)
     rng = np.random.default_rng(101)
     shape = (19, 17, 13)
     coords = random_coords(rng, 700, shape, batch=2)
@@ -100,6 +102,51 @@ def test_spdownsample_minkowski_and_spconv():
     np.testing.assert_array_equal(got, oracle.spdownsample_floor(coords, 2))
     got = F.spdownsample(dev(coords), 2, 3, 1).cpu().numpy()
     np.testing.assert_array_equal(got, oracle.kmap_downsample(coords, 3, 2, 1)[1])
+
+
+@pytest.mark.parametrize("n,shape,batch", [(1, (3, 3, 3), 1), (40000, (300, 280, 24), 1),
+                                           (30000, (90, 70, 40), 5), (3000, (4000, 3000, 900), 2),
+                                           (2000, (100000, 90000, 70000), 1)])
+@pytest.mark.parametrize("geom", [(2, 2, 0), (3, 2, 1), (5, 3, 2)])
+def test_downsample_through_grid_equals_hash_and_sort(n, shape, batch, geom, monkeypatch):
+    """The occupancy-bitmap path and the hash-and-sort path give the same output coordinates,
+    in the same order, and tables that index them alike: small grids, grids of many 2048-word
+    chunks, several batches, and grids too large for the bitmap (the call falls back)."""
+    rng = np.random.default_rng(n + batch)
+    cols = [rng.integers(0, batch, n)] + [rng.integers(0, e, n) for e in shape]
+    coords = np.unique(np.stack(cols, 1).astype(np.int32), axis=0)
+    coords = coords[rng.permutation(len(coords))]
+    ks, st, pd = t3(geom[0]), t3(geom[1]), t3(geom[2])
+    results = []
+    for through_grid in (True, False):
+        monkeypatch.setattr(backend, "downsample_through_grid", through_grid)
+        out, table = backend.downsample_coords(dev(coords), ks, st, pd)
+        omap = table.query_bxyz(out, (1, 1, 1), (1, 1, 1), (0, 0, 0))[:out.shape[0], 0]
+        results.append((out.cpu().numpy(), omap.cpu().numpy()))
+    np.testing.assert_array_equal(results[0][0], results[1][0])
+    np.testing.assert_array_equal(results[0][1], np.arange(len(results[0][0])))
+    np.testing.assert_array_equal(results[1][1], np.arange(len(results[1][0])))
+    np.testing.assert_array_equal(results[0][0], oracle.kmap_downsample(coords, ks, st, pd)[1])
+
+
+def test_downsample_grid_recovers_from_an_unfinished_call():
+    """The occupancy bitmap is shared by the calls on a stream and must be all zero between them:
+    a call that stopped after marking (here: forged, then a real one that raises because the
+    output table is too small) is noticed and the bitmap cleared before the next use."""
+    rng = np.random.default_rng(7)
+    coords = random_coords(rng, 5000, (60, 50, 40), batch=2)
+    want = oracle.kmap_downsample(coords, t3(3), t3(2), t3(1))[1]
+    args = (dev(coords), t3(3), t3(2), t3(1))
+    np.testing.assert_array_equal(backend.downsample_coords(*args)[0].cpu().numpy(), want)
+    assert backend._grid_scratch
+    for entry in backend._grid_scratch.values():
+        entry[0][:entry[1]].fill_(-1)
+        entry[2] = True
+    np.testing.assert_array_equal(backend.downsample_coords(*args)[0].cpu().numpy(), want)
+    with pytest.raises(ValueError, match="capacity of hashtable"):
+        backend.downsample_coords(*args, rsv_ratio=0.001)
+    np.testing.assert_array_equal(backend.downsample_coords(*args)[0].cpu().numpy(), want)
+    assert not any(entry[2] for entry in backend._grid_scratch.values())
 
 
 def test_table_reuse_across_levels():

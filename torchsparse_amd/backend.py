@@ -56,6 +56,9 @@ def _load():
         "tsmi_hashtable_compact_keys": [_vp, _vp, _i64, _vp, _vp],
         "tsmi_sort_keys": [_vp, _vp, _vp, _i64, _i32, _vp, _i64],
         "tsmi_downsample_finalize": [_vp, _vp, _i64, _vp, _vp, _i64, _vp],
+        "tsmi_downsample_grid_count": [_vp, _vp, _i64, _I3, _I3, _I3, _vp, _vp, _vp, _i64, _i32, _vp, _vp],
+        "tsmi_downsample_grid_emit": [_vp, _I3, _I3, _I3, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _vp,
+                                      _i64, _vp, _vp],
         "tsmi_transpose_map": [_vp, _vp, _i64, _i32, _vp, _i64],
         "tsmi_derive_bitmask": [_vp, _vp, _i64, _i32, _i32, _i64, _vp],
         "tsmi_argsort_desc": [_vp, _vp, _vp, _vp, _i32, _i64, _vp, _i64],
@@ -294,6 +297,11 @@ def downsample_coords(coords: torch.Tensor, kernel_sizes, stride, padding, coord
         cap = hash_capacity(n * (fan if _reserve_all else min(fan, 2)), rsv_ratio)
     table = GPUHashTable(cap, device=dev)
     counters = table.counters  # zero on a fresh table
+    if mode == 0 and not allow_negative and n > 0 and downsample_through_grid and not _reserve_all:
+        done = _downsample_coords_grid(coords, ks, st, pd, coords_max_host, fan, rsv_ratio, table)
+        if done is not None:
+            return done
+        counters.zero_()
     in_max = in_min = None
     host_max = None
     if mode == 3:
@@ -331,6 +339,70 @@ def downsample_coords(coords: torch.Tensor, kernel_sizes, stride, padding, coord
         _check(_C.tsmi_sort_keys(s, _ptr(uniq), _ptr(sorted_keys), n_out, 63, _ptr(temp), temp_bytes))
         _check(_C.tsmi_downsample_finalize(s, _ptr(sorted_keys), n_out, _ptr(table.keys),
                                            _ptr(table.vals), cap, _ptr(out_coords)))
+    return out_coords, table
+
+
+# Strided output coordinates go through an occupancy bitmap of the output grid when it is small
+# enough (no sort); False keeps every call on the hash-and-sort path.
+downsample_through_grid = True
+_GRID_CHUNK_WORDS = 2048
+_grid_scratch = {}  # (device index, stream) -> [int32 buffer: bitmap | chunk counts, bitmap words, in flight]
+
+
+def _grid_bitmap(dev: torch.device, words: int):
+    """The all-zero bitmap of at least ``words`` words kept for the current stream (every call
+    leaves it zero again; one that did not finish has it cleared here)."""
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(), _stream())
+    entry = _grid_scratch.get(key)
+    if entry is None or entry[1] < words:
+        entry = [torch.zeros(words + words // _GRID_CHUNK_WORDS, dtype=torch.int32, device=dev), words, False]
+        _grid_scratch[key] = entry
+    elif entry[2]:
+        entry[0].zero_()
+    return entry
+
+
+def _downsample_coords_grid(coords, ks, st, pd, coords_max_host, fan, rsv_ratio, table):
+    """downsample_coords for non-negative coordinates when the output grid has at most
+    2048 cells per candidate (and at most 2^30): mark an occupancy bitmap, count, read the
+    number of outputs back, emit rows and table entries in ascending order.  None when the grid
+    is larger than that (decided on the device; costs the same one read-back)."""
+    n = coords.shape[0]
+    dev = coords.device
+    bits = min(max(1 << (n * fan * 2048 - 1).bit_length(), 1 << 20), 1 << 30)
+    entry = _grid_bitmap(dev, bits // 32)
+    words = entry[1]
+    bitmap, chunk_counts = entry[0][:words], entry[0][words:]
+    counters = table.counters
+    in_max = counters[4:8]  # zero on a fresh table
+    s = _stream()
+    _check(_C.tsmi_coords_max(s, _ptr(coords), n, _ptr(in_max), 0))
+    host_max = _I3(*[int(v) for v in coords_max_host]) if coords_max_host is not None else None
+    entry[2] = True  # marked bits stay behind unless the emit pass below runs
+    _check(_C.tsmi_downsample_grid_count(s, _ptr(coords), n, _I3(*ks), _I3(*st), _I3(*pd), host_max,
+                                         _ptr(in_max), _ptr(bitmap), words, 0, _ptr(chunk_counts),
+                                         _ptr(counters)))
+    host = counters.tolist()
+    n_out, too_large = host[0], host[2]
+    if too_large:
+        entry[2] = False  # nothing was marked
+        return None
+    if n_out > table.capacity:
+        if fan > 2:  # more than the two outputs per input the first table reserves
+            table = GPUHashTable(hash_capacity(n * fan, rsv_ratio), device=dev)
+        if n_out > table.capacity:
+            raise ValueError(
+                "The capacity of hashtable is not sufficient. Please enlarge reserved space for "
+                "hashtable:\n # Python \nimport torchsparse_amd.backends\n"
+                "torchsparse_amd.backends.hash_rsv_ratio=#Value")
+    out_coords = torch.empty((n_out, 4), dtype=torch.int32, device=dev)
+    if n_out > 0:
+        _check(_C.tsmi_downsample_grid_emit(s, _I3(*ks), _I3(*st), _I3(*pd), host_max, _ptr(in_max),
+                                            (ctypes.c_int32 * 4)(*host[4:8]),
+                                            _ptr(bitmap), words, _ptr(chunk_counts), n_out,
+                                            _ptr(table.keys), _ptr(table.vals), table.capacity,
+                                            _ptr(out_coords), _ptr(table.counters)))
+    entry[2] = False
     return out_coords, table
 
 

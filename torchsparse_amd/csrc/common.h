@@ -37,7 +37,7 @@ inline int raise_dynamic_lds(const void *kernel, int bytes, std::atomic<uint64_t
   return TSMI_OK;
 }
 
-inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+__host__ __device__ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 // 1-D grids are capped at 2^31-1 blocks; every kernel here sizes its grid from
 // an int64 element count through this helper and refuses anything larger.

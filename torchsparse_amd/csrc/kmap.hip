@@ -157,7 +157,7 @@ __global__ void coords_max_kernel(const int4 *coords, int64_t n, int32_t *out_ma
   }
 }
 
-__device__ __forceinline__ int floor_div(int a, int b) {
+__host__ __device__ __forceinline__ int floor_div(int a, int b) {
   int q = a / b;
   return (a % b != 0 && ((a < 0) != (b < 0))) ? q - 1 : q;
 }
@@ -165,7 +165,7 @@ __device__ __forceinline__ int floor_div(int a, int b) {
 // Output range of axis a: upper bound from the host or floor((max + 2 pad - (ks-1)) / stride)
 // of the largest input coordinate; lower bound 0, or, when negative coordinates are allowed
 // (in_min_dev given), (min - 2 pad + (ks-1)) / stride rounded toward zero.
-__device__ __forceinline__ void output_range(const Geom &g, int a, int3 out_max_host,
+__host__ __device__ __forceinline__ void output_range(const Geom &g, int a, int3 out_max_host,
                                              const int32_t *in_max_dev, const int32_t *in_min_dev,
                                              int *lo, int *hi) {
   *hi = in_max_dev ? floor_div(in_max_dev[1 + a] + 2 * g.pad[a] - (g.ks[a] - 1), g.stride[a])
@@ -173,40 +173,33 @@ __device__ __forceinline__ void output_range(const Geom &g, int a, int3 out_max_
   *lo = in_min_dev ? (in_min_dev[1 + a] - 2 * g.pad[a] + (g.ks[a] - 1)) / g.stride[a] : 0;
 }
 
+// The candidate output coordinate of thread `tid`; false when the thread has none.
 // mode 0: thread per (input, exactly dividing offset); modes 1 and 2: thread per input; mode 3 (generative
 // upsampling): thread per (input, offset), o = clamp(in * stride + digit - (ks-1)/2, 0, max).
-__global__ void downsample_candidates_kernel(const int4 *in_coords, int64_t n_in, int64_t total,
-                                             Geom g, int3 out_max_host, const int32_t *in_max_dev,
-                                             const int32_t *in_min_dev, int mode, TableView t,
-                                             int32_t *counters) {
-  int64_t tid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (tid >= total) return;
-  int b, x, y, z;
+__device__ __forceinline__ bool downsample_candidate(int64_t tid, const int4 *in_coords, const Geom &g,
+                                                     int3 out_max_host, const int32_t *in_max_dev,
+                                                     const int32_t *in_min_dev, int mode, int *b,
+                                                     int *o) {
   if (mode == 3) {
     int64_t i = tid / g.kvol;
     int k = (int)(tid - i * g.kvol);
     int4 c = in_coords[i];
-    b = c.x;
+    *b = c.x;
     int d[3];
     decode_digits(k, g, d);
     int v[3] = {c.y, c.z, c.w};
-    int o[3];
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
       const int hi = a == 0 ? out_max_host.x : (a == 1 ? out_max_host.y : out_max_host.z);
       o[a] = min(max(v[a] * g.stride[a] + d[a] - (g.ks[a] - 1) / 2, 0), hi);
     }
-    x = o[0];
-    y = o[1];
-    z = o[2];
   } else if (mode != 0) {
     // one candidate per input: o = floor(in / stride).  mode 1 keeps it unbounded; mode 2
     // is the strided-convolution rule specialised to kernel size == stride, zero padding
     // (o*s <= in < o*s + k has exactly one solution), bounded like mode 0.
     int4 c = in_coords[tid];
-    b = c.x;
+    *b = c.x;
     int v[3] = {c.y, c.z, c.w};
-    int o[3];
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
       int q = v[a] / g.stride[a];
@@ -215,12 +208,9 @@ __global__ void downsample_candidates_kernel(const int4 *in_coords, int64_t n_in
       if (mode == 2) {
         int lo, hi;
         output_range(g, a, out_max_host, in_max_dev, in_min_dev, &lo, &hi);
-        if (o[a] < lo || o[a] > hi) return;
+        if (o[a] < lo || o[a] > hi) return false;
       }
     }
-    x = o[0];
-    y = o[1];
-    z = o[2];
   } else {
     // o = (in + pad + d - (ks-1)) / stride for the digits d in [0, ks) that make the division
     // exact: per axis d = r, r + stride, ... with r = (ks-1 - in - pad) mod stride, at most
@@ -233,33 +223,251 @@ __global__ void downsample_candidates_kernel(const int4 *in_coords, int64_t n_in
     int j = (int)(tid - i * fan);
     const int jj[3] = {j % f0, (j / f0) % f1, j / (f0 * f1)};
     int4 c = in_coords[i];
-    b = c.x;
+    *b = c.x;
     int v[3] = {c.y, c.z, c.w};
-    int o[3];
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
       int r = (g.ks[a] - 1 - v[a] - g.pad[a]) % g.stride[a];
       if (r < 0) r += g.stride[a];
       const int d = r + jj[a] * g.stride[a];
-      if (d >= g.ks[a]) return;
+      if (d >= g.ks[a]) return false;
       o[a] = (v[a] + g.pad[a] + d - (g.ks[a] - 1)) / g.stride[a];  // exact
       int lo, hi;
       output_range(g, a, out_max_host, in_max_dev, in_min_dev, &lo, &hi);
-      if (o[a] < lo || o[a] > hi) return;
+      if (o[a] < lo || o[a] > hi) return false;
     }
-    x = o[0];
-    y = o[1];
-    z = o[2];
   }
-  if (!coords_packable(b, x, y, z)) return;
-  unsigned long long key = pack_coords(b, x, y, z);
+  return coords_packable(*b, o[0], o[1], o[2]);
+}
+
+__global__ void downsample_candidates_kernel(const int4 *in_coords, int64_t n_in, int64_t total,
+                                             Geom g, int3 out_max_host, const int32_t *in_max_dev,
+                                             const int32_t *in_min_dev, int mode, TableView t,
+                                             int32_t *counters) {
+  int64_t tid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (tid >= total) return;
+  int b, o[3];
+  if (!downsample_candidate(tid, in_coords, g, out_max_host, in_max_dev, in_min_dev, mode, &b, o)) return;
   bool fresh;
-  uint32_t slot = table_insert(t, key, &fresh);
-  if (slot == 0xFFFFFFFFu) {
-    counters[1] = 1;
-    return;
+  if (table_insert(t, pack_coords(b, o[0], o[1], o[2]), &fresh) == 0xFFFFFFFFu) counters[1] = 1;
+}
+
+// ---- strided output coordinates through an occupancy bitmap -------------------------------
+//
+// When the output grid (batches x extents, known on the device from the largest input
+// coordinate) has at most `cap_bits` cells, the distinct outputs in ascending (b, x, y, z) order
+// are the set bits of a bitmap indexed by the mixed-radix cell number in ascending bit order: no
+// hash insertion of the candidates, no compaction, no sort.  Four passes over the used part
+// of the bitmap (clear, mark, count per 2048-word chunk, emit) and a one-block scan of the
+// chunk counts.
+constexpr int kGridChunkWords = 2048;  // 8 words per thread of a 256-thread block
+
+struct GridDims {
+  int e[3];            // extents of the three axes (largest output coordinate + 1)
+  int64_t used_words;  // bitmap words that cover every cell, rounded up to whole chunks
+  bool fits;
+};
+
+// Cell numbers stay below 2^30 (the largest bitmap), so everything after the fit test is
+// 32-bit arithmetic.
+__host__ __device__ __forceinline__ GridDims grid_dims(const Geom &g, int3 out_max_host, int has_host_max,
+                                                       const int32_t *in_max_dev, int64_t cap_words) {
+  GridDims d;
+  int64_t cells = (int64_t)in_max_dev[0] + 1;
+  bool ok = true;
+#pragma unroll
+  for (int a = 0; a < 3; ++a) {
+    int lo, hi;
+    output_range(g, a, out_max_host, has_host_max ? nullptr : in_max_dev, nullptr, &lo, &hi);
+    d.e[a] = hi + 1;
+    if (hi < 0) ok = false;  // no output at all: nothing to mark
+    // the product stays below 2^63: every factor is below 2^31 and the running product is
+    // compared with the capacity (at most 2^30) before the next factor
+    if (ok) cells *= d.e[a];
+    if (cells > cap_words * 32) ok = false;
   }
-  (void)fresh;
+  const bool empty = d.e[0] <= 0 || d.e[1] <= 0 || d.e[2] <= 0;
+  d.fits = ok || empty;
+  const uint32_t c = (ok && !empty) ? (uint32_t)cells : 0u;
+  constexpr uint32_t kChunkCells = kGridChunkWords * 32;
+  d.used_words = (int64_t)((c + kChunkCells - 1) / kChunkCells) * kGridChunkWords;  // power of two: shifts
+  return d;
+}
+
+__global__ void grid_clear_kernel(uint4 *bitmap, int64_t cap_words, Geom g, int3 out_max_host,
+                                  int has_host_max, const int32_t *in_max_dev) {
+  const GridDims d = grid_dims(g, out_max_host, has_host_max, in_max_dev, cap_words);
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i * 4 < d.used_words) bitmap[i] = make_uint4(0u, 0u, 0u, 0u);
+}
+
+// Inputs usually arrive sorted, so the candidates of neighbouring lanes fall into the same
+// bitmap word: lanes OR their bits into the last lane of each run of equal words and only
+// that lane issues the atomic (any split of the runs is still right, only less thrifty).
+__global__ void grid_mark_kernel(const int4 *in_coords, int64_t total, Geom g, int3 out_max_host,
+                                 int has_host_max, const int32_t *in_max_dev, int mode,
+                                 uint32_t *bitmap, int64_t cap_words) {
+  const int64_t tid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  const GridDims d = grid_dims(g, out_max_host, has_host_max, in_max_dev, cap_words);
+  if (!d.fits || d.used_words == 0) return;  // the same for every thread
+  int word = -1;
+  uint32_t bits = 0;
+  int b, o[3];
+  if (tid < total &&
+      downsample_candidate(tid, in_coords, g, out_max_host, has_host_max ? nullptr : in_max_dev,
+                           nullptr, mode, &b, o) &&
+      b <= in_max_dev[0]) {
+    const uint32_t cell = (((uint32_t)b * d.e[0] + o[0]) * d.e[1] + o[1]) * d.e[2] + o[2];
+    word = (int)(cell >> 5);
+    bits = 1u << (cell & 31);
+  }
+  const int lane = threadIdx.x & 63;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int w = __shfl_up(word, off);
+    const uint32_t v = __shfl_up(bits, off);
+    if (lane >= off && w == word) bits |= v;
+  }
+  const int next = __shfl_down(word, 1);
+  if (word >= 0 && (lane == 63 || next != word)) {
+    // bits are only ever set: a stale read of set bits is still right, a stale read of clear
+    // bits only costs the atomic
+    if ((bitmap[word] & bits) != bits) atomicOr(&bitmap[word], bits);
+  }
+}
+
+__device__ __forceinline__ int grid_thread_words(const uint32_t *bitmap, int64_t chunk, uint32_t *w) {
+  const uint4 *src = (const uint4 *)(bitmap + chunk * kGridChunkWords + threadIdx.x * 8);
+  const uint4 lo = src[0], hi = src[1];
+  w[0] = lo.x; w[1] = lo.y; w[2] = lo.z; w[3] = lo.w;
+  w[4] = hi.x; w[5] = hi.y; w[6] = hi.z; w[7] = hi.w;
+  int c = 0;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) c += __popc(w[j]);
+  return c;
+}
+
+__global__ __launch_bounds__(kBlock) void grid_count_kernel(const uint32_t *bitmap, int64_t cap_words,
+                                                            Geom g, int3 out_max_host, int has_host_max,
+                                                            const int32_t *in_max_dev,
+                                                            int32_t *chunk_counts) {
+  __shared__ int wave_sum[kBlock / 64];
+  const GridDims d = grid_dims(g, out_max_host, has_host_max, in_max_dev, cap_words);
+  if ((int64_t)blockIdx.x * kGridChunkWords >= d.used_words) return;
+  uint32_t w[8];
+  int c = grid_thread_words(bitmap, blockIdx.x, w);
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) c += __shfl_xor(c, off);
+  if ((threadIdx.x & 63) == 0) wave_sum[threadIdx.x >> 6] = c;
+  __syncthreads();
+  if (threadIdx.x == 0) chunk_counts[blockIdx.x] = wave_sum[0] + wave_sum[1] + wave_sum[2] + wave_sum[3];
+}
+
+// One block: chunk_counts[0 .. used chunks) -> exclusive prefix in place, total -> counters[0].
+__global__ __launch_bounds__(1024) void grid_scan_kernel(int32_t *chunk_counts, int64_t cap_words, Geom g,
+                                                         int3 out_max_host, int has_host_max,
+                                                         const int32_t *in_max_dev, int32_t *counters) {
+  __shared__ int wave_sum[16];
+  const GridDims d = grid_dims(g, out_max_host, has_host_max, in_max_dev, cap_words);
+  const int n = (int)(d.used_words / kGridChunkWords);
+  const int per = (n + 1023) / 1024;
+  const int first = threadIdx.x * per;
+  int mine = 0;
+  for (int i = first; i < min(first + per, n); ++i) mine += chunk_counts[i];
+  int incl = mine;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int v = __shfl_up(incl, off);
+    if (lane >= off) incl += v;
+  }
+  if (lane == 63) wave_sum[wave] = incl;
+  __syncthreads();
+  int base = 0;
+  for (int w = 0; w < wave; ++w) base += wave_sum[w];
+  int run = base + incl - mine;
+  for (int i = first; i < min(first + per, n); ++i) {
+    const int c = chunk_counts[i];
+    chunk_counts[i] = run;
+    run += c;
+  }
+  if (threadIdx.x == 1023) {
+    counters[0] = base + incl;
+    counters[2] = d.fits ? 0 : 1;
+  }
+}
+
+// Set bits in ascending order -> out_coords rows; every word read is cleared again.
+// Occupied cells cluster (surfaces): one thread's 256 cells can hold a hundred outputs while its
+// neighbours hold none, so the threads only list the positions of their bits in LDS (in rank
+// order, kGridList ranks at a time) and the whole block then decodes the listed cells one per
+// thread into contiguous row stores.  The table entries (coordinate -> row + 1) are a separate
+// launch of one thread per row: inside this kernel a chunk with thousands of outputs would run
+// its insertions, each a chain of dependent global accesses, in many rounds on one block.
+constexpr int kGridList = 4096;
+
+__global__ __launch_bounds__(kBlock) void grid_emit_kernel(uint32_t *bitmap, int64_t cap_words,
+                                                           const int32_t *chunk_prefix, Geom g,
+                                                           int3 out_max_host, int has_host_max,
+                                                           const int32_t *in_max_dev, GridDims host_dims,
+                                                           int have_host_dims, int4 *out_coords,
+                                                           int64_t n_out) {
+  __shared__ int wave_sum[kBlock / 64];
+  __shared__ uint16_t list[kGridList];
+  const GridDims d = have_host_dims ? host_dims
+                                    : grid_dims(g, out_max_host, has_host_max, in_max_dev, cap_words);
+  if ((int64_t)blockIdx.x * kGridChunkWords >= d.used_words) return;
+  uint32_t w[8];
+  const int mine = grid_thread_words(bitmap, blockIdx.x, w);
+  if (mine) {  // leave the bitmap all clear for the next call
+    uint4 *own = (uint4 *)(bitmap + (int64_t)blockIdx.x * kGridChunkWords + threadIdx.x * 8);
+    own[0] = make_uint4(0u, 0u, 0u, 0u);
+    own[1] = make_uint4(0u, 0u, 0u, 0u);
+  }
+  int incl = mine;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int v = __shfl_up(incl, off);
+    if (lane >= off) incl += v;
+  }
+  if (lane == 63) wave_sum[wave] = incl;
+  __syncthreads();
+  int first = incl - mine;  // rank of this thread's first bit inside the chunk
+  for (int v = 0; v < wave; ++v) first += wave_sum[v];
+  const int chunk_total = wave_sum[0] + wave_sum[1] + wave_sum[2] + wave_sum[3];
+  const int64_t chunk_cell0 = (int64_t)blockIdx.x * kGridChunkWords * 32;
+  const int64_t chunk_rank0 = chunk_prefix[blockIdx.x];
+  for (int base = 0; base < chunk_total; base += kGridList) {
+    if (first < base + kGridList && first + mine > base) {
+      int lr = first;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        uint32_t bits = w[j];
+        while (bits) {
+          const int bit = __ffs(bits) - 1;
+          bits &= bits - 1;
+          if (lr >= base && lr < base + kGridList) list[lr - base] = (uint16_t)(threadIdx.x * 256 + j * 32 + bit);
+          ++lr;
+        }
+      }
+    }
+    __syncthreads();
+    const int count = min(kGridList, chunk_total - base);
+    for (int i = threadIdx.x; i < count; i += kBlock) {
+      uint32_t cell = (uint32_t)chunk_cell0 + list[i];
+      const int64_t r = chunk_rank0 + base + i;
+      const int z = (int)(cell % d.e[2]);
+      cell /= d.e[2];
+      const int y = (int)(cell % d.e[1]);
+      cell /= d.e[1];
+      const int x = (int)(cell % d.e[0]);
+      const int b = (int)(cell / d.e[0]);
+      // always true: n_out is the total of the counts the ranks come from
+      if (r < n_out) out_coords[r] = make_int4(b, x, y, z);
+    }
+    __syncthreads();
+  }
 }
 
 // Occupied slots of a table, gathered in arbitrary order: one atomic per workgroup
@@ -837,6 +1045,99 @@ extern "C" int tsmi_downsample_finalize(tsmi_stream_t s, const int64_t *sorted_k
   hipLaunchKernelGGL(downsample_finalize_kernel, grid_for(n_out), dim3(kBlock), 0, (hipStream_t)s,
                      (const unsigned long long *)sorted_keys, n_out, t, (int4 *)out_coords);
   return check_launch("tsmi_downsample_finalize");
+}
+
+namespace {
+// Shared argument checks of the two occupancy-bitmap entry points.
+int grid_args(Geom *g, int *mode, int3 *hm, const int32_t ks[3], const int32_t stride[3],
+              const int32_t pad[3], const int32_t out_max_host[3], const int32_t *in_max_dev,
+              const void *bitmap, int64_t bitmap_words, const void *chunk_counts, const void *counters) {
+  if (int e = make_geom(g, ks, stride, pad)) return e;
+  TSMI_REQUIRE(in_max_dev && bitmap && chunk_counts && counters, "downsample_grid: null pointer");
+  TSMI_REQUIRE((uintptr_t)bitmap % 16 == 0, "downsample_grid: bitmap must be 16-byte aligned");
+  TSMI_REQUIRE(bitmap_words >= kGridChunkWords && bitmap_words % kGridChunkWords == 0 &&
+                   bitmap_words <= (int64_t(1) << 25),
+               "downsample_grid: bitmap_words must be a multiple of %d and at most 2^25", kGridChunkWords);
+  *mode = (ks[0] == stride[0] && ks[1] == stride[1] && ks[2] == stride[2] && pad[0] == 0 &&
+           pad[1] == 0 && pad[2] == 0) ? 2 : 0;
+  *hm = out_max_host ? make_int3(out_max_host[0], out_max_host[1], out_max_host[2]) : make_int3(0, 0, 0);
+  return TSMI_OK;
+}
+}  // namespace
+
+extern "C" int tsmi_downsample_grid_count(tsmi_stream_t s, const int32_t *in_coords, int64_t n_in,
+                                          const int32_t ks[3], const int32_t stride[3],
+                                          const int32_t pad[3], const int32_t out_max_host[3],
+                                          const int32_t *in_max_dev, int32_t *bitmap,
+                                          int64_t bitmap_words, int clear_first,
+                                          int32_t *chunk_counts, int32_t *counters) {
+  Geom g;
+  int mode;
+  int3 hm;
+  if (int e = grid_args(&g, &mode, &hm, ks, stride, pad, out_max_host, in_max_dev, bitmap, bitmap_words,
+                        chunk_counts, counters))
+    return e;
+  TSMI_REQUIRE(n_in >= 0 && (n_in == 0 || in_coords), "downsample_grid_count: bad coords");
+  const int has_hm = out_max_host != nullptr;
+  const int64_t per_input = mode == 2 ? 1
+                                      : (int64_t)((ks[0] + stride[0] - 1) / stride[0]) *
+                                            ((ks[1] + stride[1] - 1) / stride[1]) *
+                                            ((ks[2] + stride[2] - 1) / stride[2]);
+  const int64_t total = n_in * per_input;
+  TSMI_GRID_CHECK(total);
+  hipStream_t st = (hipStream_t)s;
+  const unsigned chunks = (unsigned)(bitmap_words / kGridChunkWords);
+  if (clear_first)
+    hipLaunchKernelGGL(grid_clear_kernel, grid_for(bitmap_words / 4), dim3(kBlock), 0, st, (uint4 *)bitmap,
+                       bitmap_words, g, hm, has_hm, in_max_dev);
+  if (total > 0)
+    hipLaunchKernelGGL(grid_mark_kernel, grid_for(total), dim3(kBlock), 0, st, (const int4 *)in_coords,
+                       total, g, hm, has_hm, in_max_dev, mode, (uint32_t *)bitmap, bitmap_words);
+  hipLaunchKernelGGL(grid_count_kernel, dim3(chunks), dim3(kBlock), 0, st, (const uint32_t *)bitmap,
+                     bitmap_words, g, hm, has_hm, in_max_dev, chunk_counts);
+  hipLaunchKernelGGL(grid_scan_kernel, dim3(1), dim3(1024), 0, st, chunk_counts, bitmap_words, g, hm,
+                     has_hm, in_max_dev, counters);
+  return check_launch("tsmi_downsample_grid_count");
+}
+
+extern "C" int tsmi_downsample_grid_emit(tsmi_stream_t s, const int32_t ks[3], const int32_t stride[3],
+                                         const int32_t pad[3], const int32_t out_max_host[3],
+                                         const int32_t *in_max_dev, const int32_t *in_max_host,
+                                         int32_t *bitmap, int64_t bitmap_words,
+                                         const int32_t *chunk_prefix, int64_t n_out, int64_t *keys,
+                                         int32_t *vals, int64_t cap, int32_t *out_coords,
+                                         int32_t *counters) {
+  Geom g;
+  int mode;
+  int3 hm;
+  TableView t;
+  if (int e = grid_args(&g, &mode, &hm, ks, stride, pad, out_max_host, in_max_dev, bitmap, bitmap_words,
+                        chunk_prefix, counters))
+    return e;
+  if (int e = make_table(&t, keys, vals, cap)) return e;
+  TSMI_REQUIRE(n_out >= 0 && (n_out == 0 || out_coords), "downsample_grid_emit: bad arguments");
+  TSMI_REQUIRE(n_out <= cap,
+               "The capacity of hashtable is not sufficient. Please enlarge reserved space for "
+               "hashtable (backends.hash_rsv_ratio): %lld outputs, capacity %lld",
+               (long long)n_out, (long long)cap);
+  if (n_out == 0) return TSMI_OK;
+  TSMI_GRID_CHECK(n_out);
+  // with the maxima on the host the extents are computed here: the kernel neither waits for
+  // them nor launches the chunks beyond the grid
+  GridDims hd = {};
+  int64_t chunks = bitmap_words / kGridChunkWords;
+  if (in_max_host) {
+    hd = grid_dims(g, hm, out_max_host != nullptr, in_max_host, bitmap_words);
+    TSMI_REQUIRE(hd.fits, "downsample_grid_emit: the grid does not fit the bitmap");
+    chunks = hd.used_words / kGridChunkWords;
+    if (chunks == 0) return TSMI_OK;
+  }
+  hipLaunchKernelGGL(grid_emit_kernel, dim3((unsigned)chunks), dim3(kBlock), 0, (hipStream_t)s,
+                     (uint32_t *)bitmap, bitmap_words, chunk_prefix, g, hm, out_max_host != nullptr,
+                     in_max_dev, hd, in_max_host != nullptr, (int4 *)out_coords, n_out);
+  hipLaunchKernelGGL(insert_coords_kernel, grid_for(n_out), dim3(kBlock), 0, (hipStream_t)s, t,
+                     (const int4 *)out_coords, n_out, counters + 1);
+  return check_launch("tsmi_downsample_grid_emit");
 }
 
 extern "C" int tsmi_transpose_map(tsmi_stream_t s, const int32_t *map, int64_t n_rows, int kvol,
