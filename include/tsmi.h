@@ -172,7 +172,7 @@ int tsmi_downsample_finalize(tsmi_stream_t s, const int64_t *sorted_keys, int64_
  * then marked and the caller takes the sorting path).  in_max_dev is the device int32[4]
  * per-column maximum of in_coords (tsmi_coords_max); out_max_host, when given, bounds the
  * three spatial axes instead.  bitmap int32[bitmap_words] (16-byte aligned, a multiple of
- * 2048 words, at most 2^25) and chunk_counts int32[bitmap_words / 2048] are scratch that
+ * 512 words, at most 2^25) and chunk_counts int32[bitmap_words / 512] are scratch that
  * tsmi_downsample_grid_emit reads back: it writes out_coords int32[n_out,4] in ascending
  * (b,x,y,z) order, inserts coordinate -> row + 1 into the EMPTY output table
  * (keys, vals, cap; counters[1] = 1 if the table was too small) and leaves the bitmap

@@ -345,7 +345,7 @@ def downsample_coords(coords: torch.Tensor, kernel_sizes, stride, padding, coord
 # Strided output coordinates go through an occupancy bitmap of the output grid when it is small
 # enough (no sort); False keeps every call on the hash-and-sort path.
 downsample_through_grid = True
-_GRID_CHUNK_WORDS = 2048
+_GRID_CHUNK_WORDS = 512
 _grid_scratch = {}  # (device index, stream) -> [int32 buffer: bitmap | chunk counts, bitmap words, in flight]
 
 

@@ -57,15 +57,18 @@ __device__ __forceinline__ uint32_t home_slot(const TableView &t, unsigned long 
 
 // Returns the slot holding `key` (inserting it if absent) or 0xFFFFFFFF when the
 // table is full.  *fresh tells whether this call created the entry.
+// kLoadFirst: read the slot with a plain load before the compare-and-swap.  That pays when
+// most calls find their key already there (de-duplicating candidates): device-scope atomics
+// are an order of magnitude slower than loads here, and a slot never changes once it is
+// non-empty, so only slots that read as empty (possibly stale) need the atomic.  Distinct
+// keys going into a mostly empty table take the atomic at once and save the round trip.
+template <bool kLoadFirst = true>
 __device__ __forceinline__ uint32_t table_insert(const TableView &t, unsigned long long key,
                                                  bool *fresh) {
   const unsigned long long stored = key + 1;
   uint32_t slot = home_slot(t, key);
   for (uint32_t probe = 0; probe < t.cap; ++probe) {
-    // A plain load first: device-scope atomics are an order of magnitude slower than
-    // loads here, and a slot never changes once it is non-empty, so only slots that
-    // read as empty (possibly stale) need the compare-and-swap.
-    unsigned long long prev = t.keys[slot];
+    unsigned long long prev = kLoadFirst ? t.keys[slot] : 0ULL;
     if (prev == 0ULL) prev = atomicCAS(&t.keys[slot], 0ULL, stored);
     if (prev == 0ULL) {
       *fresh = true;

@@ -59,7 +59,7 @@ __global__ void insert_coords_kernel(TableView t, const int4 *coords, int64_t n,
   int4 c = coords[i];  // (b, x, y, z)
   if (!coords_packable(c.x, c.y, c.z, c.w)) return;
   bool fresh;
-  uint32_t slot = table_insert(t, pack_coords(c.x, c.y, c.z, c.w), &fresh);
+  uint32_t slot = table_insert<false>(t, pack_coords(c.x, c.y, c.z, c.w), &fresh);  // rows are distinct
   if (slot == 0xFFFFFFFFu) {
     if (status) *status = 1;
     return;
@@ -258,9 +258,9 @@ __global__ void downsample_candidates_kernel(const int4 *in_coords, int64_t n_in
 // coordinate) has at most `cap_bits` cells, the distinct outputs in ascending (b, x, y, z) order
 // are the set bits of a bitmap indexed by the mixed-radix cell number in ascending bit order: no
 // hash insertion of the candidates, no compaction, no sort.  Four passes over the used part
-// of the bitmap (clear, mark, count per 2048-word chunk, emit) and a one-block scan of the
+// of the bitmap (mark, count per 512-word chunk, emit and clear) and a one-block scan of the
 // chunk counts.
-constexpr int kGridChunkWords = 2048;  // 8 words per thread of a 256-thread block
+constexpr int kGridChunkWords = 512;  // 2 words per thread of a 256-thread block
 
 struct GridDims {
   int e[3];            // extents of the three axes (largest output coordinate + 1)
@@ -337,30 +337,32 @@ __global__ void grid_mark_kernel(const int4 *in_coords, int64_t total, Geom g, i
 }
 
 __device__ __forceinline__ int grid_thread_words(const uint32_t *bitmap, int64_t chunk, uint32_t *w) {
-  const uint4 *src = (const uint4 *)(bitmap + chunk * kGridChunkWords + threadIdx.x * 8);
-  const uint4 lo = src[0], hi = src[1];
-  w[0] = lo.x; w[1] = lo.y; w[2] = lo.z; w[3] = lo.w;
-  w[4] = hi.x; w[5] = hi.y; w[6] = hi.z; w[7] = hi.w;
-  int c = 0;
-#pragma unroll
-  for (int j = 0; j < 8; ++j) c += __popc(w[j]);
-  return c;
+  const uint2 v = *(const uint2 *)(bitmap + chunk * kGridChunkWords + threadIdx.x * 2);
+  w[0] = v.x;
+  w[1] = v.y;
+  return __popc(v.x) + __popc(v.y);
 }
 
 __global__ __launch_bounds__(kBlock) void grid_count_kernel(const uint32_t *bitmap, int64_t cap_words,
                                                             Geom g, int3 out_max_host, int has_host_max,
                                                             const int32_t *in_max_dev,
                                                             int32_t *chunk_counts) {
+  // The extents live on the device, so the launch cannot be sized to the grid; a block that
+  // only learns it has nothing to do still waits ~2 us for them, and thousands of such blocks
+  // queue up behind each other.  A bounded number of blocks stride over the chunks instead.
   __shared__ int wave_sum[kBlock / 64];
   const GridDims d = grid_dims(g, out_max_host, has_host_max, in_max_dev, cap_words);
-  if ((int64_t)blockIdx.x * kGridChunkWords >= d.used_words) return;
-  uint32_t w[8];
-  int c = grid_thread_words(bitmap, blockIdx.x, w);
+  const int64_t chunks = d.used_words / kGridChunkWords;
+  for (int64_t chunk = blockIdx.x; chunk < chunks; chunk += gridDim.x) {
+    uint32_t w[2];
+    int c = grid_thread_words(bitmap, chunk, w);
 #pragma unroll
-  for (int off = 32; off > 0; off >>= 1) c += __shfl_xor(c, off);
-  if ((threadIdx.x & 63) == 0) wave_sum[threadIdx.x >> 6] = c;
-  __syncthreads();
-  if (threadIdx.x == 0) chunk_counts[blockIdx.x] = wave_sum[0] + wave_sum[1] + wave_sum[2] + wave_sum[3];
+    for (int off = 32; off > 0; off >>= 1) c += __shfl_xor(c, off);
+    if ((threadIdx.x & 63) == 0) wave_sum[threadIdx.x >> 6] = c;
+    __syncthreads();
+    if (threadIdx.x == 0) chunk_counts[chunk] = wave_sum[0] + wave_sum[1] + wave_sum[2] + wave_sum[3];
+    __syncthreads();
+  }
 }
 
 // One block: chunk_counts[0 .. used chunks) -> exclusive prefix in place, total -> counters[0].
@@ -398,14 +400,11 @@ __global__ __launch_bounds__(1024) void grid_scan_kernel(int32_t *chunk_counts, 
 }
 
 // Set bits in ascending order -> out_coords rows; every word read is cleared again.
-// Occupied cells cluster (surfaces): one thread's 256 cells can hold a hundred outputs while its
-// neighbours hold none, so the threads only list the positions of their bits in LDS (in rank
-// order, kGridList ranks at a time) and the whole block then decodes the listed cells one per
-// thread into contiguous row stores.  The table entries (coordinate -> row + 1) are a separate
-// launch of one thread per row: inside this kernel a chunk with thousands of outputs would run
-// its insertions, each a chain of dependent global accesses, in many rounds on one block.
-constexpr int kGridList = 4096;
-
+// Occupied cells cluster (surfaces): a few words of a chunk can hold most of its outputs, so
+// the block does not walk bits word by word.  It keeps the chunk's words and the exclusive
+// prefix of their bit counts in LDS, and thread i takes output rank i, i + 256, ...: a binary
+// search of the prefix finds the word, five halvings find the bit.  The table entries
+// (coordinate -> row + 1) are a separate launch of one thread per row.
 __global__ __launch_bounds__(kBlock) void grid_emit_kernel(uint32_t *bitmap, int64_t cap_words,
                                                            const int32_t *chunk_prefix, Geom g,
                                                            int3 out_max_host, int has_host_max,
@@ -413,17 +412,15 @@ __global__ __launch_bounds__(kBlock) void grid_emit_kernel(uint32_t *bitmap, int
                                                            int have_host_dims, int4 *out_coords,
                                                            int64_t n_out) {
   __shared__ int wave_sum[kBlock / 64];
-  __shared__ uint16_t list[kGridList];
+  __shared__ uint32_t words[kGridChunkWords];
+  __shared__ int before[kGridChunkWords];  // set bits of the chunk before each word
   const GridDims d = have_host_dims ? host_dims
                                     : grid_dims(g, out_max_host, has_host_max, in_max_dev, cap_words);
   if ((int64_t)blockIdx.x * kGridChunkWords >= d.used_words) return;
-  uint32_t w[8];
+  uint32_t w[2];
   const int mine = grid_thread_words(bitmap, blockIdx.x, w);
-  if (mine) {  // leave the bitmap all clear for the next call
-    uint4 *own = (uint4 *)(bitmap + (int64_t)blockIdx.x * kGridChunkWords + threadIdx.x * 8);
-    own[0] = make_uint4(0u, 0u, 0u, 0u);
-    own[1] = make_uint4(0u, 0u, 0u, 0u);
-  }
+  if (mine)  // leave the bitmap all clear for the next call
+    *(uint2 *)(bitmap + (int64_t)blockIdx.x * kGridChunkWords + threadIdx.x * 2) = make_uint2(0u, 0u);
   int incl = mine;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
@@ -433,40 +430,42 @@ __global__ __launch_bounds__(kBlock) void grid_emit_kernel(uint32_t *bitmap, int
   }
   if (lane == 63) wave_sum[wave] = incl;
   __syncthreads();
-  int first = incl - mine;  // rank of this thread's first bit inside the chunk
+  int first = incl - mine;
   for (int v = 0; v < wave; ++v) first += wave_sum[v];
+  words[threadIdx.x * 2] = w[0];
+  words[threadIdx.x * 2 + 1] = w[1];
+  before[threadIdx.x * 2] = first;
+  before[threadIdx.x * 2 + 1] = first + __popc(w[0]);
   const int chunk_total = wave_sum[0] + wave_sum[1] + wave_sum[2] + wave_sum[3];
-  const int64_t chunk_cell0 = (int64_t)blockIdx.x * kGridChunkWords * 32;
+  __syncthreads();
+  const uint32_t chunk_cell0 = (uint32_t)blockIdx.x * (kGridChunkWords * 32);
   const int64_t chunk_rank0 = chunk_prefix[blockIdx.x];
-  for (int base = 0; base < chunk_total; base += kGridList) {
-    if (first < base + kGridList && first + mine > base) {
-      int lr = first;
+  for (int i = threadIdx.x; i < chunk_total; i += kBlock) {
+    // the last word with before[word] <= i holds rank i (an empty word shares its successor's count)
+    int lo = 0;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        uint32_t bits = w[j];
-        while (bits) {
-          const int bit = __ffs(bits) - 1;
-          bits &= bits - 1;
-          if (lr >= base && lr < base + kGridList) list[lr - base] = (uint16_t)(threadIdx.x * 256 + j * 32 + bit);
-          ++lr;
-        }
+    for (int step = kGridChunkWords / 2; step > 0; step >>= 1)
+      if (before[lo + step] <= i) lo += step;
+    uint32_t x = words[lo];
+    int k = i - before[lo], pos = 0;
+#pragma unroll
+    for (int half = 16; half > 0; half >>= 1) {
+      const int c = __popc(x & ((1u << half) - 1u));
+      if (k >= c) {
+        k -= c;
+        x >>= half;
+        pos += half;
       }
     }
-    __syncthreads();
-    const int count = min(kGridList, chunk_total - base);
-    for (int i = threadIdx.x; i < count; i += kBlock) {
-      uint32_t cell = (uint32_t)chunk_cell0 + list[i];
-      const int64_t r = chunk_rank0 + base + i;
-      const int z = (int)(cell % d.e[2]);
-      cell /= d.e[2];
-      const int y = (int)(cell % d.e[1]);
-      cell /= d.e[1];
-      const int x = (int)(cell % d.e[0]);
-      const int b = (int)(cell / d.e[0]);
-      // always true: n_out is the total of the counts the ranks come from
-      if (r < n_out) out_coords[r] = make_int4(b, x, y, z);
-    }
-    __syncthreads();
+    uint32_t cell = chunk_cell0 + lo * 32 + pos;
+    const int z = (int)(cell % d.e[2]);
+    cell /= d.e[2];
+    const int y = (int)(cell % d.e[1]);
+    cell /= d.e[1];
+    const int x_ = (int)(cell % d.e[0]);
+    const int b = (int)(cell / d.e[0]);
+    // always true: n_out is the total of the counts the ranks come from
+    if (chunk_rank0 + i < n_out) out_coords[chunk_rank0 + i] = make_int4(b, x_, y, z);
   }
 }
 
@@ -1093,7 +1092,8 @@ extern "C" int tsmi_downsample_grid_count(tsmi_stream_t s, const int32_t *in_coo
   if (total > 0)
     hipLaunchKernelGGL(grid_mark_kernel, grid_for(total), dim3(kBlock), 0, st, (const int4 *)in_coords,
                        total, g, hm, has_hm, in_max_dev, mode, (uint32_t *)bitmap, bitmap_words);
-  hipLaunchKernelGGL(grid_count_kernel, dim3(chunks), dim3(kBlock), 0, st, (const uint32_t *)bitmap,
+  hipLaunchKernelGGL(grid_count_kernel, dim3(chunks < 2048u ? chunks : 2048u), dim3(kBlock), 0, st,
+                     (const uint32_t *)bitmap,
                      bitmap_words, g, hm, has_hm, in_max_dev, chunk_counts);
   hipLaunchKernelGGL(grid_scan_kernel, dim3(1), dim3(1024), 0, st, chunk_counts, bitmap_words, g, hm,
                      has_hm, in_max_dev, counters);
