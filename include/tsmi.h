@@ -169,7 +169,9 @@ int tsmi_downsample_finalize(tsmi_stream_t s, const int64_t *sorted_keys, int64_
  * clear_first is set, for callers that pass uninitialised scratch every time; otherwise the
  * caller guarantees it is all zero) and counts its set bits:
  * counters[0] = number of outputs, counters[2] = 1 when the grid does not fit (nothing is
- * then marked and the caller takes the sorting path).  in_max_dev is the device int32[4]
+ * then marked and the caller takes the sorting path).  next_in_max_dev, when given, is a
+ * zero-filled device int32[4] that receives the per-column maximum of the outputs (what
+ * tsmi_coords_max would find over out_coords).  in_max_dev is the device int32[4]
  * per-column maximum of in_coords (tsmi_coords_max); out_max_host, when given, bounds the
  * three spatial axes instead.  bitmap int32[bitmap_words] (16-byte aligned, a multiple of
  * 512 words, at most 2^25) and chunk_counts int32[bitmap_words / 512] are scratch that
@@ -183,7 +185,22 @@ int tsmi_downsample_grid_count(tsmi_stream_t s, const int32_t *in_coords, int64_
                                const int32_t ks[3], const int32_t stride[3], const int32_t pad[3],
                                const int32_t out_max_host[3], const int32_t *in_max_dev,
                                int32_t *bitmap, int64_t bitmap_words, int clear_first,
-                               int32_t *chunk_counts, int32_t *counters);
+                               int32_t *chunk_counts, int32_t *counters, int32_t *next_in_max_dev);
+/* The next level of a chain of strided convolutions with the same geometry, before the
+ * previous level's outputs exist as rows: the inputs are the set bits of the previous
+ * level's bitmap (marked by tsmi_downsample_grid_count / _count_next with next_in_max_dev =
+ * this call's in_max_dev, a zero-filled device int32[4] that receives the per-column maximum
+ * of the outputs; prev_in_max_dev is the in_max_dev of that call).  Same outputs in counters,
+ * bitmap and chunk_counts as tsmi_downsample_grid_count; a level whose predecessor did not fit
+ * marks nothing.  No counterpart in the reference, which reads the number of outputs back
+ * after every level (others/sparsemapping_cuda.cu:477-479); with this entry one read-back
+ * serves the whole chain. */
+int tsmi_downsample_grid_count_next(tsmi_stream_t s, const int32_t ks[3], const int32_t stride[3],
+                                    const int32_t pad[3], const int32_t *prev_in_max_dev,
+                                    const int32_t *prev_bitmap, int64_t prev_bitmap_words,
+                                    const int32_t *in_max_dev, int32_t *bitmap, int64_t bitmap_words,
+                                    int32_t *chunk_counts, int32_t *counters,
+                                    int32_t *next_in_max_dev);
 int tsmi_downsample_grid_emit(tsmi_stream_t s, const int32_t ks[3], const int32_t stride[3],
                               const int32_t pad[3], const int32_t out_max_host[3],
                               const int32_t *in_max_dev, const int32_t *in_max_host,

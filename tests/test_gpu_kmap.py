@@ -149,6 +149,48 @@ def test_downsample_grid_recovers_from_an_unfinished_call():
     assert not any(entry[2] for entry in backend._grid_scratch.values())
 
 
+@pytest.mark.parametrize("geom", [(2, 2, 0), (3, 2, 1), ((2, 2, 1), (2, 2, 1), (0, 0, 0))])
+def test_strided_chain_computed_ahead_equals_level_by_level(geom, monkeypatch):
+    """A chain of equal strided calls, each on the previous one's outputs: once the chain has
+    been seen, its first call computes the later levels before its one read-back.  Same
+    coordinates, same order, tables that index them, as level by level and as the oracle."""
+    rng = np.random.default_rng(11)
+    coords = lidar_like_coords(rng, 30000) if geom[0] == 2 else random_coords(rng, 20000, (150, 140, 30), 2)
+    ks, st, pd = t3(geom[0]), t3(geom[1]), t3(geom[2])
+    calls = []
+    real = backend._downsample_coords_grid
+    monkeypatch.setattr(backend, "_downsample_coords_grid",
+                        lambda *a, **k: (calls.append(a[-1] if not k else k.get("ahead")), real(*a, **k))[1])
+
+    def chain(ahead):
+        monkeypatch.setattr(backend, "downsample_chain_ahead", ahead)
+        outs, c = [], dev(coords)
+        for _ in range(4):
+            out, table = backend.downsample_coords(c, ks, st, pd)
+            rows = table.query_bxyz(out, (1, 1, 1), (1, 1, 1), (0, 0, 0))[:out.shape[0], 0]
+            outs.append((out.cpu().numpy(), rows.cpu().numpy()))
+            c = out
+        return outs
+
+    base = chain(False)
+    chain(True)  # the chain is learnt here (or was, by an earlier test)
+    del calls[:]
+    ahead = chain(True)
+    assert calls == [3], calls  # one call marks four levels, three calls return what it left
+    want = coords
+    for (a, ra), (b, rb) in zip(base, ahead):
+        want = oracle.kmap_downsample(want, ks, st, pd)[1]
+        np.testing.assert_array_equal(a, want)
+        np.testing.assert_array_equal(b, want)
+        np.testing.assert_array_equal(ra, np.arange(len(want)))
+        np.testing.assert_array_equal(rb, np.arange(len(want)))
+    # a different geometry on a level computed ahead ignores what was left for it
+    out, _ = backend.downsample_coords(dev(coords), ks, st, pd)
+    got = backend.downsample_coords(out, t3(3), t3(2), t3(0))[0].cpu().numpy()
+    np.testing.assert_array_equal(got, oracle.kmap_downsample(base[0][0], t3(3), t3(2), t3(0))[1])
+    assert not any(entry[2] for entry in backend._grid_scratch.values())
+
+
 def test_table_reuse_across_levels():
     """The table a strided map leaves behind indexes its outputs and serves the next
     submanifold map at that level without re-insertion."""

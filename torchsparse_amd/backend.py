@@ -8,6 +8,7 @@ eager fallback: if the shared object is missing, importing this module raises.
 """
 import ctypes
 import os
+import weakref
 from typing import List, Optional, Sequence, Tuple
 
 import torch
@@ -56,7 +57,9 @@ def _load():
         "tsmi_hashtable_compact_keys": [_vp, _vp, _i64, _vp, _vp],
         "tsmi_sort_keys": [_vp, _vp, _vp, _i64, _i32, _vp, _i64],
         "tsmi_downsample_finalize": [_vp, _vp, _i64, _vp, _vp, _i64, _vp],
-        "tsmi_downsample_grid_count": [_vp, _vp, _i64, _I3, _I3, _I3, _vp, _vp, _vp, _i64, _i32, _vp, _vp],
+        "tsmi_downsample_grid_count": [_vp, _vp, _i64, _I3, _I3, _I3, _vp, _vp, _vp, _i64, _i32, _vp, _vp,
+                                       _vp],
+        "tsmi_downsample_grid_count_next": [_vp, _I3, _I3, _I3, _vp, _vp, _i64, _vp, _vp, _i64, _vp, _vp, _vp],
         "tsmi_downsample_grid_emit": [_vp, _I3, _I3, _I3, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _vp,
                                       _i64, _vp, _vp],
         "tsmi_transpose_map": [_vp, _vp, _i64, _i32, _vp, _i64],
@@ -295,11 +298,19 @@ def downsample_coords(coords: torch.Tensor, kernel_sizes, stride, padding, coord
         cap = hash_capacity(n * ks[0] * ks[1] * ks[2], rsv_ratio)
     else:
         cap = hash_capacity(n * (fan if _reserve_all else min(fan, 2)), rsv_ratio)
+    through_grid = (mode == 0 and not allow_negative and n > 0 and downsample_through_grid
+                    and not _reserve_all)
+    if through_grid:
+        chain = (ks, st, pd, rsv_ratio) if coords_max_host is None else None
+        ahead = _chain_step(coords, chain)
+        if not isinstance(ahead, int):  # computed ahead when the previous level of the chain was
+            return ahead
     table = GPUHashTable(cap, device=dev)
     counters = table.counters  # zero on a fresh table
-    if mode == 0 and not allow_negative and n > 0 and downsample_through_grid and not _reserve_all:
-        done = _downsample_coords_grid(coords, ks, st, pd, coords_max_host, fan, rsv_ratio, table)
+    if through_grid:
+        done = _downsample_coords_grid(coords, ks, st, pd, coords_max_host, fan, rsv_ratio, table, ahead)
         if done is not None:
+            _chain["last"] = weakref.ref(done[0])
             return done
         counters.zero_()
     in_max = in_min = None
@@ -345,65 +356,149 @@ def downsample_coords(coords: torch.Tensor, kernel_sizes, stride, padding, coord
 # Strided output coordinates go through an occupancy bitmap of the output grid when it is small
 # enough (no sort); False keeps every call on the hash-and-sort path.
 downsample_through_grid = True
+# Networks apply the same strided convolution level after level (k2 s2 four times in a U-Net).
+# Once such a chain has been seen, the call for its first level also computes the following
+# levels (each from the previous level's bitmap) before the one read-back of the output counts,
+# so the later calls return at once and the forward synchronises once instead of once per
+# level.  Levels computed ahead and never asked for cost their kernels, not a read-back.
+downsample_chain_ahead = True
 _GRID_CHUNK_WORDS = 512
-_grid_scratch = {}  # (device index, stream) -> [int32 buffer: bitmap | chunk counts, bitmap words, in flight]
+_GRID_LEVELS = 4  # the level asked for and up to three ahead
+_grid_scratch = {}  # (device index, stream) -> [int32 buffer, bitmap words of level 0, in flight]
+_chain = {"geom": None, "last": None, "len": 0}  # the chain of equal strided calls in progress
+_chain_len = {}  # geometry -> length of the last chain that ended
+_ahead = {}  # id(coords) -> (weak reference to coords, geometry, out_coords, table)
+
+
+def _chain_step(coords, geom):
+    """Book-keeping of chains of equal strided calls (each on the previous one's outputs).  Returns
+    the (out_coords, table) computed ahead for ``coords``, or the number of levels to compute ahead
+    now."""
+    hit = _ahead.pop(id(coords), None)
+    last = _chain["last"]() if _chain["last"] is not None else None
+    if geom is not None and _chain["geom"] == geom and last is coords:
+        _chain["len"] += 1
+        if hit is not None and hit[0]() is coords and hit[1] == geom and downsample_chain_ahead:
+            _chain["last"] = weakref.ref(hit[2])
+            return hit[2], hit[3]
+        return 0
+    if _chain["geom"] is not None:
+        _chain_len[_chain["geom"]] = _chain["len"]
+    _chain["geom"], _chain["len"], _chain["last"] = geom, 1, None
+    _ahead.clear()
+    if geom is None or not downsample_chain_ahead:
+        return 0
+    return min(_chain_len.get(geom, 1) - 1, _GRID_LEVELS - 1)
+
+
+def _grid_layout(words0: int):
+    """(bitmap offset, bitmap words, chunk-count offset) of each level inside the scratch buffer:
+    a level's grid has at most a quarter of the cells of the one before in any strided geometry
+    worth chaining (half the extent on two axes or more), and a level that does not fit only
+    ends the look-ahead."""
+    out, off = [], 0
+    for level in range(_GRID_LEVELS):
+        w = max(words0 >> (2 * level), 1 << 15)
+        out.append((off, w, off + w))
+        off += w + w // _GRID_CHUNK_WORDS
+    return out, off
 
 
 def _grid_bitmap(dev: torch.device, words: int):
-    """The all-zero bitmap of at least ``words`` words kept for the current stream (every call
-    leaves it zero again; one that did not finish has it cleared here)."""
+    """The all-zero scratch (bitmaps and chunk counts of every level) whose first bitmap has at
+    least ``words`` words, kept for the current stream.  Every call leaves the bitmaps zero
+    again; one that did not finish has them cleared here."""
     key = (dev.index if dev.index is not None else torch.cuda.current_device(), _stream())
     entry = _grid_scratch.get(key)
     if entry is None or entry[1] < words:
-        entry = [torch.zeros(words + words // _GRID_CHUNK_WORDS, dtype=torch.int32, device=dev), words, False]
+        entry = [torch.zeros(_grid_layout(words)[1], dtype=torch.int32, device=dev), words, False]
         _grid_scratch[key] = entry
     elif entry[2]:
         entry[0].zero_()
     return entry
 
 
-def _downsample_coords_grid(coords, ks, st, pd, coords_max_host, fan, rsv_ratio, table):
+def _downsample_coords_grid(coords, ks, st, pd, coords_max_host, fan, rsv_ratio, table, ahead=0):
     """downsample_coords for non-negative coordinates when the output grid has at most
     2048 cells per candidate (and at most 2^30): mark an occupancy bitmap, count, read the
     number of outputs back, emit rows and table entries in ascending order.  None when the grid
-    is larger than that (decided on the device; costs the same one read-back)."""
+    is larger than that (decided on the device; costs the same one read-back).  ``ahead`` more
+    levels of the same geometry are computed before the read-back and left in ``_ahead``."""
     n = coords.shape[0]
     dev = coords.device
     bits = min(max(1 << (n * fan * 2048 - 1).bit_length(), 1 << 20), 1 << 30)
     entry = _grid_bitmap(dev, bits // 32)
-    words = entry[1]
-    bitmap, chunk_counts = entry[0][:words], entry[0][words:]
-    counters = table.counters
-    in_max = counters[4:8]  # zero on a fresh table
+    layout, _ = _grid_layout(entry[1])
+    buf = entry[0]
+    levels = 1 + ahead
+    # per level 8 counters: [n_out, table overflow, grid too large, -, max b, x, y, z of the INPUTS]
+    ctr = table.counters if levels == 1 else torch.zeros(8 * levels, dtype=torch.int32, device=dev)
     s = _stream()
-    _check(_C.tsmi_coords_max(s, _ptr(coords), n, _ptr(in_max), 0))
+    g = (_I3(*ks), _I3(*st), _I3(*pd))
     host_max = _I3(*[int(v) for v in coords_max_host]) if coords_max_host is not None else None
-    entry[2] = True  # marked bits stay behind unless the emit pass below runs
-    _check(_C.tsmi_downsample_grid_count(s, _ptr(coords), n, _I3(*ks), _I3(*st), _I3(*pd), host_max,
-                                         _ptr(in_max), _ptr(bitmap), words, 0, _ptr(chunk_counts),
-                                         _ptr(counters)))
-    host = counters.tolist()
-    n_out, too_large = host[0], host[2]
-    if too_large:
-        entry[2] = False  # nothing was marked
+
+    def part(level, what):
+        if what == "in_max":
+            return ctr[8 * level + 4:8 * level + 8] if level < levels else None
+        off, w, cc = layout[level]
+        if what == "bitmap":
+            return buf[off:off + w]
+        if what == "chunks":
+            return buf[cc:cc + w // _GRID_CHUNK_WORDS]
+        return ctr[8 * level:8 * level + 8]  # "counters"
+
+    _check(_C.tsmi_coords_max(s, _ptr(coords), n, _ptr(part(0, "in_max")), 0))
+    entry[2] = True  # marked bits stay behind unless the emit passes below run
+    _check(_C.tsmi_downsample_grid_count(s, _ptr(coords), n, *g, host_max, _ptr(part(0, "in_max")),
+                                         _ptr(part(0, "bitmap")), layout[0][1], 0,
+                                         _ptr(part(0, "chunks")), _ptr(part(0, "counters")),
+                                         _ptr(part(1, "in_max"))))
+    for level in range(1, levels):
+        _check(_C.tsmi_downsample_grid_count_next(
+            s, *g, _ptr(part(level - 1, "in_max")), _ptr(part(level - 1, "bitmap")), layout[level - 1][1],
+            _ptr(part(level, "in_max")), _ptr(part(level, "bitmap")), layout[level][1],
+            _ptr(part(level, "chunks")), _ptr(part(level, "counters")), _ptr(part(level + 1, "in_max"))))
+    host = ctr.tolist()
+    if host[2]:
+        entry[2] = False  # nothing was marked, at any level
         return None
-    if n_out > table.capacity:
-        if fan > 2:  # more than the two outputs per input the first table reserves
-            table = GPUHashTable(hash_capacity(n * fan, rsv_ratio), device=dev)
-        if n_out > table.capacity:
+
+    def emit(level, n_in, tbl):
+        n_out = host[8 * level]
+        if n_out > tbl.capacity and fan > 2:  # more than the two outputs per input reserved
+            tbl = GPUHashTable(hash_capacity(n_in * fan, rsv_ratio), device=dev)
+        if n_out > tbl.capacity:
             raise ValueError(
                 "The capacity of hashtable is not sufficient. Please enlarge reserved space for "
                 "hashtable:\n # Python \nimport torchsparse_amd.backends\n"
                 "torchsparse_amd.backends.hash_rsv_ratio=#Value")
-    out_coords = torch.empty((n_out, 4), dtype=torch.int32, device=dev)
-    if n_out > 0:
-        _check(_C.tsmi_downsample_grid_emit(s, _I3(*ks), _I3(*st), _I3(*pd), host_max, _ptr(in_max),
-                                            (ctypes.c_int32 * 4)(*host[4:8]),
-                                            _ptr(bitmap), words, _ptr(chunk_counts), n_out,
-                                            _ptr(table.keys), _ptr(table.vals), table.capacity,
-                                            _ptr(out_coords), _ptr(table.counters)))
-    entry[2] = False
-    return out_coords, table
+        out = torch.empty((n_out, 4), dtype=torch.int32, device=dev)
+        if n_out > 0:
+            _check(_C.tsmi_downsample_grid_emit(
+                s, *g, host_max, _ptr(part(level, "in_max")),
+                (ctypes.c_int32 * 4)(*host[8 * level + 4:8 * level + 8]), _ptr(part(level, "bitmap")),
+                layout[level][1], _ptr(part(level, "chunks")), n_out, _ptr(tbl.keys), _ptr(tbl.vals),
+                tbl.capacity, _ptr(out), _ptr(tbl.counters)))
+        return out, tbl
+
+    first = emit(0, n, table)
+    prev = first[0]
+    clean = True
+    for level in range(1, levels):
+        if prev.shape[0] == 0:
+            break  # no inputs: nothing was marked from here on
+        if host[8 * level + 2]:
+            break  # this level's grid did not fit its bitmap: it and the later ones marked nothing
+        n_in = prev.shape[0]
+        try:
+            nxt = emit(level, n_in, GPUHashTable(hash_capacity(n_in * min(fan, 2), rsv_ratio), device=dev))
+        except ValueError:  # not asked for yet: let the call that asks raise it
+            clean = False  # this level's marks (and the later ones') are still in the bitmaps
+            break
+        _ahead[id(prev)] = (weakref.ref(prev), (ks, st, pd, rsv_ratio), nxt[0], nxt[1])
+        prev = nxt[0]
+    entry[2] = not clean
+    return first
 
 
 def build_kernel_map_downsample_hashmap(in_table: Optional[GPUHashTable], coords, coords_min,

@@ -173,6 +173,66 @@ __host__ __device__ __forceinline__ void output_range(const Geom &g, int a, int3
   *lo = in_min_dev ? (in_min_dev[1 + a] - 2 * g.pad[a] + (g.ks[a] - 1)) / g.stride[a] : 0;
 }
 
+// Candidate j of the input coordinate c = (b, x, y, z) for modes 0, 1 and 2 (one candidate,
+// j = 0, in modes 1 and 2) inside the output range [lo, hi] per axis (unused in mode 1); false
+// when there is none.
+__device__ __forceinline__ bool strided_candidate_in(int4 c, int j, const Geom &g, const int *lo,
+                                                     const int *hi, int mode, int *b, int *o) {
+  *b = c.x;
+  const int v[3] = {c.y, c.z, c.w};
+  if (mode != 0) {
+    // one candidate per input: o = floor(in / stride).  mode 1 keeps it unbounded; mode 2
+    // is the strided-convolution rule specialised to kernel size == stride, zero padding
+    // (o*s <= in < o*s + k has exactly one solution), bounded like mode 0.
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+      int q = v[a] / g.stride[a];
+      if (v[a] % g.stride[a] != 0 && v[a] < 0) --q;
+      o[a] = q;
+      if (mode == 2 && (o[a] < lo[a] || o[a] > hi[a])) return false;
+    }
+  } else {
+    // o = (in + pad + d - (ks-1)) / stride for the digits d in [0, ks) that make the division
+    // exact: per axis d = r, r + stride, ... with r = (ks-1 - in - pad) mod stride, at most
+    // ceil(ks / stride) of them; j numbers the combinations of such digits.
+    const int f0 = (g.ks[0] + g.stride[0] - 1) / g.stride[0];
+    const int f1 = (g.ks[1] + g.stride[1] - 1) / g.stride[1];
+    const int jj[3] = {j % f0, (j / f0) % f1, j / (f0 * f1)};
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+      int r = (g.ks[a] - 1 - v[a] - g.pad[a]) % g.stride[a];
+      if (r < 0) r += g.stride[a];
+      const int d = r + jj[a] * g.stride[a];
+      if (d >= g.ks[a]) return false;
+      o[a] = (v[a] + g.pad[a] + d - (g.ks[a] - 1)) / g.stride[a];  // exact
+      if (o[a] < lo[a] || o[a] > hi[a]) return false;
+    }
+  }
+  return coords_packable(*b, o[0], o[1], o[2]);
+}
+
+__device__ __forceinline__ void output_ranges(const Geom &g, int3 out_max_host, const int32_t *in_max_dev,
+                                              const int32_t *in_min_dev, int mode, int *lo, int *hi) {
+#pragma unroll
+  for (int a = 0; a < 3; ++a) {
+    lo[a] = hi[a] = 0;
+    if (mode != 1) output_range(g, a, out_max_host, in_max_dev, in_min_dev, &lo[a], &hi[a]);
+  }
+}
+
+__device__ __forceinline__ bool strided_candidate(int4 c, int j, const Geom &g, int3 out_max_host,
+                                                  const int32_t *in_max_dev, const int32_t *in_min_dev,
+                                                  int mode, int *b, int *o) {
+  int lo[3], hi[3];
+  output_ranges(g, out_max_host, in_max_dev, in_min_dev, mode, lo, hi);
+  return strided_candidate_in(c, j, g, lo, hi, mode, b, o);
+}
+
+__device__ __forceinline__ int strided_fan(const Geom &g) {
+  return ((g.ks[0] + g.stride[0] - 1) / g.stride[0]) * ((g.ks[1] + g.stride[1] - 1) / g.stride[1]) *
+         ((g.ks[2] + g.stride[2] - 1) / g.stride[2]);
+}
+
 // The candidate output coordinate of thread `tid`; false when the thread has none.
 // mode 0: thread per (input, exactly dividing offset); modes 1 and 2: thread per input; mode 3 (generative
 // upsampling): thread per (input, offset), o = clamp(in * stride + digit - (ks-1)/2, 0, max).
@@ -193,51 +253,13 @@ __device__ __forceinline__ bool downsample_candidate(int64_t tid, const int4 *in
       const int hi = a == 0 ? out_max_host.x : (a == 1 ? out_max_host.y : out_max_host.z);
       o[a] = min(max(v[a] * g.stride[a] + d[a] - (g.ks[a] - 1) / 2, 0), hi);
     }
-  } else if (mode != 0) {
-    // one candidate per input: o = floor(in / stride).  mode 1 keeps it unbounded; mode 2
-    // is the strided-convolution rule specialised to kernel size == stride, zero padding
-    // (o*s <= in < o*s + k has exactly one solution), bounded like mode 0.
-    int4 c = in_coords[tid];
-    *b = c.x;
-    int v[3] = {c.y, c.z, c.w};
-#pragma unroll
-    for (int a = 0; a < 3; ++a) {
-      int q = v[a] / g.stride[a];
-      if (v[a] % g.stride[a] != 0 && v[a] < 0) --q;
-      o[a] = q;
-      if (mode == 2) {
-        int lo, hi;
-        output_range(g, a, out_max_host, in_max_dev, in_min_dev, &lo, &hi);
-        if (o[a] < lo || o[a] > hi) return false;
-      }
-    }
-  } else {
-    // o = (in + pad + d - (ks-1)) / stride for the digits d in [0, ks) that make the division
-    // exact: per axis d = r, r + stride, ... with r = (ks-1 - in - pad) mod stride, at most
-    // ceil(ks / stride) of them.  One thread per (input, combination of such digits).
-    const int f0 = (g.ks[0] + g.stride[0] - 1) / g.stride[0];
-    const int f1 = (g.ks[1] + g.stride[1] - 1) / g.stride[1];
-    const int f2 = (g.ks[2] + g.stride[2] - 1) / g.stride[2];
-    const int fan = f0 * f1 * f2;
-    int64_t i = tid / fan;
-    int j = (int)(tid - i * fan);
-    const int jj[3] = {j % f0, (j / f0) % f1, j / (f0 * f1)};
-    int4 c = in_coords[i];
-    *b = c.x;
-    int v[3] = {c.y, c.z, c.w};
-#pragma unroll
-    for (int a = 0; a < 3; ++a) {
-      int r = (g.ks[a] - 1 - v[a] - g.pad[a]) % g.stride[a];
-      if (r < 0) r += g.stride[a];
-      const int d = r + jj[a] * g.stride[a];
-      if (d >= g.ks[a]) return false;
-      o[a] = (v[a] + g.pad[a] + d - (g.ks[a] - 1)) / g.stride[a];  // exact
-      int lo, hi;
-      output_range(g, a, out_max_host, in_max_dev, in_min_dev, &lo, &hi);
-      if (o[a] < lo || o[a] > hi) return false;
-    }
+    return coords_packable(*b, o[0], o[1], o[2]);
   }
-  return coords_packable(*b, o[0], o[1], o[2]);
+  if (mode != 0) return strided_candidate(in_coords[tid], 0, g, out_max_host, in_max_dev, in_min_dev, mode, b, o);
+  const int fan = strided_fan(g);
+  const int64_t i = tid / fan;
+  return strided_candidate(in_coords[i], (int)(tid - i * fan), g, out_max_host, in_max_dev, in_min_dev,
+                           mode, b, o);
 }
 
 __global__ void downsample_candidates_kernel(const int4 *in_coords, int64_t n_in, int64_t total,
@@ -304,23 +326,45 @@ __global__ void grid_clear_kernel(uint4 *bitmap, int64_t cap_words, Geom g, int3
 // Inputs usually arrive sorted, so the candidates of neighbouring lanes fall into the same
 // bitmap word: lanes OR their bits into the last lane of each run of equal words and only
 // that lane issues the atomic (any split of the runs is still right, only less thrifty).
+// Per-column maximum of the block's (b, x, y, z), raised into out_max[4] (zero before the
+// launch; threads without a coordinate pass zeros).  Every thread of the block must call it.
+__device__ __forceinline__ void block_raise_max(int b, int x, int y, int z, int32_t *out_max) {
+  __shared__ int wave_max[kBlock / 64][4];
+  int v[4] = {b, x, y, z};
+#pragma unroll
+  for (int a = 0; a < 4; ++a) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v[a] = max(v[a], __shfl_xor(v[a], off));
+    if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6][a] = v[a];
+  }
+  __syncthreads();
+  if (threadIdx.x < 4) {
+    const int m = max(max(wave_max[0][threadIdx.x], wave_max[1][threadIdx.x]),
+                      max(wave_max[2][threadIdx.x], wave_max[3][threadIdx.x]));
+    // the maxima only grow: a stale read that is already large enough spares the atomic
+    if (m > 0 && m > out_max[threadIdx.x]) atomicMax(&out_max[threadIdx.x], m);
+  }
+}
+
 __global__ void grid_mark_kernel(const int4 *in_coords, int64_t total, Geom g, int3 out_max_host,
                                  int has_host_max, const int32_t *in_max_dev, int mode,
-                                 uint32_t *bitmap, int64_t cap_words) {
+                                 uint32_t *bitmap, int64_t cap_words, int32_t *next_in_max) {
   const int64_t tid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   const GridDims d = grid_dims(g, out_max_host, has_host_max, in_max_dev, cap_words);
   if (!d.fits || d.used_words == 0) return;  // the same for every thread
   int word = -1;
   uint32_t bits = 0;
   int b, o[3];
-  if (tid < total &&
-      downsample_candidate(tid, in_coords, g, out_max_host, has_host_max ? nullptr : in_max_dev,
-                           nullptr, mode, &b, o) &&
-      b <= in_max_dev[0]) {
+  const bool have = tid < total &&
+                    downsample_candidate(tid, in_coords, g, out_max_host,
+                                         has_host_max ? nullptr : in_max_dev, nullptr, mode, &b, o) &&
+                    b <= in_max_dev[0];
+  if (have) {
     const uint32_t cell = (((uint32_t)b * d.e[0] + o[0]) * d.e[1] + o[1]) * d.e[2] + o[2];
     word = (int)(cell >> 5);
     bits = 1u << (cell & 31);
   }
+  if (next_in_max) block_raise_max(have ? b : 0, have ? o[0] : 0, have ? o[1] : 0, have ? o[2] : 0, next_in_max);
   const int lane = threadIdx.x & 63;
 #pragma unroll
   for (int off = 1; off < 64; off <<= 1) {
@@ -334,6 +378,92 @@ __global__ void grid_mark_kernel(const int4 *in_coords, int64_t total, Geom g, i
     // bits only costs the atomic
     if ((bitmap[word] & bits) != bits) atomicOr(&bitmap[word], bits);
   }
+}
+
+__device__ __forceinline__ int grid_thread_words(const uint32_t *bitmap, int64_t chunk, uint32_t *w);
+
+// The same marking for the NEXT level of a chain of equal strided convolutions: its inputs are
+// the set bits of the previous level's bitmap (prev_in_max: the maxima that bitmap's extents
+// derive from; in_max: the maxima of its set bits, raised by the launch that marked it).
+// A bounded number of blocks strides over the previous bitmap's chunks; like the emit kernel,
+// a block keeps the chunk's words and the prefix of their bit counts in LDS and thread i takes
+// the chunk's set bits i, i + 256, ... - a walk of each thread's own words would leave the
+// threads over dense words with tens of divisions-heavy candidates and the rest with none.
+__global__ __launch_bounds__(kBlock) void grid_mark_next_kernel(
+    const uint32_t *prev_bitmap, int64_t prev_cap_words, const int32_t *prev_in_max, Geom g, int mode,
+    const int32_t *in_max, uint32_t *bitmap, int64_t cap_words, int32_t *next_in_max) {
+  __shared__ int wave_sum[kBlock / 64];
+  __shared__ uint32_t words[kGridChunkWords];
+  __shared__ int before[kGridChunkWords];
+  const int3 none = make_int3(0, 0, 0);
+  const GridDims pd = grid_dims(g, none, 0, prev_in_max, prev_cap_words);
+  const GridDims d = grid_dims(g, none, 0, in_max, cap_words);
+  if (!pd.fits || !d.fits || d.used_words == 0) return;  // the same for every thread
+  const int fan = mode == 2 ? 1 : strided_fan(g);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const uint32_t e0 = pd.e[0], e1 = pd.e[1], e2 = pd.e[2];
+  int range_lo[3], range_hi[3];
+  output_ranges(g, none, in_max, nullptr, mode, range_lo, range_hi);
+  const int max_batch = in_max[0];
+  int mb = 0, mx = 0, my = 0, mz = 0;
+  const int64_t chunks = pd.used_words / kGridChunkWords;
+  for (int64_t chunk = blockIdx.x; chunk < chunks; chunk += gridDim.x) {
+    uint32_t w[2];
+    const int mine = grid_thread_words(prev_bitmap, chunk, w);
+    int incl = mine;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const int v = __shfl_up(incl, off);
+      if (lane >= off) incl += v;
+    }
+    if (lane == 63) wave_sum[wave] = incl;
+    __syncthreads();
+    int first = incl - mine;
+    for (int v = 0; v < wave; ++v) first += wave_sum[v];
+    words[threadIdx.x * 2] = w[0];
+    words[threadIdx.x * 2 + 1] = w[1];
+    before[threadIdx.x * 2] = first;
+    before[threadIdx.x * 2 + 1] = first + __popc(w[0]);
+    const int chunk_total = wave_sum[0] + wave_sum[1] + wave_sum[2] + wave_sum[3];
+    __syncthreads();
+    for (int i = threadIdx.x; i < chunk_total; i += kBlock) {
+      int lo = 0;
+#pragma unroll
+      for (int step = kGridChunkWords / 2; step > 0; step >>= 1)
+        if (before[lo + step] <= i) lo += step;
+      uint32_t x = words[lo];
+      int k = i - before[lo], pos = 0;
+#pragma unroll
+      for (int half = 16; half > 0; half >>= 1) {
+        const int c = __popc(x & ((1u << half) - 1u));
+        if (k >= c) {
+          k -= c;
+          x >>= half;
+          pos += half;
+        }
+      }
+      uint32_t cell = ((uint32_t)chunk * kGridChunkWords + lo) * 32 + pos;
+      int4 c;
+      c.w = (int)(cell % e2);
+      cell /= e2;
+      c.z = (int)(cell % e1);
+      cell /= e1;
+      c.y = (int)(cell % e0);
+      c.x = (int)(cell / e0);
+      for (int j = 0; j < fan; ++j) {
+        int b, o[3];
+        if (!strided_candidate_in(c, j, g, range_lo, range_hi, mode, &b, o) || b > max_batch) continue;
+        const uint32_t out = (((uint32_t)b * d.e[0] + o[0]) * d.e[1] + o[1]) * d.e[2] + o[2];
+        atomicOr(&bitmap[out >> 5], 1u << (out & 31));  // result unused: nothing waits for it
+        mb = max(mb, b);
+        mx = max(mx, o[0]);
+        my = max(my, o[1]);
+        mz = max(mz, o[2]);
+      }
+    }
+    __syncthreads();  // the LDS arrays are rewritten by the next chunk
+  }
+  if (next_in_max) block_raise_max(mb, mx, my, mz, next_in_max);
 }
 
 __device__ __forceinline__ int grid_thread_words(const uint32_t *bitmap, int64_t chunk, uint32_t *w) {
@@ -1069,7 +1199,8 @@ extern "C" int tsmi_downsample_grid_count(tsmi_stream_t s, const int32_t *in_coo
                                           const int32_t pad[3], const int32_t out_max_host[3],
                                           const int32_t *in_max_dev, int32_t *bitmap,
                                           int64_t bitmap_words, int clear_first,
-                                          int32_t *chunk_counts, int32_t *counters) {
+                                          int32_t *chunk_counts, int32_t *counters,
+                                          int32_t *next_in_max_dev) {
   Geom g;
   int mode;
   int3 hm;
@@ -1091,13 +1222,44 @@ extern "C" int tsmi_downsample_grid_count(tsmi_stream_t s, const int32_t *in_coo
                        bitmap_words, g, hm, has_hm, in_max_dev);
   if (total > 0)
     hipLaunchKernelGGL(grid_mark_kernel, grid_for(total), dim3(kBlock), 0, st, (const int4 *)in_coords,
-                       total, g, hm, has_hm, in_max_dev, mode, (uint32_t *)bitmap, bitmap_words);
+                       total, g, hm, has_hm, in_max_dev, mode, (uint32_t *)bitmap, bitmap_words,
+                       next_in_max_dev);
   hipLaunchKernelGGL(grid_count_kernel, dim3(chunks < 2048u ? chunks : 2048u), dim3(kBlock), 0, st,
                      (const uint32_t *)bitmap,
                      bitmap_words, g, hm, has_hm, in_max_dev, chunk_counts);
   hipLaunchKernelGGL(grid_scan_kernel, dim3(1), dim3(1024), 0, st, chunk_counts, bitmap_words, g, hm,
                      has_hm, in_max_dev, counters);
   return check_launch("tsmi_downsample_grid_count");
+}
+
+extern "C" int tsmi_downsample_grid_count_next(tsmi_stream_t s, const int32_t ks[3],
+                                               const int32_t stride[3], const int32_t pad[3],
+                                               const int32_t *prev_in_max_dev, const int32_t *prev_bitmap,
+                                               int64_t prev_bitmap_words, const int32_t *in_max_dev,
+                                               int32_t *bitmap, int64_t bitmap_words,
+                                               int32_t *chunk_counts, int32_t *counters,
+                                               int32_t *next_in_max_dev) {
+  Geom g;
+  int mode;
+  int3 hm;
+  if (int e = grid_args(&g, &mode, &hm, ks, stride, pad, nullptr, in_max_dev, bitmap, bitmap_words,
+                        chunk_counts, counters))
+    return e;
+  TSMI_REQUIRE(prev_in_max_dev && prev_bitmap && prev_bitmap_words >= kGridChunkWords &&
+                   prev_bitmap_words % kGridChunkWords == 0 && prev_bitmap_words <= (int64_t(1) << 25),
+               "downsample_grid_count_next: bad previous bitmap");
+  hipStream_t st = (hipStream_t)s;
+  const int64_t prev_chunks = prev_bitmap_words / kGridChunkWords;
+  hipLaunchKernelGGL(grid_mark_next_kernel, dim3((unsigned)(prev_chunks < 2048 ? prev_chunks : 2048)),
+                     dim3(kBlock), 0, st, (const uint32_t *)prev_bitmap, prev_bitmap_words,
+                     prev_in_max_dev, g, mode, in_max_dev, (uint32_t *)bitmap, bitmap_words,
+                     next_in_max_dev);
+  const unsigned chunks = (unsigned)(bitmap_words / kGridChunkWords);
+  hipLaunchKernelGGL(grid_count_kernel, dim3(chunks < 2048u ? chunks : 2048u), dim3(kBlock), 0, st,
+                     (const uint32_t *)bitmap, bitmap_words, g, hm, 0, in_max_dev, chunk_counts);
+  hipLaunchKernelGGL(grid_scan_kernel, dim3(1), dim3(1024), 0, st, chunk_counts, bitmap_words, g, hm, 0,
+                     in_max_dev, counters);
+  return check_launch("tsmi_downsample_grid_count_next");
 }
 
 extern "C" int tsmi_downsample_grid_emit(tsmi_stream_t s, const int32_t ks[3], const int32_t stride[3],
