@@ -129,10 +129,11 @@ def test_downsample_through_grid_equals_hash_and_sort(n, shape, batch, geom, mon
     np.testing.assert_array_equal(results[0][0], oracle.kmap_downsample(coords, ks, st, pd)[1])
 
 
-def test_downsample_grid_recovers_from_an_unfinished_call():
+def test_downsample_grid_recovers_from_an_unfinished_call(monkeypatch):
     """The occupancy bitmap is shared by the calls on a stream and must be all zero between them:
     a call that stopped after marking (here: forged, then a real one that raises because the
     output table is too small) is noticed and the bitmap cleared before the next use."""
+    monkeypatch.setattr(backend, "downsample_chain_ahead", False)
     rng = np.random.default_rng(7)
     coords = random_coords(rng, 5000, (60, 50, 40), batch=2)
     want = oracle.kmap_downsample(coords, t3(3), t3(2), t3(1))[1]
@@ -189,6 +190,13 @@ def test_strided_chain_computed_ahead_equals_level_by_level(geom, monkeypatch):
     got = backend.downsample_coords(out, t3(3), t3(2), t3(0))[0].cpu().numpy()
     np.testing.assert_array_equal(got, oracle.kmap_downsample(base[0][0], t3(3), t3(2), t3(0))[1])
     assert not any(entry[2] for entry in backend._grid_scratch.values())
+    # levels computed ahead and never asked for are dropped by the next chain
+    chain(True)
+    out, _ = backend.downsample_coords(dev(coords), ks, st, pd)
+    assert backend._ahead
+    np.testing.assert_array_equal(backend.downsample_coords(dev(coords), ks, st, pd)[0].cpu().numpy(), base[0][0])
+    chain(True)
+    assert not any(entry[2] for entry in backend._grid_scratch.values()) and not backend._ahead
 
 
 def test_table_reuse_across_levels():
