@@ -489,6 +489,34 @@ int tsmi_to_dense_forward(tsmi_stream_t s, const void *feats, const int32_t *coo
 int tsmi_to_dense_backward(tsmi_stream_t s, const void *top_grad, const int32_t *coords, int64_t n,
                            int c, const int32_t *spatial_range, int dtype, void *bottom_grad);
 
+/* ---- batch normalisation of feats [n, c] in training mode ------------------------------
+ * Replaces what nn/modules/norm.py:13-17 reaches through torch.nn.BatchNorm1d on
+ * SparseTensor.feats (forward with batch statistics, running-statistics update, backward).
+ * x, y, dy, dx: [n, c] row-major of `dtype`, 16-byte aligned, c a multiple of 16 bytes' worth
+ * of elements (8 for 16-bit types, 4 for fp32) and at most 256 such pieces.  weight, bias,
+ * running_mean, running_var: [c] of `param_dtype`, each may be null (no affine term, no
+ * running statistics).  partial: fp32 scratch of tsmi_bn_partial_elems(c) elements.  Sums run
+ * in fp32 in a fixed order: results are identical from run to run.
+ *
+ * forward:  stats[4c] (fp32) receives mean[c] and invstd[c] (biased variance,
+ *           1/sqrt(var + eps)), which the backward takes, and 2c values of scratch;
+ *           y = (x - mean) * invstd * weight + bias;
+ *           running_mean = (1 - momentum) * running_mean + momentum * mean,
+ *           running_var likewise with the unbiased variance.
+ * backward: sums[5c] (fp32) receives sum_rows dy (the bias gradient) in [0:c], sum_rows
+ *           dy * xhat (the weight gradient) in [c:2c], xhat = (x - mean) * invstd, and 3c values
+ *           of scratch; grads, when given, receives the same two gradients as [2c] of
+ *           param_dtype;
+ *           dx = weight * invstd * (dy - sums[0:c] / n - xhat * sums[c:2c] / n). */
+int64_t tsmi_bn_partial_elems(int c);
+int tsmi_bn_forward_train(tsmi_stream_t s, const void *x, int64_t n, int c, int dtype,
+                          const void *weight, const void *bias, int param_dtype, void *running_mean,
+                          void *running_var, float momentum, float eps, float *partial, float *stats,
+                          void *y);
+int tsmi_bn_backward(tsmi_stream_t s, const void *dy, const void *x, int64_t n, int c, int dtype,
+                     const void *weight, int param_dtype, const float *mean, const float *invstd,
+                     float *partial, float *sums, void *grads, void *dx);
+
 #pragma GCC visibility pop
 #ifdef __cplusplus
 }

@@ -94,6 +94,10 @@ def _load():
         "tsmi_devoxelize_backward": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _vp],
         "tsmi_to_dense_forward": [_vp, _vp, _vp, _i64, _i32, _I4, _i32, _vp],
         "tsmi_to_dense_backward": [_vp, _vp, _vp, _i64, _i32, _I4, _i32, _vp],
+        "tsmi_bn_forward_train": [_vp, _vp, _i64, _i32, _i32, _vp, _vp, _i32, _vp, _vp, _f32, _f32, _vp, _vp,
+                                  _vp],
+        "tsmi_bn_partial_elems": [_i32],
+        "tsmi_bn_backward": [_vp, _vp, _vp, _i64, _i32, _i32, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _vp],
         "tsmi_gs_gather": [_vp, _vp, _vp, _i64, _i32, _i32, _i32, _vp],
         "tsmi_gs_gemm": [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _i32, _i32, _vp],
         "tsmi_gs_scatter": [_vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _vp, _vp, _i32, _vp],
@@ -1137,3 +1141,51 @@ def to_dense_backward_cuda(top_grad: torch.Tensor, idx: torch.Tensor, spatial_ra
     rng = [int(v) for v in (spatial_range.tolist() if torch.is_tensor(spatial_range) else spatial_range)]
     _check(_C.tsmi_to_dense_backward(_stream(), _ptr(g), _ptr(idx), out.shape[0], out.shape[1], _I4(*rng),
                                      _dtype_code(g), _ptr(out)))
+
+
+# ------------------------------------------------------------------ batch normalisation
+
+
+def bn_supported(x: torch.Tensor, *params) -> bool:
+    """Whether the batch-norm kernels take this [N, C] matrix: GPU, contiguous, a supported
+    type, N >= 2, C a multiple of 16 bytes' worth of elements (at most 256 such pieces), and
+    every parameter / running statistic given of one supported type."""
+    if not (x.is_cuda and x.dim() == 2 and x.dtype in _DTYPE_CODE and x.is_contiguous() and x.shape[0] >= 2):
+        return False
+    v = 4 if x.dtype == torch.float32 else 8
+    if x.shape[1] < v or x.shape[1] % v or x.shape[1] // v > 256 or x.data_ptr() % 16:
+        return False
+    given = [p for p in params if p is not None]
+    return all(p.is_cuda and p.dtype in _DTYPE_CODE and p.dtype == given[0].dtype and p.is_contiguous()
+               and p.numel() == x.shape[1] for p in given)
+
+
+def bn_forward_train(x, weight, bias, running_mean, running_var, momentum: float, eps: float):
+    """(y, mean, invstd): batch statistics over the rows of x [N, C], running statistics updated in
+    place — what torch.nn.functional.batch_norm(training=True) does for nn/modules/norm.py:13-17."""
+    n, c = x.shape
+    given = [p for p in (weight, bias, running_mean, running_var) if p is not None]
+    pcode = _dtype_code(given[0]) if given else F32
+    work = torch.empty(_C.tsmi_bn_partial_elems(c), dtype=torch.float32, device=x.device)
+    stats = torch.empty(4 * c, dtype=torch.float32, device=x.device)
+    y = torch.empty_like(x)
+    _check(_C.tsmi_bn_forward_train(_stream(), _ptr(x), n, c, _dtype_code(x), _ptr(weight), _ptr(bias), pcode,
+                                    _ptr(running_mean), _ptr(running_var), float(momentum), float(eps),
+                                    _ptr(work), _ptr(stats), _ptr(y)))
+    return y, stats[:c], stats[c:2 * c]
+
+
+def bn_backward(dy, x, weight, mean, invstd):
+    """(dx, sum_rows dy * xhat, sum_rows dy): the input, weight and bias gradients (the last two in
+    the weight's type; fp32 without a weight)."""
+    n, c = x.shape
+    work = torch.empty(_C.tsmi_bn_partial_elems(c), dtype=torch.float32, device=x.device)
+    sums = torch.empty(5 * c, dtype=torch.float32, device=x.device)
+    dx = torch.empty_like(x)
+    pcode = _dtype_code(weight) if weight is not None else F32
+    grads = torch.empty(2 * c, dtype=weight.dtype, device=x.device) if weight is not None else None
+    _check(_C.tsmi_bn_backward(_stream(), _ptr(dy), _ptr(x), n, c, _dtype_code(x), _ptr(weight), pcode,
+                               _ptr(mean), _ptr(invstd), _ptr(work), _ptr(sums), _ptr(grads), _ptr(dx)))
+    if grads is not None:
+        return dx, grads[c:], grads[:c]
+    return dx, sums[c:2 * c], sums[:c]

@@ -19,6 +19,7 @@ SOURCES = [
     "kmap.hip",
     "sort.hip",
     "pointops.hip",
+    "norm.hip",
     "conv_api.cpp",
     "conv_igemm_f16.hip",
     "conv_igemm_bf16.hip",
