@@ -8,6 +8,7 @@ eager fallback: if the shared object is missing, importing this module raises.
 """
 import ctypes
 import os
+import threading
 import weakref
 from typing import List, Optional, Sequence, Tuple
 
@@ -422,7 +423,15 @@ def _grid_bitmap(dev: torch.device, words: int):
     return entry
 
 
+_grid_lock = threading.Lock()  # one call at a time between marking a scratch bitmap and emitting from it
+
+
 def _downsample_coords_grid(coords, ks, st, pd, coords_max_host, fan, rsv_ratio, table, ahead=0):
+    with _grid_lock:
+        return _downsample_coords_grid_locked(coords, ks, st, pd, coords_max_host, fan, rsv_ratio, table, ahead)
+
+
+def _downsample_coords_grid_locked(coords, ks, st, pd, coords_max_host, fan, rsv_ratio, table, ahead=0):
     """downsample_coords for non-negative coordinates when the output grid has at most
     2048 cells per candidate (and at most 2^30): mark an occupancy bitmap, count, read the
     number of outputs back, emit rows and table entries in ascending order.  None when the grid
