@@ -192,3 +192,40 @@ def test_kernel_maps_of_arbitrary_geometry(mods, seed):
         nb, sz = oracle.pair_lists(want_map[:n_out])
         assert np.array_equal(pl["nbsizes"].cpu().numpy(), sz), what
         assert np.array_equal(pl["nbmaps_inter"].cpu().numpy(), nb), what
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_chains_of_equal_strided_layers(mods, seed):
+    """One to four equal strided layers, each on the previous one's output coordinates, three
+    passes: the later passes take the levels that the first call of the chain computed ahead
+    through the occupancy bitmaps.  Coordinates, their order and the output tables against the
+    oracle, level by level."""
+    from torchsparse_amd import backend
+    rng = np.random.default_rng(4000 + seed)
+    for _ in range(6):
+        ks = tuple(int(v) for v in rng.integers(1, 6, 3))
+        st = tuple(int(v) for v in rng.integers(1, 4, 3))
+        if all(s == 1 for s in st):
+            st = (2, st[1], st[2])
+        pd = tuple(int(v) for v in rng.integers(0, 3, 3))
+        n = int(rng.choice([1, 7, 300, 5000, 40000]))
+        ext = tuple(int(v) for v in rng.choice([3, 17, 64, 300, 2000], 3))
+        batch = int(rng.integers(1, 4))
+        cols = [rng.integers(0, batch, n)] + [rng.integers(0, e, n) for e in ext]
+        coords = np.unique(np.stack(cols, 1).astype(np.int32), axis=0)
+        coords = coords[rng.permutation(len(coords))]
+        want, c = [], coords
+        for _ in range(int(rng.integers(1, 5))):
+            c = oracle.kmap_downsample(c, ks, st, pd)[1]
+            want.append(c)
+            if len(c) == 0:
+                break
+        for rep in range(3):
+            c = torch.from_numpy(coords).cuda()
+            for level, w in enumerate(want):
+                out, table = backend.downsample_coords(c, ks, st, pd)
+                rows = table.query_bxyz(out, (1, 1, 1), (1, 1, 1), (0, 0, 0))[:out.shape[0], 0]
+                case = f"ks={ks} st={st} pd={pd} n={len(coords)} ext={ext} pass={rep} level={level}"
+                np.testing.assert_array_equal(out.cpu().numpy(), w, err_msg=case)
+                np.testing.assert_array_equal(rows.cpu().numpy(), np.arange(len(w)), err_msg=case)
+                c = out
