@@ -136,3 +136,55 @@ def test_synthetic_workloads_are_seeded_and_sized():
     assert len(np.unique(a, axis=0)) == len(a)
     c = uniform_voxels(20000, 128, seed=0)
     assert c.shape == (20000, 4) and len(np.unique(c, axis=0)) == 20000 and c[:, 1:].max() < 128
+
+
+def test_strided_chain_bookkeeping_with_interleaved_chains():
+    """The look-ahead of chains of equal strided convolutions is book-keeping per (device,
+    stream).  Two states fed interleaved chains never see each other's levels; inside one
+    state a chain interrupted by another geometry hands out nothing computed for the old one."""
+    import weakref
+    from torchsparse_amd import backend
+    geom_a, geom_b = ((2, 2, 2), (2, 2, 2), (0, 0, 0), 2.0), ((3, 3, 3), (2, 2, 2), (1, 1, 1), 2.0)
+    mk = lambda: torch.zeros(1, 4, dtype=torch.int32)
+
+    def run_chain(state, geom, length, levels):
+        """Calls chain_step like downsample_coords does; returns what each call got."""
+        got, c = [], levels[0]
+        for i in range(length):
+            r = state.chain_step(c, geom)
+            got.append(r)
+            if isinstance(r, int):
+                for j in range(r):  # what the grid path leaves behind for the levels ahead
+                    state.ahead[id(levels[i + j + 1])] = (weakref.ref(levels[i + j + 1]), geom,
+                                                          levels[i + j + 2], "table%d" % (i + j + 2))
+                state.chain_last = weakref.ref(levels[i + 1])
+            c = levels[i + 1]
+        return got
+
+    s1, s2 = backend._StridedState(), backend._StridedState()
+    lv1, lv2 = [mk() for _ in range(6)], [mk() for _ in range(6)]
+    assert run_chain(s1, geom_a, 4, lv1) == [0, 0, 0, 0]       # nothing known yet
+    assert run_chain(s2, geom_b, 2, lv2) == [0, 0]
+    second = run_chain(s1, geom_a, 4, lv1)                      # learnt: 3 levels ahead, then hits
+    assert second[0] == 3 and [r[0] is lv1[i + 1] for i, r in enumerate(second[1:], 1)] == [True] * 3
+    assert s1.ahead_hits == 3 and s2.ahead_hits == 0 and not s2.ahead
+    third = run_chain(s2, geom_b, 2, lv2)                       # the other state learnt its own length
+    assert third[0] == 1 and third[1][0] is lv2[2] and s1.chain_len == {geom_a: 4}
+    # one state, chains interleaved: A starts (computes ahead), B interrupts, A's next level asks
+    assert s1.chain_step(lv1[0], geom_a) == 3
+    for j in range(1, 4):
+        s1.ahead[id(lv1[j])] = (weakref.ref(lv1[j]), geom_a, lv1[j + 1], "t")
+    s1.chain_last = weakref.ref(lv1[1])
+    assert s1.chain_step(lv2[0], geom_b) == 0 and not s1.ahead  # B starts: A's levels are dropped
+    r = s1.chain_step(lv1[1], geom_a)                           # A resumes as a new chain
+    assert isinstance(r, int)
+    # a level computed ahead for a tensor that died is not handed to a new tensor at its address
+    s3 = backend._StridedState()
+    dead = mk()
+    s3.ahead[id(dead)] = (weakref.ref(dead), geom_a, lv1[1], "t")
+    s3.chain_geom, s3.chain_last = geom_a, weakref.ref(dead)
+    key = id(dead)
+    del dead
+    fresh = mk()
+    s3.ahead[id(fresh)] = s3.ahead.pop(key)  # worst case: the allocator reused the address
+    assert isinstance(s3.chain_step(fresh, geom_a), int)

@@ -139,15 +139,15 @@ def test_downsample_grid_recovers_from_an_unfinished_call(monkeypatch):
     want = oracle.kmap_downsample(coords, t3(3), t3(2), t3(1))[1]
     args = (dev(coords), t3(3), t3(2), t3(1))
     np.testing.assert_array_equal(backend.downsample_coords(*args)[0].cpu().numpy(), want)
-    assert backend._grid_scratch
-    for entry in backend._grid_scratch.values():
-        entry[0][:entry[1]].fill_(-1)
-        entry[2] = True
+    assert backend._stream_states
+    for state in backend._stream_states.values():
+        state.grid_buf[:state.grid_words].fill_(-1)
+        state.grid_dirty = True
     np.testing.assert_array_equal(backend.downsample_coords(*args)[0].cpu().numpy(), want)
     with pytest.raises(ValueError, match="capacity of hashtable"):
         backend.downsample_coords(*args, rsv_ratio=0.001)
     np.testing.assert_array_equal(backend.downsample_coords(*args)[0].cpu().numpy(), want)
-    assert not any(entry[2] for entry in backend._grid_scratch.values())
+    assert not any(state.grid_dirty for state in backend._stream_states.values())
 
 
 @pytest.mark.parametrize("geom", [(2, 2, 0), (3, 2, 1), ((2, 2, 1), (2, 2, 1), (0, 0, 0))])
@@ -162,6 +162,7 @@ def test_strided_chain_computed_ahead_equals_level_by_level(geom, monkeypatch):
     real = backend._downsample_coords_grid
     monkeypatch.setattr(backend, "_downsample_coords_grid",
                         lambda *a, **k: (calls.append(a[-1] if not k else k.get("ahead")), real(*a, **k))[1])
+    backend.release_scratch()  # no chain history from earlier tests
 
     def chain(ahead):
         monkeypatch.setattr(backend, "downsample_chain_ahead", ahead)
@@ -174,7 +175,7 @@ def test_strided_chain_computed_ahead_equals_level_by_level(geom, monkeypatch):
         return outs
 
     base = chain(False)
-    chain(True)  # the chain is learnt here (or was, by an earlier test)
+    chain(True)  # the chain is learnt here
     del calls[:]
     ahead = chain(True)
     assert calls == [3], calls  # one call marks four levels, three calls return what it left
@@ -189,14 +190,15 @@ def test_strided_chain_computed_ahead_equals_level_by_level(geom, monkeypatch):
     out, _ = backend.downsample_coords(dev(coords), ks, st, pd)
     got = backend.downsample_coords(out, t3(3), t3(2), t3(0))[0].cpu().numpy()
     np.testing.assert_array_equal(got, oracle.kmap_downsample(base[0][0], t3(3), t3(2), t3(0))[1])
-    assert not any(entry[2] for entry in backend._grid_scratch.values())
+    assert not any(state.grid_dirty for state in backend._stream_states.values())
     # levels computed ahead and never asked for are dropped by the next chain
     chain(True)
     out, _ = backend.downsample_coords(dev(coords), ks, st, pd)
-    assert backend._ahead
+    state, = backend._stream_states.values()
+    assert state.ahead and state.ahead_hits > 0
     np.testing.assert_array_equal(backend.downsample_coords(dev(coords), ks, st, pd)[0].cpu().numpy(), base[0][0])
     chain(True)
-    assert not any(entry[2] for entry in backend._grid_scratch.values()) and not backend._ahead
+    assert not state.grid_dirty and not state.ahead
 
 
 def test_table_reuse_across_levels():

@@ -6,6 +6,7 @@ PyTorch is used for device memory and the current HIP stream; every computation
 below happens in the hand-written HIP kernels of ``csrc/``.  There is no CPU or
 eager fallback: if the shared object is missing, importing this module raises.
 """
+import collections
 import ctypes
 import os
 import threading
@@ -305,19 +306,24 @@ def downsample_coords(coords: torch.Tensor, kernel_sizes, stride, padding, coord
         cap = hash_capacity(n * (fan if _reserve_all else min(fan, 2)), rsv_ratio)
     through_grid = (mode == 0 and not allow_negative and n > 0 and downsample_through_grid
                     and not _reserve_all)
+    table = None
     if through_grid:
-        chain = (ks, st, pd, rsv_ratio) if coords_max_host is None else None
-        ahead = _chain_step(coords, chain)
-        if not isinstance(ahead, int):  # computed ahead when the previous level of the chain was
-            return ahead
-    table = GPUHashTable(cap, device=dev)
+        with _state_lock:
+            state = _strided_state(dev)
+            chain = (ks, st, pd, rsv_ratio) if coords_max_host is None else None
+            ahead = state.chain_step(coords, chain)
+            if not isinstance(ahead, int):  # computed ahead when the previous level of the chain was
+                return ahead
+            table = GPUHashTable(cap, device=dev)
+            done = _downsample_coords_grid(state, coords, ks, st, pd, coords_max_host, fan, rsv_ratio,
+                                           table, ahead)
+            if done is not None:
+                state.chain_last = weakref.ref(done[0])
+                return done
+        table.counters.zero_()
+    if table is None:
+        table = GPUHashTable(cap, device=dev)
     counters = table.counters  # zero on a fresh table
-    if through_grid:
-        done = _downsample_coords_grid(coords, ks, st, pd, coords_max_host, fan, rsv_ratio, table, ahead)
-        if done is not None:
-            _chain["last"] = weakref.ref(done[0])
-            return done
-        counters.zero_()
     in_max = in_min = None
     host_max = None
     if mode == 3:
@@ -369,31 +375,84 @@ downsample_through_grid = True
 downsample_chain_ahead = True
 _GRID_CHUNK_WORDS = 512
 _GRID_LEVELS = 4  # the level asked for and up to three ahead
-_grid_scratch = {}  # (device index, stream) -> [int32 buffer, bitmap words of level 0, in flight]
-_chain = {"geom": None, "last": None, "len": 0}  # the chain of equal strided calls in progress
-_chain_len = {}  # geometry -> length of the last chain that ended
-_ahead = {}  # id(coords) -> (weak reference to coords, geometry, out_coords, table)
+_MAX_STREAM_STATES = 8  # (device, stream) pairs whose scratch is kept; the least recently used goes
 
 
-def _chain_step(coords, geom):
-    """Book-keeping of chains of equal strided calls (each on the previous one's outputs).  Returns
-    the (out_coords, table) computed ahead for ``coords``, or the number of levels to compute ahead
-    now."""
-    hit = _ahead.pop(id(coords), None)
-    last = _chain["last"]() if _chain["last"] is not None else None
-    if geom is not None and _chain["geom"] == geom and last is coords:
-        _chain["len"] += 1
-        if hit is not None and hit[0]() is coords and hit[1] == geom and downsample_chain_ahead:
-            _chain["last"] = weakref.ref(hit[2])
-            return hit[2], hit[3]
-        return 0
-    if _chain["geom"] is not None:
-        _chain_len[_chain["geom"]] = _chain["len"]
-    _chain["geom"], _chain["len"], _chain["last"] = geom, 1, None
-    _ahead.clear()
-    if geom is None or not downsample_chain_ahead:
-        return 0
-    return min(_chain_len.get(geom, 1) - 1, _GRID_LEVELS - 1)
+class _StridedState:
+    """What the strided-coordinate path keeps between calls, for ONE (device, stream): the
+    occupancy-bitmap scratch, the chain of equal strided calls in progress, the lengths of the
+    chains seen, and the levels computed ahead.  Everything in it was produced by work queued
+    on that stream, so a later call on the same stream is ordered after it; calls on another
+    stream (or device) get a state of their own and never see these tensors."""
+    __slots__ = ("grid_buf", "grid_words", "grid_dirty", "chain_geom", "chain_last", "chain_count",
+                 "chain_len", "ahead", "ahead_hits")
+
+    def __init__(self):
+        self.grid_buf = None      # int32 scratch: bitmaps and chunk counts of every level
+        self.grid_words = 0       # bitmap words of level 0 the scratch was laid out for
+        self.grid_dirty = False   # a call marked bits and did not reach its emit passes
+        self.chain_geom = None    # geometry of the chain in progress
+        self.chain_last = None    # weak reference to the last output of that chain
+        self.chain_count = 0
+        self.chain_len = {}       # geometry -> length of the last chain that ended
+        self.ahead = {}           # id(coords) -> (weakref(coords), geometry, out_coords, table)
+        self.ahead_hits = 0       # calls answered from `ahead` (diagnostic)
+
+    def chain_step(self, coords, geom):
+        """Book-keeping of chains of equal strided calls (each on the previous one's outputs).
+        Returns the (out_coords, table) computed ahead for ``coords``, or the number of levels
+        to compute ahead now."""
+        hit = self.ahead.pop(id(coords), None)
+        last = self.chain_last() if self.chain_last is not None else None
+        if geom is not None and self.chain_geom == geom and last is coords:
+            self.chain_count += 1
+            if hit is not None and hit[0]() is coords and hit[1] == geom and downsample_chain_ahead:
+                self.chain_last = weakref.ref(hit[2])
+                self.ahead_hits += 1
+                return hit[2], hit[3]
+            return 0
+        if self.chain_geom is not None:
+            self.chain_len[self.chain_geom] = self.chain_count
+        self.chain_geom, self.chain_count, self.chain_last = geom, 1, None
+        self.ahead.clear()
+        if geom is None or not downsample_chain_ahead:
+            return 0
+        return min(self.chain_len.get(geom, 1) - 1, _GRID_LEVELS - 1)
+
+    def bitmap(self, dev: torch.device, words: int):
+        """The all-zero scratch whose first bitmap has at least ``words`` words.  Every call
+        leaves the bitmaps zero again; one that did not finish has them cleared here."""
+        if self.grid_buf is None or self.grid_words < words:
+            self.grid_buf = torch.zeros(_grid_layout(words)[1], dtype=torch.int32, device=dev)
+            self.grid_words, self.grid_dirty = words, False
+        elif self.grid_dirty:
+            self.grid_buf.zero_()
+            self.grid_dirty = False
+        return self.grid_buf
+
+
+_stream_states = collections.OrderedDict()  # (device index, stream) -> _StridedState
+_state_lock = threading.RLock()  # guards _stream_states and every _StridedState
+
+
+def _strided_state(dev: torch.device) -> _StridedState:
+    """State of the current stream of ``dev`` (call with _state_lock held)."""
+    key = (dev.index if dev.index is not None else _cur_device(), _stream())
+    st = _stream_states.get(key)
+    if st is None:
+        st = _stream_states[key] = _StridedState()
+        while len(_stream_states) > _MAX_STREAM_STATES:
+            _stream_states.popitem(last=False)
+    else:
+        _stream_states.move_to_end(key)
+    return st
+
+
+def release_scratch() -> None:
+    """Drop the scratch bitmaps, the levels computed ahead and the chain history of every
+    stream (up to ~170 MB of device memory per stream that ran a large strided map)."""
+    with _state_lock:
+        _stream_states.clear()
 
 
 def _grid_layout(words0: int):
@@ -409,40 +468,18 @@ def _grid_layout(words0: int):
     return out, off
 
 
-def _grid_bitmap(dev: torch.device, words: int):
-    """The all-zero scratch (bitmaps and chunk counts of every level) whose first bitmap has at
-    least ``words`` words, kept for the current stream.  Every call leaves the bitmaps zero
-    again; one that did not finish has them cleared here."""
-    key = (dev.index if dev.index is not None else torch.cuda.current_device(), _stream())
-    entry = _grid_scratch.get(key)
-    if entry is None or entry[1] < words:
-        entry = [torch.zeros(_grid_layout(words)[1], dtype=torch.int32, device=dev), words, False]
-        _grid_scratch[key] = entry
-    elif entry[2]:
-        entry[0].zero_()
-    return entry
-
-
-_grid_lock = threading.Lock()  # one call at a time between marking a scratch bitmap and emitting from it
-
-
-def _downsample_coords_grid(coords, ks, st, pd, coords_max_host, fan, rsv_ratio, table, ahead=0):
-    with _grid_lock:
-        return _downsample_coords_grid_locked(coords, ks, st, pd, coords_max_host, fan, rsv_ratio, table, ahead)
-
-
-def _downsample_coords_grid_locked(coords, ks, st, pd, coords_max_host, fan, rsv_ratio, table, ahead=0):
+def _downsample_coords_grid(state, coords, ks, st, pd, coords_max_host, fan, rsv_ratio, table, ahead=0):
     """downsample_coords for non-negative coordinates when the output grid has at most
     2048 cells per candidate (and at most 2^30): mark an occupancy bitmap, count, read the
     number of outputs back, emit rows and table entries in ascending order.  None when the grid
     is larger than that (decided on the device; costs the same one read-back).  ``ahead`` more
-    levels of the same geometry are computed before the read-back and left in ``_ahead``."""
+    levels of the same geometry are computed before the read-back and left in ``state.ahead``.
+    Runs with _state_lock held: one call at a time between marking a bitmap and emitting."""
     n = coords.shape[0]
     dev = coords.device
     bits = min(max(1 << (n * fan * 2048 - 1).bit_length(), 1 << 20), 1 << 30)
-    entry = _grid_bitmap(dev, bits // 32)
-    layout, _ = _grid_layout(entry[1])
-    buf = entry[0]
+    buf = state.bitmap(dev, bits // 32)
+    layout, _ = _grid_layout(state.grid_words)
     levels = 1 + ahead
     # per level 8 counters: [n_out, table overflow, grid too large, -, max b, x, y, z of the INPUTS]
     ctr = table.counters if levels == 1 else torch.zeros(8 * levels, dtype=torch.int32, device=dev)
@@ -461,7 +498,7 @@ def _downsample_coords_grid_locked(coords, ks, st, pd, coords_max_host, fan, rsv
         return ctr[8 * level:8 * level + 8]  # "counters"
 
     _check(_C.tsmi_coords_max(s, _ptr(coords), n, _ptr(part(0, "in_max")), 0))
-    entry[2] = True  # marked bits stay behind unless the emit passes below run
+    state.grid_dirty = True  # marked bits stay behind unless the emit passes below run
     _check(_C.tsmi_downsample_grid_count(s, _ptr(coords), n, *g, host_max, _ptr(part(0, "in_max")),
                                          _ptr(part(0, "bitmap")), layout[0][1], 0,
                                          _ptr(part(0, "chunks")), _ptr(part(0, "counters")),
@@ -473,7 +510,7 @@ def _downsample_coords_grid_locked(coords, ks, st, pd, coords_max_host, fan, rsv
             _ptr(part(level, "chunks")), _ptr(part(level, "counters")), _ptr(part(level + 1, "in_max"))))
     host = ctr.tolist()
     if host[2]:
-        entry[2] = False  # nothing was marked, at any level
+        state.grid_dirty = False  # nothing was marked, at any level
         return None
 
     def emit(level, n_in, tbl):
@@ -508,9 +545,9 @@ def _downsample_coords_grid_locked(coords, ks, st, pd, coords_max_host, fan, rsv
         except ValueError:  # not asked for yet: let the call that asks raise it
             clean = False  # this level's marks (and the later ones') are still in the bitmaps
             break
-        _ahead[id(prev)] = (weakref.ref(prev), (ks, st, pd, rsv_ratio), nxt[0], nxt[1])
+        state.ahead[id(prev)] = (weakref.ref(prev), (ks, st, pd, rsv_ratio), nxt[0], nxt[1])
         prev = nxt[0]
-    entry[2] = not clean
+    state.grid_dirty = not clean
     return first
 
 

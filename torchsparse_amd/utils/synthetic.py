@@ -81,34 +81,41 @@ def lidar_scan_voxels(seed: int = 1, voxel: float = 0.05, n_beams: int = 64, n_a
     return np.concatenate([np.zeros((len(vox), 1), np.int64), vox], 1).astype(np.int32)
 
 
-def multisweep_voxels(seed: int = 2, batch: int = 2, n_sweeps: int = 10) -> Tuple[np.ndarray, tuple]:
-    """Per sample: `n_sweeps` sweeps of a 32-beam sensor (ego moves 0.5 m per sweep)
-    merged inside +-54 m x +-54 m x [-5, 3] m and voxelised at (0.075, 0.075, 0.2) m.
-    Rows are (b, z, y, x) in a (41, 1440, 1440) grid, the layout detection backbones
-    use.  Returns (coords, spatial_range)."""
+def multisweep_voxels(seed: int = 2, batch: int = 2, target: int = 250_000, max_sweeps: int = 80,
+                      n_azimuth: int = 2180, range_noise: float = 0.03) -> Tuple[np.ndarray, tuple]:
+    """Per sample: sweeps of a 32-beam sensor (the ego moves 0.5 m per sweep past 40 boxes,
+    Gaussian range noise of `range_noise` metres) are merged inside +-54 m x +-54 m x [-5, 3] m
+    and voxelised at (0.075, 0.075, 0.2) m until the sample holds `target` voxels (or
+    `max_sweeps` were merged).  Rows are (b, z, y, x) in a
+    (41, 1440, 1440) grid, the layout detection backbones use.
+    Returns (coords, spatial_range)."""
     rng = np.random.default_rng(seed)
-    dirs = _sensor_dirs(32, -30.0, 10.0, 1090)
+    dirs = _sensor_dirs(32, -30.0, 10.0, n_azimuth)
     grid = (41, 1440, 1440)
     out = []
     for b in range(batch):
         lo, hi = _random_boxes(rng, 40, 4.0, 52.0)
-        pts = []
-        for s in range(n_sweeps):
+        keys = np.zeros(0, np.int64)
+        for s in range(max_sweeps):
             origin = np.array([0.5 * s, 0.0, 1.8])
-            jitter = rng.normal(0, 0.002, dirs.shape)
-            d = dirs + jitter
+            d = dirs + rng.normal(0, 0.002, dirs.shape)
             d /= np.linalg.norm(d, axis=1, keepdims=True)
-            pts.append(_raycast(origin, d, lo, hi, 1.0, 75.0))
-        p = np.concatenate(pts, 0)
-        p[:, 2] -= 1.8 + 3.0  # sensor frame, ground near z = -4.8... keep inside [-5, 3]
-        p[:, 2] += 3.0
-        keep = (np.abs(p[:, 0]) < 54) & (np.abs(p[:, 1]) < 54) & (p[:, 2] > -5) & (p[:, 2] < 3)
-        p = p[keep]
-        ix = np.floor((p[:, 0] + 54) / 0.075).astype(np.int64)
-        iy = np.floor((p[:, 1] + 54) / 0.075).astype(np.int64)
-        iz = np.floor((p[:, 2] + 5) / 0.2).astype(np.int64)
-        zyx = np.unique(np.stack([iz, iy, ix], 1), axis=0)
-        zyx = zyx[(zyx[:, 0] < grid[0]) & (zyx[:, 1] < grid[1]) & (zyx[:, 2] < grid[2])]
+            p = _raycast(origin, d, lo, hi, 1.0, 75.0)
+            if range_noise > 0:
+                ray = p - origin
+                rng_m = np.linalg.norm(ray, axis=1, keepdims=True)
+                p = origin + ray / rng_m * (rng_m + rng.normal(0, range_noise, rng_m.shape))
+            p[:, 2] -= 1.8  # sensor frame: the ground lies near z = -1.8, inside [-5, 3]
+            keep = (np.abs(p[:, 0]) < 54) & (np.abs(p[:, 1]) < 54) & (p[:, 2] > -5) & (p[:, 2] < 3)
+            p = p[keep]
+            ix = np.floor((p[:, 0] + 54) / 0.075).astype(np.int64)
+            iy = np.floor((p[:, 1] + 54) / 0.075).astype(np.int64)
+            iz = np.floor((p[:, 2] + 5) / 0.2).astype(np.int64)
+            ok = (iz < grid[0]) & (iy < grid[1]) & (ix < grid[2])
+            keys = np.union1d(keys, ((iz * grid[1] + iy) * grid[2] + ix)[ok])
+            if len(keys) >= target:
+                break
+        zyx = np.stack([keys // (grid[1] * grid[2]), (keys // grid[2]) % grid[1], keys % grid[2]], 1)
         out.append(np.concatenate([np.full((len(zyx), 1), b), zyx], 1))
     return np.concatenate(out, 0).astype(np.int32), (batch,) + grid
 
