@@ -376,6 +376,19 @@ int tsmi_wgrad_pairs_pad(tsmi_stream_t s, const int32_t *nbmaps_inter, int64_t n
 int tsmi_wgrad_pairs_build(tsmi_stream_t s, const int32_t *map, int64_t n_rows, int kvol,
                            int32_t *block_counts, int32_t *nbsizes, int32_t *pairs,
                            int32_t *seg_steps);
+/* tsmi_wgrad_pairs_build without the caller's scratch buffer, for callers that cannot
+ * allocate device memory (code under HIP graph capture, serving loops and harnesses that
+ * forbid hipMalloc).  It has no counterpart in the reference.  The per-block counts live in
+ * an array built into the library (4 MiB of device memory on every GPU the library runs
+ * on, held until the process ends); inputs and outputs are still the caller's.  Limit:
+ * K_vol * ceil(n_rows / 256) <= 1,048,576 (e.g. 9.9M map rows at K_vol = 27), otherwise
+ * TSMI_ERR_INVALID_ARGUMENT.  The call allocates nothing; its first call on a device looks
+ * the array's address up (hipGetSymbolAddress) and should therefore happen outside stream
+ * capture.  All calls on one GPU share the array: calls that overlap on one GPU (two
+ * streams, two threads) race, calls queued on one stream do not.  Same outputs, bit for
+ * bit, as tsmi_wgrad_pairs_build. */
+int tsmi_wgrad_pairs_build_static(tsmi_stream_t s, const int32_t *map, int64_t n_rows, int kvol,
+                                  int32_t *nbsizes, int32_t *pairs, int32_t *seg_steps);
 int64_t tsmi_conv_wgrad_pairs_workspace_elems(int64_t pair_cap, int kvol, int cin, int cout,
                                               int dtype);
 int tsmi_conv_wgrad_pairs(tsmi_stream_t s, const void *x, const void *dy, const int32_t *pairs,

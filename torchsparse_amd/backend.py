@@ -81,6 +81,7 @@ def _load():
                                            _vp],
         "tsmi_conv_wgrad": [_vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _i32, _i32, _vp, _i64, _vp],
         "tsmi_wgrad_pairs_build": [_vp, _vp, _i64, _i32, _vp, _vp, _vp, _vp],
+        "tsmi_wgrad_pairs_build_static": [_vp, _vp, _i64, _i32, _vp, _vp, _vp],
         "tsmi_wgrad_pairs_pad": [_vp, _vp, _i64, _vp, _i32, _vp, _vp],
         "tsmi_conv_wgrad_pairs": [_vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _i32, _vp,
                                   _i64, _vp],

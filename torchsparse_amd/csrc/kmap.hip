@@ -1442,6 +1442,50 @@ extern "C" int tsmi_wgrad_pairs_build(tsmi_stream_t s, const int32_t *map, int64
   return check_launch("tsmi_wgrad_pairs_build");
 }
 
+// ---- the entry point that allocates nothing -------------------------------------------------
+// Scratch of the pair-list build (per-block counts of every offset) for callers that cannot
+// bring a buffer of their own.  Each GPU holds its own copy of the array at its own address;
+// host code only ever uses the per-device address obtained below, never the array's name.
+constexpr int64_t kStaticScratchInts = int64_t(1) << 20;  // 4 MiB per GPU
+static __device__ __align__(256) int32_t scratch[kStaticScratchInts];
+constexpr int kStaticScratchMaxDevices = 64;
+static std::atomic<int32_t *> g_scratch_ptr[kStaticScratchMaxDevices];
+
+// Device address of `scratch` on the current device, looked up once per device.
+static int static_scratch(int32_t **out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return tsmi::fail(TSMI_ERR_HIP, "static scratch: %s", hipGetErrorString(e));
+  TSMI_REQUIRE(dev >= 0 && dev < kStaticScratchMaxDevices, "static scratch: device %d out of range", dev);
+  int32_t *p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    void *addr = nullptr;
+    e = hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !addr)
+      return tsmi::fail(TSMI_ERR_HIP, "static scratch: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    p = static_cast<int32_t *>(addr);
+    g_scratch_ptr[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return TSMI_OK;
+}
+
+extern "C" int tsmi_wgrad_pairs_build_static(tsmi_stream_t s, const int32_t *map, int64_t n_rows,
+                                             int kvol, int32_t *nbsizes, int32_t *pairs,
+                                             int32_t *seg_steps) {
+  TSMI_REQUIRE(kvol >= 1 && kvol <= kWgradMaxKvol && n_rows >= 0,
+               "wgrad_pairs_build_static: bad sizes (kernel volume %d, at most %d)", kvol, kWgradMaxKvol);
+  const int64_t need = (int64_t)kvol * ceil_div(n_rows, kBlock);
+  TSMI_REQUIRE(need <= kStaticScratchInts,
+               "wgrad_pairs_build_static: K_vol * ceil(n_rows / 256) = %lld exceeds the %lld "
+               "entries of the built-in scratch; use tsmi_wgrad_pairs_build with a buffer",
+               (long long)need, (long long)kStaticScratchInts);
+  int32_t *block_counts = nullptr;
+  if (int e = static_scratch(&block_counts)) return e;
+  // every entry the kernels read is written by the counting pass first: nothing to clear
+  return tsmi_wgrad_pairs_build(s, map, n_rows, kvol, block_counts, nbsizes, pairs, seg_steps);
+}
+
 extern "C" int tsmi_wgrad_pairs_pad(tsmi_stream_t s, const int32_t *nbmaps_inter, int64_t nnz,
                                     const int32_t *nbsizes, int kvol, int32_t *pairs,
                                     int32_t *seg_steps) {
