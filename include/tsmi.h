@@ -58,8 +58,12 @@ int tsmi_hashtable_clear(tsmi_stream_t s, int64_t *keys, int32_t *vals, int64_t 
 /* Insert coords[i] -> i+1 for i < n.
  * Replaces subm_hashmap_kmap_stage1 (others/sparsemapping_cuda.cu:129-140) and
  * GPUHashTable::insert_coords (hashmap/hashmap_cuda.cuh:149-169).
- * `status` (device int32[1], pre-zeroed by the caller or NULL) is set to 1 when a
- * key could not be placed because the table is full. */
+ * `status` (device int32[1], pre-zeroed by the caller or NULL) collects two bits: 1 when a
+ * key could not be placed because the table is full, 2 when a row cannot be packed into a
+ * table key (x, y or z outside [-2^17, 2^17) or batch outside [0, 512)) and was left out.
+ * The reference ravels over the measured extents and takes any int32 coordinate
+ * (others/sparsemapping_cuda.cu:12-26); a caller that does not check bit 2 gets maps
+ * that miss those rows. */
 int tsmi_hashtable_insert_coords(tsmi_stream_t s, int64_t *keys, int32_t *vals, int64_t cap,
                                  const int32_t *coords, int64_t n, int32_t *status);
 
@@ -100,6 +104,19 @@ int tsmi_kmap_query_subm(tsmi_stream_t s, const int64_t *keys, const int32_t *va
                          const int32_t *coords, int64_t n, int64_t n_pad, const int32_t ks[3],
                          int32_t *out_in_map);
 
+/* A whole submanifold map in one call: empty the table and fill the map with -1 (one
+ * launch), insert coords[i] -> i+1, query (mirrored for an all-odd kernel, all offsets
+ * otherwise; pad = (ks-1)/2 for an odd kernel volume, 0 for an even one).  keys / vals need
+ * not be initialised.  `status` as in tsmi_hashtable_insert_coords, except that this call
+ * clears it first.  Same table and map, bit
+ * for bit, as tsmi_hashtable_clear + tsmi_hashtable_insert_coords + tsmi_kmap_query_subm (or
+ * tsmi_kmap_query).  Replaces build_kernel_map_subm_hashmap with to_insert = true
+ * (others/sparsemapping_cuda.cu:303-345) together with the torch.zeros of its table
+ * (kmap/func/hashmap_on_the_fly.py:59-67). */
+int tsmi_kmap_build_subm(tsmi_stream_t s, int64_t *keys, int32_t *vals, int64_t cap,
+                         const int32_t *coords, int64_t n, int64_t n_pad, const int32_t ks[3],
+                         int32_t *out_in_map, int32_t *status);
+
 /* Per-column maximum of non-negative coords -> out_max int32[4] (device).  n may be 0 (result 0).
  * clear_first = 0 when out_max already holds zeros (saves the fill launch).
  * Replaces coords.max(0).values (hashmap_on_the_fly.py:33). */
@@ -108,8 +125,11 @@ int tsmi_coords_max(tsmi_stream_t s, const int32_t *coords, int64_t n, int32_t *
 
 /* Candidate output coordinates of a strided convolution, de-duplicated by inserting
  * them, packed as (b<<54 | x'<<36 | y'<<18 | z') with x' = x + 2^17, into the (empty) OUTPUT table
- * (keys, cap); vals are not touched.  counters[1] (device int32[2], zero on entry) is
- * set to 1 if the table overflowed.
+ * (keys, cap); vals are not touched.  counters (device int32[4], zero on entry):
+ * counters[1] is set to 1 if the table overflowed, counters[3] to 1 if an input row or one
+ * of its in-range candidates cannot be packed (x, y or z outside [-2^17, 2^17), batch
+ * outside [0, 512)) — the reference has no such limit (others/sparsemapping_cuda.cu:12-26)
+ * and the caller must treat it as an error.
  *   mode 0: o = (in + pad + digit - (ks-1)) / stride where divisible and
  *           out_min <= o <= out_max per axis — downsample_grid_kmap_stage1_specialized_fast
  *           (others/sparsemapping_cuda.cu:60-107) and get_output_coords_kernel
@@ -169,7 +189,9 @@ int tsmi_downsample_finalize(tsmi_stream_t s, const int64_t *sorted_keys, int64_
  * clear_first is set, for callers that pass uninitialised scratch every time; otherwise the
  * caller guarantees it is all zero) and counts its set bits:
  * counters[0] = number of outputs, counters[2] = 1 when the grid does not fit (nothing is
- * then marked and the caller takes the sorting path).  next_in_max_dev, when given, is a
+ * then marked and the caller takes the sorting path), counters[3] = 1 when an input row or
+ * an in-range candidate cannot be packed into a table key (as in tsmi_downsample_candidates;
+ * the caller zeroes counters[3] before the call).  next_in_max_dev, when given, is a
  * zero-filled device int32[4] that receives the per-column maximum of the outputs (what
  * tsmi_coords_max would find over out_coords).  in_max_dev is the device int32[4]
  * per-column maximum of in_coords (tsmi_coords_max); out_max_host, when given, bounds the

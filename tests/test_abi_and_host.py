@@ -188,3 +188,21 @@ def test_strided_chain_bookkeeping_with_interleaved_chains():
     fresh = mk()
     s3.ahead[id(fresh)] = s3.ahead.pop(key)  # worst case: the allocator reused the address
     assert isinstance(s3.chain_step(fresh, geom_a), int)
+
+
+def test_coordinate_range_bookkeeping_on_the_host():
+    """Which coordinate tensors count as checked: the same object, unchanged; nothing else."""
+    from torchsparse_amd import backend
+    a = torch.zeros((5, 4), dtype=torch.int32)
+    assert not backend._range_known(a)
+    backend._mark_range_ok(a)
+    assert backend._range_known(a)
+    assert not backend._range_known(a.clone())
+    a[0, 0] = 1
+    assert not backend._range_known(a)
+    for _ in range(600):  # the table of checked tensors stays bounded
+        backend._mark_range_ok(torch.zeros((1, 4), dtype=torch.int32))
+    assert len(backend._range_ok) <= 512
+    msg = str(backend._range_error())
+    assert "-131072" in msg and "131072)" in msg and "512" in msg
+    assert backend.COORD_LIMIT == 1 << 17 and backend.BATCH_LIMIT == 512

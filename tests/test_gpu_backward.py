@@ -278,6 +278,34 @@ def test_autograd_through_transposed_conv_and_relu_residual(mods):
     assert rel_rms(_f32(x.grad), dx) < 1e-4
 
 
+@pytest.mark.parametrize("flow", ["ImplicitGEMM", "GatherScatter", "FetchOnDemand"])
+def test_only_bias_and_residual_trainable(mods, flow):
+    """Frozen features and kernel, trainable bias and residual: the reference adds both with
+    torch ops, so both get a gradient (d loss / d bias = column sums of the ReLU-masked g)."""
+    ts, backend, spnn, F = mods
+    rng = np.random.default_rng(3)
+    coords = random_coords(rng, 700, (14, 12, 9))
+    n = len(coords)
+    torch.manual_seed(2)
+    layer = spnn.Conv3d(16, 8, 3, bias=True).cuda()
+    layer.kernel.requires_grad_(False)
+    cfg = F.conv_config.get_default_conv_config()
+    cfg.dataflow = getattr(F.Dataflow, flow)
+    x = torch.from_numpy(rng.standard_normal((n, 16)).astype(np.float32)).cuda()
+    res = torch.from_numpy(rng.standard_normal((n, 8)).astype(np.float32)).cuda().requires_grad_(True)
+    out = F.conv3d(ts.SparseTensor(x, dev(coords)), layer.kernel, kernel_size=3, bias=layer.bias,
+                   residual=res, activation="relu", config=cfg)
+    g = torch.from_numpy(rng.standard_normal((n, 8)).astype(np.float32)).cuda()
+    (out.feats * g).sum().backward()
+    pre = oracle.conv_implicit_gemm(_f32(x), _f32(layer.kernel), oracle.kmap_subm(coords, 3), n) \
+        + _f32(layer.bias) + _f32(res)
+    assert rel_rms(_f32(out.feats), np.maximum(pre, 0)) < 1e-4
+    gpre = _f32(g) * (pre > 0)
+    assert layer.kernel.grad is None
+    assert rel_rms(_f32(res.grad), gpre) < 1e-4
+    assert rel_rms(_f32(layer.bias.grad), gpre.sum(0)) < 1e-4
+
+
 @pytest.mark.parametrize("geom", [(3, 1, 1), (2, 2, 0), (3, 2, 1)])
 @pytest.mark.parametrize("splits", [(1, 1), (3, 2)])
 @pytest.mark.parametrize("cin,cout", [(16, 24), (32, 64)])

@@ -212,6 +212,7 @@ def test_single_layer_vs_dense_conv(mods, kmap_mode):
             ref = _dense_reference(coords, feats.astype(np.float32), filters.astype(np.float32), k, s, shape)
             want = np.stack([ref[0, :, c[1], c[2], c[3]] for c in oc])
             got = _f32(out.feats)
+            assert rel_rms(got, want) <= 1e-2, (k, s)  # the per-case bound: fp16 storage, fp32 sums
             acc_adiff += np.abs(got - want).sum() / want.size
             acc_rdiff += np.abs(got - want).max() / np.abs(got).mean()
             count += 1
@@ -224,7 +225,7 @@ def test_pointwise_and_module_init(mods):
     torch.manual_seed(0)
     layer = spnn.Conv3d(32, 64, 1, bias=True).to("cuda")
     assert layer.kernel.shape == (32, 64)
-    assert float(layer.kernel.abs().max()) <= 1 / np.sqrt(32) + 1e-6
+    assert float(layer.kernel.detach().abs().max()) <= 1 / np.sqrt(32) + 1e-6
     x = torch.randn(100, 32, device="cuda")
     coords = dev(random_coords(np.random.default_rng(1), 100, (8, 8, 8)))
     out = layer(ts.SparseTensor(x, coords))

@@ -379,3 +379,101 @@ def test_sort_keys_small_and_large(n):
                                     backend._ptr(temp), temp_bytes))
     np.testing.assert_array_equal(d_out.cpu().numpy(), np.sort(keys))
     assert torch.equal(d_in.cpu(), torch.from_numpy(keys))  # the input is left alone
+
+
+# Coordinates the packed table key cannot hold (18 bits per axis, 9 for the batch) must stop the
+# call with a ValueError, in every builder; the reference takes any int32 coordinate
+# (others/sparsemapping_cuda.cu:12-26), so a silent drop would be a wrong map with status 0.
+BAD_ROWS = [(0, 131072, 3, 3), (0, 3, -131073, 3), (0, 3, 3, 1 << 20), (512, 3, 3, 3), (-1, 3, 3, 3)]
+
+
+def _coords_with(bad_row):
+    rng = np.random.default_rng(5)
+    coords = random_coords(rng, 300, (12, 12, 12))
+    coords[137] = bad_row
+    return coords
+
+
+@pytest.mark.parametrize("bad_row", BAD_ROWS)
+def test_unpackable_coordinates_raise_in_the_submanifold_build(bad_row):
+    coords = dev(_coords_with(bad_row))
+    with pytest.raises(ValueError, match="packed hash key"):
+        F.build_kernel_map(coords, coords.shape[0], 3, 1, 0, mode="hashmap_on_the_fly")
+    table = backend.GPUHashTable(backend.hash_capacity(coords.shape[0]), device="cuda")
+    with pytest.raises(ValueError, match="packed hash key"):
+        table.insert_bxyz(coords)
+    with pytest.raises(ValueError, match="packed hash key"):
+        table.insert_coords(coords[:, [1, 2, 3, 0]].contiguous())
+
+
+@pytest.mark.parametrize("bad_row", BAD_ROWS)
+@pytest.mark.parametrize("through_grid", [True, False])
+@pytest.mark.parametrize("mode", ["hashmap_on_the_fly", "hashmap"])
+def test_unpackable_coordinates_raise_in_the_strided_builds(bad_row, through_grid, mode, monkeypatch):
+    monkeypatch.setattr(backend, "downsample_through_grid", through_grid)
+    coords = dev(_coords_with(bad_row))
+    with pytest.raises(ValueError, match="packed hash key"):
+        F.build_kernel_map(coords, coords.shape[0], 2, 2, 0, mode=mode)
+    with pytest.raises(ValueError, match="packed hash key"):
+        F.build_kernel_map(coords, coords.shape[0], 3, 2, 1, mode=mode)
+    backend.release_scratch()  # a refused call leaves marks in the stream's bitmap: start clean
+
+
+def test_coordinates_at_the_edge_of_the_packed_range_are_exact():
+    """The largest and smallest packable coordinates, in every builder, against the oracle."""
+    rng = np.random.default_rng(6)
+    base = random_coords(rng, 400, (9, 9, 9))
+    hi = base.copy()
+    hi[:, 1:] += 131072 - 9
+    kmap = F.build_kernel_map(dev(hi), len(hi), 3, 1, 0, mode="hashmap_on_the_fly")
+    np.testing.assert_array_equal(kmap["out_in_map"].cpu().numpy(), oracle.kmap_subm(hi, 3))
+    for through_grid in (True, False):
+        backend.downsample_through_grid = through_grid
+        try:
+            kmap = F.build_kernel_map(dev(hi), len(hi), 2, 2, 0, mode="hashmap_on_the_fly")
+        finally:
+            backend.downsample_through_grid = True
+        want_map, want_coords = oracle.kmap_downsample(hi, 2, 2, 0)
+        np.testing.assert_array_equal(kmap["coords"].cpu().numpy(), want_coords)
+        np.testing.assert_array_equal(kmap["out_in_map"].cpu().numpy(), want_map)
+    lo = base.copy()
+    lo[:, 1:] -= 131072
+    lo[:, 0] = 511
+    kmap = F.build_kernel_map(dev(lo), len(lo), 3, 1, 0, mode="hashmap_on_the_fly")
+    want = oracle.kmap_subm(lo, 3, coords_min=lo.min(0), coords_max=lo.max(0))
+    np.testing.assert_array_equal(kmap["out_in_map"].cpu().numpy(), want)
+
+
+def test_a_checked_tensor_is_not_read_back_again_and_a_changed_one_is():
+    rng = np.random.default_rng(7)
+    coords = dev(random_coords(rng, 500, (10, 10, 10)))
+    assert not backend._range_known(coords)
+    F.build_kernel_map(coords, coords.shape[0], 3, 1, 0, mode="hashmap_on_the_fly")
+    assert backend._range_known(coords)
+    coords[3, 1] = 1 << 18  # an in-place write bumps the version: the tensor is checked again
+    assert not backend._range_known(coords)
+    with pytest.raises(ValueError, match="packed hash key"):
+        F.build_kernel_map(coords, coords.shape[0], 3, 1, 0, mode="hashmap_on_the_fly")
+    # outputs of a strided build are known to be in range: their own builds do not synchronise
+    good = dev(random_coords(rng, 500, (10, 10, 10)))
+    kmap = F.build_kernel_map(good, good.shape[0], 2, 2, 0, mode="hashmap_on_the_fly")
+    assert backend._range_known(good) and backend._range_known(kmap["coords"])
+
+
+def test_fused_submanifold_build_equals_the_separate_calls():
+    """tsmi_kmap_build_subm against clear + insert + query on the same rows: table and map."""
+    rng = np.random.default_rng(8)
+    for n, ks in ((0, 3), (1, 3), (777, 3), (5000, (3, 1, 5)), (3001, 2), (2000, (2, 3, 3))):
+        coords = dev(random_coords(rng, n, (30, 20, 10))) if n else torch.zeros((0, 4), dtype=torch.int32,
+                                                                                 device="cuda")
+        table, omap = backend.GPUHashTable.build_subm(coords, ks)
+        ref = backend.GPUHashTable(backend.hash_capacity(n), device="cuda")
+        ref.insert_bxyz(coords)
+        want = ref.query_subm_bxyz(coords, t3(ks))
+        assert torch.equal(omap, want), (n, ks)
+        # slots may differ only where two keys raced for one; the key -> value relation may not
+        assert torch.equal(torch.sort(table.keys)[0], torch.sort(ref.keys)[0])
+        looked = table.query_bxyz(coords, (1, 1, 1), (1, 1, 1), (0, 0, 0))
+        assert torch.equal(looked[:n, 0], torch.arange(n, dtype=torch.int32, device="cuda"))
+        if n:
+            np.testing.assert_array_equal(omap.cpu().numpy(), oracle.kmap_subm(coords.cpu().numpy(), t3(ks)))

@@ -82,6 +82,7 @@ def _load():
         "tsmi_conv_wgrad": [_vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _i32, _i32, _vp, _i64, _vp],
         "tsmi_wgrad_pairs_build": [_vp, _vp, _i64, _i32, _vp, _vp, _vp, _vp],
         "tsmi_wgrad_pairs_build_static": [_vp, _vp, _i64, _i32, _vp, _vp, _vp],
+        "tsmi_kmap_build_subm": [_vp, _vp, _vp, _i64, _vp, _i64, _i64, _I3, _vp, _vp],
         "tsmi_wgrad_pairs_pad": [_vp, _vp, _i64, _vp, _i32, _vp, _vp],
         "tsmi_conv_wgrad_pairs": [_vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _i32, _vp,
                                   _i64, _vp],
@@ -170,19 +171,67 @@ def hash_capacity(n: int, ratio: float = 2.0) -> int:
 # --------------------------------------------------------------------- hash table
 
 
+# The table key packs 18 bits per spatial axis and 9 for the batch index.  The reference
+# ravels over the measured extents and takes any int32 coordinate
+# (others/sparsemapping_cuda.cu:12-26); here a row outside the packed range must stop the
+# call: the kernels flag it and the shim raises.  A flag costs a read-back, so a coordinate
+# tensor is checked once: tensors that passed (and the ones the strided builders produced
+# from them) are remembered by identity, version and address.
+COORD_LIMIT = 1 << 17
+BATCH_LIMIT = 512
+_range_ok = {}  # id(tensor) -> (weak reference, version, address)
+
+
+def _range_error() -> ValueError:
+    return ValueError(
+        f"coordinates outside the range of the packed hash key: x, y, z must lie in "
+        f"[{-COORD_LIMIT}, {COORD_LIMIT}) and the batch index in [0, {BATCH_LIMIT})")
+
+
+def _range_known(coords: torch.Tensor) -> bool:
+    hit = _range_ok.get(id(coords))
+    return (hit is not None and hit[0]() is coords and hit[1] == coords._version
+            and hit[2] == coords.data_ptr())
+
+
+def _mark_range_ok(coords: torch.Tensor) -> None:
+    if len(_range_ok) >= 512:
+        for key in [k for k, v in _range_ok.items() if v[0]() is None]:
+            del _range_ok[key]
+        if len(_range_ok) >= 512:
+            _range_ok.clear()
+    _range_ok[id(coords)] = (weakref.ref(coords), coords._version, coords.data_ptr())
+
+
+def _settle_insert(coords: torch.Tensor, status: torch.Tensor) -> None:
+    """After an insert pass over ``coords`` that collected its flags in ``status``: read them
+    (one synchronisation) unless these rows are known to be in range."""
+    if _range_known(coords):
+        return
+    flags = int(status.item())
+    if flags & 2:
+        raise _range_error()
+    if flags & 1:
+        raise ValueError("The capacity of hashtable is not sufficient.")
+    _mark_range_ok(coords)
+
+
 class GPUHashTable:
     """Non-owning view of (keys int64[cap], vals int32[cap]) or, given an int, an
     owning table of that capacity — hashmap/hashmap_cuda.cuh:65-121."""
 
-    def __init__(self, keys, vals: Optional[torch.Tensor] = None, device="cuda"):
+    def __init__(self, keys, vals: Optional[torch.Tensor] = None, device="cuda", zero: bool = True):
         self.counters = None
         if isinstance(keys, int):
-            # one zero-filled allocation: keys (int64 view), vals, 8 spare counters
+            # one allocation: keys (int64 view), vals, 8 spare counters; zero-filled unless the
+            # caller's first pass over the table clears it (build_subm)
             cap = make_divisible(max(int(keys), 8), 8)
-            buf = torch.zeros(3 * cap + 8, dtype=torch.int32, device=device)
+            buf = (torch.zeros if zero else torch.empty)(3 * cap + 8, dtype=torch.int32, device=device)
             self.keys = buf[:2 * cap].view(torch.int64)
             self.vals = buf[2 * cap:3 * cap]
-            self.counters = buf[3 * cap:]
+            if zero:
+                self.counters = buf[3 * cap:]
+            self._status = buf[3 * cap + 3:3 * cap + 4]
         else:
             self.keys = _need(keys, torch.int64, "hashmap_keys")
             self.vals = _need(vals, torch.int32, "hashmap_vals")
@@ -197,9 +246,32 @@ class GPUHashTable:
         _check(_C.tsmi_hashtable_clear(_stream(), _ptr(self.keys), _ptr(self.vals), self.capacity))
 
     def insert_bxyz(self, coords: torch.Tensor) -> None:
+        given = coords
         coords = _need(coords, torch.int32, "coords")
+        known = _range_known(given)
+        status = None
+        if not known:
+            status = torch.zeros(1, dtype=torch.int32, device=coords.device)
         _check(_C.tsmi_hashtable_insert_coords(_stream(), _ptr(self.keys), _ptr(self.vals),
-                                               self.capacity, _ptr(coords), coords.shape[0], None))
+                                               self.capacity, _ptr(coords), coords.shape[0], _ptr(status)))
+        if not known:
+            _settle_insert(given, status)
+
+    @classmethod
+    def build_subm(cls, coords: torch.Tensor, kernel_size, rsv_ratio: float = 2.0):
+        """(table over ``coords``, stride-1 map of ``kernel_size``) in one call: the table is
+        emptied and the map filled by one launch, then insert, then query."""
+        given = coords
+        coords = _need(coords, torch.int32, "coords")
+        ks = _triple(kernel_size)
+        n = coords.shape[0]
+        table = cls(hash_capacity(n, rsv_ratio), device=coords.device, zero=False)
+        n_pad = make_divisible(n, 128)
+        omap = torch.empty((n_pad, ks[0] * ks[1] * ks[2]), dtype=torch.int32, device=coords.device)
+        _check(_C.tsmi_kmap_build_subm(_stream(), _ptr(table.keys), _ptr(table.vals), table.capacity,
+                                       _ptr(coords), n, n_pad, _I3(*ks), _ptr(omap), _ptr(table._status)))
+        _settle_insert(given, table._status)
+        return table, omap
 
     def query_subm_bxyz(self, coords, kernel_size) -> torch.Tensor:
         """Stride-1 map over the table's own coordinates (row i inserted with value i).  Odd
@@ -348,7 +420,10 @@ def downsample_coords(coords: torch.Tensor, kernel_sizes, stride, padding, coord
     scratch = torch.empty(2 * cap + temp_bytes // 8 + 1, dtype=torch.int64, device=dev)
     uniq, sorted_keys, temp = scratch[:cap], scratch[cap:2 * cap], scratch[2 * cap:]
     _check(_C.tsmi_hashtable_compact_keys(s, _ptr(table.keys), cap, _ptr(uniq), _ptr(counters)))
-    n_out, overflow = counters[:2].tolist()
+    n_out, overflow, _, unpackable = counters[:4].tolist()
+    if unpackable:
+        raise _range_error()
+    _mark_range_ok(coords)
     if overflow and mode == 0 and fan > 2 and not _reserve_all:
         return downsample_coords(coords, kernel_sizes, stride, padding, coords_max_host, mode, rsv_ratio,
                                  allow_negative, _reserve_all=True)
@@ -362,6 +437,7 @@ def downsample_coords(coords: torch.Tensor, kernel_sizes, stride, padding, coord
         _check(_C.tsmi_sort_keys(s, _ptr(uniq), _ptr(sorted_keys), n_out, 63, _ptr(temp), temp_bytes))
         _check(_C.tsmi_downsample_finalize(s, _ptr(sorted_keys), n_out, _ptr(table.keys),
                                            _ptr(table.vals), cap, _ptr(out_coords)))
+    _mark_range_ok(out_coords)  # unpacked from keys
     return out_coords, table
 
 
@@ -513,6 +589,10 @@ def _downsample_coords_grid(state, coords, ks, st, pd, coords_max_host, fan, rsv
     if host[2]:
         state.grid_dirty = False  # nothing was marked, at any level
         return None
+    if host[3]:  # a row or an in-range output the packed key cannot hold
+        raise _range_error()  # the marks stay: grid_dirty has the next call clear them
+    if host[0] > 0:  # the marking pass looked at every input row
+        _mark_range_ok(coords)
 
     def emit(level, n_in, tbl):
         n_out = host[8 * level]
@@ -533,6 +613,7 @@ def _downsample_coords_grid(state, coords, ks, st, pd, coords_max_host, fan, rsv
         return out, tbl
 
     first = emit(0, n, table)
+    _mark_range_ok(first[0])  # cells of a grid whose every in-range candidate was packable
     prev = first[0]
     clean = True
     for level in range(1, levels):
@@ -547,6 +628,10 @@ def _downsample_coords_grid(state, coords, ks, st, pd, coords_max_host, fan, rsv
             clean = False  # this level's marks (and the later ones') are still in the bitmaps
             break
         state.ahead[id(prev)] = (weakref.ref(prev), (ks, st, pd, rsv_ratio), nxt[0], nxt[1])
+        # the later levels are not flagged on the device; their inputs' maxima are on the host
+        if (host[8 * level + 4] < BATCH_LIMIT and
+                all(host[8 * level + 5 + a] + 2 * pd[a] < COORD_LIMIT for a in range(3))):
+            _mark_range_ok(nxt[0])
         prev = nxt[0]
     state.grid_dirty = not clean
     return first

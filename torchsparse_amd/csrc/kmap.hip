@@ -57,14 +57,28 @@ __global__ void insert_coords_kernel(TableView t, const int4 *coords, int64_t n,
   int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (i >= n) return;
   int4 c = coords[i];  // (b, x, y, z)
-  if (!coords_packable(c.x, c.y, c.z, c.w)) return;
+  if (!coords_packable(c.x, c.y, c.z, c.w)) {
+    if (status) atomicOr(status, 2);  // a row the packed key cannot hold: the caller must not go on
+    return;
+  }
   bool fresh;
   uint32_t slot = table_insert<false>(t, pack_coords(c.x, c.y, c.z, c.w), &fresh);  // rows are distinct
   if (slot == 0xFFFFFFFFu) {
-    if (status) *status = 1;
+    if (status) atomicOr(status, 1);
     return;
   }
   t.vals[slot] = (int32_t)(i + 1);
+}
+
+// What a submanifold build needs before its insert pass, in one launch: an empty table and a
+// map of -1.  Both are 16-byte stores; thread i takes the i-th int4 of each region it covers.
+__global__ void subm_prepare_kernel(int4 *keys, int64_t keys4, int4 *vals, int64_t vals4, int4 *map,
+                                    int64_t map4, int32_t *status) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i == 0 && status) *status = 0;
+  if (i < keys4) keys[i] = make_int4(0, 0, 0, 0);
+  if (i < vals4) vals[i] = make_int4(0, 0, 0, 0);
+  if (i < map4) map[i] = make_int4(-1, -1, -1, -1);
 }
 
 __global__ void insert_keys_kernel(TableView t, const long long *user_keys, int64_t n,
@@ -176,8 +190,10 @@ __host__ __device__ __forceinline__ void output_range(const Geom &g, int a, int3
 // Candidate j of the input coordinate c = (b, x, y, z) for modes 0, 1 and 2 (one candidate,
 // j = 0, in modes 1 and 2) inside the output range [lo, hi] per axis (unused in mode 1); false
 // when there is none.
+// *unpackable (when given) is set if the candidate exists but the packed key cannot hold it.
 __device__ __forceinline__ bool strided_candidate_in(int4 c, int j, const Geom &g, const int *lo,
-                                                     const int *hi, int mode, int *b, int *o) {
+                                                     const int *hi, int mode, int *b, int *o,
+                                                     bool *unpackable = nullptr) {
   *b = c.x;
   const int v[3] = {c.y, c.z, c.w};
   if (mode != 0) {
@@ -208,7 +224,9 @@ __device__ __forceinline__ bool strided_candidate_in(int4 c, int j, const Geom &
       if (o[a] < lo[a] || o[a] > hi[a]) return false;
     }
   }
-  return coords_packable(*b, o[0], o[1], o[2]);
+  const bool ok = coords_packable(*b, o[0], o[1], o[2]);
+  if (!ok && unpackable) *unpackable = true;
+  return ok;
 }
 
 __device__ __forceinline__ void output_ranges(const Geom &g, int3 out_max_host, const int32_t *in_max_dev,
@@ -222,10 +240,10 @@ __device__ __forceinline__ void output_ranges(const Geom &g, int3 out_max_host, 
 
 __device__ __forceinline__ bool strided_candidate(int4 c, int j, const Geom &g, int3 out_max_host,
                                                   const int32_t *in_max_dev, const int32_t *in_min_dev,
-                                                  int mode, int *b, int *o) {
+                                                  int mode, int *b, int *o, bool *unpackable = nullptr) {
   int lo[3], hi[3];
   output_ranges(g, out_max_host, in_max_dev, in_min_dev, mode, lo, hi);
-  return strided_candidate_in(c, j, g, lo, hi, mode, b, o);
+  return strided_candidate_in(c, j, g, lo, hi, mode, b, o, unpackable);
 }
 
 __device__ __forceinline__ int strided_fan(const Geom &g) {
@@ -239,7 +257,7 @@ __device__ __forceinline__ int strided_fan(const Geom &g) {
 __device__ __forceinline__ bool downsample_candidate(int64_t tid, const int4 *in_coords, const Geom &g,
                                                      int3 out_max_host, const int32_t *in_max_dev,
                                                      const int32_t *in_min_dev, int mode, int *b,
-                                                     int *o) {
+                                                     int *o, bool *unpackable = nullptr) {
   if (mode == 3) {
     int64_t i = tid / g.kvol;
     int k = (int)(tid - i * g.kvol);
@@ -253,13 +271,17 @@ __device__ __forceinline__ bool downsample_candidate(int64_t tid, const int4 *in
       const int hi = a == 0 ? out_max_host.x : (a == 1 ? out_max_host.y : out_max_host.z);
       o[a] = min(max(v[a] * g.stride[a] + d[a] - (g.ks[a] - 1) / 2, 0), hi);
     }
-    return coords_packable(*b, o[0], o[1], o[2]);
+    const bool ok = coords_packable(*b, o[0], o[1], o[2]);
+    if (unpackable && (!ok || !coords_packable(c.x, c.y, c.z, c.w))) *unpackable = true;
+    return ok;
   }
-  if (mode != 0) return strided_candidate(in_coords[tid], 0, g, out_max_host, in_max_dev, in_min_dev, mode, b, o);
-  const int fan = strided_fan(g);
+  const int fan = mode == 0 ? strided_fan(g) : 1;
   const int64_t i = tid / fan;
-  return strided_candidate(in_coords[i], (int)(tid - i * fan), g, out_max_host, in_max_dev, in_min_dev,
-                           mode, b, o);
+  const int4 c = in_coords[i];
+  // an input the packed key cannot hold is missing from every table built from these rows
+  if (unpackable && !coords_packable(c.x, c.y, c.z, c.w)) *unpackable = true;
+  return strided_candidate(c, (int)(tid - i * fan), g, out_max_host, in_max_dev, in_min_dev, mode, b, o,
+                           unpackable);
 }
 
 __global__ void downsample_candidates_kernel(const int4 *in_coords, int64_t n_in, int64_t total,
@@ -269,7 +291,11 @@ __global__ void downsample_candidates_kernel(const int4 *in_coords, int64_t n_in
   int64_t tid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   if (tid >= total) return;
   int b, o[3];
-  if (!downsample_candidate(tid, in_coords, g, out_max_host, in_max_dev, in_min_dev, mode, &b, o)) return;
+  bool unpackable = false;
+  const bool have = downsample_candidate(tid, in_coords, g, out_max_host, in_max_dev, in_min_dev, mode, &b,
+                                         o, &unpackable);
+  if (unpackable) counters[3] = 1;  // the caller must not go on: rows or outputs would be missing
+  if (!have) return;
   bool fresh;
   if (table_insert(t, pack_coords(b, o[0], o[1], o[2]), &fresh) == 0xFFFFFFFFu) counters[1] = 1;
 }
@@ -348,17 +374,21 @@ __device__ __forceinline__ void block_raise_max(int b, int x, int y, int z, int3
 
 __global__ void grid_mark_kernel(const int4 *in_coords, int64_t total, Geom g, int3 out_max_host,
                                  int has_host_max, const int32_t *in_max_dev, int mode,
-                                 uint32_t *bitmap, int64_t cap_words, int32_t *next_in_max) {
+                                 uint32_t *bitmap, int64_t cap_words, int32_t *next_in_max,
+                                 int32_t *counters) {
   const int64_t tid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
   const GridDims d = grid_dims(g, out_max_host, has_host_max, in_max_dev, cap_words);
   if (!d.fits || d.used_words == 0) return;  // the same for every thread
   int word = -1;
   uint32_t bits = 0;
   int b, o[3];
+  bool unpackable = false;
   const bool have = tid < total &&
                     downsample_candidate(tid, in_coords, g, out_max_host,
-                                         has_host_max ? nullptr : in_max_dev, nullptr, mode, &b, o) &&
+                                         has_host_max ? nullptr : in_max_dev, nullptr, mode, &b, o,
+                                         &unpackable) &&
                     b <= in_max_dev[0];
+  if (unpackable) counters[3] = 1;
   if (have) {
     const uint32_t cell = (((uint32_t)b * d.e[0] + o[0]) * d.e[1] + o[1]) * d.e[2] + o[2];
     word = (int)(cell >> 5);
@@ -1097,6 +1127,53 @@ extern "C" int tsmi_kmap_query_subm(tsmi_stream_t s, const int64_t *keys, const 
   return check_launch("tsmi_kmap_query_subm");
 }
 
+extern "C" int tsmi_kmap_build_subm(tsmi_stream_t s, int64_t *keys, int32_t *vals, int64_t cap,
+                                    const int32_t *coords, int64_t n, int64_t n_pad,
+                                    const int32_t ks[3], int32_t *out_in_map, int32_t *status) {
+  TableView t;
+  Geom g;
+  if (int e = make_table(&t, keys, vals, cap)) return e;
+  TSMI_REQUIRE(ks && ks[0] >= 1 && ks[1] >= 1 && ks[2] >= 1, "kmap_build_subm: bad kernel size");
+  const bool odd = ks[0] % 2 == 1 && ks[1] % 2 == 1 && ks[2] % 2 == 1;
+  const bool odd_volume = ((int64_t)ks[0] * ks[1] * ks[2]) % 2 == 1;
+  const int32_t one[3] = {1, 1, 1};
+  const int32_t pad[3] = {odd_volume ? (ks[0] - 1) / 2 : 0, odd_volume ? (ks[1] - 1) / 2 : 0,
+                          odd_volume ? (ks[2] - 1) / 2 : 0};
+  if (int e = make_geom(&g, ks, one, pad)) return e;
+  TSMI_REQUIRE(n >= 0 && n_pad >= n, "kmap_build_subm: n_pad < n");
+  TSMI_REQUIRE(n == 0 || coords, "kmap_build_subm: null coords");
+  TSMI_REQUIRE(n <= cap, "The capacity of hashtable is not sufficient (%lld keys, capacity %lld)",
+               (long long)n, (long long)cap);
+  const int64_t cells = n_pad * g.kvol;
+  TSMI_REQUIRE(cells == 0 || out_in_map, "kmap_build_subm: null out_in_map");
+  TSMI_REQUIRE((uintptr_t)keys % 16 == 0 && (uintptr_t)vals % 16 == 0 && (uintptr_t)out_in_map % 16 == 0,
+               "kmap_build_subm: table and map must be 16-byte aligned");
+  // capacity is a multiple of 8 and n_pad * kvol a multiple of 4 (n_pad is a multiple of 128
+  // in every caller; any other n_pad takes the scalar fill below)
+  const bool vec_map = cells % 4 == 0;
+  const int64_t keys4 = cap / 2, vals4 = cap / 4, map4 = (odd && vec_map) ? cells / 4 : 0;
+  const int64_t prep = std::max(keys4, std::max(vals4, map4));
+  TSMI_GRID_CHECK(std::max(prep, cells));
+  hipLaunchKernelGGL(subm_prepare_kernel, grid_for(prep), dim3(kBlock), 0, (hipStream_t)s, (int4 *)keys,
+                     keys4, (int4 *)vals, vals4, (int4 *)out_in_map, map4, status);
+  if (odd && !vec_map && cells > 0)
+    hipLaunchKernelGGL(fill_kernel<int32_t>, grid_for(cells), dim3(kBlock), 0, (hipStream_t)s,
+                       out_in_map, cells, -1);
+  if (n > 0)
+    hipLaunchKernelGGL(insert_coords_kernel, grid_for(n), dim3(kBlock), 0, (hipStream_t)s, t,
+                       (const int4 *)coords, n, status);
+  if (odd) {
+    const int64_t total = n * (g.kvol / 2 + 1);
+    if (total > 0)
+      hipLaunchKernelGGL(kmap_query_subm_kernel, grid_for(total), dim3(kBlock), 0, (hipStream_t)s, t,
+                         (const int4 *)coords, n, total, g, out_in_map);
+  } else if (cells > 0) {
+    hipLaunchKernelGGL(kmap_query_kernel, grid_for(cells), dim3(kBlock), 0, (hipStream_t)s, t,
+                       (const int4 *)coords, n, cells, g, out_in_map);
+  }
+  return check_launch("tsmi_kmap_build_subm");
+}
+
 extern "C" int tsmi_coords_max(tsmi_stream_t s, const int32_t *coords, int64_t n,
                                int32_t *out_max, int clear_first) {
   TSMI_REQUIRE(out_max && n >= 0 && (n == 0 || coords), "coords_max: bad arguments");
@@ -1223,7 +1300,7 @@ extern "C" int tsmi_downsample_grid_count(tsmi_stream_t s, const int32_t *in_coo
   if (total > 0)
     hipLaunchKernelGGL(grid_mark_kernel, grid_for(total), dim3(kBlock), 0, st, (const int4 *)in_coords,
                        total, g, hm, has_hm, in_max_dev, mode, (uint32_t *)bitmap, bitmap_words,
-                       next_in_max_dev);
+                       next_in_max_dev, counters);
   hipLaunchKernelGGL(grid_count_kernel, dim3(chunks < 2048u ? chunks : 2048u), dim3(kBlock), 0, st,
                      (const uint32_t *)bitmap,
                      bitmap_words, g, hm, has_hm, in_max_dev, chunk_counts);

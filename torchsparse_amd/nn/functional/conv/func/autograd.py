@@ -113,8 +113,12 @@ def differentiable(forward_impl: Callable):
     """Wrap a dataflow's forward: with autograd active the convolution goes through
     SparseConvFunction and bias / residual / ReLU are applied by autograd-aware ops."""
     def apply(input, weight, kmap, config, transposed=False, bias=None, residual=None, relu=False):
-        if torch.is_grad_enabled() and (input.requires_grad or weight.requires_grad):
-            out = SparseConvFunction.apply(input, weight, kmap, config, transposed, forward_impl)
+        if torch.is_grad_enabled() and any(
+                t is not None and t.requires_grad for t in (input, weight, bias, residual)):
+            if input.requires_grad or weight.requires_grad:
+                out = SparseConvFunction.apply(input, weight, kmap, config, transposed, forward_impl)
+            else:  # only the bias or the residual is trainable: they enter through torch ops below
+                out = forward_impl(input, weight, kmap, config, transposed, None, None, False)
             if bias is not None:
                 out = out + bias.to(out.dtype)
             if residual is not None:

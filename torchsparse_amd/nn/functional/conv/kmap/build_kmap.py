@@ -168,7 +168,11 @@ def build_kernel_map(_coords: torch.Tensor, input_node_num: int,
 
     # table over the input coordinates: reuse or build
     fresh = hashmap_keys is None or hashmap_vals is None
-    if fresh:
+    out_in_map = None
+    if fresh and subm and (mode == "hashmap_on_the_fly" or all(k % 2 == 1 for k in kernel_size)):
+        # table and map in one call (an even kernel in "hashmap" mode is centred differently)
+        in_table, out_in_map = backend.GPUHashTable.build_subm(coords, kernel_size, backends.hash_rsv_ratio)
+    elif fresh:
         in_table = backend.GPUHashTable(backend.hash_capacity(n_in, backends.hash_rsv_ratio),
                                         device=coords.device)
         in_table.insert_bxyz(coords)
@@ -195,7 +199,9 @@ def build_kernel_map(_coords: torch.Tensor, input_node_num: int,
     if subm and mode == "hashmap":
         pad_eff = tuple((k - 1) // 2 for k in kernel_size)
 
-    if subm and all(k % 2 == 1 for k in kernel_size):
+    if out_in_map is not None:
+        pass
+    elif subm and all(k % 2 == 1 for k in kernel_size):
         out_in_map = in_table.query_subm_bxyz(out_coords, kernel_size)  # centred in both modes
     else:
         out_in_map = in_table.query_bxyz(out_coords, kernel_size, stride, pad_eff)
