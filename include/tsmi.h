@@ -117,6 +117,29 @@ int tsmi_kmap_build_subm(tsmi_stream_t s, int64_t *keys, int32_t *vals, int64_t 
                          const int32_t *coords, int64_t n, int64_t n_pad, const int32_t ks[3],
                          int32_t *out_in_map, int32_t *status);
 
+/* flags[0] (device int32[1], zeroed by the caller) |= 1 when the rows of coords do not ascend
+ * strictly in (b, x, y, z), |= 2 when a row cannot be packed into a table key (see
+ * tsmi_hashtable_insert_coords).  What a caller reads once per coordinate tensor to choose
+ * between tsmi_kmap_sorted and the hash-table builders; no counterpart in the reference. */
+int tsmi_coords_check(tsmi_stream_t s, const int32_t *coords, int64_t n, int32_t *flags);
+
+/* out_in_map[o, k] = i with in_coords[i] == out_coords[o] * stride - pad + digits(k), -1 when
+ * there is none — the map of tsmi_kmap_query (same digit order, same padding rows), computed
+ * WITHOUT a hash table for inputs whose rows ascend strictly in (b, x, y, z) and are all
+ * packable, and outputs that ascend too (out_coords == in_coords for a submanifold map;
+ * tsmi_downsample_grid_emit and tsmi_downsample_finalize emit ascending rows): the input row
+ * of a target is found by binary search inside a short segment of the input that a block of
+ * output rows stages in LDS.  One launch, every entry of the n_out_pad rows written.
+ * Replaces build_kernel_map_subm_hashmap and stages 1 and 3 of
+ * build_kernel_map_downsample_hashmap (others/sparsemapping_cuda.cu:303-345, 429-507) for
+ * such inputs.  tsmi_kmap_sorted_supported: 1 when the kernel size fits the kernel's LDS
+ * layout (ks[0] <= 6, ks[1] <= 8, volume <= 7168). */
+int tsmi_kmap_sorted_supported(const int32_t ks[3]);
+int tsmi_kmap_sorted(tsmi_stream_t s, const int32_t *in_coords, int64_t n_in,
+                     const int32_t *out_coords, int64_t n_out, int64_t n_out_pad,
+                     const int32_t ks[3], const int32_t stride[3], const int32_t pad[3],
+                     int32_t *out_in_map);
+
 /* Per-column maximum of non-negative coords -> out_max int32[4] (device).  n may be 0 (result 0).
  * clear_first = 0 when out_max already holds zeros (saves the fill launch).
  * Replaces coords.max(0).values (hashmap_on_the_fly.py:33). */
@@ -199,7 +222,7 @@ int tsmi_downsample_finalize(tsmi_stream_t s, const int64_t *sorted_keys, int64_
  * 512 words, at most 2^25) and chunk_counts int32[bitmap_words / 512] are scratch that
  * tsmi_downsample_grid_emit reads back: it writes out_coords int32[n_out,4] in ascending
  * (b,x,y,z) order, inserts coordinate -> row + 1 into the EMPTY output table
- * (keys, vals, cap; counters[1] = 1 if the table was too small) and leaves the bitmap
+ * (keys, vals, cap; counters[1] = 1 if the table was too small; keys == NULL: no table) and leaves the bitmap
  * all zero again, so that one bitmap can serve call after call without clear_first.
  * in_max_host, when given, is a host copy of in_max_dev (read back with the counters): the
  * extents are then computed on the host and only the chunks inside the grid are launched. */

@@ -1,0 +1,193 @@
+"""Kernel maps searched over sorted coordinates (tsmi_kmap_sorted: no hash table) against the
+CPU oracle, bit-exact, and against the hash-table builders on the same rows.  Inputs ascend
+strictly in (b, x, y, z), which is what voxelisation by a ravelled key produces and what selects
+this path in build_kernel_map."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import lidar_like_coords, random_coords
+
+pytestmark = pytest.mark.gpu
+
+backend = None
+F = None
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _load():
+    global backend, F
+    from torchsparse_amd import backend as b
+    from torchsparse_amd.nn import functional as f
+    backend, F = b, f
+
+
+def dev(a, dtype=torch.int32):
+    return torch.from_numpy(np.ascontiguousarray(a)).to("cuda", dtype)
+
+
+def t3(v):
+    return (v,) * 3 if isinstance(v, int) else tuple(v)
+
+
+def ascending(coords):
+    """Rows in ascending (b, x, y, z) order."""
+    return coords[np.lexsort((coords[:, 3], coords[:, 2], coords[:, 1], coords[:, 0]))]
+
+
+def build(coords, ks, stride, pad, **kw):
+    kmap = F.build_kernel_map(dev(coords), len(coords), t3(ks), t3(stride), t3(pad), mode="hashmap_on_the_fly", **kw)
+    assert kmap["in_hashmap"] is None  # searched: no table over the inputs
+    return kmap
+
+
+@pytest.mark.parametrize("ks", [3, 2, 5, (3, 1, 1), (1, 3, 1), (2, 3, 3), (3, 5, 3), (1, 1, 1), (5, 7, 2)])
+@pytest.mark.parametrize("batch", [1, 3])
+def test_subm_map_over_sorted_rows_matches_oracle(ks, batch):
+    rng = np.random.default_rng(200)
+    coords = ascending(random_coords(rng, 900, (14, 12, 10), batch))
+    kmap = build(coords, ks, 1, 0)
+    np.testing.assert_array_equal(kmap["out_in_map"].cpu().numpy(), oracle.kmap_subm(coords, t3(ks)))
+    assert kmap["sizes"] == (len(coords), len(coords)) and kmap["out_in_map"].shape[0] % 128 == 0
+
+
+DOWN_CASES = [(2, 2, 0), (3, 2, 1), (3, 3, 1), (5, 2, 2), (5, 3, 2), (2, 3, 0), (3, 2, 0),
+              ((3, 1, 1), (2, 1, 1), (0, 0, 0)), ((3, 3, 3), (2, 2, 2), (0, 1, 1)),
+              ((1, 3, 1), (1, 2, 1), 0), ((4, 2, 6), (2, 2, 3), (1, 0, 2))]
+
+
+@pytest.mark.parametrize("ks,stride,pad", DOWN_CASES)
+@pytest.mark.parametrize("with_range", [False, True])
+@pytest.mark.parametrize("through_grid", [True, False])
+def test_strided_map_over_sorted_rows_matches_oracle(ks, stride, pad, with_range, through_grid, monkeypatch):
+    monkeypatch.setattr(backend, "downsample_through_grid", through_grid)
+    rng = np.random.default_rng(201)
+    shape = (19, 17, 13)
+    coords = ascending(random_coords(rng, 700, shape, batch=2))
+    ks, stride, pad = t3(ks), t3(stride), t3(pad)
+    sr = (2,) + shape if with_range else None
+    kmap = build(coords, ks, stride, pad, spatial_range=sr)
+    new_sr = None
+    if with_range:
+        new_sr = (2,) + tuple((shape[a] + 2 * pad[a] - (ks[a] - 1) - 1) // stride[a] + 1 for a in range(3))
+    want_map, want_coords = oracle.kmap_downsample(coords, ks, stride, pad, spatial_range=new_sr)
+    np.testing.assert_array_equal(kmap["coords"].cpu().numpy(), want_coords)
+    np.testing.assert_array_equal(kmap["out_in_map"].cpu().numpy(), want_map)
+
+
+def test_unsorted_or_repeated_rows_take_the_tables():
+    rng = np.random.default_rng(202)
+    coords = ascending(random_coords(rng, 500, (10, 10, 10)))
+    swapped = coords.copy()
+    swapped[[100, 101]] = swapped[[101, 100]]
+    repeated = np.concatenate([coords[:200], coords[199:]])
+    for rows in (swapped, repeated):
+        t = dev(rows)
+        assert not backend.coords_ascending(t)
+        kmap = F.build_kernel_map(t, len(rows), 3, 1, 0, mode="hashmap_on_the_fly")
+        assert kmap["in_hashmap"] is not None
+    assert backend.coords_ascending(dev(coords))
+    assert backend.coords_ascending(dev(coords[:1])) and backend.coords_ascending(dev(coords[:0]))
+
+
+def test_segments_longer_than_the_staging_area_are_searched_in_memory():
+    """A thin slab next to a dense one: the block that holds the thin slab's rows needs the
+    whole dense slab as its segment for the x-digit that points there."""
+    ys, zs = np.meshgrid(np.arange(120), np.arange(60), indexing="ij")
+    dense = np.stack([np.zeros(ys.size), np.full(ys.size, 5), ys.ravel(), zs.ravel()], 1)
+    thin_y = np.arange(0, 120, 3)
+    thin = np.stack([np.zeros(thin_y.size), np.full(thin_y.size, 4), thin_y, np.full(thin_y.size, 7)], 1)
+    far = np.stack([np.zeros(50), np.full(50, 9), np.arange(50), np.arange(50)], 1)
+    coords = ascending(np.concatenate([thin, dense, far]).astype(np.int32))
+    kmap = build(coords, 3, 1, 0)
+    np.testing.assert_array_equal(kmap["out_in_map"].cpu().numpy(), oracle.kmap_subm(coords, 3))
+    kmap = build(coords, (3, 3, 3), (1, 2, 2), (1, 1, 1))
+    want_map, want_coords = oracle.kmap_downsample(coords, (3, 3, 3), (1, 2, 2), (1, 1, 1))
+    np.testing.assert_array_equal(kmap["coords"].cpu().numpy(), want_coords)
+    np.testing.assert_array_equal(kmap["out_in_map"].cpu().numpy(), want_map)
+
+
+@pytest.mark.parametrize("n,extent", [(1, (3, 3, 3)), (2, (2, 2, 2)), (255, (9, 9, 9)), (256, (9, 9, 9)),
+                                      (257, (9, 9, 9)), (70000, (300, 300, 12)), (300000, (900, 900, 30))])
+def test_sizes_around_the_sampling_levels(n, extent):
+    """One and two sampling levels (more than 65536 rows: second-level samples every other row
+    and beyond), tiny inputs, sizes around one block."""
+    rng = np.random.default_rng(n)
+    coords = ascending(random_coords(rng, n, extent))
+    kmap = build(coords, 3, 1, 0)
+    np.testing.assert_array_equal(kmap["out_in_map"].cpu().numpy(), oracle.kmap_subm(coords, 3))
+    kmap = build(coords, 2, 2, 0)
+    want_map, want_coords = oracle.kmap_downsample(coords, 2, 2, 0)
+    np.testing.assert_array_equal(kmap["coords"].cpu().numpy(), want_coords)
+    np.testing.assert_array_equal(kmap["out_in_map"].cpu().numpy(), want_map)
+
+
+def test_sorted_search_equals_the_table_builders_on_random_geometries():
+    """Per-axis kernel, stride and padding drawn at random; the searched map against the
+    hash-table map of the same rows (itself pinned by the oracle elsewhere)."""
+    rng = np.random.default_rng(203)
+    for case in range(40):
+        ks = tuple(int(v) for v in rng.integers(1, 5, 3))
+        st = tuple(int(v) for v in rng.integers(1, 4, 3))
+        pd = tuple(int(v) for v in rng.integers(0, 3, 3))
+        n = int(rng.integers(1, 6000))
+        extent = tuple(int(v) for v in rng.integers(3, 60, 3))
+        n = min(n, int(np.prod(extent)))
+        coords = ascending(random_coords(rng, n, extent, batch=int(rng.integers(1, 3))))
+        if case % 2:
+            coords[:, 1:] -= np.array(extent) // 2  # negative coordinates: the biased key keeps the order
+        ins = dev(coords)
+        outs = dev(ascending(random_coords(rng, max(n // 2, 1), extent)))
+        table = backend.GPUHashTable(backend.hash_capacity(len(coords)), device="cuda")
+        table.insert_bxyz(ins)
+        want = table.query_bxyz(outs, ks, st, pd)
+        got = backend.kmap_sorted(ins, outs, ks, st, pd)
+        assert torch.equal(got, want), (case, ks, st, pd, n, extent)
+
+
+def test_negative_coordinates_and_the_edge_of_the_packed_range():
+    import torchsparse_amd as ts
+    rng = np.random.default_rng(204)
+    base = random_coords(rng, 600, (11, 11, 11))
+    lo = base.copy()
+    lo[:, 1:] -= 131072
+    lo = ascending(lo)
+    kmap = build(lo, 3, 1, 0)
+    np.testing.assert_array_equal(kmap["out_in_map"].cpu().numpy(),
+                                  oracle.kmap_subm(lo, 3, coords_min=lo.min(0), coords_max=lo.max(0)))
+    hi = base.copy()
+    hi[:, 1:] += 131072 - 11
+    hi[:, 0] = 511
+    hi = ascending(hi)
+    kmap = build(hi, 3, 1, 0)
+    np.testing.assert_array_equal(kmap["out_in_map"].cpu().numpy(), oracle.kmap_subm(hi, 3))
+    kmap = build(hi, 2, 2, 0)
+    want_map, want_coords = oracle.kmap_downsample(hi, 2, 2, 0)
+    np.testing.assert_array_equal(kmap["coords"].cpu().numpy(), want_coords)
+    np.testing.assert_array_equal(kmap["out_in_map"].cpu().numpy(), want_map)
+    mid = base.copy()
+    mid[:, 1:] -= 5
+    mid = ascending(mid)
+    ts.set_allow_negative_coordinates(True)
+    try:
+        kmap = build(mid, 3, 2, 1)
+        want_map, want_coords = oracle.kmap_downsample(mid, 3, 2, 1, allow_negative=True)
+    finally:
+        ts.set_allow_negative_coordinates(False)
+    np.testing.assert_array_equal(kmap["coords"].cpu().numpy(), want_coords)
+    np.testing.assert_array_equal(kmap["out_in_map"].cpu().numpy(), want_map)
+
+
+def test_scan_like_surface_and_switch():
+    rng = np.random.default_rng(205)
+    coords = ascending(lidar_like_coords(rng, 60000))
+    kmap = build(coords, 3, 1, 0)
+    np.testing.assert_array_equal(kmap["out_in_map"].cpu().numpy(), oracle.kmap_subm(coords, 3))
+    backend.kmap_through_sorted = False
+    try:
+        hashed = F.build_kernel_map(dev(coords), len(coords), 3, 1, 0, mode="hashmap_on_the_fly")
+    finally:
+        backend.kmap_through_sorted = True
+    assert hashed["in_hashmap"] is not None
+    assert torch.equal(hashed["out_in_map"], kmap["out_in_map"])

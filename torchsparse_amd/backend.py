@@ -83,6 +83,9 @@ def _load():
         "tsmi_wgrad_pairs_build": [_vp, _vp, _i64, _i32, _vp, _vp, _vp, _vp],
         "tsmi_wgrad_pairs_build_static": [_vp, _vp, _i64, _i32, _vp, _vp, _vp],
         "tsmi_kmap_build_subm": [_vp, _vp, _vp, _i64, _vp, _i64, _i64, _I3, _vp, _vp],
+        "tsmi_coords_check": [_vp, _vp, _i64, _vp],
+        "tsmi_kmap_sorted_supported": [_I3],
+        "tsmi_kmap_sorted": [_vp, _vp, _i64, _vp, _i64, _i64, _I3, _I3, _I3, _vp],
         "tsmi_wgrad_pairs_pad": [_vp, _vp, _i64, _vp, _i32, _vp, _vp],
         "tsmi_conv_wgrad_pairs": [_vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _i32, _vp,
                                   _i64, _vp],
@@ -175,11 +178,15 @@ def hash_capacity(n: int, ratio: float = 2.0) -> int:
 # ravels over the measured extents and takes any int32 coordinate
 # (others/sparsemapping_cuda.cu:12-26); here a row outside the packed range must stop the
 # call: the kernels flag it and the shim raises.  A flag costs a read-back, so a coordinate
-# tensor is checked once: tensors that passed (and the ones the strided builders produced
-# from them) are remembered by identity, version and address.
+# tensor is looked at once: what is known of it — it is in range; its rows ascend strictly in
+# (b, x, y, z) or do not — is remembered by identity, version and address.  The strided
+# builders produce ascending rows in range and say so for their outputs.
 COORD_LIMIT = 1 << 17
 BATCH_LIMIT = 512
-_range_ok = {}  # id(tensor) -> (weak reference, version, address)
+_range_ok = {}  # id(tensor) -> (weak reference, version, address, ascending: True / False / None = not known)
+# Kernel maps of ascending inputs are built by binary search over the coordinates themselves
+# (no hash table); False sends every map through the tables.
+kmap_through_sorted = True
 
 
 def _range_error() -> ValueError:
@@ -188,19 +195,66 @@ def _range_error() -> ValueError:
         f"[{-COORD_LIMIT}, {COORD_LIMIT}) and the batch index in [0, {BATCH_LIMIT})")
 
 
-def _range_known(coords: torch.Tensor) -> bool:
+def _range_entry(coords: torch.Tensor):
     hit = _range_ok.get(id(coords))
-    return (hit is not None and hit[0]() is coords and hit[1] == coords._version
-            and hit[2] == coords.data_ptr())
+    if (hit is not None and hit[0]() is coords and hit[1] == coords._version
+            and hit[2] == coords.data_ptr()):
+        return hit
+    return None
 
 
-def _mark_range_ok(coords: torch.Tensor) -> None:
+def _range_known(coords: torch.Tensor) -> bool:
+    return _range_entry(coords) is not None
+
+
+def _mark_range_ok(coords: torch.Tensor, ascending: Optional[bool] = None) -> None:
+    """``coords`` is in range; ``ascending`` says whether its rows ascend strictly (None keeps
+    what is already known)."""
+    if ascending is None:
+        hit = _range_entry(coords)
+        if hit is not None:
+            return
     if len(_range_ok) >= 512:
         for key in [k for k, v in _range_ok.items() if v[0]() is None]:
             del _range_ok[key]
         if len(_range_ok) >= 512:
             _range_ok.clear()
-    _range_ok[id(coords)] = (weakref.ref(coords), coords._version, coords.data_ptr())
+    _range_ok[id(coords)] = (weakref.ref(coords), coords._version, coords.data_ptr(), ascending)
+
+
+def coords_ascending(coords: torch.Tensor) -> bool:
+    """Whether the rows of ``coords`` ascend strictly in (b, x, y, z); raises ValueError for a
+    row outside the packed key's range.  One kernel and one read-back the first time a tensor
+    is seen, nothing afterwards."""
+    hit = _range_entry(coords)
+    if hit is not None and hit[3] is not None:
+        return hit[3]
+    rows = _need(coords, torch.int32, "coords")
+    flags = torch.zeros(1, dtype=torch.int32, device=rows.device)
+    _check(_C.tsmi_coords_check(_stream(), _ptr(rows), rows.shape[0], _ptr(flags)))
+    bits = int(flags.item())
+    if bits & 2:
+        raise _range_error()
+    _mark_range_ok(coords, ascending=not (bits & 1))
+    return not (bits & 1)
+
+
+def kmap_sorted_supported(kernel_size) -> bool:
+    return bool(kmap_through_sorted and _C.tsmi_kmap_sorted_supported(_I3(*_triple(kernel_size))))
+
+
+def kmap_sorted(in_coords: torch.Tensor, out_coords: torch.Tensor, kernel_size, stride, pad) -> torch.Tensor:
+    """out_in_map int32 [ceil128(N_out), K_vol] of ascending in-range inputs and ascending
+    outputs, by binary search over the input rows: no hash table, one launch."""
+    in_coords = _need(in_coords, torch.int32, "coords")
+    out_coords = _need(out_coords, torch.int32, "coords")
+    ks, st, pd = _triple(kernel_size), _triple(stride), _triple(pad)
+    n_out = out_coords.shape[0]
+    n_pad = make_divisible(n_out, 128)
+    omap = torch.empty((n_pad, ks[0] * ks[1] * ks[2]), dtype=torch.int32, device=out_coords.device)
+    _check(_C.tsmi_kmap_sorted(_stream(), _ptr(in_coords), in_coords.shape[0], _ptr(out_coords), n_out,
+                               n_pad, _I3(*ks), _I3(*st), _I3(*pd), _ptr(omap)))
+    return omap
 
 
 def _settle_insert(coords: torch.Tensor, status: torch.Tensor) -> None:
@@ -356,9 +410,10 @@ def coords_max(coords: torch.Tensor) -> torch.Tensor:
 
 def downsample_coords(coords: torch.Tensor, kernel_sizes, stride, padding, coords_max_host=None,
                       mode: int = 0, rsv_ratio: float = 2.0, allow_negative: bool = False,
-                      _reserve_all: bool = False):
+                      _reserve_all: bool = False, want_table: bool = True):
     """Output coordinates of a strided convolution in ascending (b,x,y,z) order and
-    the hash table that indexes them.  Returns (out_coords, GPUHashTable).
+    the hash table that indexes them.  Returns (out_coords, GPUHashTable); with
+    ``want_table=False`` the table may be None (callers that search the sorted rows).
     One host read-back (the number of outputs) — the reference has two
     (others/sparsemapping_cuda.cu:477-479).  With ``allow_negative`` the outputs are bounded
     below by the reference's coords_min (hashmap_on_the_fly.py:39-43) instead of 0."""
@@ -386,14 +441,16 @@ def downsample_coords(coords: torch.Tensor, kernel_sizes, stride, padding, coord
             chain = (ks, st, pd, rsv_ratio) if coords_max_host is None else None
             ahead = state.chain_step(coords, chain)
             if not isinstance(ahead, int):  # computed ahead when the previous level of the chain was
+                if want_table and ahead[1] is None:
+                    tbl = GPUHashTable(hash_capacity(ahead[0].shape[0], rsv_ratio), device=dev)
+                    tbl.insert_bxyz(ahead[0])
+                    return ahead[0], tbl
                 return ahead
-            table = GPUHashTable(cap, device=dev)
             done = _downsample_coords_grid(state, coords, ks, st, pd, coords_max_host, fan, rsv_ratio,
-                                           table, ahead)
+                                           cap, ahead, want_table)
             if done is not None:
                 state.chain_last = weakref.ref(done[0])
                 return done
-        table.counters.zero_()
     if table is None:
         table = GPUHashTable(cap, device=dev)
     counters = table.counters  # zero on a fresh table
@@ -437,7 +494,7 @@ def downsample_coords(coords: torch.Tensor, kernel_sizes, stride, padding, coord
         _check(_C.tsmi_sort_keys(s, _ptr(uniq), _ptr(sorted_keys), n_out, 63, _ptr(temp), temp_bytes))
         _check(_C.tsmi_downsample_finalize(s, _ptr(sorted_keys), n_out, _ptr(table.keys),
                                            _ptr(table.vals), cap, _ptr(out_coords)))
-    _mark_range_ok(out_coords)  # unpacked from keys
+    _mark_range_ok(out_coords, ascending=True)  # unpacked from sorted keys
     return out_coords, table
 
 
@@ -545,7 +602,8 @@ def _grid_layout(words0: int):
     return out, off
 
 
-def _downsample_coords_grid(state, coords, ks, st, pd, coords_max_host, fan, rsv_ratio, table, ahead=0):
+def _downsample_coords_grid(state, coords, ks, st, pd, coords_max_host, fan, rsv_ratio, cap, ahead=0,
+                            want_table=True):
     """downsample_coords for non-negative coordinates when the output grid has at most
     2048 cells per candidate (and at most 2^30): mark an occupancy bitmap, count, read the
     number of outputs back, emit rows and table entries in ascending order.  None when the grid
@@ -559,7 +617,7 @@ def _downsample_coords_grid(state, coords, ks, st, pd, coords_max_host, fan, rsv
     layout, _ = _grid_layout(state.grid_words)
     levels = 1 + ahead
     # per level 8 counters: [n_out, table overflow, grid too large, -, max b, x, y, z of the INPUTS]
-    ctr = table.counters if levels == 1 else torch.zeros(8 * levels, dtype=torch.int32, device=dev)
+    ctr = torch.zeros(8 * levels, dtype=torch.int32, device=dev)
     s = _stream()
     g = (_I3(*ks), _I3(*st), _I3(*pd))
     host_max = _I3(*[int(v) for v in coords_max_host]) if coords_max_host is not None else None
@@ -594,26 +652,29 @@ def _downsample_coords_grid(state, coords, ks, st, pd, coords_max_host, fan, rsv
     if host[0] > 0:  # the marking pass looked at every input row
         _mark_range_ok(coords)
 
-    def emit(level, n_in, tbl):
+    def emit(level, n_in, capacity):
         n_out = host[8 * level]
-        if n_out > tbl.capacity and fan > 2:  # more than the two outputs per input reserved
-            tbl = GPUHashTable(hash_capacity(n_in * fan, rsv_ratio), device=dev)
-        if n_out > tbl.capacity:
+        if n_out > capacity and fan > 2:  # more than the two outputs per input reserved
+            capacity = hash_capacity(n_in * fan, rsv_ratio)
+        if n_out > capacity:  # the reference's limit, with or without a table to overflow
             raise ValueError(
                 "The capacity of hashtable is not sufficient. Please enlarge reserved space for "
                 "hashtable:\n # Python \nimport torchsparse_amd.backends\n"
                 "torchsparse_amd.backends.hash_rsv_ratio=#Value")
+        tbl = GPUHashTable(capacity, device=dev) if want_table else None
         out = torch.empty((n_out, 4), dtype=torch.int32, device=dev)
         if n_out > 0:
             _check(_C.tsmi_downsample_grid_emit(
                 s, *g, host_max, _ptr(part(level, "in_max")),
                 (ctypes.c_int32 * 4)(*host[8 * level + 4:8 * level + 8]), _ptr(part(level, "bitmap")),
-                layout[level][1], _ptr(part(level, "chunks")), n_out, _ptr(tbl.keys), _ptr(tbl.vals),
-                tbl.capacity, _ptr(out), _ptr(tbl.counters)))
+                layout[level][1], _ptr(part(level, "chunks")), n_out,
+                _ptr(tbl.keys) if tbl is not None else None, _ptr(tbl.vals) if tbl is not None else None,
+                capacity, _ptr(out), _ptr(tbl.counters) if tbl is not None else _ptr(part(level, "counters"))))
         return out, tbl
 
-    first = emit(0, n, table)
-    _mark_range_ok(first[0])  # cells of a grid whose every in-range candidate was packable
+    first = emit(0, n, cap)
+    # cells of a grid whose every in-range candidate was packable, in ascending order
+    _mark_range_ok(first[0], ascending=True)
     prev = first[0]
     clean = True
     for level in range(1, levels):
@@ -623,7 +684,7 @@ def _downsample_coords_grid(state, coords, ks, st, pd, coords_max_host, fan, rsv
             break  # this level's grid did not fit its bitmap: it and the later ones marked nothing
         n_in = prev.shape[0]
         try:
-            nxt = emit(level, n_in, GPUHashTable(hash_capacity(n_in * min(fan, 2), rsv_ratio), device=dev))
+            nxt = emit(level, n_in, hash_capacity(n_in * min(fan, 2), rsv_ratio))
         except ValueError:  # not asked for yet: let the call that asks raise it
             clean = False  # this level's marks (and the later ones') are still in the bitmaps
             break
@@ -631,7 +692,7 @@ def _downsample_coords_grid(state, coords, ks, st, pd, coords_max_host, fan, rsv
         # the later levels are not flagged on the device; their inputs' maxima are on the host
         if (host[8 * level + 4] < BATCH_LIMIT and
                 all(host[8 * level + 5 + a] + 2 * pd[a] < COORD_LIMIT for a in range(3))):
-            _mark_range_ok(nxt[0])
+            _mark_range_ok(nxt[0], ascending=True)
         prev = nxt[0]
     state.grid_dirty = not clean
     return first

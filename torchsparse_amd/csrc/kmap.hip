@@ -989,6 +989,8 @@ __global__ void scan_quantified_kernel(int kvol, const int32_t *nbsizes, int q, 
   }
 }
 
+#include "kmap_sorted.inc"
+
 int make_table(TableView *t, const int64_t *keys, const int32_t *vals, int64_t cap) {
   TSMI_REQUIRE(keys != nullptr && vals != nullptr, "hash table: null keys/vals");
   TSMI_REQUIRE(cap >= 8 && cap % 8 == 0 && cap < (int64_t(1) << 31),
@@ -1174,6 +1176,54 @@ extern "C" int tsmi_kmap_build_subm(tsmi_stream_t s, int64_t *keys, int32_t *val
   return check_launch("tsmi_kmap_build_subm");
 }
 
+extern "C" int tsmi_coords_check(tsmi_stream_t s, const int32_t *coords, int64_t n, int32_t *flags) {
+  TSMI_REQUIRE(flags && n >= 0 && (n == 0 || coords), "coords_check: bad arguments");
+  if (n == 0) return TSMI_OK;
+  TSMI_GRID_CHECK(n);
+  hipLaunchKernelGGL(coords_check_kernel, grid_for(n), dim3(kBlock), 0, (hipStream_t)s,
+                     (const int4 *)coords, n, flags);
+  return check_launch("tsmi_coords_check");
+}
+
+extern "C" int tsmi_kmap_sorted_supported(const int32_t ks[3]) {
+  if (!ks || ks[0] < 1 || ks[1] < 1 || ks[2] < 1) return 0;
+  const int64_t kvol = (int64_t)ks[0] * ks[1] * ks[2];
+  return ks[0] <= kSortedMaxKs0 && ks[1] <= kSortedMaxKs1 && kvol <= kSortedTileInts;
+}
+
+extern "C" int tsmi_kmap_sorted(tsmi_stream_t s, const int32_t *in_coords, int64_t n_in,
+                                const int32_t *out_coords, int64_t n_out, int64_t n_out_pad,
+                                const int32_t ks[3], const int32_t stride[3], const int32_t pad[3],
+                                int32_t *out_in_map) {
+  SortedArgs a;
+  if (int e = make_geom(&a.g, ks, stride, pad)) return e;
+  TSMI_REQUIRE(tsmi_kmap_sorted_supported(ks), "kmap_sorted: kernel size (%d, %d, %d) not supported",
+               ks[0], ks[1], ks[2]);
+  TSMI_REQUIRE(n_in >= 0 && n_in < (int64_t(1) << 31) && (n_in == 0 || in_coords), "kmap_sorted: bad in_coords");
+  TSMI_REQUIRE(n_out >= 0 && n_out_pad >= n_out && n_out_pad < (int64_t(1) << 31),
+               "kmap_sorted: n_out_pad < n_out");
+  TSMI_REQUIRE(n_out == 0 || out_coords, "kmap_sorted: null out_coords");
+  if (n_out_pad == 0) return TSMI_OK;
+  TSMI_REQUIRE(out_in_map, "kmap_sorted: null out_in_map");
+  a.in_coords = (const int4 *)in_coords;
+  a.out_coords = (const int4 *)out_coords;
+  a.map = out_in_map;
+  a.n_in = n_in;
+  a.n_out = n_out;
+  a.n_out_pad = n_out_pad;
+  a.rows = std::min(kBlock, kSortedTileInts / a.g.kvol);
+  const int64_t blocks = ceil_div(n_out_pad, a.rows);
+  TSMI_REQUIRE(grid_fits(blocks), "kmap_sorted: too many rows for one launch");
+  const dim3 grid((unsigned)blocks), block(kBlock);
+  const int cube = (ks[0] == ks[1] && ks[1] == ks[2] && a.rows == kBlock) ? ks[0] : 0;
+  switch (cube) {
+    case 2: hipLaunchKernelGGL(kmap_sorted_kernel<2>, grid, block, 0, (hipStream_t)s, a); break;
+    case 3: hipLaunchKernelGGL(kmap_sorted_kernel<3>, grid, block, 0, (hipStream_t)s, a); break;
+    default: hipLaunchKernelGGL(kmap_sorted_kernel<0>, grid, block, 0, (hipStream_t)s, a); break;
+  }
+  return check_launch("tsmi_kmap_sorted");
+}
+
 extern "C" int tsmi_coords_max(tsmi_stream_t s, const int32_t *coords, int64_t n,
                                int32_t *out_max, int clear_first) {
   TSMI_REQUIRE(out_max && n >= 0 && (n == 0 || coords), "coords_max: bad arguments");
@@ -1353,9 +1403,11 @@ extern "C" int tsmi_downsample_grid_emit(tsmi_stream_t s, const int32_t ks[3], c
   if (int e = grid_args(&g, &mode, &hm, ks, stride, pad, out_max_host, in_max_dev, bitmap, bitmap_words,
                         chunk_prefix, counters))
     return e;
-  if (int e = make_table(&t, keys, vals, cap)) return e;
+  const bool want_table = keys != nullptr;
+  if (want_table)
+    if (int e = make_table(&t, keys, vals, cap)) return e;
   TSMI_REQUIRE(n_out >= 0 && (n_out == 0 || out_coords), "downsample_grid_emit: bad arguments");
-  TSMI_REQUIRE(n_out <= cap,
+  TSMI_REQUIRE(!want_table || n_out <= cap,
                "The capacity of hashtable is not sufficient. Please enlarge reserved space for "
                "hashtable (backends.hash_rsv_ratio): %lld outputs, capacity %lld",
                (long long)n_out, (long long)cap);
@@ -1374,8 +1426,9 @@ extern "C" int tsmi_downsample_grid_emit(tsmi_stream_t s, const int32_t ks[3], c
   hipLaunchKernelGGL(grid_emit_kernel, dim3((unsigned)chunks), dim3(kBlock), 0, (hipStream_t)s,
                      (uint32_t *)bitmap, bitmap_words, chunk_prefix, g, hm, out_max_host != nullptr,
                      in_max_dev, hd, in_max_host != nullptr, (int4 *)out_coords, n_out);
-  hipLaunchKernelGGL(insert_coords_kernel, grid_for(n_out), dim3(kBlock), 0, (hipStream_t)s, t,
-                     (const int4 *)out_coords, n_out, counters + 1);
+  if (want_table)
+    hipLaunchKernelGGL(insert_coords_kernel, grid_for(n_out), dim3(kBlock), 0, (hipStream_t)s, t,
+                       (const int4 *)out_coords, n_out, counters + 1);
   return check_launch("tsmi_downsample_grid_emit");
 }
 

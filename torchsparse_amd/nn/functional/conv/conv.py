@@ -98,8 +98,10 @@ def conv3d(input: SparseTensor, weight: torch.Tensor,
                 ifsort=config["ifsort"], split_mask_num=config["split_mask_num"],
                 split_mask_num_bwd=config["split_mask_num_bwd"])
             caches.kmaps[key] = kmap
-            caches.hashmaps.setdefault(input.stride, kmap["in_hashmap"])
-            caches.hashmaps.setdefault(out_stride, kmap["out_hashmap"])
+            # tables exist only where a map was built through one (unsorted coordinates, "hashmap" mode)
+            for level, table in ((input.stride, kmap["in_hashmap"]), (out_stride, kmap["out_hashmap"])):
+                if table is not None and caches.hashmaps.get(level) is None:
+                    caches.hashmaps[level] = table
         out_feats = conv_fn.apply(feats, weight, kmap, config, False, bias, residual, relu)
         output = SparseTensor._make(out_feats, kmap["coords"], out_stride, kmap["spatial_range"], caches)
     elif generative:

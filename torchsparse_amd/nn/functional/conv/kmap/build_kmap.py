@@ -166,52 +166,76 @@ def build_kernel_map(_coords: torch.Tensor, input_node_num: int,
     coords = _coords.contiguous()
     n_in = coords.shape[0]
 
-    # table over the input coordinates: reuse or build
     fresh = hashmap_keys is None or hashmap_vals is None
     out_in_map = None
-    if fresh and subm and (mode == "hashmap_on_the_fly" or all(k % 2 == 1 for k in kernel_size)):
-        # table and map in one call (an even kernel in "hashmap" mode is centred differently)
-        in_table, out_in_map = backend.GPUHashTable.build_subm(coords, kernel_size, backends.hash_rsv_ratio)
-    elif fresh:
-        in_table = backend.GPUHashTable(backend.hash_capacity(n_in, backends.hash_rsv_ratio),
-                                        device=coords.device)
-        in_table.insert_bxyz(coords)
+    in_table = out_table = None
+    # Ascending input rows (voxelisation by a ravelled key, every strided builder here): the
+    # map is searched over the rows themselves and no table is built at all.
+    by_search = (mode == "hashmap_on_the_fly" and n_in > 0 and backend.kmap_sorted_supported(kernel_size)
+                 and backend.coords_ascending(_coords))
+    if by_search:
+        if subm:
+            out_coords = coords
+            out_in_map = backend.kmap_sorted(coords, coords, kernel_size, stride, backend._subm_pad(kernel_size))
+        else:
+            host_max = None if new_range is None else tuple(x - 1 for x in new_range[1:])
+            from torchsparse_amd.tensor import get_allow_negative_coordinates
+            out_coords, out_table = backend.downsample_coords(
+                coords, kernel_size, stride, padding, host_max, 0, backends.hash_rsv_ratio,
+                allow_negative=get_allow_negative_coordinates(), want_table=False)
+            out_in_map = backend.kmap_sorted(coords, out_coords, kernel_size, stride, padding)
+        if not fresh:
+            in_table = backend.GPUHashTable(hashmap_keys, hashmap_vals)
     else:
-        in_table = backend.GPUHashTable(hashmap_keys, hashmap_vals)
-    kmap["in_hashmap"] = (in_table.keys, in_table.vals)
+        # table over the input coordinates: reuse or build
+        if fresh and subm and (mode == "hashmap_on_the_fly" or all(k % 2 == 1 for k in kernel_size)):
+            # table and map in one call (an even kernel in "hashmap" mode is centred differently)
+            in_table, out_in_map = backend.GPUHashTable.build_subm(coords, kernel_size, backends.hash_rsv_ratio)
+        elif fresh:
+            in_table = backend.GPUHashTable(backend.hash_capacity(n_in, backends.hash_rsv_ratio),
+                                            device=coords.device)
+            in_table.insert_bxyz(coords)
+        else:
+            in_table = backend.GPUHashTable(hashmap_keys, hashmap_vals)
 
-    if subm:
-        out_coords = coords
-        pad_eff = backend._subm_pad(kernel_size)
-        out_table = in_table
-    elif mode == "hashmap_on_the_fly":
-        host_max = None if new_range is None else tuple(x - 1 for x in new_range[1:])
-        from torchsparse_amd.tensor import get_allow_negative_coordinates
-        out_coords, out_table = backend.downsample_coords(
-            coords, kernel_size, stride, padding, host_max, 0, backends.hash_rsv_ratio,
-            allow_negative=get_allow_negative_coordinates())
-        pad_eff = padding
-    else:  # "hashmap": coordinates first, then a padding-free centred lookup
-        from .downsample import spdownsample
-        out_coords, out_table = spdownsample(coords, stride, kernel_size, padding, new_range,
-                                             downsample_mode, return_table=True)
-        pad_eff = tuple((k - 1) // 2 for k in kernel_size)
-    if subm and mode == "hashmap":
-        pad_eff = tuple((k - 1) // 2 for k in kernel_size)
+        if subm:
+            out_coords = coords
+            pad_eff = backend._subm_pad(kernel_size)
+            out_table = in_table
+        elif mode == "hashmap_on_the_fly":
+            host_max = None if new_range is None else tuple(x - 1 for x in new_range[1:])
+            from torchsparse_amd.tensor import get_allow_negative_coordinates
+            out_coords, out_table = backend.downsample_coords(
+                coords, kernel_size, stride, padding, host_max, 0, backends.hash_rsv_ratio,
+                allow_negative=get_allow_negative_coordinates())
+            pad_eff = padding
+        else:  # "hashmap": coordinates first, then a padding-free centred lookup
+            from .downsample import spdownsample
+            out_coords, out_table = spdownsample(coords, stride, kernel_size, padding, new_range,
+                                                 downsample_mode, return_table=True)
+            pad_eff = tuple((k - 1) // 2 for k in kernel_size)
+        if subm and mode == "hashmap":
+            pad_eff = tuple((k - 1) // 2 for k in kernel_size)
 
-    if out_in_map is not None:
-        pass
-    elif subm and all(k % 2 == 1 for k in kernel_size):
-        out_in_map = in_table.query_subm_bxyz(out_coords, kernel_size)  # centred in both modes
-    else:
-        out_in_map = in_table.query_bxyz(out_coords, kernel_size, stride, pad_eff)
+        if out_in_map is not None:
+            pass
+        elif subm and all(k % 2 == 1 for k in kernel_size):
+            out_in_map = in_table.query_subm_bxyz(out_coords, kernel_size)  # centred in both modes
+        else:
+            out_in_map = in_table.query_bxyz(out_coords, kernel_size, stride, pad_eff)
+
+    def pair(table):
+        return None if table is None else (table.keys, table.vals)
+
     kmap["out_in_map"] = out_in_map
     kmap["subm"] = subm  # stride 1: outputs are the inputs, the centre offset is the identity
     kmap["coords"] = out_coords if not subm else _coords
     kmap["sizes"] = (input_node_num, out_coords.shape[0])
-    kmap["out_hashmap"] = (out_table.keys, out_table.vals)
-    kmap["hashmap_keys"], kmap["hashmap_vals"] = (
-        (in_table.keys, in_table.vals) if (subm or mode == "hashmap") else (out_table.keys, out_table.vals))
+    # tables of the input / output coordinates: None when the map was searched over sorted rows
+    kmap["in_hashmap"] = pair(in_table)
+    kmap["out_hashmap"] = pair(in_table if (subm and out_table is None) else out_table)
+    owner = in_table if (subm or mode == "hashmap") else out_table
+    kmap["hashmap_keys"], kmap["hashmap_vals"] = pair(owner) if owner is not None else (None, None)
 
     if dataflow == Dataflow.ImplicitGEMM:
         if ifsort:
