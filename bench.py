@@ -183,12 +183,68 @@ def layer_sweep(ts, spnn, F, backend, coords_dev, n):
             kbytes = 4.0 * kvol * (km["out_in_map"].shape[0] + n_pad)  # read one map, write the other
         else:
             kbytes = kmap_bytes_down(n, n_out, n_pad, cap, nnz, kvol)
-        out.append({"layer": name, "n_in": n_in, "n_out": n_out, "nnz": nnz,
-                    "kmap_ms": round(kmap_ms, 4), "kmap_GBps": round(kbytes / kmap_ms / 1e6, 1),
-                    "conv_ms": round(conv_ms, 4),
-                    "eff_TFLOPs": round(flops / conv_ms / 1e9, 2),
-                    "min_bytes_GBps": round(nbytes / conv_ms / 1e6, 1)})
+        row = {"layer": name, "n_in": n_in, "n_out": n_out, "nnz": nnz,
+               "kmap_ms": round(kmap_ms, 4), "kmap_GBps": round(kbytes / kmap_ms / 1e6, 1),
+               "conv_ms": round(conv_ms, 4),
+               "eff_TFLOPs": round(flops / conv_ms / 1e9, 2),
+               "min_bytes_GBps": round(nbytes / conv_ms / 1e6, 1)}
+        row.update(pair_dataflows(ts, spnn, F, backend, layer, inp, mid if transposed else None,
+                                  k, s, transposed, cin, cout, flops))
+        out.append(row)
         del y
+    return out
+
+
+def pair_dataflows(ts, spnn, F, backend, layer, inp, mid, k, s, transposed, cin, cout, flops):
+    """The same layer through the two pair-list dataflows (warm map products): the whole layer,
+    and for gather-scatter its gather and scatter kernels on their own with the bytes they have
+    to move — gather: every pair's input row read and written plus its index
+    (nnz * (2 * Cin * 2 + 4)); scatter: every product row and its mask entry read, every output
+    row written (nnz * (Cout * 2 + 4) + N_out * Cout * 2)."""
+    out = {}
+    key = ((1, 1, 1), (k,) * 3, (s,) * 3, (1, 1, 1))
+    for flow, tag in ((F.Dataflow.GatherScatter, "gather_scatter"), (F.Dataflow.FetchOnDemand, "fetch_on_demand")):
+        cfg = F.conv_config.get_default_conv_config()
+        cfg.dataflow = flow
+        twin = spnn.Conv3d(cin, cout, k, stride=s, transposed=transposed, config=cfg).cuda().half()
+        twin.kernel.data.copy_(layer.kernel.data)
+        if transposed:
+            lower = spnn.Conv3d(1, cin, k, stride=s, config=cfg).cuda().half()
+            fine = ts.SparseTensor(torch.zeros(mid._caches.cmaps[(1, 1, 1)][0].shape[0], 1, device="cuda",
+                                               dtype=torch.float16), mid._caches.cmaps[(1, 1, 1)][0])
+            coarse = lower(fine)  # this dataflow's products of the strided map
+            x = ts.SparseTensor(inp.feats, coarse.coords, stride=coarse.stride)
+            x._caches = coarse._caches
+        else:
+            x = ts.SparseTensor(inp.feats, inp.coords)
+        with torch.no_grad():
+            twin(x)  # builds the pair lists once
+            ms = event_ms(lambda: twin(x), iters=20)
+        out[tag + "_ms"] = round(ms, 4)
+        out[tag + "_eff_TFLOPs"] = round(flops / ms / 1e9, 2)
+        if flow == F.Dataflow.GatherScatter:
+            km = x._caches.kmaps[key]
+            nb = km["nbmaps"]
+            nnz = nb.shape[0]
+            n_rows_out = km["sizes"][0] if transposed else km["sizes"][1]
+            code = 1
+            C = backend._C
+            st = backend._stream()
+            gathered = torch.empty((max(nnz, 1), cin), dtype=torch.float16, device="cuda")
+            products = torch.randn((max(nnz, 1), cout), dtype=torch.float16, device="cuda")
+            y = torch.empty((n_rows_out, cout), dtype=torch.float16, device="cuda")
+            feats = inp.feats
+            g_ms = event_ms(lambda: C.tsmi_gs_gather(st, feats.data_ptr(), nb.data_ptr(), nnz, cin, code,
+                                                     int(transposed), gathered.data_ptr()), iters=20)
+            mask = km["input_mask"] if transposed else km["output_mask"]
+            center = k ** 3 // 2 if (s == 1 and k % 2 == 1) else -1
+            s_ms = event_ms(lambda: C.tsmi_gs_scatter(st, products.data_ptr(), km["nbaddrs"].data_ptr(),
+                                                      mask.data_ptr(), n_rows_out, k ** 3, cout, code, center,
+                                                      None, None, 0, y.data_ptr()), iters=20)
+            out["gather_ms"] = round(g_ms, 4)
+            out["gather_GBps"] = round(nnz * (2 * cin * 2 + 4) / g_ms / 1e6, 1)
+            out["scatter_ms"] = round(s_ms, 4)
+            out["scatter_GBps"] = round((nnz * (cout * 2 + 4) + n_rows_out * cout * 2) / s_ms / 1e6, 1)
     return out
 
 
