@@ -412,6 +412,7 @@ def dominant_layer_roofline(ts, F, records, caches, pmc_target=None):
         key = (r["level"], r["ks"], r["stride"], r["transposed"], r["cin"], r["cout"])
         groups.setdefault(key, []).append(r)
     best = None
+    every = []
     for key, rs in groups.items():
         level, ks, stride, transposed, cin, cout = key
         r = rs[0]
@@ -430,8 +431,14 @@ def dominant_layer_roofline(ts, F, records, caches, pmc_target=None):
                 f"level{level} n_out={r['n_out']} nnz={nnz}")
         if pmc_target not in (None, "auto"):
             total = 1.0 if desc == pmc_target else 0.0
+        flops, nbytes = conv_work(r["n_in"], r["n_out"], omap.shape[0], nnz, kvol, cin, cout, 2)
+        one = roofline_of(flops, nbytes, ms)
+        every.append({"kernel": desc, "launches_per_step": len(rs), "launch_ms": round(ms, 5),
+                      "step_ms": round(ms * len(rs), 4), "bound": one["bound"],
+                      "achieved": round(one["achieved"], 2), "peak": one["peak"], "unit": one["unit"],
+                      "frac": round(one["frac"], 4),
+                      "dense_map_TFLOPs": round(2.0 * omap.shape[0] * kvol * cin * cout / (ms * 1e-3) / 1e12, 1)})
         if best is None or total > best["total_ms"]:
-            flops, nbytes = conv_work(r["n_in"], r["n_out"], omap.shape[0], nnz, kvol, cin, cout, 2)
             best = {"total_ms": total, "ms": ms, "launches": len(rs), "flops": flops, "bytes": nbytes,
                     "run": run, "issued": 2.0 * omap.shape[0] * kvol * cin * cout,
                     "desc": desc}
@@ -447,7 +454,12 @@ def dominant_layer_roofline(ts, F, records, caches, pmc_target=None):
         return {"kernel": best["desc"]}
     roof = roofline_of(best["flops"], best["bytes"], best["ms"])
     roof["traffic"] = PMC_TRAFFIC_BYTES.get(best["desc"])
+    if roof["traffic"] is None:
+        roof["traffic_note"] = "no FETCH_SIZE / WRITE_SIZE pass recorded for this kernel and shape"
     roof["kernel"] = best["desc"]
+    # every convolution group of the step, largest share first: the deep, wide layers run
+    # furthest below their roofline and carry the largest share of the step
+    roof["all_groups"] = sorted(every, key=lambda e: -e["step_ms"])
     roof["launch_ms"] = round(best["ms"], 5)
     roof["launches_per_step"] = best["launches"]
     roof["algorithmic_bytes"] = best["bytes"]

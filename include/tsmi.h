@@ -138,7 +138,15 @@ int tsmi_kmap_sorted_supported(const int32_t ks[3]);
 int tsmi_kmap_sorted(tsmi_stream_t s, const int32_t *in_coords, int64_t n_in,
                      const int32_t *out_coords, int64_t n_out, int64_t n_out_pad,
                      const int32_t ks[3], const int32_t stride[3], const int32_t pad[3],
-                     int32_t *out_in_map);
+                     const int64_t *samples, int32_t *out_in_map);
+/* Optional for tsmi_kmap_sorted, and only for inputs of more than 131072 rows (smaller ones
+ * need none: tsmi_kmap_sorted_samples_elems returns 0): the keys every block of that kernel
+ * searches before it stages its segment, gathered once per INPUT into
+ * samples int64[tsmi_kmap_sorted_samples_elems(n_in)] — every map over the same input rows
+ * (the submanifold and the strided map of a level) can share them.  With samples == NULL the
+ * kernel reads the same keys row by row (one cache line per key and block). */
+int64_t tsmi_kmap_sorted_samples_elems(int64_t n_in);
+int tsmi_kmap_sorted_samples(tsmi_stream_t s, const int32_t *in_coords, int64_t n_in, int64_t *samples);
 
 /* Per-column maximum of non-negative coords -> out_max int32[4] (device).  n may be 0 (result 0).
  * clear_first = 0 when out_max already holds zeros (saves the fill launch).

@@ -47,6 +47,8 @@ def _load():
     lib.tsmi_wgrad_pairs_capacity.argtypes = [_i64, _i32]
     lib.tsmi_conv_wgrad_pairs_workspace_elems.restype = _i64
     lib.tsmi_conv_wgrad_pairs_workspace_elems.argtypes = [_i64, _i32, _i32, _i32, _i32]
+    lib.tsmi_kmap_sorted_samples_elems.restype = _i64
+    lib.tsmi_kmap_sorted_samples_elems.argtypes = [_i64]
     sig = {
         "tsmi_hashtable_clear": [_vp, _vp, _vp, _i64],
         "tsmi_hashtable_insert_coords": [_vp, _vp, _vp, _i64, _vp, _i64, _vp],
@@ -85,7 +87,8 @@ def _load():
         "tsmi_kmap_build_subm": [_vp, _vp, _vp, _i64, _vp, _i64, _i64, _I3, _vp, _vp],
         "tsmi_coords_check": [_vp, _vp, _i64, _vp],
         "tsmi_kmap_sorted_supported": [_I3],
-        "tsmi_kmap_sorted": [_vp, _vp, _i64, _vp, _i64, _i64, _I3, _I3, _I3, _vp],
+        "tsmi_kmap_sorted": [_vp, _vp, _i64, _vp, _i64, _i64, _I3, _I3, _I3, _vp, _vp],
+        "tsmi_kmap_sorted_samples": [_vp, _vp, _i64, _vp],
         "tsmi_wgrad_pairs_pad": [_vp, _vp, _i64, _vp, _i32, _vp, _vp],
         "tsmi_conv_wgrad_pairs": [_vp, _vp, _vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _i32, _vp,
                                   _i64, _vp],
@@ -252,9 +255,36 @@ def kmap_sorted(in_coords: torch.Tensor, out_coords: torch.Tensor, kernel_size, 
     n_out = out_coords.shape[0]
     n_pad = make_divisible(n_out, 128)
     omap = torch.empty((n_pad, ks[0] * ks[1] * ks[2]), dtype=torch.int32, device=out_coords.device)
+    samples = _sorted_samples(in_coords)
     _check(_C.tsmi_kmap_sorted(_stream(), _ptr(in_coords), in_coords.shape[0], _ptr(out_coords), n_out,
-                               n_pad, _I3(*ks), _I3(*st), _I3(*pd), _ptr(omap)))
+                               n_pad, _I3(*ks), _I3(*st), _I3(*pd), _ptr(samples), _ptr(omap)))
     return omap
+
+
+_samples_of = {}  # id(coords) -> (weak reference, version, address, stream, samples)
+
+
+def _sorted_samples(coords: torch.Tensor) -> Optional[torch.Tensor]:
+    """The search samples of a large input (None below 131073 rows), gathered once per
+    coordinate tensor and stream: the submanifold and the strided map of a level share them."""
+    n = coords.shape[0]
+    elems = _C.tsmi_kmap_sorted_samples_elems(n)
+    if elems == 0:
+        return None
+    stream = _stream()
+    hit = _samples_of.get(id(coords))
+    if (hit is not None and hit[0]() is coords and hit[1] == coords._version
+            and hit[2] == coords.data_ptr() and hit[3] == stream):
+        return hit[4]
+    samples = torch.empty(elems, dtype=torch.int64, device=coords.device)
+    _check(_C.tsmi_kmap_sorted_samples(stream, _ptr(coords), n, _ptr(samples)))
+    if len(_samples_of) >= 64:
+        for key in [k for k, v in _samples_of.items() if v[0]() is None]:
+            del _samples_of[key]
+        if len(_samples_of) >= 64:
+            _samples_of.clear()
+    _samples_of[id(coords)] = (weakref.ref(coords), coords._version, coords.data_ptr(), stream, samples)
+    return samples
 
 
 def _settle_insert(coords: torch.Tensor, status: torch.Tensor) -> None:

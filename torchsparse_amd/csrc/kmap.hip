@@ -1191,10 +1191,28 @@ extern "C" int tsmi_kmap_sorted_supported(const int32_t ks[3]) {
   return ks[0] <= kSortedMaxKs0 && ks[1] <= kSortedMaxKs1 && kvol <= kSortedTileInts;
 }
 
+extern "C" int64_t tsmi_kmap_sorted_samples_elems(int64_t n_in) {
+  if (n_in <= (int64_t)kSortedSamples * kSortedDirect || n_in >= (int64_t(1) << 31)) return 0;
+  return (int64_t)kSortedSamples * (1 + kSortedCell);
+}
+
+extern "C" int tsmi_kmap_sorted_samples(tsmi_stream_t s, const int32_t *in_coords, int64_t n_in,
+                                        int64_t *samples) {
+  TSMI_REQUIRE(tsmi_kmap_sorted_samples_elems(n_in) > 0, "kmap_sorted_samples: inputs of this size need none");
+  TSMI_REQUIRE(in_coords && samples, "kmap_sorted_samples: null pointer");
+  const int n = (int)n_in;
+  const int sa = (n + kSortedSamples - 1) / kSortedSamples, n_a = (n + sa - 1) / sa;
+  const int sb = (sa + kSortedCell - 1) / kSortedCell;
+  hipLaunchKernelGGL(kmap_sorted_samples_kernel, grid_for((int64_t)n_a * kSortedCell), dim3(kBlock), 0,
+                     (hipStream_t)s, (const int4 *)in_coords, n, sa, sb, n_a,
+                     (unsigned long long *)samples, (unsigned long long *)samples + kSortedSamples);
+  return check_launch("tsmi_kmap_sorted_samples");
+}
+
 extern "C" int tsmi_kmap_sorted(tsmi_stream_t s, const int32_t *in_coords, int64_t n_in,
                                 const int32_t *out_coords, int64_t n_out, int64_t n_out_pad,
                                 const int32_t ks[3], const int32_t stride[3], const int32_t pad[3],
-                                int32_t *out_in_map) {
+                                const int64_t *samples, int32_t *out_in_map) {
   SortedArgs a;
   if (int e = make_geom(&a.g, ks, stride, pad)) return e;
   TSMI_REQUIRE(tsmi_kmap_sorted_supported(ks), "kmap_sorted: kernel size (%d, %d, %d) not supported",
@@ -1212,6 +1230,9 @@ extern "C" int tsmi_kmap_sorted(tsmi_stream_t s, const int32_t *in_coords, int64
   a.n_out = n_out;
   a.n_out_pad = n_out_pad;
   a.rows = std::min(kBlock, kSortedTileInts / a.g.kvol);
+  const bool sampled = samples != nullptr && tsmi_kmap_sorted_samples_elems(n_in) > 0;
+  a.first = sampled ? (const unsigned long long *)samples : nullptr;
+  a.cell = sampled ? (const unsigned long long *)samples + kSortedSamples : nullptr;
   const int64_t blocks = ceil_div(n_out_pad, a.rows);
   TSMI_REQUIRE(grid_fits(blocks), "kmap_sorted: too many rows for one launch");
   const dim3 grid((unsigned)blocks), block(kBlock);
