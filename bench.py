@@ -57,6 +57,11 @@ def parse():
                     help="run only a 256 MiB device copy (5 launches) and one conv kernel (5 launches) "
                          "for a hardware-counter pass; KERNEL is the description a normal run prints "
                          "in roofline.kernel, or 'auto' for the kernel that run would pick")
+    ap.add_argument("--pmc-kernels", action="store_true",
+                    help="for a hardware-counter pass over the kernels outside the dominant convolution: "
+                         "a 256 MiB device copy (5 launches), then 5 launches each of the kernel-map "
+                         "builders (searched and hashed, scan and 1M voxels), the gather and scatter "
+                         "kernels (64 channels) and the 1M-voxel 256 -> 256 convolution")
     ap.add_argument("--sorted", type=int, default=-1,
                     help="1: run the implicit GEMM over row-sorted maps (conv_mode 1); 0: unsorted; "
                          "-1: the default of this benchmark")
@@ -474,6 +479,66 @@ def dominant_layer_roofline(ts, F, records, caches, pmc_target=None):
     return roof
 
 
+def pmc_kernels(ts, spnn, F, backend, coords, n):
+    """The launches a counter pass (rocprofv3 --pmc) looks at, five of each after five 256 MiB
+    copies whose known size scales the counters: kernel maps of the scan and of the 1M-voxel
+    input (searched over sorted rows, then through the hash table), the strided k2 s2 chain
+    of the scan, gather and scatter of a 64 -> 64 layer, the 1M-voxel 256 -> 256 convolution."""
+    from torchsparse_amd.utils import synthetic
+    src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda")
+    dst = torch.empty_like(src)
+    for _ in range(5):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    del src, dst
+    big = torch.from_numpy(synthetic.sphere_shell_voxels(seed=3)).cuda()
+    for rows in (coords, big):
+        for searched in (True, False):
+            backend.kmap_through_sorted = searched
+            for _ in range(5):
+                F.build_kernel_map(rows, rows.shape[0], 3, 1, 1, mode="hashmap_on_the_fly")
+            torch.cuda.synchronize()
+    backend.kmap_through_sorted = True
+    for _ in range(5):
+        level = coords
+        for _ in range(4):
+            level = F.build_kernel_map(level, level.shape[0], 2, 2, 0, mode="hashmap_on_the_fly")["coords"]
+    torch.cuda.synchronize()
+    cfg = F.conv_config.get_default_conv_config()
+    cfg.dataflow = F.Dataflow.GatherScatter
+    layer = spnn.Conv3d(64, 64, 3, config=cfg).cuda().half()
+    x = ts.SparseTensor(torch.randn(n, 64, device="cuda", dtype=torch.float16), coords)
+    with torch.no_grad():
+        for _ in range(6):
+            layer(x)
+    torch.cuda.synchronize()
+    km = F.build_kernel_map(big, big.shape[0], 3, 1, 1, mode="hashmap_on_the_fly")
+    xb = torch.randn(big.shape[0], 256, device="cuda", dtype=torch.float16)
+    w = torch.randn(27, 256, 256, device="cuda", dtype=torch.float16) * 0.02
+    for _ in range(5):
+        backend.conv_forward_implicit_gemm_cuda(xb, w, km["out_in_map"], big.shape[0], 256)
+    torch.cuda.synchronize()
+    print(json.dumps({"pmc_kernels": "done", "scan_voxels": n, "big_voxels": int(big.shape[0])}))
+
+
+def kmap_roofline(F, backend, coords, n):
+    """The submanifold k3 map of the scan (one launch over ascending rows): HIP-event time of
+    the build, priced with the bytes a hash-table build has to touch (coordinates, table
+    init, inserts, one probe per queried neighbour of the half kernel, the map) and with the
+    least any builder moves (coordinates in, map out)."""
+    ms = event_ms(lambda: F.build_kernel_map(coords, n, 3, 1, 1, mode="hashmap_on_the_fly"), iters=30, warm=5)
+    n_pad = (n + 127) // 128 * 128
+    hashed = kmap_bytes_subm(n, n_pad, backend.hash_capacity(n), 27)
+    least = 16.0 * n + 4.0 * 27 * n_pad
+    searched = backend.kmap_sorted_supported(3) and backend.coords_ascending(coords)
+    return {"bound": "hbm", "achieved": round(hashed / ms / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(hashed / ms / 1e6 / HBM_PEAK_GBS, 4), "traffic": None,
+            "kernel": ("kmap_sorted_kernel<3>" if searched else "subm_prepare + insert_coords + kmap_query_subm")
+                      + f" k3 s1 n={n}",
+            "launch_ms": round(ms, 5), "algorithmic_bytes": hashed,
+            "coords_plus_map_bytes": least, "coords_plus_map_GBps": round(least / ms / 1e6, 1)}
+
+
 def cpu_baseline(records, level_coords):
     """The oracle's CPU convolution (gather -> GEMM -> scatter, fp32, threads over rows)
     and kernel-map builders over the network's sparse conv layers and maps, once."""
@@ -594,10 +659,12 @@ def main():
     if args.sorted == 1:
         F.set_conv_mode(1)
 
-    def timed(net, steps, warmup):
+    def timed(net, steps, warmup, fresh_coords=False):
         def step():
             with torch.no_grad():
-                x = ts.SparseTensor(feats, coords)
+                # a coordinate tensor is checked (range, row order: one small kernel and one
+                # read-back) the first time the library sees it; fresh_coords pays that every step
+                x = ts.SparseTensor(feats, coords.clone() if fresh_coords else coords)
                 return head(net(x)[-1].feats)
         for _ in range(warmup):
             step()
@@ -608,6 +675,9 @@ def main():
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) * 1e3 / steps
 
+    if args.pmc_kernels:
+        pmc_kernels(ts, spnn, F, backend, coords, n)
+        return
     if args.pmc_target:
         with torch.no_grad():
             inp = ts.SparseTensor(feats, coords)
@@ -618,6 +688,7 @@ def main():
 
     ms_per_step = timed(model, args.steps, args.warmup)
     ms_unfused = timed(unfused, max(args.steps // 2, 1), 2)
+    ms_fresh = timed(model, args.steps, 2, fresh_coords=True)
 
     with torch.no_grad():
         inp = ts.SparseTensor(feats, coords)
@@ -626,6 +697,7 @@ def main():
         roof = None if args.no_roofline else dominant_layer_roofline(ts, F, records, inp._caches)
         level_coords = {lvl: c[0].cpu().numpy() for lvl, c in inp._caches.cmaps.items()}
         layers = None if args.no_layers else layer_sweep(ts, spnn, F, backend, coords, n)
+        roof_kmap = None if args.no_roofline else kmap_roofline(F, backend, coords, n)
     backward = None if args.no_backward else backward_sweep(ts, spnn, F, backend, coords, n, feats)
     pointops = None if args.no_pointops else pointops_sweep(F)
     configs = None if args.no_configs else other_configs(ts, spnn, F, backend)
@@ -658,8 +730,10 @@ def main():
                                "kernel maps rebuilt every step",
                    "voxels": n, "warm_map_ms_per_step": round(warm_ms, 4),
                    "unfused_ms_per_step": round(ms_unfused, 4),
+                   "fresh_coordinate_tensor_ms_per_step": round(ms_fresh, 4),
                    "conv_mode": F.get_conv_mode().value},
-        "roofline": roof, "cpu_baseline": cpu, "layers": layers, "backward": backward,
+        "roofline": roof, "roofline_kmap": roof_kmap, "cpu_baseline": cpu, "layers": layers,
+        "backward": backward,
         "tuned": tuned, "pointops": pointops, "other_configs": configs,
     }
     print(json.dumps(result))

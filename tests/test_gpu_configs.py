@@ -146,6 +146,13 @@ def test_million_voxel_256_channel_layer(mods):
     want = _rows_expected(x1.float().cpu().numpy(), w.float().cpu().numpy(), got_rows)
     got = y1[torch.from_numpy(rows).cuda()].float().cpu().numpy()
     assert rel_rms(got, want) < 1e-2
+    # the same layer over the row-sorted map (the 128 x 256 tiles of a large 256-channel layer
+    # in both modes): the rows are the same sums
+    ks = F.build_kernel_map(coords, n, 3, 1, 1, mode="hashmap_on_the_fly", ifsort=True)
+    ys = backend.conv_forward_implicit_gemm_sorted_cuda(x1, w, ks["reorder_out_in_map"], ks["reduced_sorted_mask"],
+                                                        ks["reorder_loc"], n, 256)
+    assert rel_rms(ys.float().cpu().numpy(), y1.float().cpu().numpy()) < 1e-3
+    del ys, ks
     # linearity in the features (power-of-two scale: exact in fp16)
     x2 = torch.randn(n, 256, device="cuda", dtype=torch.float16)
     y2 = backend.conv_forward_implicit_gemm_cuda(x2, w, omap, n, 256)
