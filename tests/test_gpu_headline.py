@@ -263,13 +263,15 @@ def test_minkunet_forward_on_the_scan(mods, scan):
 
     backend.release_scratch()
     step()  # the first forward learns the chain of strided layers ...
+    step()  # ... the second computes levels 2, 3, 4 ahead in its first strided call ...
     handles = [m.register_forward_hook(hook, with_kwargs=True)
                for m in model.modules() if isinstance(m, spnn.Conv3d)]
-    inp, outs, logits = step()  # ... the second computes levels 2, 3, 4 ahead in its first strided call
+    inp, outs, logits = step()  # ... the third queues that call's first half when the stem's map is built
     for h in handles:
         h.remove()
     state, = backend._stream_states.values()
-    assert state.ahead_hits == 3, state.ahead_hits  # one strided call computed, three were answered ahead
+    assert state.ahead_hits == 6, state.ahead_hits  # per forward one strided call computed, three answered ahead
+    assert state.lookahead_hits == 1 and state.pending is None  # bench.py's steady state
 
     # --- the nine kernel maps and the coordinate levels, bit-exact
     caches = inp._caches

@@ -477,3 +477,64 @@ def test_fused_submanifold_build_equals_the_separate_calls():
         assert torch.equal(looked[:n, 0], torch.arange(n, dtype=torch.int32, device="cuda"))
         if n:
             np.testing.assert_array_equal(omap.cpu().numpy(), oracle.kmap_subm(coords.cpu().numpy(), t3(ks)))
+
+
+def test_chain_started_at_the_submanifold_build():
+    """The strided chain's first half queued when the submanifold map of the same rows is built
+    (what a U-Net's stem does): same coordinates and maps as without, a look-ahead nobody asks for
+    leaves no marks behind, and other rows or another geometry in between do not take it."""
+    rng = np.random.default_rng(21)
+    rows = lidar_like_coords(rng, 30000)
+    rows = rows[np.lexsort((rows[:, 3], rows[:, 2], rows[:, 1], rows[:, 0]))]
+    want = []
+    level = rows
+    for _ in range(3):
+        m, level = oracle.kmap_downsample(level, 2, 2, 0)
+        want.append((m, level))
+    backend.release_scratch()
+
+    def forward(coords, strided=3, geom=(2, 2, 0)):
+        F.build_kernel_map(coords, coords.shape[0], 3, 1, 1, mode="hashmap_on_the_fly")
+        got, level = [], coords
+        for _ in range(strided):
+            km = F.build_kernel_map(level, level.shape[0], geom[0], geom[1], geom[2], mode="hashmap_on_the_fly")
+            got.append(km)
+            level = km["coords"]
+        return got
+
+    coords = dev(rows)
+    for _ in range(4):
+        got = forward(coords)
+        for km, (m, c) in zip(got, want):
+            np.testing.assert_array_equal(km["coords"].cpu().numpy(), c)
+            np.testing.assert_array_equal(km["out_in_map"].cpu().numpy(), m)
+    state, = backend._stream_states.values()
+    assert state.lookahead_hits == 2 and state.pending is None  # forwards three and four
+    # a forward that stops after the stem leaves a look-ahead behind; the next strided call of
+    # other rows must not take it, and must find clean bitmaps
+    F.build_kernel_map(coords, coords.shape[0], 3, 1, 1, mode="hashmap_on_the_fly")
+    assert state.pending is not None
+    other = rows[: len(rows) // 2].copy()
+    other[:, 1] += 3
+    km = F.build_kernel_map(dev(other), len(other), 2, 2, 0, mode="hashmap_on_the_fly")
+    m, c = oracle.kmap_downsample(other, 2, 2, 0)
+    np.testing.assert_array_equal(km["coords"].cpu().numpy(), c)
+    np.testing.assert_array_equal(km["out_in_map"].cpu().numpy(), m)
+    assert state.pending is None
+    # the same rows with another geometry: the look-ahead is for k2 s2 and is dropped
+    F.build_kernel_map(coords, coords.shape[0], 3, 1, 1, mode="hashmap_on_the_fly")
+    km = F.build_kernel_map(coords, coords.shape[0], 3, 2, 1, mode="hashmap_on_the_fly")
+    m, c = oracle.kmap_downsample(rows, 3, 2, 1)
+    np.testing.assert_array_equal(km["coords"].cpu().numpy(), c)
+    np.testing.assert_array_equal(km["out_in_map"].cpu().numpy(), m)
+    # and switched off, nothing is queued early
+    backend.downsample_lookahead_at_subm = False
+    try:
+        forward(coords)
+        assert state.pending is None
+        hits = state.lookahead_hits
+        forward(coords)
+        assert state.lookahead_hits == hits
+    finally:
+        backend.downsample_lookahead_at_subm = True
+    assert not any(st.grid_dirty for st in backend._stream_states.values())

@@ -210,19 +210,27 @@ def _range_known(coords: torch.Tensor) -> bool:
     return _range_entry(coords) is not None
 
 
-def _mark_range_ok(coords: torch.Tensor, ascending: Optional[bool] = None) -> None:
+def _range_origin(coords: torch.Tensor) -> Optional[str]:
+    """"user": a caller's tensor that coords_ascending looked at; "library": rows a strided
+    builder produced; None: not known."""
+    hit = _range_entry(coords)
+    return None if hit is None else hit[4]
+
+
+def _mark_range_ok(coords: torch.Tensor, ascending: Optional[bool] = None, origin: str = "library") -> None:
     """``coords`` is in range; ``ascending`` says whether its rows ascend strictly (None keeps
     what is already known)."""
     if ascending is None:
         hit = _range_entry(coords)
         if hit is not None:
             return
+        origin = "user"  # vouched for by a flag read-back over a caller's rows
     if len(_range_ok) >= 512:
         for key in [k for k, v in _range_ok.items() if v[0]() is None]:
             del _range_ok[key]
         if len(_range_ok) >= 512:
             _range_ok.clear()
-    _range_ok[id(coords)] = (weakref.ref(coords), coords._version, coords.data_ptr(), ascending)
+    _range_ok[id(coords)] = (weakref.ref(coords), coords._version, coords.data_ptr(), ascending, origin)
 
 
 def coords_ascending(coords: torch.Tensor) -> bool:
@@ -238,7 +246,7 @@ def coords_ascending(coords: torch.Tensor) -> bool:
     bits = int(flags.item())
     if bits & 2:
         raise _range_error()
-    _mark_range_ok(coords, ascending=not (bits & 1))
+    _mark_range_ok(coords, ascending=not (bits & 1), origin="user")
     return not (bits & 1)
 
 
@@ -469,6 +477,7 @@ def downsample_coords(coords: torch.Tensor, kernel_sizes, stride, padding, coord
         with _state_lock:
             state = _strided_state(dev)
             chain = (ks, st, pd, rsv_ratio) if coords_max_host is None else None
+            job, state.pending = state.pending, None
             ahead = state.chain_step(coords, chain)
             if not isinstance(ahead, int):  # computed ahead when the previous level of the chain was
                 if want_table and ahead[1] is None:
@@ -476,8 +485,17 @@ def downsample_coords(coords: torch.Tensor, kernel_sizes, stride, padding, coord
                     tbl.insert_bxyz(ahead[0])
                     return ahead[0], tbl
                 return ahead
-            done = _downsample_coords_grid(state, coords, ks, st, pd, coords_max_host, fan, rsv_ratio,
-                                           cap, ahead, want_table)
+            if chain is not None and _range_origin(coords) == "user":
+                state.root_chain = chain  # what strided_lookahead starts next time
+            if (job is not None and job.coords is coords and job.geom == (ks, st, pd)
+                    and job.coords_max_host is None and coords_max_host is None
+                    and job.levels == 1 + ahead and state.pending_rsv == rsv_ratio):
+                state.lookahead_hits += 1
+                done = _grid_finish(state, job, rsv_ratio, cap, want_table)
+            else:
+                # (a look-ahead that does not fit this call left marks behind: bitmap() clears them)
+                done = _downsample_coords_grid(state, coords, ks, st, pd, coords_max_host, fan, rsv_ratio,
+                                               cap, ahead, want_table)
             if done is not None:
                 state.chain_last = weakref.ref(done[0])
                 return done
@@ -549,7 +567,8 @@ class _StridedState:
     on that stream, so a later call on the same stream is ordered after it; calls on another
     stream (or device) get a state of their own and never see these tensors."""
     __slots__ = ("grid_buf", "grid_words", "grid_dirty", "chain_geom", "chain_last", "chain_count",
-                 "chain_len", "ahead", "ahead_hits")
+                 "chain_len", "ahead", "ahead_hits", "host_counters", "pending", "pending_rsv", "root_chain",
+                 "lookahead_hits")
 
     def __init__(self):
         self.grid_buf = None      # int32 scratch: bitmaps and chunk counts of every level
@@ -561,6 +580,11 @@ class _StridedState:
         self.chain_len = {}       # geometry -> length of the last chain that ended
         self.ahead = {}           # id(coords) -> (weakref(coords), geometry, out_coords, table)
         self.ahead_hits = 0       # calls answered from `ahead` (diagnostic)
+        self.host_counters = None  # pinned int32 buffer the counters are copied into
+        self.pending = None       # _GridJob started at a submanifold build, not yet asked for
+        self.pending_rsv = None
+        self.root_chain = None    # geometry of the last chain that started from a caller's own rows
+        self.lookahead_hits = 0   # chains whose first half was already queued (diagnostic)
 
     def chain_step(self, coords, geom):
         """Book-keeping of chains of equal strided calls (each on the previous one's outputs).
@@ -632,38 +656,37 @@ def _grid_layout(words0: int):
     return out, off
 
 
-def _downsample_coords_grid(state, coords, ks, st, pd, coords_max_host, fan, rsv_ratio, cap, ahead=0,
-                            want_table=True):
-    """downsample_coords for non-negative coordinates when the output grid has at most
-    2048 cells per candidate (and at most 2^30): mark an occupancy bitmap, count, read the
-    number of outputs back, emit rows and table entries in ascending order.  None when the grid
-    is larger than that (decided on the device; costs the same one read-back).  ``ahead`` more
-    levels of the same geometry are computed before the read-back and left in ``state.ahead``.
-    Runs with _state_lock held: one call at a time between marking a bitmap and emitting."""
+class _GridJob:
+    """The first half of a strided-coordinate build through the occupancy bitmaps — extents,
+    marks and counts of every level queued, the counters on their way to pinned host memory —
+    whose second half (emit) needs the counts on the host."""
+    __slots__ = ("coords", "geom", "coords_max_host", "fan", "levels", "ctr", "host", "event", "stream")
+
+
+def _strided_fan(ks, st) -> int:
+    fan = 1
+    for k, s in zip(ks, st):
+        fan *= -(-k // s)
+    return fan
+
+
+def _grid_start(state, coords, ks, st, pd, coords_max_host, fan, ahead) -> _GridJob:
+    """Queue the marking and counting passes of ``1 + ahead`` levels and the copy of their
+    counters to the host; nothing waits.  Runs with _state_lock held."""
     n = coords.shape[0]
     dev = coords.device
     bits = min(max(1 << (n * fan * 2048 - 1).bit_length(), 1 << 20), 1 << 30)
     buf = state.bitmap(dev, bits // 32)
     layout, _ = _grid_layout(state.grid_words)
     levels = 1 + ahead
-    # per level 8 counters: [n_out, table overflow, grid too large, -, max b, x, y, z of the INPUTS]
+    # per level 8 counters: [n_out, table overflow, grid too large, unpackable, max b, x, y, z of the INPUTS]
     ctr = torch.zeros(8 * levels, dtype=torch.int32, device=dev)
     s = _stream()
     g = (_I3(*ks), _I3(*st), _I3(*pd))
     host_max = _I3(*[int(v) for v in coords_max_host]) if coords_max_host is not None else None
-
-    def part(level, what):
-        if what == "in_max":
-            return ctr[8 * level + 4:8 * level + 8] if level < levels else None
-        off, w, cc = layout[level]
-        if what == "bitmap":
-            return buf[off:off + w]
-        if what == "chunks":
-            return buf[cc:cc + w // _GRID_CHUNK_WORDS]
-        return ctr[8 * level:8 * level + 8]  # "counters"
-
+    part = lambda level, what: _grid_part(buf, ctr, layout, levels, level, what)  # noqa: E731
     _check(_C.tsmi_coords_max(s, _ptr(coords), n, _ptr(part(0, "in_max")), 0))
-    state.grid_dirty = True  # marked bits stay behind unless the emit passes below run
+    state.grid_dirty = True  # marked bits stay behind unless the emit passes run
     _check(_C.tsmi_downsample_grid_count(s, _ptr(coords), n, *g, host_max, _ptr(part(0, "in_max")),
                                          _ptr(part(0, "bitmap")), layout[0][1], 0,
                                          _ptr(part(0, "chunks")), _ptr(part(0, "counters")),
@@ -673,7 +696,49 @@ def _downsample_coords_grid(state, coords, ks, st, pd, coords_max_host, fan, rsv
             s, *g, _ptr(part(level - 1, "in_max")), _ptr(part(level - 1, "bitmap")), layout[level - 1][1],
             _ptr(part(level, "in_max")), _ptr(part(level, "bitmap")), layout[level][1],
             _ptr(part(level, "chunks")), _ptr(part(level, "counters")), _ptr(part(level + 1, "in_max"))))
-    host = ctr.tolist()
+    job = _GridJob()
+    job.coords, job.geom, job.coords_max_host, job.fan = coords, (ks, st, pd), coords_max_host, fan
+    job.levels, job.ctr, job.stream = levels, ctr, s
+    # pinned memory is allocated once per stream state (allocating it is slow); the copy is
+    # asynchronous and an event marks its end, so a job started early is usually complete by
+    # the time its counts are asked for and the host never waits for the queue to drain
+    if state.host_counters is None:
+        state.host_counters = torch.empty(8 * _GRID_LEVELS, dtype=torch.int32, pin_memory=True)
+    job.host = state.host_counters[:8 * levels]
+    job.host.copy_(ctr, non_blocking=True)
+    job.event = torch.cuda.Event()
+    job.event.record()
+    return job
+
+
+def _grid_part(buf, ctr, layout, levels, level, what):
+    if what == "in_max":
+        return ctr[8 * level + 4:8 * level + 8] if level < levels else None
+    off, w, cc = layout[level]
+    if what == "bitmap":
+        return buf[off:off + w]
+    if what == "chunks":
+        return buf[cc:cc + w // _GRID_CHUNK_WORDS]
+    return ctr[8 * level:8 * level + 8]  # "counters"
+
+
+def _grid_finish(state, job: _GridJob, rsv_ratio, cap, want_table):
+    """The second half: wait for the counters, emit the rows of every level.  Returns what
+    downsample_coords returns for the first level (None: the grid did not fit) and leaves
+    the later levels in ``state.ahead``.  Runs with _state_lock held."""
+    coords = job.coords
+    ks, st, pd = job.geom
+    fan, levels, ctr = job.fan, job.levels, job.ctr
+    n = coords.shape[0]
+    dev = coords.device
+    buf = state.grid_buf
+    layout, _ = _grid_layout(state.grid_words)
+    s = job.stream
+    g = (_I3(*ks), _I3(*st), _I3(*pd))
+    host_max = _I3(*[int(v) for v in job.coords_max_host]) if job.coords_max_host is not None else None
+    part = lambda level, what: _grid_part(buf, ctr, layout, levels, level, what)  # noqa: E731
+    job.event.synchronize()
+    host = job.host.tolist()
     if host[2]:
         state.grid_dirty = False  # nothing was marked, at any level
         return None
@@ -726,6 +791,50 @@ def _downsample_coords_grid(state, coords, ks, st, pd, coords_max_host, fan, rsv
         prev = nxt[0]
     state.grid_dirty = not clean
     return first
+
+
+def _downsample_coords_grid(state, coords, ks, st, pd, coords_max_host, fan, rsv_ratio, cap, ahead=0,
+                            want_table=True):
+    """downsample_coords for non-negative coordinates when the output grid has at most
+    2048 cells per candidate (and at most 2^30): mark an occupancy bitmap, count, read the
+    number of outputs back, emit rows and table entries in ascending order.  None when the grid
+    is larger than that (decided on the device; costs the same one read-back).  ``ahead`` more
+    levels of the same geometry are computed before the read-back and left in ``state.ahead``.
+    Runs with _state_lock held: one call at a time between marking a bitmap and emitting."""
+    job = _grid_start(state, coords, ks, st, pd, coords_max_host, fan, ahead)
+    return _grid_finish(state, job, rsv_ratio, cap, want_table)
+
+
+# A network that starts with submanifold layers and then enters a chain of strided ones (a
+# U-Net's stem and encoder) asks for the chain's coordinates a few convolutions after the
+# first map of the same rows.  Once such a chain has been seen, the first half of its build
+# (marks, counts, the copy of the counters) is queued when the submanifold map of those rows is
+# built, so the counts are on the host by the time the strided layer asks and the forward no
+# longer stops to wait for the queue to drain.  A look-ahead nobody asks for costs its kernels
+# and a clear of the bitmaps.
+downsample_lookahead_at_subm = True
+
+
+def strided_lookahead(coords: torch.Tensor) -> None:
+    """Called when a submanifold map is built over ``coords``: start the strided chain that
+    followed such rows last time on this stream, if any."""
+    if not (downsample_lookahead_at_subm and downsample_through_grid and downsample_chain_ahead):
+        return
+    if coords.shape[0] == 0:
+        return
+    with _state_lock:
+        state = _strided_state(coords.device)
+        root = state.root_chain  # geometry of the last chain that started from rows like these
+        if root is None or _range_origin(coords) != "user":
+            return
+        if state.pending is not None:
+            if state.pending.coords is coords:
+                return
+            state.pending = None  # never asked for; its marks are cleared by the next bitmap() call
+        ks, st, pd, rsv_ratio = root
+        ahead = min(state.chain_len.get(root, 1) - 1, _GRID_LEVELS - 1)
+        state.pending = _grid_start(state, coords, ks, st, pd, None, _strided_fan(ks, st), ahead)
+        state.pending_rsv = rsv_ratio
 
 
 def build_kernel_map_downsample_hashmap(in_table: Optional[GPUHashTable], coords, coords_min,

@@ -175,6 +175,7 @@ def build_kernel_map(_coords: torch.Tensor, input_node_num: int,
                  and backend.coords_ascending(_coords))
     if by_search:
         if subm:
+            backend.strided_lookahead(_coords)  # the strided chain that follows such rows, queued early
             out_coords = coords
             out_in_map = backend.kmap_sorted(coords, coords, kernel_size, stride, backend._subm_pad(kernel_size))
         else:
