@@ -233,12 +233,19 @@ int tsmi_downsample_finalize(tsmi_stream_t s, const int64_t *sorted_keys, int64_
  * (keys, vals, cap; counters[1] = 1 if the table was too small; keys == NULL: no table) and leaves the bitmap
  * all zero again, so that one bitmap can serve call after call without clear_first.
  * in_max_host, when given, is a host copy of in_max_dev (read back with the counters): the
- * extents are then computed on the host and only the chunks inside the grid are launched. */
+ * extents are then computed on the host and only the chunks inside the grid are launched.
+ * Chains without a read-back in between: tsmi_downsample_grid_emit with n_out = -capacity
+ * emits every set bit into out_coords int32[capacity, 4] while the count is still on the
+ * device (no table; capacity >= the count, e.g. the number of inputs when every input has one
+ * output), and tsmi_downsample_grid_count with n_in_dev (device int32[1], e.g. counters[0] of
+ * the previous level; n_in is then the capacity of in_coords) marks from such rows.  NULL:
+ * n_in rows. */
 int tsmi_downsample_grid_count(tsmi_stream_t s, const int32_t *in_coords, int64_t n_in,
                                const int32_t ks[3], const int32_t stride[3], const int32_t pad[3],
                                const int32_t out_max_host[3], const int32_t *in_max_dev,
                                int32_t *bitmap, int64_t bitmap_words, int clear_first,
-                               int32_t *chunk_counts, int32_t *counters, int32_t *next_in_max_dev);
+                               int32_t *chunk_counts, int32_t *counters, int32_t *next_in_max_dev,
+                               const int32_t *n_in_dev);
 /* The next level of a chain of strided convolutions with the same geometry, before the
  * previous level's outputs exist as rows: the inputs are the set bits of the previous
  * level's bitmap (marked by tsmi_downsample_grid_count / _count_next with next_in_max_dev =

@@ -62,7 +62,7 @@ def _load():
         "tsmi_sort_keys": [_vp, _vp, _vp, _i64, _i32, _vp, _i64],
         "tsmi_downsample_finalize": [_vp, _vp, _i64, _vp, _vp, _i64, _vp],
         "tsmi_downsample_grid_count": [_vp, _vp, _i64, _I3, _I3, _I3, _vp, _vp, _vp, _i64, _i32, _vp, _vp,
-                                       _vp],
+                                       _vp, _vp],
         "tsmi_downsample_grid_count_next": [_vp, _I3, _I3, _I3, _vp, _vp, _i64, _vp, _vp, _i64, _vp, _vp, _vp],
         "tsmi_downsample_grid_emit": [_vp, _I3, _I3, _I3, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _vp,
                                       _i64, _vp, _vp],
@@ -660,7 +660,7 @@ class _GridJob:
     """The first half of a strided-coordinate build through the occupancy bitmaps — extents,
     marks and counts of every level queued, the counters on their way to pinned host memory —
     whose second half (emit) needs the counts on the host."""
-    __slots__ = ("coords", "geom", "coords_max_host", "fan", "levels", "ctr", "host", "event", "stream")
+    __slots__ = ("coords", "geom", "coords_max_host", "fan", "levels", "ctr", "host", "event", "stream", "rows")
 
 
 def _strided_fan(ks, st) -> int:
@@ -670,7 +670,7 @@ def _strided_fan(ks, st) -> int:
     return fan
 
 
-def _grid_start(state, coords, ks, st, pd, coords_max_host, fan, ahead) -> _GridJob:
+def _grid_start(state, coords, ks, st, pd, coords_max_host, fan, ahead, early=False) -> _GridJob:
     """Queue the marking and counting passes of ``1 + ahead`` levels and the copy of their
     counters to the host; nothing waits.  Runs with _state_lock held."""
     n = coords.shape[0]
@@ -690,24 +690,53 @@ def _grid_start(state, coords, ks, st, pd, coords_max_host, fan, ahead) -> _Grid
     _check(_C.tsmi_downsample_grid_count(s, _ptr(coords), n, *g, host_max, _ptr(part(0, "in_max")),
                                          _ptr(part(0, "bitmap")), layout[0][1], 0,
                                          _ptr(part(0, "chunks")), _ptr(part(0, "counters")),
-                                         _ptr(part(1, "in_max"))))
-    for level in range(1, levels):
-        _check(_C.tsmi_downsample_grid_count_next(
-            s, *g, _ptr(part(level - 1, "in_max")), _ptr(part(level - 1, "bitmap")), layout[level - 1][1],
-            _ptr(part(level, "in_max")), _ptr(part(level, "bitmap")), layout[level][1],
-            _ptr(part(level, "chunks")), _ptr(part(level, "counters")), _ptr(part(level + 1, "in_max"))))
+                                         _ptr(part(1, "in_max")), None))
+    # One output per input (kernel size == stride, no padding: a level never has more rows than
+    # the one before): every level's rows are emitted at once into a buffer of n rows while
+    # their count is still on the device, and the next level marks from those rows.  Nothing is
+    # left to launch once the counts are on the host.  Other geometries mark the next level
+    # from the previous level's bitmap and emit after the read-back; so does a single level,
+    # whose emit pass is cheaper once the host knows the extents.
+    rows = None
+    if (levels > 1 and fan == 1 and ks == st and pd == (0, 0, 0) and coords_max_host is None
+            and downsample_emit_before_readback):
+        rows = []
+        src = coords
+        for level in range(levels):
+            if level > 0:
+                _check(_C.tsmi_downsample_grid_count(
+                    s, _ptr(src), n, *g, None, _ptr(part(level, "in_max")), _ptr(part(level, "bitmap")),
+                    layout[level][1], 0, _ptr(part(level, "chunks")), _ptr(part(level, "counters")),
+                    _ptr(part(level + 1, "in_max")), _ptr(part(level - 1, "counters"))))
+            out = torch.empty((n, 4), dtype=torch.int32, device=dev)
+            _check(_C.tsmi_downsample_grid_emit(
+                s, *g, None, _ptr(part(level, "in_max")), None, _ptr(part(level, "bitmap")),
+                layout[level][1], _ptr(part(level, "chunks")), -n, None, None, 0, _ptr(out),
+                _ptr(part(level, "counters"))))
+            rows.append(out)
+            src = out
+    else:
+        for level in range(1, levels):
+            _check(_C.tsmi_downsample_grid_count_next(
+                s, *g, _ptr(part(level - 1, "in_max")), _ptr(part(level - 1, "bitmap")), layout[level - 1][1],
+                _ptr(part(level, "in_max")), _ptr(part(level, "bitmap")), layout[level][1],
+                _ptr(part(level, "chunks")), _ptr(part(level, "counters")), _ptr(part(level + 1, "in_max"))))
     job = _GridJob()
+    job.rows = rows
     job.coords, job.geom, job.coords_max_host, job.fan = coords, (ks, st, pd), coords_max_host, fan
     job.levels, job.ctr, job.stream = levels, ctr, s
-    # pinned memory is allocated once per stream state (allocating it is slow); the copy is
-    # asynchronous and an event marks its end, so a job started early is usually complete by
-    # the time its counts are asked for and the host never waits for the queue to drain
-    if state.host_counters is None:
-        state.host_counters = torch.empty(8 * _GRID_LEVELS, dtype=torch.int32, pin_memory=True)
-    job.host = state.host_counters[:8 * levels]
-    job.host.copy_(ctr, non_blocking=True)
-    job.event = torch.cuda.Event()
-    job.event.record()
+    job.host = job.event = None
+    if early:
+        # a job started ahead of its use copies its counters to pinned memory (allocated once
+        # per stream state: allocating it is slow) and marks the end of the copy with an event,
+        # so the counts are usually on the host by the time they are asked for; a job whose
+        # counts are needed at once reads them back directly, which is the quicker way then
+        if state.host_counters is None:
+            state.host_counters = torch.empty(8 * _GRID_LEVELS, dtype=torch.int32, pin_memory=True)
+        job.host = state.host_counters[:8 * levels]
+        job.host.copy_(ctr, non_blocking=True)
+        job.event = torch.cuda.Event()
+        job.event.record()
     return job
 
 
@@ -737,8 +766,11 @@ def _grid_finish(state, job: _GridJob, rsv_ratio, cap, want_table):
     g = (_I3(*ks), _I3(*st), _I3(*pd))
     host_max = _I3(*[int(v) for v in job.coords_max_host]) if job.coords_max_host is not None else None
     part = lambda level, what: _grid_part(buf, ctr, layout, levels, level, what)  # noqa: E731
-    job.event.synchronize()
-    host = job.host.tolist()
+    if job.event is not None:
+        job.event.synchronize()
+        host = job.host.tolist()
+    else:
+        host = ctr.tolist()
     if host[2]:
         state.grid_dirty = False  # nothing was marked, at any level
         return None
@@ -749,6 +781,14 @@ def _grid_finish(state, job: _GridJob, rsv_ratio, cap, want_table):
 
     def emit(level, n_in, capacity):
         n_out = host[8 * level]
+        if job.rows is not None:  # emitted before the read-back: the level is a view of its buffer
+            out = job.rows[level][:n_out]
+            tbl = None
+            if want_table:
+                _mark_range_ok(out, ascending=True)  # (known: the insert below does not read a flag back)
+                tbl = GPUHashTable(capacity, device=dev)
+                tbl.insert_bxyz(out)
+            return out, tbl
         if n_out > capacity and fan > 2:  # more than the two outputs per input reserved
             capacity = hash_capacity(n_in * fan, rsv_ratio)
         if n_out > capacity:  # the reference's limit, with or without a table to overflow
@@ -789,7 +829,8 @@ def _grid_finish(state, job: _GridJob, rsv_ratio, cap, want_table):
                 all(host[8 * level + 5 + a] + 2 * pd[a] < COORD_LIMIT for a in range(3))):
             _mark_range_ok(nxt[0], ascending=True)
         prev = nxt[0]
-    state.grid_dirty = not clean
+    # rows emitted before the read-back cleared every bitmap they read, asked for or not
+    state.grid_dirty = (not clean) and job.rows is None
     return first
 
 
@@ -813,6 +854,9 @@ def _downsample_coords_grid(state, coords, ks, st, pd, coords_max_host, fan, rsv
 # longer stops to wait for the queue to drain.  A look-ahead nobody asks for costs its kernels
 # and a clear of the bitmaps.
 downsample_lookahead_at_subm = True
+# Chains in which every input has exactly one output emit each level's rows before the counts
+# are read back (False: mark the next level from the bitmap, emit afterwards).
+downsample_emit_before_readback = True
 
 
 def strided_lookahead(coords: torch.Tensor) -> None:
@@ -833,7 +877,7 @@ def strided_lookahead(coords: torch.Tensor) -> None:
             state.pending = None  # never asked for; its marks are cleared by the next bitmap() call
         ks, st, pd, rsv_ratio = root
         ahead = min(state.chain_len.get(root, 1) - 1, _GRID_LEVELS - 1)
-        state.pending = _grid_start(state, coords, ks, st, pd, None, _strided_fan(ks, st), ahead)
+        state.pending = _grid_start(state, coords, ks, st, pd, None, _strided_fan(ks, st), ahead, early=True)
         state.pending_rsv = rsv_ratio
 
 

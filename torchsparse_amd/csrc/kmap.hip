@@ -375,8 +375,11 @@ __device__ __forceinline__ void block_raise_max(int b, int x, int y, int z, int3
 __global__ void grid_mark_kernel(const int4 *in_coords, int64_t total, Geom g, int3 out_max_host,
                                  int has_host_max, const int32_t *in_max_dev, int mode,
                                  uint32_t *bitmap, int64_t cap_words, int32_t *next_in_max,
-                                 int32_t *counters) {
+                                 int32_t *counters, const int32_t *n_in_dev) {
   const int64_t tid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  // the rows may be the emit pass's output of the previous level of a chain, whose count has
+  // not been read back: `total` is then the capacity and the count comes from the device
+  if (n_in_dev) total = min(total, (int64_t)*n_in_dev * (mode == 0 ? strided_fan(g) : 1));
   const GridDims d = grid_dims(g, out_max_host, has_host_max, in_max_dev, cap_words);
   if (!d.fits || d.used_words == 0) return;  // the same for every thread
   int word = -1;
@@ -576,13 +579,15 @@ __global__ __launch_bounds__(kBlock) void grid_emit_kernel(uint32_t *bitmap, int
   __shared__ int before[kGridChunkWords];  // set bits of the chunk before each word
   const GridDims d = have_host_dims ? host_dims
                                     : grid_dims(g, out_max_host, has_host_max, in_max_dev, cap_words);
-  if ((int64_t)blockIdx.x * kGridChunkWords >= d.used_words) return;
-  uint32_t w[2];
-  const int mine = grid_thread_words(bitmap, blockIdx.x, w);
-  if (mine)  // leave the bitmap all clear for the next call
-    *(uint2 *)(bitmap + (int64_t)blockIdx.x * kGridChunkWords + threadIdx.x * 2) = make_uint2(0u, 0u);
-  int incl = mine;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // one block per chunk when the host knows the extents; otherwise a bounded number of blocks
+  // strides over the chunks the device-side extents cover
+  for (int64_t chunk = blockIdx.x; chunk * kGridChunkWords < d.used_words; chunk += gridDim.x) {
+  uint32_t w[2];
+  const int mine = grid_thread_words(bitmap, chunk, w);
+  if (mine)  // leave the bitmap all clear for the next call
+    *(uint2 *)(bitmap + chunk * kGridChunkWords + threadIdx.x * 2) = make_uint2(0u, 0u);
+  int incl = mine;
 #pragma unroll
   for (int off = 1; off < 64; off <<= 1) {
     const int v = __shfl_up(incl, off);
@@ -598,8 +603,8 @@ __global__ __launch_bounds__(kBlock) void grid_emit_kernel(uint32_t *bitmap, int
   before[threadIdx.x * 2 + 1] = first + __popc(w[0]);
   const int chunk_total = wave_sum[0] + wave_sum[1] + wave_sum[2] + wave_sum[3];
   __syncthreads();
-  const uint32_t chunk_cell0 = (uint32_t)blockIdx.x * (kGridChunkWords * 32);
-  const int64_t chunk_rank0 = chunk_prefix[blockIdx.x];
+  const uint32_t chunk_cell0 = (uint32_t)chunk * (kGridChunkWords * 32);
+  const int64_t chunk_rank0 = chunk_prefix[chunk];
   for (int i = threadIdx.x; i < chunk_total; i += kBlock) {
     // the last word with before[word] <= i holds rank i (an empty word shares its successor's count)
     int lo = 0;
@@ -624,8 +629,11 @@ __global__ __launch_bounds__(kBlock) void grid_emit_kernel(uint32_t *bitmap, int
     cell /= d.e[1];
     const int x_ = (int)(cell % d.e[0]);
     const int b = (int)(cell / d.e[0]);
-    // always true: n_out is the total of the counts the ranks come from
+    // always true: n_out is the total of the counts the ranks come from (or the capacity of
+    // out_coords when the total is still on the device)
     if (chunk_rank0 + i < n_out) out_coords[chunk_rank0 + i] = make_int4(b, x_, y, z);
+  }
+  __syncthreads();  // the LDS arrays are rewritten by the next chunk
   }
 }
 
@@ -1348,7 +1356,7 @@ extern "C" int tsmi_downsample_grid_count(tsmi_stream_t s, const int32_t *in_coo
                                           const int32_t *in_max_dev, int32_t *bitmap,
                                           int64_t bitmap_words, int clear_first,
                                           int32_t *chunk_counts, int32_t *counters,
-                                          int32_t *next_in_max_dev) {
+                                          int32_t *next_in_max_dev, const int32_t *n_in_dev) {
   Geom g;
   int mode;
   int3 hm;
@@ -1371,7 +1379,7 @@ extern "C" int tsmi_downsample_grid_count(tsmi_stream_t s, const int32_t *in_coo
   if (total > 0)
     hipLaunchKernelGGL(grid_mark_kernel, grid_for(total), dim3(kBlock), 0, st, (const int4 *)in_coords,
                        total, g, hm, has_hm, in_max_dev, mode, (uint32_t *)bitmap, bitmap_words,
-                       next_in_max_dev, counters);
+                       next_in_max_dev, counters, n_in_dev);
   hipLaunchKernelGGL(grid_count_kernel, dim3(chunks < 2048u ? chunks : 2048u), dim3(kBlock), 0, st,
                      (const uint32_t *)bitmap,
                      bitmap_words, g, hm, has_hm, in_max_dev, chunk_counts);
@@ -1427,6 +1435,17 @@ extern "C" int tsmi_downsample_grid_emit(tsmi_stream_t s, const int32_t ks[3], c
   const bool want_table = keys != nullptr;
   if (want_table)
     if (int e = make_table(&t, keys, vals, cap)) return e;
+  // n_out < 0: the count is still on the device and out_coords holds -n_out rows; every chunk
+  // the device-side extents cover is emitted by a bounded grid, no table is filled
+  const bool on_device = n_out < 0;
+  if (on_device) {
+    TSMI_REQUIRE(!want_table && !in_max_host && out_coords, "downsample_grid_emit: a device-side count takes no table");
+    const int64_t chunks_cap = bitmap_words / kGridChunkWords;
+    hipLaunchKernelGGL(grid_emit_kernel, dim3((unsigned)std::min<int64_t>(chunks_cap, 2048)), dim3(kBlock), 0,
+                       (hipStream_t)s, (uint32_t *)bitmap, bitmap_words, chunk_prefix, g, hm,
+                       out_max_host != nullptr, in_max_dev, GridDims{}, 0, (int4 *)out_coords, -n_out);
+    return check_launch("tsmi_downsample_grid_emit");
+  }
   TSMI_REQUIRE(n_out >= 0 && (n_out == 0 || out_coords), "downsample_grid_emit: bad arguments");
   TSMI_REQUIRE(!want_table || n_out <= cap,
                "The capacity of hashtable is not sufficient. Please enlarge reserved space for "
