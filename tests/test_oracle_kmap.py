@@ -86,6 +86,23 @@ def test_downsample_k_equals_s_is_floor_unique():
     np.testing.assert_array_equal(oracle.spdownsample_floor(coords, 2), np.unique(c, axis=0))
 
 
+def test_downsample_k_equals_s_drops_inputs_at_an_even_maximum():
+    # kmap/func/hashmap_on_the_fly.py:27-37 derives the output bound from the input maximum as
+    # (max + 2 pad - (k - 1)) // stride: with k = s = 2 an input whose coordinate is the (even)
+    # maximum of its axis maps to max / 2, one past that bound, and gets no output.  A strided
+    # map therefore does NOT give every input a pair, and its transposed map has empty rows.
+    coords = np.array([[0, 0, 0, 0], [0, 3, 5, 1], [0, 6, 2, 1], [0, 6, 5, 0]], np.int32)  # max x = 6
+    omap, ocoords = oracle.kmap_downsample(coords, 2, 2, 0)
+    np.testing.assert_array_equal(ocoords, [[0, 0, 0, 0], [0, 1, 2, 0]])
+    assert sorted(omap[omap >= 0].tolist()) == [0, 1]
+    t = oracle.transpose_map(omap, len(coords))
+    assert ((t[:4] >= 0).sum(1) == [1, 1, 0, 0]).all()
+    # an odd maximum on every axis keeps all of them
+    coords[:, 1:] += np.array([1, 0, 0], np.int32)
+    omap, _ = oracle.kmap_downsample(coords, 2, 2, 0)
+    assert (omap >= 0).sum() == 4
+
+
 @pytest.mark.parametrize("ks,stride", [(2, 2), (3, 2), (3, 1), (2, 1), (5, 3)])
 def test_lookup_coords_bruteforce(ks, stride):
     rng = RNG(13)
