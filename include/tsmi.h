@@ -473,6 +473,38 @@ int tsmi_conv_fetch_on_demand(tsmi_stream_t s, const void *x, const void *w_pack
                               const void *bias, const void *residual, int relu, void *partial,
                               void *y);
 
+/* Convolution over pair segments: the form the implicit-GEMM dataflow takes on small, wide
+ * layers (a few thousand to a few ten thousand rows, 128 or more channels), where a dense
+ * pass over all K_vol offsets of every row tile would stream the whole weight tensor once
+ * per tile.  tsmi_pair_segments compacts the pairs of a kernel map (int32 [n_rows, K_vol],
+ * negative = none) per kernel offset, in one launch and without a host read-back:
+ * in_rows[k * seg_rows + j] = map value of the j-th pair of offset k, pos[k * n_rows + row] =
+ * j (-1: the row has no pair at k), counts[k] = pairs of offset k.  seg_rows >= n_rows is the
+ * fixed capacity of a segment (a multiple of 64 for the convolution below); in_rows holds
+ * K_vol * seg_rows int32 (only the first counts[k] of a segment are written), pos
+ * K_vol * n_rows, counts K_vol.  The order of the pairs inside a segment is not fixed
+ * (blocks reserve their share with an atomic add); pos names each pair's place, and every
+ * result computed through the two arrays is the same whatever the order.
+ * tsmi_conv_implicit_gemm_segments: products[k * seg_rows + j, :] = X[in_rows[k * seg_rows + j], :]
+ * W[k] for j < counts[k] (one launch: a workgroup takes a run of 64-pair tiles and keeps the
+ * weights of their offset in registers), then Y[o, :] = sum over k of products[k * seg_rows +
+ * pos[k * n_out + o], :] + bias + residual, optional ReLU (second launch; fp32 sums in the
+ * order of k, atomic free).  `products` holds K_vol * seg_rows * cout elements of the I/O
+ * type, of which only the rows of existing pairs are touched.  tsmi_conv_segments_supported:
+ * 1 for the shapes that have a variant (fp16 / bf16, K_vol <= 64, cin one of 128, 192, 256,
+ * 384, cout a multiple of 8).  Same sums as conv_forward_implicit_gemm_cuda
+ * (convolution/convolution_forward_implicit_gemm_cuda.cu:1527-1986) with the per-offset
+ * products rounded to the I/O type as conv_forward_fetch_on_demand_cuda's are
+ * (convolution/convolution_forward_fetch_on_demand_cuda.cu:1981-2119). */
+int tsmi_conv_segments_supported(int kvol, int cin, int cout, int dtype);
+int tsmi_pair_segments(tsmi_stream_t s, const int32_t *map, int64_t n_rows, int kvol,
+                       int64_t seg_rows, int32_t *counts, int32_t *in_rows, int32_t *pos);
+int tsmi_conv_implicit_gemm_segments(tsmi_stream_t s, const void *x, const void *w_packed,
+                                     const int32_t *in_rows, const int32_t *counts,
+                                     const int32_t *pos, int64_t seg_rows, int64_t n_out, int kvol,
+                                     int cin, int cout, int dtype, const void *bias,
+                                     const void *residual, int relu, void *products, void *y);
+
 /* Gather-GEMM-scatter, step 1: buffer[nbaddrs[k] + p, :] = X[in(k,p), :].
  * Replaces gather_all_kernel_pad_sep_with_mask / gather_kernel
  * (convolution/convolution_gather_scatter_cuda.cu:17-40,70-112). */

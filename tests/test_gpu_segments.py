@@ -1,0 +1,184 @@
+"""GPU parity of the pair-segment form of the implicit-GEMM dataflow (tsmi_pair_segments,
+tsmi_conv_implicit_gemm_segments) against the CPU oracle.
+
+Integer products are compared exactly (counts per offset, the place of every pair, the input
+row stored at that place); the order of the pairs inside a segment is not fixed, so it is the
+relation between the two arrays that is checked, not their raw contents.  Features: 1e-2
+(fp16) / 3e-2 (bf16) of the RMS of the oracle's output, which is fed the inputs already
+rounded to the I/O type."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import random_coords, rel_rms
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float16: 1e-2, torch.bfloat16: 3e-2}
+
+
+@pytest.fixture(scope="module")
+def mods():
+    from torchsparse_amd import backend
+    from torchsparse_amd.nn import functional as F
+    return backend, F
+
+
+def dev(a, dtype=torch.int32):
+    return torch.from_numpy(np.ascontiguousarray(a)).to("cuda", dtype)
+
+
+def _f32(t):
+    return t.detach().float().cpu().numpy()
+
+
+def _check_segments(backend, omap_np, n_rows):
+    omap = dev(omap_np)
+    counts, in_rows, pos, seg_rows = backend.pair_segments(omap, n_rows)
+    counts, in_rows, pos = counts.cpu().numpy(), in_rows.cpu().numpy(), pos.cpu().numpy()
+    kvol = omap_np.shape[1]
+    assert seg_rows >= n_rows and seg_rows % 64 == 0
+    assert in_rows.shape == (kvol, seg_rows) and pos.shape == (kvol, n_rows)
+    m = omap_np[:n_rows]
+    np.testing.assert_array_equal(counts, (m >= 0).sum(0))
+    for k in range(kvol):
+        has = m[:, k] >= 0
+        assert (pos[k][~has] == -1).all()
+        places = pos[k][has]
+        # the places of an offset's pairs are 0 .. count-1, each once
+        np.testing.assert_array_equal(np.sort(places), np.arange(counts[k]))
+        np.testing.assert_array_equal(in_rows[k][places], m[has, k])
+
+
+@pytest.mark.parametrize("ks,stride,n", [(3, 1, 2500), (3, 1, 1), (2, 2, 3000), ((3, 1, 3), 1, 700),
+                                         (5, 1, 400), (3, 2, 2000)])
+def test_pair_segments_hold_every_pair_once(mods, ks, stride, n):
+    backend, F = mods
+    rng = np.random.default_rng(n + 17)
+    coords = random_coords(rng, n, (24, 20, 12))
+    if stride == 1:
+        omap = oracle.kmap_subm(coords, ks)
+        n_rows = n
+    else:
+        pad = 0 if ks == 2 else 1
+        omap, out_coords = oracle.kmap_downsample(coords, ks, stride, pad)
+        n_rows = len(out_coords)
+    _check_segments(backend, omap, n_rows)
+
+
+def test_pair_segments_of_offsets_without_pairs(mods):
+    backend, _ = mods
+    # isolated voxels: only the centre offset has pairs
+    coords = np.array([[0, 4 * i, 0, 0] for i in range(130)], np.int32)
+    omap = oracle.kmap_subm(coords, 3)
+    assert (omap[:130] >= 0).sum() == 130
+    _check_segments(backend, omap, 130)
+
+
+def test_pair_segments_are_built_once_per_map(mods):
+    backend, _ = mods
+    rng = np.random.default_rng(5)
+    omap = dev(oracle.kmap_subm(random_coords(rng, 300, (10, 10, 10)), 3))
+    a = backend.pair_segments(omap, 300)
+    assert backend.pair_segments(omap, 300) is a
+    assert backend.pair_segments(omap, 256) is not a  # another row count: rebuilt
+    with pytest.raises(ValueError):
+        backend.pair_segments(omap, omap.shape[0] + 1)
+
+
+SHAPES = [(3000, 128, 128), (2100, 256, 256), (1300, 192, 128), (777, 384, 256), (1500, 128, 136),
+          (64, 256, 128), (1, 128, 128)]
+
+
+@pytest.mark.parametrize("n,cin,cout", SHAPES)
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_convolution_over_segments_matches_oracle(mods, n, cin, cout, dtype):
+    backend, F = mods
+    rng = np.random.default_rng(n + cin + cout)
+    coords = random_coords(rng, n, (22, 18, 12))
+    omap_np = oracle.kmap_subm(coords, 3)
+    omap = dev(omap_np)
+    x = torch.from_numpy(rng.standard_normal((n, cin)).astype(np.float32)).to("cuda", dtype)
+    bound = 1.0 / np.sqrt(cin * 27)
+    w = torch.from_numpy(rng.uniform(-bound, bound, (27, cin, cout)).astype(np.float32)).to("cuda", dtype)
+    assert backend._C.tsmi_conv_segments_supported(27, cin, cout, backend._dtype_code(x)) == 1
+    wp = backend.pack_weights(w)
+    y = backend.conv_implicit_gemm_segments(x, wp, 27, cin, cout, omap, n)
+    want = oracle.conv_implicit_gemm(_f32(x), _f32(w), omap_np, n)
+    assert y.dtype == dtype and y.shape == (n, cout)
+    assert rel_rms(_f32(y), want) < TOL[dtype]
+    # epilogue: bias, residual and ReLU
+    bias = torch.from_numpy(rng.standard_normal(cout).astype(np.float32)).to("cuda", dtype)
+    res = torch.from_numpy(rng.standard_normal((n, cout)).astype(np.float32)).to("cuda", dtype)
+    y2 = backend.conv_implicit_gemm_segments(x, wp, 27, cin, cout, omap, n, bias, res, True)
+    want2 = np.maximum(want + _f32(bias)[None, :] + _f32(res), 0)
+    assert rel_rms(_f32(y2), want2) < TOL[dtype]
+
+
+def test_segments_and_dense_pass_agree_through_the_public_call(mods):
+    """conv_forward_implicit_gemm_cuda takes the segment form for small, wide layers; switched
+    off it runs the dense pass.  Both against the oracle, and close to each other."""
+    backend, F = mods
+    rng = np.random.default_rng(99)
+    n, cin, cout = 4000, 256, 256
+    coords = random_coords(rng, n, (30, 30, 10))
+    omap_np = oracle.kmap_subm(coords, 3)
+    omap = dev(omap_np)
+    x = torch.from_numpy(rng.standard_normal((n, cin)).astype(np.float32)).cuda().half()
+    w = torch.from_numpy(rng.uniform(-0.01, 0.01, (27, cin, cout)).astype(np.float32)).cuda().half()
+    want = oracle.conv_implicit_gemm(_f32(x), _f32(w), omap_np, n)
+    assert backend._segments_pay(x, 27, cin, cout, n)
+    seg = backend.conv_forward_implicit_gemm_cuda(x, w, omap, n, cout)
+    assert id(omap) in backend._segments_of  # the segment form ran (and kept its lists)
+    keep = backend.igemm_through_segments
+    backend.igemm_through_segments = False
+    try:
+        assert not backend._segments_pay(x, 27, cin, cout, n)
+        dense = backend.conv_forward_implicit_gemm_cuda(x, w, omap, n, cout)
+    finally:
+        backend.igemm_through_segments = keep
+    assert rel_rms(_f32(seg), want) < 1e-2 and rel_rms(_f32(dense), want) < 1e-2
+    assert rel_rms(_f32(seg), _f32(dense)) < 1e-2
+
+
+def test_strided_and_transposed_maps_over_segments(mods):
+    """A strided map (K_vol 8, fewer outputs than inputs) and its transposed map (every row at
+    most one pair), called directly."""
+    backend, F = mods
+    rng = np.random.default_rng(321)
+    coords = random_coords(rng, 5000, (40, 30, 12))
+    omap_np, out_coords = oracle.kmap_downsample(coords, 2, 2, 0)
+    n_in, n_out = len(coords), len(out_coords)
+    cin, cout = 128, 256
+    x = torch.from_numpy(rng.standard_normal((n_in, cin)).astype(np.float32)).cuda().half()
+    w = torch.from_numpy(rng.uniform(-0.03, 0.03, (8, cin, cout)).astype(np.float32)).cuda().half()
+    y = backend.conv_implicit_gemm_segments(x, backend.pack_weights(w), 8, cin, cout, dev(omap_np), n_out)
+    want = oracle.conv_implicit_gemm(_f32(x), _f32(w), omap_np, n_out)
+    assert rel_rms(_f32(y), want) < 1e-2
+    map_t = oracle.transpose_map(omap_np, n_in)
+    xt = torch.from_numpy(rng.standard_normal((n_out, cout)).astype(np.float32)).cuda().half()
+    wt = torch.from_numpy(rng.uniform(-0.03, 0.03, (8, cout, cin)).astype(np.float32)).cuda().half()
+    yt = backend.conv_implicit_gemm_segments(xt, backend.pack_weights(wt), 8, cout, cin, dev(map_t), n_in)
+    want_t = oracle.conv_implicit_gemm(_f32(xt), _f32(wt), map_t, n_in)
+    assert rel_rms(_f32(yt), want_t) < 1e-2
+
+
+def test_shapes_without_a_variant_are_refused_and_fall_back(mods):
+    backend, F = mods
+    code = 1  # fp16
+    for kvol, cin, cout in ((27, 96, 128), (27, 64, 128), (27, 512, 128), (125, 128, 128), (27, 128, 130)):
+        assert backend._C.tsmi_conv_segments_supported(kvol, cin, cout, code) == 0, (kvol, cin, cout)
+    assert backend._C.tsmi_conv_segments_supported(27, 128, 128, 0) == 0  # fp32: the dense pass only
+    rng = np.random.default_rng(8)
+    n = 500
+    coords = random_coords(rng, n, (12, 12, 8))
+    omap_np = oracle.kmap_subm(coords, 3)
+    x = torch.from_numpy(rng.standard_normal((n, 96)).astype(np.float32)).cuda().half()
+    w = torch.from_numpy(rng.uniform(-0.02, 0.02, (27, 96, 128)).astype(np.float32)).cuda().half()
+    with pytest.raises(ValueError):
+        backend.conv_implicit_gemm_segments(x, backend.pack_weights(w), 27, 96, 128, dev(omap_np), n)
+    assert not backend._segments_pay(x, 27, 96, 128, n)
+    y = backend.conv_forward_implicit_gemm_cuda(x, w, dev(omap_np), n, 128)  # the dense pass
+    want = oracle.conv_implicit_gemm(_f32(x), _f32(w), omap_np, n)
+    assert rel_rms(_f32(y), want) < 1e-2

@@ -8,6 +8,7 @@ eager fallback: if the shared object is missing, importing this module raises.
 """
 import collections
 import ctypes
+import functools
 import os
 import threading
 import weakref
@@ -94,6 +95,10 @@ def _load():
                                   _i64, _vp],
         "tsmi_conv_fetch_on_demand": [_vp, _vp, _vp, _vp, _i64, _vp, _vp, _i64, _vp, _i64, _i32,
                                       _i32, _i32, _i32, _i32, _i32, _vp, _vp, _i32, _vp, _vp],
+        "tsmi_conv_segments_supported": [_i32, _i32, _i32, _i32],
+        "tsmi_pair_segments": [_vp, _vp, _i64, _i32, _i64, _vp, _vp, _vp],
+        "tsmi_conv_implicit_gemm_segments": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _i32,
+                                             _i32, _vp, _vp, _i32, _vp, _vp],
         "tsmi_hash_coords": [_vp, _vp, _i64, _vp],
         "tsmi_kernel_hash": [_vp, _vp, _i64, _vp, _i32, _vp],
         "tsmi_count": [_vp, _vp, _i64, _vp, _i32],
@@ -1064,14 +1069,43 @@ def _epilogue_args(bias, residual, x, n_out, cout):
     return _ptr(bias), _ptr(residual)
 
 
+_SCRATCH = {}  # (device index, stream) -> uint8 tensor, grown on demand
+# held while a call that goes through the scratch buffer queues its launches: two host threads
+# that feed one stream must not interleave the launches of two such calls
+_scratch_lock = threading.Lock()
+
+
+def _scratch(device, stream: int, nbytes: int) -> int:
+    """Address of at least ``nbytes`` of device memory that the convolutions queued on one stream
+    share for their intermediate results (partial sums, per-pair products): every such launch
+    pair writes before it reads, and the stream runs them one after the other, so the buffer
+    needs no allocation per call.  It only grows; a replaced buffer goes back to torch's
+    stream-ordered allocator like any temporary."""
+    key = (device.index, stream)
+    t = _SCRATCH.get(key)
+    if t is None or t.numel() < nbytes:
+        t = _SCRATCH[key] = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+    return t.data_ptr()
+
+
+@functools.lru_cache(maxsize=4096)
+def _workspace_elems(n_out: int, kvol: int, cin: int, cout: int, code: int) -> int:
+    return _C.tsmi_conv_workspace_elems(n_out, n_out, kvol, 1, cin, cout, code, 0)
+
+
+@functools.lru_cache(maxsize=4096)
+def _segments_supported(kvol: int, cin: int, cout: int, code: int) -> bool:
+    return bool(_C.tsmi_conv_segments_supported(kvol, cin, cout, code))
+
+
 _TILE_COUNTERS = {}
 _N_TILE_COUNTERS = 4096
 
 
-def _tile_counters(device):
+def _tile_counters(device, stream: int):
     """Zero-filled int32 array shared by the split convolutions of one stream (each
     launch leaves it zero again)."""
-    key = (device.index, _stream())
+    key = (device.index, stream)
     t = _TILE_COUNTERS.get(key)
     if t is None:
         t = _TILE_COUNTERS[key] = torch.zeros(_N_TILE_COUNTERS, dtype=torch.int32, device=device)
@@ -1090,21 +1124,94 @@ def conv_forward_implicit_gemm_cuda(in_feats, kernel, out_in_map, num_out_feats,
     return _implicit_gemm(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias, residual, relu)
 
 
+# Small, wide layers of the implicit-GEMM dataflow run over pair segments (a per-offset
+# compaction of the map, built once per map and kept with it) instead of the dense pass over
+# all offsets of every row tile.  False: always the dense pass.
+igemm_through_segments = True
+
+_segments_of = {}  # id(map) -> (weak reference, version, address, stream, rows, segments)
+
+
+def pair_segments(out_in_map: torch.Tensor, n_rows: int):
+    """(counts int32 [K_vol], in_rows int32 [K_vol, seg_rows], pos int32 [K_vol, n_rows],
+    seg_rows) of a kernel map's first ``n_rows`` rows: per kernel offset the input rows of
+    its pairs, compacted, and for every (offset, row) the place of the pair in that list
+    (-1: none).  Built in one launch, once per map tensor and stream."""
+    out_in_map = _need(out_in_map, torch.int32, "out_in_map")
+    stream = _stream()
+    hit = _segments_of.get(id(out_in_map))
+    if (hit is not None and hit[0]() is out_in_map and hit[1] == out_in_map._version
+            and hit[2] == out_in_map.data_ptr() and hit[3] == stream and hit[4] == n_rows):
+        return hit[5]
+    kvol = out_in_map.shape[1]
+    if n_rows > out_in_map.shape[0]:
+        raise ValueError(f"the map has {out_in_map.shape[0]} rows, fewer than the {n_rows} asked for")
+    seg_rows = make_divisible(max(n_rows, 1), 128)
+    dev = out_in_map.device
+    counts = torch.empty(kvol, dtype=torch.int32, device=dev)
+    in_rows = torch.empty((kvol, seg_rows), dtype=torch.int32, device=dev)
+    pos = torch.empty((kvol, n_rows), dtype=torch.int32, device=dev)
+    _check(_C.tsmi_pair_segments(stream, _ptr(out_in_map), n_rows, kvol, seg_rows, _ptr(counts),
+                                 _ptr(in_rows), _ptr(pos)))
+    seg = (counts, in_rows, pos, seg_rows)
+    if len(_segments_of) >= 64:
+        for key in [k for k, v in _segments_of.items() if v[0]() is None]:
+            del _segments_of[key]
+        if len(_segments_of) >= 64:
+            _segments_of.clear()
+    _segments_of[id(out_in_map)] = (weakref.ref(out_in_map), out_in_map._version, out_in_map.data_ptr(),
+                                    stream, n_rows, seg)
+    return seg
+
+
+def _segments_pay(x, kvol, cin, cout, num_out_feats) -> bool:
+    """Whether a layer runs over pair segments: 16-bit features, a 3^3 or larger kernel, few rows
+    and many channels (the regime in which the dense pass is bound by the weight slabs it streams
+    per row tile).  Measured on the levels of an 89,834-voxel scan: 8,045 rows 256 -> 256 32 vs
+    43 us, 384 -> 256 39 vs 57, 19,815 rows 128 -> 128 30 vs 36, 192 -> 128 33 vs 47, 3,105 rows
+    256 -> 256 22 vs 28; 8,045 rows 128 -> 128 (21 vs 20) stays with the dense pass."""
+    return bool(igemm_through_segments and kvol >= 27 and 0 < num_out_feats < 65536 and cout >= 128
+                and (cin * cout > 128 * 128 or num_out_feats >= 12000)
+                and _segments_supported(kvol, cin, cout, _dtype_code(x)))
+
+
+def conv_implicit_gemm_segments(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias=None,
+                                residual=None, relu=False) -> torch.Tensor:
+    """The implicit-GEMM sums over pair segments: one launch multiplies every pair's input row
+    by its offset's weights (a workgroup reads one offset's weights only), a second adds each
+    output row's products."""
+    counts, in_rows, pos, seg_rows = pair_segments(out_in_map, num_out_feats)
+    y = torch.empty((num_out_feats, cout), dtype=x.dtype, device=x.device)
+    stream = _stream()
+    pb, pr = _epilogue_args(bias, residual, x, num_out_feats, cout)
+    with _scratch_lock:
+        products = _scratch(x.device, stream, kvol * seg_rows * cout * x.element_size())
+        _check(_C.tsmi_conv_implicit_gemm_segments(stream, x.data_ptr(), wp.data_ptr(), in_rows.data_ptr(),
+                                                   counts.data_ptr(), pos.data_ptr(), seg_rows,
+                                                   num_out_feats, kvol, cin, cout, _dtype_code(x), pb, pr,
+                                                   int(relu), products, y.data_ptr()))
+    return y
+
+
 def _implicit_gemm(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias=None, residual=None,
                    relu=False) -> torch.Tensor:
+    if _segments_pay(x, kvol, cin, cout, num_out_feats):
+        return conv_implicit_gemm_segments(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias,
+                                           residual, relu)
     y = torch.empty((num_out_feats, cout), dtype=x.dtype, device=x.device)
     code = _dtype_code(x)
-    ws, ws_elems = None, 0
-    if num_out_feats < 65536:  # only maps with few row tiles use the offset split
-        ws_elems = _C.tsmi_conv_workspace_elems(num_out_feats, num_out_feats, kvol, 1, cin, cout, code, 0)
-        if ws_elems > 0:
-            ws = torch.empty(ws_elems, dtype=torch.float32, device=x.device)
+    stream = _stream()
     pb, pr = _epilogue_args(bias, residual, x, num_out_feats, cout)
-    _check(_C.tsmi_conv_implicit_gemm(_stream(), _ptr(x), _ptr(wp), _ptr(out_in_map),
-                                      out_in_map.shape[0], num_out_feats, kvol, cin, cout, code,
-                                      pb, pr, int(relu), _ptr(ws), ws_elems,
-                                      _ptr(_tile_counters(x.device)) if ws is not None else None,
-                                      _N_TILE_COUNTERS, _ptr(y)))
+    args = (stream, x.data_ptr(), wp.data_ptr(), out_in_map.data_ptr(), out_in_map.shape[0], num_out_feats,
+            kvol, cin, cout, code, pb, pr, int(relu))
+    ws_elems = _workspace_elems(num_out_feats, kvol, cin, cout, code) if num_out_feats < 65536 else 0
+    if ws_elems > 0:  # (only maps with few row tiles use the offset split)
+        with _scratch_lock:
+            _check(_C.tsmi_conv_implicit_gemm(*args, _scratch(x.device, stream, 4 * ws_elems), ws_elems,
+                                              _tile_counters(x.device, stream).data_ptr(),
+                                              _N_TILE_COUNTERS, y.data_ptr()))
+    else:
+        _check(_C.tsmi_conv_implicit_gemm(*args, None, 0, None, _N_TILE_COUNTERS, y.data_ptr()))
     return y
 
 
@@ -1184,7 +1291,7 @@ def _implicit_gemm_sorted(x, wp, kvol, cin, cout, reorder_out_in_map, reduced_ma
                                              _ptr(reduced_mask), _ptr(reorder_loc), n_pad,
                                              num_out_feats, kvol, split, cin, cout, code,
                                              pb, pr, int(relu), _ptr(ws), ws_elems,
-                                             _ptr(_tile_counters(x.device)) if ws is not None else None,
+                                             _ptr(_tile_counters(x.device, _stream())) if ws is not None else None,
                                              _N_TILE_COUNTERS, _ptr(y)))
     return y
 

@@ -166,6 +166,35 @@ extern "C" int tsmi_conv_fetch_on_demand(tsmi_stream_t s, const void *x, const v
                       residual, relu, y);
 }
 
+extern "C" int tsmi_conv_segments_supported(int kvol, int cin, int cout, int dtype) {
+  const ConvOps *ops = ops_for(dtype);
+  if (!ops || kvol < 1 || cin < 1 || cout < 1) return 0;
+  return ops->segments_supported(kvol, cin, cout);
+}
+
+extern "C" int tsmi_conv_implicit_gemm_segments(tsmi_stream_t s, const void *x, const void *w_packed,
+                                               const int32_t *in_rows, const int32_t *counts,
+                                               const int32_t *pos, int64_t seg_rows, int64_t n_out,
+                                               int kvol, int cin, int cout, int dtype,
+                                               const void *bias, const void *residual, int relu,
+                                               void *products, void *y) {
+  const ConvOps *ops = ops_for(dtype);
+  if (int e = check_shapes("conv_implicit_gemm_segments", ops, kvol, cin, cout)) return e;
+  TSMI_REQUIRE(n_out >= 0 && seg_rows >= n_out && seg_rows % 64 == 0,
+               "conv_implicit_gemm_segments: bad sizes (n_out %lld, seg_rows %lld)", (long long)n_out,
+               (long long)seg_rows);
+  if (n_out == 0) return TSMI_OK;
+  TSMI_REQUIRE(x && w_packed && in_rows && counts && pos && products && y,
+               "conv_implicit_gemm_segments: null pointer");
+  TSMI_REQUIRE(aligned16(x) && aligned16(w_packed) && aligned16(products) && aligned16(y),
+               "conv_implicit_gemm_segments: x, w_packed, products and y must be 16-byte aligned");
+  if (int e = ops->segments((hipStream_t)s, x, w_packed, in_rows, counts, seg_rows, kvol, cin, cout,
+                            products))
+    return e;
+  return ops->segment_sum((hipStream_t)s, products, pos, n_out, kvol, seg_rows, cout, bias, residual,
+                          relu, y);
+}
+
 extern "C" int tsmi_gs_gather(tsmi_stream_t s, const void *x, const int32_t *nbmaps_inter,
                               int64_t nnz, int cin, int dtype, int transpose, void *buffer) {
   const ConvOps *ops = ops_for(dtype);

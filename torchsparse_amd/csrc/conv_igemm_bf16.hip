@@ -38,6 +38,7 @@ struct TraitsBF16 {
 #include "conv_small_cin.inc"
 #include "conv_tile.inc"
 #include "conv_igemm2.inc"
+#include "conv_segments.inc"
 #include "conv_plan.inc"
 #include "conv_wgrad.inc"
 #include "conv_wgrad_pairs.inc"

@@ -42,6 +42,16 @@ struct ConvOps {
   int (*wgrad_pairs)(hipStream_t s, const void *x, const void *dy, const int32_t *pairs,
                      const int32_t *seg_steps, int64_t pair_cap, int x_col, int kvol, int cin,
                      int cout, float *partial, int64_t partial_elems, void *dw);
+  // 1 when `segments` has a variant for the shape
+  int (*segments_supported)(int kvol, int cin, int cout);
+  // products[k * seg_rows + j, :] = X[in_rows[k * seg_rows + j], :] W[k] for j < counts[k]
+  int (*segments)(hipStream_t s, const void *x, const void *wp, const int32_t *in_rows,
+                  const int32_t *counts, int64_t seg_rows, int kvol, int cin, int cout,
+                  void *products);
+  // y[o, :] = sum over k of products[k * seg_rows + pos[k * n_out + o], :] where pos >= 0
+  int (*segment_sum)(hipStream_t s, const void *products, const int32_t *pos, int64_t n_out, int kvol,
+                     int64_t seg_rows, int cout, const void *bias, const void *residual, int relu,
+                     void *y);
 };
 
 const ConvOps &conv_ops_f16();

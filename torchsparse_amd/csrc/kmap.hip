@@ -784,6 +784,70 @@ __global__ __launch_bounds__(kBlock) void pair_count_kernel(const int32_t *map, 
   }
 }
 
+// The pairs of every kernel offset, compacted into that offset's fixed segment, in one launch:
+// in_rows[k * seg_rows + j] = map[row][k] of the j-th pair of offset k, pos[k * n_rows + row] = j
+// (-1 where the row has no pair at k), counts[k] (zero on entry) = pairs of offset k.  A block
+// reserves its share of each segment with one atomic add per offset, so the order of the blocks'
+// shares inside a segment varies from launch to launch; pos names the place either way.
+// KV > 0: the kernel volume, known at compile time: a thread keeps its row's entries in
+// registers (one round trip to memory, no staging).  KV == 0: any volume, staged through LDS
+// in chunks of kPairChunk offsets.
+template <int KV>
+__global__ __launch_bounds__(kBlock) void pair_segments_kernel(const int32_t *map, int64_t n_rows,
+                                                               int kvol, int64_t seg_rows,
+                                                               int32_t *counts, int32_t *in_rows,
+                                                               int32_t *pos) {
+  constexpr int kChunk = KV > 0 ? KV : kPairChunk;
+  __shared__ int32_t tile[KV > 0 ? 1 : kBlock * kPairStride];
+  __shared__ int wave_cnt[kBlock / 64][kChunk];
+  __shared__ int wave_base[kBlock / 64][kChunk];
+  const int64_t row0 = (int64_t)blockIdx.x * kBlock, row = row0 + threadIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const unsigned long long below = (1ULL << lane) - 1ULL;
+  for (int k0 = 0; k0 < kvol; k0 += kChunk) {
+    const int kc = KV > 0 ? KV : min(kChunk, kvol - k0);
+    int32_t m[KV > 0 ? KV : 1];
+    if (KV > 0) {
+#pragma unroll
+      for (int j = 0; j < KV; ++j) m[j] = row < n_rows ? map[row * KV + j] : -1;
+    } else {
+      __syncthreads();  // the previous chunk's tile and bases are no longer read
+      pair_stage_rows(map, row0, n_rows, kvol, k0, kc, tile);
+      __syncthreads();
+    }
+    auto entry = [&](int j) __attribute__((always_inline)) -> int32_t {
+      return KV > 0 ? m[KV > 0 ? j : 0] : tile[threadIdx.x * kPairStride + j];
+    };
+#pragma unroll
+    for (int j = 0; j < kChunk; ++j) {
+      if (j >= kc) break;
+      const int c = __popcll(__ballot(entry(j) >= 0));
+      if (lane == 0) wave_cnt[wave][j] = c;
+    }
+    __syncthreads();
+    if (threadIdx.x < kc) {
+      const int t = threadIdx.x;
+      const int a = wave_cnt[0][t], b = wave_cnt[1][t], c = wave_cnt[2][t], d = wave_cnt[3][t];
+      const int total = a + b + c + d;
+      const int base = total > 0 ? atomicAdd(&counts[k0 + t], total) : 0;
+      wave_base[0][t] = base;
+      wave_base[1][t] = base + a;
+      wave_base[2][t] = base + a + b;
+      wave_base[3][t] = base + a + b + c;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kChunk; ++j) {
+      if (j >= kc) break;
+      const int32_t v = entry(j);
+      const unsigned long long b = __ballot(v >= 0);
+      const int rank = wave_base[wave][j] + __popcll(b & below);
+      if (v >= 0) in_rows[(int64_t)(k0 + j) * seg_rows + rank] = v;
+      if (row < n_rows) pos[(int64_t)(k0 + j) * n_rows + row] = v >= 0 ? rank : -1;
+    }
+  }
+}
+
 // Block k: exclusive scan of offset k's per-block counts in place (positions relative to the
 // start of the offset's list); nbsizes[k] = their sum.
 __global__ __launch_bounds__(1024) void pair_scan_kernel(int32_t *counts, int kvol, int64_t nblk,
@@ -1583,6 +1647,36 @@ extern "C" int tsmi_pair_lists_fill(tsmi_stream_t s, const int32_t *map, int64_t
                        nbmaps_planar, n_in, n_out, input_mask, output_mask, skip_k);
   }
   return check_launch("tsmi_pair_lists_fill");
+}
+
+extern "C" int tsmi_pair_segments(tsmi_stream_t s, const int32_t *map, int64_t n_rows, int kvol,
+                                  int64_t seg_rows, int32_t *counts, int32_t *in_rows, int32_t *pos) {
+  TSMI_REQUIRE(kvol >= 1 && kvol <= kPairMaxKvol && n_rows >= 0 && seg_rows >= n_rows,
+               "pair_segments: bad sizes (kernel volume %d, at most %d; %lld rows, segments of %lld)",
+               kvol, kPairMaxKvol, (long long)n_rows, (long long)seg_rows);
+  TSMI_REQUIRE((int64_t)kvol * seg_rows < (int64_t(1) << 31), "pair_segments: kvol * seg_rows exceeds int32");
+  TSMI_REQUIRE(counts, "pair_segments: null counts");
+  hipLaunchKernelGGL(fill_kernel<int32_t>, grid_for(kvol), dim3(kBlock), 0, (hipStream_t)s, counts,
+                     (int64_t)kvol, 0);
+  if (n_rows == 0) return check_launch("tsmi_pair_segments");
+  TSMI_REQUIRE(map && in_rows && pos, "pair_segments: null pointer");
+  const int64_t nblk = ceil_div(n_rows, kBlock);
+  TSMI_REQUIRE(grid_fits(nblk), "pair_segments: too many rows");
+  const dim3 grid((unsigned)nblk), block(kBlock);
+  switch (kvol) {
+    case 27:
+      hipLaunchKernelGGL(pair_segments_kernel<27>, grid, block, 0, (hipStream_t)s, map, n_rows, kvol,
+                         seg_rows, counts, in_rows, pos);
+      break;
+    case 8:
+      hipLaunchKernelGGL(pair_segments_kernel<8>, grid, block, 0, (hipStream_t)s, map, n_rows, kvol,
+                         seg_rows, counts, in_rows, pos);
+      break;
+    default:
+      hipLaunchKernelGGL(pair_segments_kernel<0>, grid, block, 0, (hipStream_t)s, map, n_rows, kvol,
+                         seg_rows, counts, in_rows, pos);
+  }
+  return check_launch("tsmi_pair_segments");
 }
 
 extern "C" int64_t tsmi_wgrad_pairs_capacity(int64_t n_rows, int kvol) {
