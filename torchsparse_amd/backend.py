@@ -573,7 +573,7 @@ class _StridedState:
     stream (or device) get a state of their own and never see these tensors."""
     __slots__ = ("grid_buf", "grid_words", "grid_dirty", "chain_geom", "chain_last", "chain_count",
                  "chain_len", "ahead", "ahead_hits", "host_counters", "pending", "pending_rsv", "root_chain",
-                 "lookahead_hits")
+                 "lookahead_hits", "side", "grid_event", "grid_old")
 
     def __init__(self):
         self.grid_buf = None      # int32 scratch: bitmaps and chunk counts of every level
@@ -590,6 +590,9 @@ class _StridedState:
         self.pending_rsv = None
         self.root_chain = None    # geometry of the last chain that started from a caller's own rows
         self.lookahead_hits = 0   # chains whose first half was already queued (diagnostic)
+        self.side = None          # second stream of the device, for chains queued ahead of their use
+        self.grid_event = None    # end of the last work queued on the bitmap scratch, on either stream
+        self.grid_old = None      # the scratch before it last grew (kept until the next growth)
 
     def chain_step(self, coords, geom):
         """Book-keeping of chains of equal strided calls (each on the previous one's outputs).
@@ -616,6 +619,7 @@ class _StridedState:
         """The all-zero scratch whose first bitmap has at least ``words`` words.  Every call
         leaves the bitmaps zero again; one that did not finish has them cleared here."""
         if self.grid_buf is None or self.grid_words < words:
+            self.grid_old = self.grid_buf  # work queued on the other stream may still hold its address
             self.grid_buf = torch.zeros(_grid_layout(words)[1], dtype=torch.int32, device=dev)
             self.grid_words, self.grid_dirty = words, False
         elif self.grid_dirty:
@@ -680,6 +684,8 @@ def _grid_start(state, coords, ks, st, pd, coords_max_host, fan, ahead, early=Fa
     counters to the host; nothing waits.  Runs with _state_lock held."""
     n = coords.shape[0]
     dev = coords.device
+    if state.grid_event is not None:  # the scratch may last have been used on the other stream
+        torch.cuda.current_stream(dev).wait_event(state.grid_event)
     bits = min(max(1 << (n * fan * 2048 - 1).bit_length(), 1 << 20), 1 << 30)
     buf = state.bitmap(dev, bits // 32)
     layout, _ = _grid_layout(state.grid_words)
@@ -689,13 +695,14 @@ def _grid_start(state, coords, ks, st, pd, coords_max_host, fan, ahead, early=Fa
     s = _stream()
     g = (_I3(*ks), _I3(*st), _I3(*pd))
     host_max = _I3(*[int(v) for v in coords_max_host]) if coords_max_host is not None else None
-    part = lambda level, what: _grid_part(buf, ctr, layout, levels, level, what)  # noqa: E731
-    _check(_C.tsmi_coords_max(s, _ptr(coords), n, _ptr(part(0, "in_max")), 0))
+    buf_ptr, ctr_ptr = buf.data_ptr(), ctr.data_ptr()
+    part = lambda level, what: _grid_part(buf_ptr, ctr_ptr, layout, levels, level, what)  # noqa: E731
+    _check(_C.tsmi_coords_max(s, _ptr(coords), n, part(0, "in_max"), 0))
     state.grid_dirty = True  # marked bits stay behind unless the emit passes run
-    _check(_C.tsmi_downsample_grid_count(s, _ptr(coords), n, *g, host_max, _ptr(part(0, "in_max")),
-                                         _ptr(part(0, "bitmap")), layout[0][1], 0,
-                                         _ptr(part(0, "chunks")), _ptr(part(0, "counters")),
-                                         _ptr(part(1, "in_max")), None))
+    _check(_C.tsmi_downsample_grid_count(s, _ptr(coords), n, *g, host_max, part(0, "in_max"),
+                                         part(0, "bitmap"), layout[0][1], 0,
+                                         part(0, "chunks"), part(0, "counters"),
+                                         part(1, "in_max"), None))
     # One output per input (kernel size == stride, no padding: a level never has more rows than
     # the one before): every level's rows are emitted at once into a buffer of n rows while
     # their count is still on the device, and the next level marks from those rows.  Nothing is
@@ -710,22 +717,22 @@ def _grid_start(state, coords, ks, st, pd, coords_max_host, fan, ahead, early=Fa
         for level in range(levels):
             if level > 0:
                 _check(_C.tsmi_downsample_grid_count(
-                    s, _ptr(src), n, *g, None, _ptr(part(level, "in_max")), _ptr(part(level, "bitmap")),
-                    layout[level][1], 0, _ptr(part(level, "chunks")), _ptr(part(level, "counters")),
-                    _ptr(part(level + 1, "in_max")), _ptr(part(level - 1, "counters"))))
+                    s, _ptr(src), n, *g, None, part(level, "in_max"), part(level, "bitmap"),
+                    layout[level][1], 0, part(level, "chunks"), part(level, "counters"),
+                    part(level + 1, "in_max"), part(level - 1, "counters")))
             out = torch.empty((n, 4), dtype=torch.int32, device=dev)
             _check(_C.tsmi_downsample_grid_emit(
-                s, *g, None, _ptr(part(level, "in_max")), None, _ptr(part(level, "bitmap")),
-                layout[level][1], _ptr(part(level, "chunks")), -n, None, None, 0, _ptr(out),
-                _ptr(part(level, "counters"))))
+                s, *g, None, part(level, "in_max"), None, part(level, "bitmap"),
+                layout[level][1], part(level, "chunks"), -n, None, None, 0, _ptr(out),
+                part(level, "counters")))
             rows.append(out)
             src = out
     else:
         for level in range(1, levels):
             _check(_C.tsmi_downsample_grid_count_next(
-                s, *g, _ptr(part(level - 1, "in_max")), _ptr(part(level - 1, "bitmap")), layout[level - 1][1],
-                _ptr(part(level, "in_max")), _ptr(part(level, "bitmap")), layout[level][1],
-                _ptr(part(level, "chunks")), _ptr(part(level, "counters")), _ptr(part(level + 1, "in_max"))))
+                s, *g, part(level - 1, "in_max"), part(level - 1, "bitmap"), layout[level - 1][1],
+                part(level, "in_max"), part(level, "bitmap"), layout[level][1],
+                part(level, "chunks"), part(level, "counters"), part(level + 1, "in_max")))
     job = _GridJob()
     job.rows = rows
     job.coords, job.geom, job.coords_max_host, job.fan = coords, (ks, st, pd), coords_max_host, fan
@@ -742,18 +749,25 @@ def _grid_start(state, coords, ks, st, pd, coords_max_host, fan, ahead, early=Fa
         job.host.copy_(ctr, non_blocking=True)
         job.event = torch.cuda.Event()
         job.event.record()
+        state.grid_event = job.event
+    elif state.side is not None:  # (a state that never used its side stream needs no events)
+        state.grid_event = torch.cuda.Event()
+        state.grid_event.record()
     return job
 
 
-def _grid_part(buf, ctr, layout, levels, level, what):
+def _grid_part(buf_ptr, ctr_ptr, layout, levels, level, what):
+    """Address of one part of the bitmap scratch (int32 words at ``buf_ptr``) or of the counters
+    (8 int32 per level at ``ctr_ptr``): plain integers, no tensor views (a view costs more
+    host time than the launch it feeds)."""
     if what == "in_max":
-        return ctr[8 * level + 4:8 * level + 8] if level < levels else None
+        return ctr_ptr + 4 * (8 * level + 4) if level < levels else None
     off, w, cc = layout[level]
     if what == "bitmap":
-        return buf[off:off + w]
+        return buf_ptr + 4 * off
     if what == "chunks":
-        return buf[cc:cc + w // _GRID_CHUNK_WORDS]
-    return ctr[8 * level:8 * level + 8]  # "counters"
+        return buf_ptr + 4 * cc
+    return ctr_ptr + 4 * 8 * level  # "counters"
 
 
 def _grid_finish(state, job: _GridJob, rsv_ratio, cap, want_table):
@@ -770,7 +784,8 @@ def _grid_finish(state, job: _GridJob, rsv_ratio, cap, want_table):
     s = job.stream
     g = (_I3(*ks), _I3(*st), _I3(*pd))
     host_max = _I3(*[int(v) for v in job.coords_max_host]) if job.coords_max_host is not None else None
-    part = lambda level, what: _grid_part(buf, ctr, layout, levels, level, what)  # noqa: E731
+    buf_ptr, ctr_ptr = buf.data_ptr(), ctr.data_ptr()
+    part = lambda level, what: _grid_part(buf_ptr, ctr_ptr, layout, levels, level, what)  # noqa: E731
     if job.event is not None:
         job.event.synchronize()
         host = job.host.tolist()
@@ -805,11 +820,11 @@ def _grid_finish(state, job: _GridJob, rsv_ratio, cap, want_table):
         out = torch.empty((n_out, 4), dtype=torch.int32, device=dev)
         if n_out > 0:
             _check(_C.tsmi_downsample_grid_emit(
-                s, *g, host_max, _ptr(part(level, "in_max")),
-                (ctypes.c_int32 * 4)(*host[8 * level + 4:8 * level + 8]), _ptr(part(level, "bitmap")),
-                layout[level][1], _ptr(part(level, "chunks")), n_out,
+                s, *g, host_max, part(level, "in_max"),
+                (ctypes.c_int32 * 4)(*host[8 * level + 4:8 * level + 8]), part(level, "bitmap"),
+                layout[level][1], part(level, "chunks"), n_out,
                 _ptr(tbl.keys) if tbl is not None else None, _ptr(tbl.vals) if tbl is not None else None,
-                capacity, _ptr(out), _ptr(tbl.counters) if tbl is not None else _ptr(part(level, "counters"))))
+                capacity, _ptr(out), _ptr(tbl.counters) if tbl is not None else part(level, "counters")))
         return out, tbl
 
     first = emit(0, n, cap)
@@ -836,6 +851,9 @@ def _grid_finish(state, job: _GridJob, rsv_ratio, cap, want_table):
         prev = nxt[0]
     # rows emitted before the read-back cleared every bitmap they read, asked for or not
     state.grid_dirty = (not clean) and job.rows is None
+    if state.side is not None and job.rows is None:  # emit passes ran on this stream just now
+        state.grid_event = torch.cuda.Event()
+        state.grid_event.record()
     return first
 
 
@@ -862,6 +880,9 @@ downsample_lookahead_at_subm = True
 # Chains in which every input has exactly one output emit each level's rows before the counts
 # are read back (False: mark the next level from the bitmap, emit afterwards).
 downsample_emit_before_readback = True
+# Such a chain, queued at the submanifold build, runs on a second stream of the device (False:
+# on the caller's stream, behind everything already queued there).
+downsample_side_stream = True
 
 
 def strided_lookahead(coords: torch.Tensor) -> None:
@@ -882,7 +903,26 @@ def strided_lookahead(coords: torch.Tensor) -> None:
             state.pending = None  # never asked for; its marks are cleared by the next bitmap() call
         ks, st, pd, rsv_ratio = root
         ahead = min(state.chain_len.get(root, 1) - 1, _GRID_LEVELS - 1)
-        state.pending = _grid_start(state, coords, ks, st, pd, None, _strided_fan(ks, st), ahead, early=True)
+        fan = _strided_fan(ks, st)
+        # A chain that emits its rows before the read-back needs nothing but these rows, and rows
+        # of origin "user" were read back (with a synchronisation) when the library first saw
+        # them: they are complete whatever the stream still has queued.  Such a chain runs on a
+        # second stream, beside the tail of the previous forward, instead of behind it; the
+        # caller's stream never waits for it on the device: the host waits for the counters
+        # (the last thing the side stream does) before it queues anything that reads the rows.
+        aside = (downsample_side_stream and ahead > 0 and fan == 1 and ks == st and pd == (0, 0, 0)
+                 and downsample_emit_before_readback)
+        if aside:
+            main = torch.cuda.current_stream(coords.device)
+            if state.side is None:
+                state.side = torch.cuda.Stream(device=coords.device)
+            with torch.cuda.stream(state.side):
+                job = _grid_start(state, coords, ks, st, pd, None, fan, ahead, early=True)
+            for rows in job.rows or ():
+                rows.record_stream(main)  # allocated on the side stream, read and freed on the caller's
+        else:
+            job = _grid_start(state, coords, ks, st, pd, None, fan, ahead, early=True)
+        state.pending = job
         state.pending_rsv = rsv_ratio
 
 

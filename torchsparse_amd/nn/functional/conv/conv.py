@@ -10,7 +10,7 @@ from .func import (FetchOnDemandConvolutionFuntion, GatherScatterConvolutionFunt
                    ImplicitGEMMConvolutionFuntion)
 from .kmap import build_kernel_map, transpose_kernel_map
 
-__all__ = ["conv3d"]
+__all__ = ["conv3d", "conv3d_cached"]
 
 _DATAFLOWS = {
     _cfg.Dataflow.ImplicitGEMM: ImplicitGEMMConvolutionFuntion,
@@ -131,4 +131,64 @@ def conv3d(input: SparseTensor, weight: torch.Tensor,
 
     if output.stride not in caches.cmaps:
         caches.cmaps[output.stride] = (output.coords, output.spatial_range)
+    return output
+
+
+def conv3d_cached(input: SparseTensor, kernel: torch.Tensor, bias: Optional[torch.Tensor],
+                  kernel_size: Tuple[int, int, int], stride: Tuple[int, int, int],
+                  dilation: Tuple[int, int, int], transposed: bool, config: Optional[Dict],
+                  residual: Optional[torch.Tensor], activation: Optional[str]) -> Optional[SparseTensor]:
+    """The hot case of ``conv3d`` with most of its bookkeeping left out: an inference call
+    (no gradient flows) of a real-kernel, non-generative layer in the unsorted implicit-GEMM
+    dataflow whose kernel map is already in the tensor's cache and whose operands need no
+    conversion.  Returns None for everything else (the caller then takes ``conv3d``); what it
+    returns is what ``conv3d`` returns.  Kernel size, stride and dilation come as 3-tuples."""
+    if config is None:
+        config = _cfg.get_global_conv_config()
+        if config is None:
+            config = _cfg._shared_default_config(get_conv_mode())
+    if config["dataflow"] != _cfg.Dataflow.ImplicitGEMM or config["ifsort"] or kernel.dim() != 3:
+        return None
+    feats = input.feats
+    dtype = feats.dtype
+    if (not feats.is_cuda or dtype != kernel.dtype or not feats.is_contiguous()
+            or (bias is not None and bias.dtype != dtype)
+            or (residual is not None and (residual.dtype != dtype or not residual.is_contiguous()))):
+        return None
+    if torch.is_grad_enabled() and (feats.requires_grad or kernel.requires_grad
+                                    or (bias is not None and bias.requires_grad)
+                                    or (residual is not None and residual.requires_grad)):
+        return None
+    caches = input._caches
+    ist = input.stride
+    if not transposed:
+        kmap = caches.kmaps.get((ist, kernel_size, stride, dilation))
+        if kmap is None:
+            return None
+        omap = kmap["out_in_map"]
+        n_out = kmap["sizes"][1]
+        out_stride = (ist[0] * stride[0], ist[1] * stride[1], ist[2] * stride[2])
+        out_coords, out_range = kmap["coords"], kmap["spatial_range"]
+    else:
+        out_stride = (ist[0] // stride[0], ist[1] // stride[1], ist[2] // stride[2])
+        kmap = caches.kmaps.get((out_stride, kernel_size, stride, dilation))
+        level = caches.cmaps.get(out_stride)
+        if kmap is None or level is None:
+            return None
+        omap = kmap.get("out_in_map_t")
+        if omap is None:
+            return None
+        n_out = kmap["sizes"][0]
+        out_coords, out_range = level
+    if ist not in caches.cmaps:
+        caches.cmaps[ist] = (input.coords, input.spatial_range)
+    from torchsparse_amd import backend
+    kvol, cin, cout = kernel.shape
+    if feats.shape[1] != cin:
+        return None  # (conv3d raises the reference's error)
+    out_feats = backend._implicit_gemm(feats, backend.pack_weights(kernel), kvol, cin, cout, omap, n_out,
+                                       bias, residual, activation == "relu")
+    output = SparseTensor._make(out_feats, out_coords, out_stride, out_range, caches)
+    if out_stride not in caches.cmaps:
+        caches.cmaps[out_stride] = (out_coords, out_range)
     return output

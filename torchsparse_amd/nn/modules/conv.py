@@ -30,6 +30,7 @@ class Conv3d(nn.Module):
         self.kernel_size = make_ntuple(kernel_size, ndim=3)
         self.stride = make_ntuple(stride, ndim=3)
         self.dilation = dilation
+        self._dilation3 = make_ntuple(dilation, ndim=3)
         user_pad = make_ntuple(padding, ndim=3)
         self.padding = tuple((k - 1) // 2 if (k % 2 == 1 and s == 1) else p
                              for k, s, p in zip(self.kernel_size, self.stride, user_pad))
@@ -71,6 +72,13 @@ class Conv3d(nn.Module):
         return ", ".join(parts)
 
     def forward(self, input: SparseTensor, residual: torch.Tensor = None) -> SparseTensor:
+        if not self.training and not self.generative and self.activation in (None, "relu"):
+            # a layer whose map is already cached, in inference: the short way (None: not that case)
+            dilation = getattr(self, "_dilation3", None) or make_ntuple(self.dilation, ndim=3)
+            out = F.conv3d_cached(input, self.kernel, self.bias, self.kernel_size, self.stride,
+                                  dilation, self.transposed, self._config, residual, self.activation)
+            if out is not None:
+                return out
         return F.conv3d(input, weight=self.kernel, kernel_size=self.kernel_size, bias=self.bias,
                         stride=self.stride, padding=self.padding, dilation=self.dilation,
                         transposed=self.transposed, generative=self.generative,
