@@ -484,7 +484,10 @@ int tsmi_conv_fetch_on_demand(tsmi_stream_t s, const void *x, const void *w_pack
  * K_vol * seg_rows int32 (only the first counts[k] of a segment are written), pos
  * K_vol * n_rows, counts K_vol.  The order of the pairs inside a segment is not fixed
  * (blocks reserve their share with an atomic add); pos names each pair's place, and every
- * result computed through the two arrays is the same whatever the order.
+ * result computed through the two arrays is the same whatever the order.  `pool`: NULL, or
+ * K_vol + 1 int32 that are zero on entry and zero again when the call has run (the blocks
+ * add up there and the last one moves the sums into `counts`); with NULL `counts` is cleared
+ * by a launch of its own first.  Calls that share a pool must not overlap.
  * tsmi_conv_implicit_gemm_segments: products[k * seg_rows + j, :] = X[in_rows[k * seg_rows + j], :]
  * W[k] for j < counts[k] (one launch: a workgroup takes a run of 64-pair tiles and keeps the
  * weights of their offset in registers), then Y[o, :] = sum over k of products[k * seg_rows +
@@ -498,7 +501,8 @@ int tsmi_conv_fetch_on_demand(tsmi_stream_t s, const void *x, const void *w_pack
  * (convolution/convolution_forward_fetch_on_demand_cuda.cu:1981-2119). */
 int tsmi_conv_segments_supported(int kvol, int cin, int cout, int dtype);
 int tsmi_pair_segments(tsmi_stream_t s, const int32_t *map, int64_t n_rows, int kvol,
-                       int64_t seg_rows, int32_t *counts, int32_t *in_rows, int32_t *pos);
+                       int64_t seg_rows, int32_t *pool, int32_t *counts, int32_t *in_rows,
+                       int32_t *pos);
 int tsmi_conv_implicit_gemm_segments(tsmi_stream_t s, const void *x, const void *w_packed,
                                      const int32_t *in_rows, const int32_t *counts,
                                      const int32_t *pos, int64_t seg_rows, int64_t n_out, int kvol,

@@ -96,7 +96,7 @@ def _load():
         "tsmi_conv_fetch_on_demand": [_vp, _vp, _vp, _vp, _i64, _vp, _vp, _i64, _vp, _i64, _i32,
                                       _i32, _i32, _i32, _i32, _i32, _vp, _vp, _i32, _vp, _vp],
         "tsmi_conv_segments_supported": [_i32, _i32, _i32, _i32],
-        "tsmi_pair_segments": [_vp, _vp, _i64, _i32, _i64, _vp, _vp, _vp],
+        "tsmi_pair_segments": [_vp, _vp, _i64, _i32, _i64, _vp, _vp, _vp, _vp],
         "tsmi_conv_implicit_gemm_segments": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _i32,
                                              _i32, _vp, _vp, _i32, _vp, _vp],
         "tsmi_hash_coords": [_vp, _vp, _i64, _vp],
@@ -1170,33 +1170,68 @@ def conv_forward_implicit_gemm_cuda(in_feats, kernel, out_in_map, num_out_feats,
 igemm_through_segments = True
 
 _segments_of = {}  # id(map) -> (weak reference, version, address, stream, rows, segments)
+_SEGMENT_POOLS = {}  # (device index, stream) -> zero int32 tensor the builder's blocks add up in
 
 
-def pair_segments(out_in_map: torch.Tensor, n_rows: int):
-    """(counts int32 [K_vol], in_rows int32 [K_vol, seg_rows], pos int32 [K_vol, n_rows],
-    seg_rows) of a kernel map's first ``n_rows`` rows: per kernel offset the input rows of
-    its pairs, compacted, and for every (offset, row) the place of the pair in that list
-    (-1: none).  Built in one launch, once per map tensor and stream."""
-    out_in_map = _need(out_in_map, torch.int32, "out_in_map")
+class PairSegments:
+    """Per-offset pair lists of a kernel map (tsmi_pair_segments), in one int32 allocation:
+    ``counts`` [K_vol], ``in_rows`` [K_vol, seg_rows], ``pos`` [K_vol, n_rows] (views, made when
+    asked for; the convolution works from the addresses)."""
+    __slots__ = ("buffer", "kvol", "n_rows", "seg_rows", "counts_ptr", "in_rows_ptr", "pos_ptr")
+
+    def __init__(self, kvol: int, n_rows: int, seg_rows: int, device):
+        self.kvol, self.n_rows, self.seg_rows = kvol, n_rows, seg_rows
+        head = make_divisible(kvol, 64)  # keeps the two lists 256-byte aligned
+        self.buffer = torch.empty(head + kvol * seg_rows + kvol * n_rows, dtype=torch.int32, device=device)
+        self.counts_ptr = self.buffer.data_ptr()
+        self.in_rows_ptr = self.counts_ptr + 4 * head
+        self.pos_ptr = self.in_rows_ptr + 4 * kvol * seg_rows
+
+    @property
+    def counts(self) -> torch.Tensor:
+        return self.buffer[:self.kvol]
+
+    @property
+    def in_rows(self) -> torch.Tensor:
+        head = make_divisible(self.kvol, 64)
+        return self.buffer[head:head + self.kvol * self.seg_rows].view(self.kvol, self.seg_rows)
+
+    @property
+    def pos(self) -> torch.Tensor:
+        start = make_divisible(self.kvol, 64) + self.kvol * self.seg_rows
+        return self.buffer[start:start + self.kvol * self.n_rows].view(self.kvol, self.n_rows)
+
+    def __iter__(self):  # (counts, in_rows, pos, seg_rows)
+        return iter((self.counts, self.in_rows, self.pos, self.seg_rows))
+
+
+def pair_segments(out_in_map: torch.Tensor, n_rows: int) -> PairSegments:
+    """The pair segments of a kernel map's first ``n_rows`` rows: per kernel offset the input
+    rows of its pairs, compacted (``in_rows``), their number (``counts``) and for every (offset,
+    row) the place of the pair in that list (``pos``, -1: none).  Built in one launch, once per
+    map tensor and stream."""
     stream = _stream()
     hit = _segments_of.get(id(out_in_map))
     if (hit is not None and hit[0]() is out_in_map and hit[1] == out_in_map._version
             and hit[2] == out_in_map.data_ptr() and hit[3] == stream and hit[4] == n_rows):
         return hit[5]
+    out_in_map = _need(out_in_map, torch.int32, "out_in_map")
     kvol = out_in_map.shape[1]
     if n_rows > out_in_map.shape[0]:
         raise ValueError(f"the map has {out_in_map.shape[0]} rows, fewer than the {n_rows} asked for")
-    seg_rows = make_divisible(max(n_rows, 1), 128)
     dev = out_in_map.device
-    counts = torch.empty(kvol, dtype=torch.int32, device=dev)
-    in_rows = torch.empty((kvol, seg_rows), dtype=torch.int32, device=dev)
-    pos = torch.empty((kvol, n_rows), dtype=torch.int32, device=dev)
-    _check(_C.tsmi_pair_segments(stream, _ptr(out_in_map), n_rows, kvol, seg_rows, _ptr(counts),
-                                 _ptr(in_rows), _ptr(pos)))
-    seg = (counts, in_rows, pos, seg_rows)
+    seg = PairSegments(kvol, n_rows, make_divisible(max(n_rows, 1), 128), dev)
+    key = (dev.index, stream)
+    pool = _SEGMENT_POOLS.get(key)
+    if pool is None:
+        pool = _SEGMENT_POOLS[key] = torch.zeros(520, dtype=torch.int32, device=dev)
+    with _scratch_lock:  # (the pool is shared by the builds of one stream)
+        _check(_C.tsmi_pair_segments(stream, out_in_map.data_ptr(), n_rows, kvol, seg.seg_rows,
+                                     pool.data_ptr() if kvol < 520 else None, seg.counts_ptr,
+                                     seg.in_rows_ptr, seg.pos_ptr))
     if len(_segments_of) >= 64:
-        for key in [k for k, v in _segments_of.items() if v[0]() is None]:
-            del _segments_of[key]
+        for k in [k for k, v in _segments_of.items() if v[0]() is None]:
+            del _segments_of[k]
         if len(_segments_of) >= 64:
             _segments_of.clear()
     _segments_of[id(out_in_map)] = (weakref.ref(out_in_map), out_in_map._version, out_in_map.data_ptr(),
@@ -1220,14 +1255,15 @@ def conv_implicit_gemm_segments(x, wp, kvol, cin, cout, out_in_map, num_out_feat
     """The implicit-GEMM sums over pair segments: one launch multiplies every pair's input row
     by its offset's weights (a workgroup reads one offset's weights only), a second adds each
     output row's products."""
-    counts, in_rows, pos, seg_rows = pair_segments(out_in_map, num_out_feats)
+    seg = pair_segments(out_in_map, num_out_feats)
+    seg_rows = seg.seg_rows
     y = torch.empty((num_out_feats, cout), dtype=x.dtype, device=x.device)
     stream = _stream()
     pb, pr = _epilogue_args(bias, residual, x, num_out_feats, cout)
     with _scratch_lock:
         products = _scratch(x.device, stream, kvol * seg_rows * cout * x.element_size())
-        _check(_C.tsmi_conv_implicit_gemm_segments(stream, x.data_ptr(), wp.data_ptr(), in_rows.data_ptr(),
-                                                   counts.data_ptr(), pos.data_ptr(), seg_rows,
+        _check(_C.tsmi_conv_implicit_gemm_segments(stream, x.data_ptr(), wp.data_ptr(), seg.in_rows_ptr,
+                                                   seg.counts_ptr, seg.pos_ptr, seg_rows,
                                                    num_out_feats, kvol, cin, cout, _dtype_code(x), pb, pr,
                                                    int(relu), products, y.data_ptr()))
     return y

@@ -792,11 +792,14 @@ __global__ __launch_bounds__(kBlock) void pair_count_kernel(const int32_t *map, 
 // KV > 0: the kernel volume, known at compile time: a thread keeps its row's entries in
 // registers (one round trip to memory, no staging).  KV == 0: any volume, staged through LDS
 // in chunks of kPairChunk offsets.
+// `pool` (NULL, or kvol + 1 int32 that are zero on entry): the blocks then add up in the pool,
+// and the block that finishes last moves the sums into `counts` and leaves the pool zero for
+// the next launch, so that `counts` needs no clearing beforehand.
 template <int KV>
 __global__ __launch_bounds__(kBlock) void pair_segments_kernel(const int32_t *map, int64_t n_rows,
                                                                int kvol, int64_t seg_rows,
-                                                               int32_t *counts, int32_t *in_rows,
-                                                               int32_t *pos) {
+                                                               int32_t *pool, int32_t *counts,
+                                                               int32_t *in_rows, int32_t *pos) {
   constexpr int kChunk = KV > 0 ? KV : kPairChunk;
   __shared__ int32_t tile[KV > 0 ? 1 : kBlock * kPairStride];
   __shared__ int wave_cnt[kBlock / 64][kChunk];
@@ -829,7 +832,7 @@ __global__ __launch_bounds__(kBlock) void pair_segments_kernel(const int32_t *ma
       const int t = threadIdx.x;
       const int a = wave_cnt[0][t], b = wave_cnt[1][t], c = wave_cnt[2][t], d = wave_cnt[3][t];
       const int total = a + b + c + d;
-      const int base = total > 0 ? atomicAdd(&counts[k0 + t], total) : 0;
+      const int base = total > 0 ? atomicAdd(&(pool ? pool : counts)[k0 + t], total) : 0;
       wave_base[0][t] = base;
       wave_base[1][t] = base + a;
       wave_base[2][t] = base + a + b;
@@ -844,6 +847,19 @@ __global__ __launch_bounds__(kBlock) void pair_segments_kernel(const int32_t *ma
       const int rank = wave_base[wave][j] + __popcll(b & below);
       if (v >= 0) in_rows[(int64_t)(k0 + j) * seg_rows + rank] = v;
       if (row < n_rows) pos[(int64_t)(k0 + j) * n_rows + row] = v >= 0 ? rank : -1;
+    }
+  }
+  if (pool) {
+    __shared__ int last;
+    __syncthreads();  // this block's adds are issued
+    if (threadIdx.x == 0) {
+      __threadfence();
+      last = atomicAdd(&pool[kvol], 1) == (int)gridDim.x - 1;
+    }
+    __syncthreads();
+    if (last) {  // every other block's adds precede its ticket: the sums are complete
+      for (int k = threadIdx.x; k < kvol; k += kBlock) counts[k] = atomicExch(&pool[k], 0);
+      if (threadIdx.x == 0) atomicExch(&pool[kvol], 0);
     }
   }
 }
@@ -1650,14 +1666,16 @@ extern "C" int tsmi_pair_lists_fill(tsmi_stream_t s, const int32_t *map, int64_t
 }
 
 extern "C" int tsmi_pair_segments(tsmi_stream_t s, const int32_t *map, int64_t n_rows, int kvol,
-                                  int64_t seg_rows, int32_t *counts, int32_t *in_rows, int32_t *pos) {
+                                  int64_t seg_rows, int32_t *pool, int32_t *counts, int32_t *in_rows,
+                                  int32_t *pos) {
   TSMI_REQUIRE(kvol >= 1 && kvol <= kPairMaxKvol && n_rows >= 0 && seg_rows >= n_rows,
                "pair_segments: bad sizes (kernel volume %d, at most %d; %lld rows, segments of %lld)",
                kvol, kPairMaxKvol, (long long)n_rows, (long long)seg_rows);
   TSMI_REQUIRE((int64_t)kvol * seg_rows < (int64_t(1) << 31), "pair_segments: kvol * seg_rows exceeds int32");
   TSMI_REQUIRE(counts, "pair_segments: null counts");
-  hipLaunchKernelGGL(fill_kernel<int32_t>, grid_for(kvol), dim3(kBlock), 0, (hipStream_t)s, counts,
-                     (int64_t)kvol, 0);
+  if (!pool || n_rows == 0)
+    hipLaunchKernelGGL(fill_kernel<int32_t>, grid_for(kvol), dim3(kBlock), 0, (hipStream_t)s, counts,
+                       (int64_t)kvol, 0);
   if (n_rows == 0) return check_launch("tsmi_pair_segments");
   TSMI_REQUIRE(map && in_rows && pos, "pair_segments: null pointer");
   const int64_t nblk = ceil_div(n_rows, kBlock);
@@ -1666,15 +1684,15 @@ extern "C" int tsmi_pair_segments(tsmi_stream_t s, const int32_t *map, int64_t n
   switch (kvol) {
     case 27:
       hipLaunchKernelGGL(pair_segments_kernel<27>, grid, block, 0, (hipStream_t)s, map, n_rows, kvol,
-                         seg_rows, counts, in_rows, pos);
+                         seg_rows, pool, counts, in_rows, pos);
       break;
     case 8:
       hipLaunchKernelGGL(pair_segments_kernel<8>, grid, block, 0, (hipStream_t)s, map, n_rows, kvol,
-                         seg_rows, counts, in_rows, pos);
+                         seg_rows, pool, counts, in_rows, pos);
       break;
     default:
       hipLaunchKernelGGL(pair_segments_kernel<0>, grid, block, 0, (hipStream_t)s, map, n_rows, kvol,
-                         seg_rows, counts, in_rows, pos);
+                         seg_rows, pool, counts, in_rows, pos);
   }
   return check_launch("tsmi_pair_segments");
 }

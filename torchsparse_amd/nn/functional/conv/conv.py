@@ -147,7 +147,7 @@ def conv3d_cached(input: SparseTensor, kernel: torch.Tensor, bias: Optional[torc
         config = _cfg.get_global_conv_config()
         if config is None:
             config = _cfg._shared_default_config(get_conv_mode())
-    if config["dataflow"] != _cfg.Dataflow.ImplicitGEMM or config["ifsort"] or kernel.dim() != 3:
+    if config["dataflow"] != _cfg.Dataflow.ImplicitGEMM or config["ifsort"]:
         return None
     feats = input.feats
     dtype = feats.dtype
@@ -161,6 +161,15 @@ def conv3d_cached(input: SparseTensor, kernel: torch.Tensor, bias: Optional[torc
         return None
     caches = input._caches
     ist = input.stride
+    if kernel.dim() != 3:  # a 1x1x1 stride-1 layer: no map, the outputs are the inputs
+        if kernel_size != (1, 1, 1) or stride != (1, 1, 1) or dilation != (1, 1, 1) or feats.shape[0] == 0 \
+                or feats.shape[1] != kernel.shape[0]:
+            return None
+        from torchsparse_amd import backend
+        if ist not in caches.cmaps:
+            caches.cmaps[ist] = (input.coords, input.spatial_range)
+        out_feats = backend.conv_pointwise_cuda(feats, kernel, bias, residual, activation == "relu")
+        return SparseTensor._make(out_feats, input.coords, ist, input.spatial_range, caches)
     if not transposed:
         kmap = caches.kmaps.get((ist, kernel_size, stride, dilation))
         if kmap is None:
