@@ -62,6 +62,9 @@ def parse():
                          "a 256 MiB device copy (5 launches), then 5 launches each of the kernel-map "
                          "builders (searched and hashed, scan and 1M voxels), the gather and scatter "
                          "kernels (64 channels) and the 1M-voxel 256 -> 256 convolution")
+    ap.add_argument("--dense-deep", action="store_true",
+                    help="run the small wide layers as a dense pass over the map instead of over pair "
+                         "segments (for the counter passes that compare the two forms)")
     ap.add_argument("--sorted", type=int, default=-1,
                     help="1: run the implicit GEMM over row-sorted maps (conv_mode 1); 0: unsorted; "
                          "-1: the default of this benchmark")
@@ -660,6 +663,8 @@ def main():
     head = torch.nn.Linear(96, 19).cuda().half().eval()
     if args.sorted == 1:
         F.set_conv_mode(1)
+    if args.dense_deep:
+        backend.igemm_through_segments = False
 
     def timed(net, steps, warmup, fresh_coords=False):
         def step():
