@@ -442,7 +442,7 @@ def dominant_layer_roofline(ts, F, records, caches, pmc_target=None):
         flops, nbytes = conv_work(r["n_in"], r["n_out"], omap.shape[0], nnz, kvol, cin, cout, 2)
         one = roofline_of(flops, nbytes, ms)
         form = ("pair segments (segment_products_kernel + segment_sum_kernel)"
-                if backend._segments_pay(x, kvol, cin, cout, r["n_out"]) else "dense pass over the map")
+                if backend._segments_pay(x, kvol, cin, cout, r["n_out"], omap) else "dense pass over the map")
         every.append({"kernel": desc, "form": form, "launches_per_step": len(rs), "launch_ms": round(ms, 5),
                       "step_ms": round(ms * len(rs), 4), "bound": one["bound"],
                       "achieved": round(one["achieved"], 2), "peak": one["peak"], "unit": one["unit"],

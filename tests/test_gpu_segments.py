@@ -128,13 +128,20 @@ def test_segments_and_dense_pass_agree_through_the_public_call(mods):
     x = torch.from_numpy(rng.standard_normal((n, cin)).astype(np.float32)).cuda().half()
     w = torch.from_numpy(rng.uniform(-0.01, 0.01, (27, cin, cout)).astype(np.float32)).cuda().half()
     want = oracle.conv_implicit_gemm(_f32(x), _f32(w), omap_np, n)
-    assert backend._segments_pay(x, 27, cin, cout, n)
-    seg = backend.conv_forward_implicit_gemm_cuda(x, w, omap, n, cout)
-    assert id(omap) in backend._segments_of  # the segment form ran (and kept its lists)
     keep = backend.igemm_through_segments
-    backend.igemm_through_segments = False
     try:
-        assert not backend._segments_pay(x, 27, cin, cout, n)
+        backend.igemm_through_segments = True  # the default: only maps known to be thin
+        assert not backend._segments_pay(x, 27, cin, cout, n, omap)
+        backend.hint_sparse_map(omap)
+        assert backend._segments_pay(x, 27, cin, cout, n, omap)
+        seg = backend.conv_forward_implicit_gemm_cuda(x, w, omap, n, cout)
+        assert id(omap) in backend._segments_of  # the segment form ran (and kept its lists)
+        other = omap.clone()  # an unmarked map of the same content: dense, unless told "always"
+        assert not backend._segments_pay(x, 27, cin, cout, n, other)
+        backend.igemm_through_segments = "always"
+        assert backend._segments_pay(x, 27, cin, cout, n, other)
+        backend.igemm_through_segments = False
+        assert not backend._segments_pay(x, 27, cin, cout, n, omap)
         dense = backend.conv_forward_implicit_gemm_cuda(x, w, omap, n, cout)
     finally:
         backend.igemm_through_segments = keep
@@ -178,7 +185,39 @@ def test_shapes_without_a_variant_are_refused_and_fall_back(mods):
     w = torch.from_numpy(rng.uniform(-0.02, 0.02, (27, 96, 128)).astype(np.float32)).cuda().half()
     with pytest.raises(ValueError):
         backend.conv_implicit_gemm_segments(x, backend.pack_weights(w), 27, 96, 128, dev(omap_np), n)
-    assert not backend._segments_pay(x, 27, 96, 128, n)
+    assert not backend._segments_pay(x, 27, 96, 128, n, dev(omap_np))
     y = backend.conv_forward_implicit_gemm_cuda(x, w, dev(omap_np), n, 128)  # the dense pass
     want = oracle.conv_implicit_gemm(_f32(x), _f32(w), omap_np, n)
     assert rel_rms(_f32(y), want) < 1e-2
+
+
+def test_maps_over_thinned_rows_are_marked_sparse_and_solid_ones_are_not(mods):
+    """build_kernel_map marks the submanifold map of a level that a kernel = stride layer
+    produced when the level kept at least 0.3 rows per input row (surfaces, scattered voxels);
+    a solid volume keeps 1/8 and stays with the dense pass."""
+    backend, F = mods
+    import torchsparse_amd as ts
+    from torchsparse_amd import nn as spnn
+    rng = np.random.default_rng(77)
+    scattered = random_coords(rng, 3000, (60, 60, 40))
+    g = np.stack(np.meshgrid(np.arange(16), np.arange(16), np.arange(12), indexing="ij"), -1).reshape(-1, 3)
+    solid = np.concatenate([np.zeros((len(g), 1), np.int64), g], 1).astype(np.int32)
+    for coords_np, marked in ((scattered, True), (solid, False)):
+        order = np.lexsort((coords_np[:, 3], coords_np[:, 2], coords_np[:, 1], coords_np[:, 0]))
+        coords = dev(coords_np[order])
+        x = ts.SparseTensor(torch.zeros(len(coords_np), 4, device="cuda", dtype=torch.float16), coords)
+        down = spnn.Conv3d(4, 128, 2, stride=2).cuda().half().eval()
+        deep = spnn.Conv3d(128, 256, 3).cuda().half().eval()
+        with torch.no_grad():
+            mid = down(x)
+            thinning = backend.level_thinning(mid.coords)
+            assert thinning is not None and abs(thinning - mid.coords.shape[0] / len(coords_np)) < 1e-9
+            assert (thinning >= 0.3) == marked
+            out = deep(mid)
+        omap = mid._caches.kmaps[((2, 2, 2), (3, 3, 3), (1, 1, 1), (1, 1, 1))]["out_in_map"]
+        hit = backend._sparse_maps.get(id(omap))
+        assert (hit is not None and hit() is omap) == marked
+        assert backend._segments_pay(mid.feats, 27, 128, 256, mid.feats.shape[0], omap) == marked
+        want = oracle.conv_implicit_gemm(_f32(mid.feats), _f32(deep.kernel), omap.cpu().numpy(), mid.feats.shape[0])
+        assert rel_rms(_f32(out.feats), want) < 1e-2
+    assert backend.level_thinning(dev(scattered)) is None  # a caller's own rows: nothing known

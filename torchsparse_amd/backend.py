@@ -830,6 +830,9 @@ def _grid_finish(state, job: _GridJob, rsv_ratio, cap, want_table):
     first = emit(0, n, cap)
     # cells of a grid whose every in-range candidate was packable, in ascending order
     _mark_range_ok(first[0], ascending=True)
+    thin = fan == 1 and ks == st and pd == (0, 0, 0)  # every output stands for one block of cells
+    if thin:
+        _note_level(first[0], n)
     prev = first[0]
     clean = True
     for level in range(1, levels):
@@ -844,6 +847,8 @@ def _grid_finish(state, job: _GridJob, rsv_ratio, cap, want_table):
             clean = False  # this level's marks (and the later ones') are still in the bitmaps
             break
         state.ahead[id(prev)] = (weakref.ref(prev), (ks, st, pd, rsv_ratio), nxt[0], nxt[1])
+        if thin:
+            _note_level(nxt[0], n_in)
         # the later levels are not flagged on the device; their inputs' maxima are on the host
         if (host[8 * level + 4] < BATCH_LIMIT and
                 all(host[8 * level + 5 + a] + 2 * pd[a] < COORD_LIMIT for a in range(3))):
@@ -1166,7 +1171,8 @@ def conv_forward_implicit_gemm_cuda(in_feats, kernel, out_in_map, num_out_feats,
 
 # Small, wide layers of the implicit-GEMM dataflow run over pair segments (a per-offset
 # compaction of the map, built once per map and kept with it) instead of the dense pass over
-# all offsets of every row tile.  False: always the dense pass.
+# all offsets of every row tile, where the map is known to have few pairs per row (True), wherever
+# the kernels have a variant ("always"), or never (False).
 igemm_through_segments = True
 
 _segments_of = {}  # id(map) -> (weak reference, version, address, stream, rows, segments)
@@ -1239,15 +1245,61 @@ def pair_segments(out_in_map: torch.Tensor, n_rows: int) -> PairSegments:
     return seg
 
 
-def _segments_pay(x, kvol, cin, cout, num_out_feats) -> bool:
+_level_thinning = {}  # id(coords) -> (weak reference, rows kept per input row by the layer that made them)
+_sparse_maps = {}     # id(map) -> weak reference: maps over rows known to have few neighbours
+
+
+def _note_level(out_coords: torch.Tensor, n_in: int) -> None:
+    """``out_coords`` came out of a kernel size = stride, pad 0 layer over ``n_in`` rows."""
+    if len(_level_thinning) >= 256:
+        for key in [k for k, v in _level_thinning.items() if v[0]() is None]:
+            del _level_thinning[key]
+        if len(_level_thinning) >= 256:
+            _level_thinning.clear()
+    _level_thinning[id(out_coords)] = (weakref.ref(out_coords), out_coords.shape[0] / max(n_in, 1))
+
+
+def level_thinning(coords: torch.Tensor) -> Optional[float]:
+    """N_out / N_in of the kernel size = stride, pad 0 strided layer that produced ``coords``
+    (None: not such rows).  Each output of such a layer stands for a block of prod(stride) cells,
+    so N_out / N_in = 1 / (occupied cells per occupied block): 1/8 for solid volumes under 2^3
+    blocks, 0.4 - 0.5 for surfaces (a LiDAR scan's levels: 0.50, 0.44, 0.41, 0.39)."""
+    hit = _level_thinning.get(id(coords))
+    return hit[1] if hit is not None and hit[0]() is coords else None
+
+
+def hint_sparse_map(out_in_map: torch.Tensor) -> None:
+    """Mark a kernel map as one over thin rows (few neighbours per row): the implicit-GEMM
+    dataflow then runs its small, wide layers over pair segments."""
+    if len(_sparse_maps) >= 256:
+        for key in [k for k, v in _sparse_maps.items() if v() is None]:
+            del _sparse_maps[key]
+        if len(_sparse_maps) >= 256:
+            _sparse_maps.clear()
+    _sparse_maps[id(out_in_map)] = weakref.ref(out_in_map)
+
+
+def _segments_pay(x, kvol, cin, cout, num_out_feats, out_in_map=None) -> bool:
     """Whether a layer runs over pair segments: 16-bit features, a 3^3 or larger kernel, few rows
     and many channels (the regime in which the dense pass is bound by the weight slabs it streams
-    per row tile).  Measured on the levels of an 89,834-voxel scan: 8,045 rows 256 -> 256 32 vs
-    43 us, 384 -> 256 39 vs 57, 19,815 rows 128 -> 128 30 vs 36, 192 -> 128 33 vs 47, 3,105 rows
-    256 -> 256 22 vs 28; 8,045 rows 128 -> 128 (21 vs 20) stays with the dense pass."""
-    return bool(igemm_through_segments and kvol >= 27 and 0 < num_out_feats < 65536 and cout >= 128
-                and (cin * cout > 128 * 128 or num_out_feats >= 12000)
-                and _segments_supported(kvol, cin, cout, _dtype_code(x)))
+    per row tile) and a map with few pairs per row.  The cost of the pair form grows with the
+    number of pairs (every product row crosses memory twice), the dense pass keeps its sums in
+    registers: measured on the levels of an 89,834-voxel scan (24 % of the map entries are pairs):
+    8,045 rows 256 -> 256 32 vs 43 us, 384 -> 256 39 vs 57, 19,815 rows 128 -> 128 30 vs 36,
+    192 -> 128 33 vs 47, 3,105 rows 256 -> 256 22 vs 28 (8,045 rows 128 -> 128, 21 vs 20, stays
+    dense); on a detection backbone's 55,578-row level (61 %): 128 -> 128 134 vs 85.  The number of
+    pairs is not known on the host, so ``igemm_through_segments = True`` takes the pair form only
+    for maps marked by hint_sparse_map (build_kernel_map marks those over rows that thin out like
+    surfaces, see level_thinning); "always" takes it wherever a variant exists."""
+    mode = igemm_through_segments
+    if not mode or not (kvol >= 27 and 0 < num_out_feats < 65536 and cout >= 128
+                        and (cin * cout > 128 * 128 or num_out_feats >= 12000)
+                        and _segments_supported(kvol, cin, cout, _dtype_code(x))):
+        return False
+    if mode == "always":
+        return True
+    hit = _sparse_maps.get(id(out_in_map)) if out_in_map is not None else None
+    return hit is not None and hit() is out_in_map
 
 
 def conv_implicit_gemm_segments(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias=None,
@@ -1271,7 +1323,7 @@ def conv_implicit_gemm_segments(x, wp, kvol, cin, cout, out_in_map, num_out_feat
 
 def _implicit_gemm(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias=None, residual=None,
                    relu=False) -> torch.Tensor:
-    if _segments_pay(x, kvol, cin, cout, num_out_feats):
+    if _segments_pay(x, kvol, cin, cout, num_out_feats, out_in_map):
         return conv_implicit_gemm_segments(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias,
                                            residual, relu)
     y = torch.empty((num_out_feats, cout), dtype=x.dtype, device=x.device)

@@ -178,6 +178,11 @@ def build_kernel_map(_coords: torch.Tensor, input_node_num: int,
             backend.strided_lookahead(_coords)  # the strided chain that follows such rows, queued early
             out_coords = coords
             out_in_map = backend.kmap_sorted(coords, coords, kernel_size, stride, backend._subm_pad(kernel_size))
+            # rows that thinned out like a surface on their way here (at most 1 / 0.3 occupied
+            # cells per occupied block of the strided layer before) have few neighbours each
+            thinning = backend.level_thinning(_coords)
+            if thinning is not None and thinning >= 0.3:
+                backend.hint_sparse_map(out_in_map)
         else:
             host_max = None if new_range is None else tuple(x - 1 for x in new_range[1:])
             from torchsparse_amd.tensor import get_allow_negative_coordinates
