@@ -413,6 +413,79 @@ __global__ void grid_mark_kernel(const int4 *in_coords, int64_t total, Geom g, i
   }
 }
 
+// grid_mark_kernel for the strided-convolution rule (mode 0) with several candidates per
+// input, one thread per INPUT: the outputs along each axis (at most kMaxFanAxis) are worked out
+// once and the thread walks their combinations; candidates that share a bitmap word (neighbours
+// along z) are merged before the pre-checked atomic, and the block raises the maxima once per
+// input instead of once per candidate.  Marks exactly the bits grid_mark_kernel marks.
+constexpr int kMaxFanAxis = 4;
+
+__global__ __launch_bounds__(kBlock) void grid_mark_fan_kernel(
+    const int4 *in_coords, int64_t n_in, Geom g, int3 out_max_host, int has_host_max,
+    const int32_t *in_max_dev, uint32_t *bitmap, int64_t cap_words, int32_t *next_in_max,
+    int32_t *counters) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  const GridDims d = grid_dims(g, out_max_host, has_host_max, in_max_dev, cap_words);
+  if (!d.fits || d.used_words == 0) return;  // the same for every thread
+  int lo[3], hi[3];
+  output_ranges(g, out_max_host, has_host_max ? nullptr : in_max_dev, nullptr, 0, lo, hi);
+  int mb = 0, m0 = 0, m1 = 0, m2 = 0;
+  bool unpackable = false;
+  if (i < n_in) {
+    const int4 c = in_coords[i];
+    // an input the packed key cannot hold is missing from every table built from these rows
+    if (!coords_packable(c.x, c.y, c.z, c.w)) unpackable = true;
+    const int v[3] = {c.y, c.z, c.w};
+    int cnt[3] = {0, 0, 0};
+    int ov[3][kMaxFanAxis];
+#pragma unroll
+    for (int a = 0; a < 3; ++a) {
+      // o = (in + pad + digit - (ks-1)) / stride for the digits that make the division exact
+      int r = (g.ks[a] - 1 - v[a] - g.pad[a]) % g.stride[a];
+      if (r < 0) r += g.stride[a];
+#pragma unroll
+      for (int j = 0; j < kMaxFanAxis; ++j) {
+        const int digit = r + j * g.stride[a];
+        if (digit >= g.ks[a]) break;
+        const int o = (v[a] + g.pad[a] + digit - (g.ks[a] - 1)) / g.stride[a];  // exact
+        if (o >= lo[a] && o <= hi[a]) ov[a][cnt[a]++] = o;
+      }
+    }
+    if (c.x <= in_max_dev[0]) {
+      for (int i0 = 0; i0 < cnt[0]; ++i0) {
+        for (int i1 = 0; i1 < cnt[1]; ++i1) {
+          int word = -1;
+          uint32_t bits = 0;
+          for (int i2 = 0; i2 < cnt[2]; ++i2) {
+            const int o0 = ov[0][i0], o1 = ov[1][i1], o2 = ov[2][i2];
+            if (!coords_packable(c.x, o0, o1, o2)) {
+              unpackable = true;
+              continue;
+            }
+            const uint32_t cell = (((uint32_t)c.x * d.e[0] + o0) * d.e[1] + o1) * d.e[2] + o2;
+            const int w = (int)(cell >> 5);
+            if (w != word) {
+              // bits are only ever set: a stale read of set bits is still right, a stale read
+              // of clear bits only costs the atomic
+              if (word >= 0 && (bitmap[word] & bits) != bits) atomicOr(&bitmap[word], bits);
+              word = w;
+              bits = 0;
+            }
+            bits |= 1u << (cell & 31);
+            mb = max(mb, c.x);
+            m0 = max(m0, o0);
+            m1 = max(m1, o1);
+            m2 = max(m2, o2);
+          }
+          if (word >= 0 && (bitmap[word] & bits) != bits) atomicOr(&bitmap[word], bits);
+        }
+      }
+    }
+  }
+  if (unpackable) counters[3] = 1;
+  if (next_in_max) block_raise_max(mb, m0, m1, m2, next_in_max);
+}
+
 __device__ __forceinline__ int grid_thread_words(const uint32_t *bitmap, int64_t chunk, uint32_t *w);
 
 // The same marking for the NEXT level of a chain of equal strided convolutions: its inputs are
@@ -1430,6 +1503,11 @@ int grid_args(Geom *g, int *mode, int3 *hm, const int32_t ks[3], const int32_t s
 }
 }  // namespace
 
+static int64_t per_input_fan(const int32_t ks[3], const int32_t stride[3]) {
+  return (int64_t)((ks[0] + stride[0] - 1) / stride[0]) * ((ks[1] + stride[1] - 1) / stride[1]) *
+         ((ks[2] + stride[2] - 1) / stride[2]);
+}
+
 extern "C" int tsmi_downsample_grid_count(tsmi_stream_t s, const int32_t *in_coords, int64_t n_in,
                                           const int32_t ks[3], const int32_t stride[3],
                                           const int32_t pad[3], const int32_t out_max_host[3],
@@ -1445,18 +1523,20 @@ extern "C" int tsmi_downsample_grid_count(tsmi_stream_t s, const int32_t *in_coo
     return e;
   TSMI_REQUIRE(n_in >= 0 && (n_in == 0 || in_coords), "downsample_grid_count: bad coords");
   const int has_hm = out_max_host != nullptr;
-  const int64_t per_input = mode == 2 ? 1
-                                      : (int64_t)((ks[0] + stride[0] - 1) / stride[0]) *
-                                            ((ks[1] + stride[1] - 1) / stride[1]) *
-                                            ((ks[2] + stride[2] - 1) / stride[2]);
-  const int64_t total = n_in * per_input;
+  const int64_t total = n_in * (mode == 2 ? 1 : per_input_fan(ks, stride));
   TSMI_GRID_CHECK(total);
   hipStream_t st = (hipStream_t)s;
   const unsigned chunks = (unsigned)(bitmap_words / kGridChunkWords);
   if (clear_first)
     hipLaunchKernelGGL(grid_clear_kernel, grid_for(bitmap_words / 4), dim3(kBlock), 0, st, (uint4 *)bitmap,
                        bitmap_words, g, hm, has_hm, in_max_dev);
-  if (total > 0)
+  bool per_input = mode == 0 && per_input_fan(ks, stride) > 1 && !n_in_dev;
+  for (int a = 0; a < 3; ++a) per_input = per_input && (ks[a] + stride[a] - 1) / stride[a] <= kMaxFanAxis;
+  if (total > 0 && per_input)
+    hipLaunchKernelGGL(grid_mark_fan_kernel, grid_for(n_in), dim3(kBlock), 0, st, (const int4 *)in_coords,
+                       n_in, g, hm, has_hm, in_max_dev, (uint32_t *)bitmap, bitmap_words, next_in_max_dev,
+                       counters);
+  else if (total > 0)
     hipLaunchKernelGGL(grid_mark_kernel, grid_for(total), dim3(kBlock), 0, st, (const int4 *)in_coords,
                        total, g, hm, has_hm, in_max_dev, mode, (uint32_t *)bitmap, bitmap_words,
                        next_in_max_dev, counters, n_in_dev);
