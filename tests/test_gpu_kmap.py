@@ -479,10 +479,21 @@ def test_fused_submanifold_build_equals_the_separate_calls():
             np.testing.assert_array_equal(omap.cpu().numpy(), oracle.kmap_subm(coords.cpu().numpy(), t3(ks)))
 
 
-def test_chain_started_at_the_submanifold_build():
+@pytest.mark.parametrize("side", [True, False])
+def test_chain_started_at_the_submanifold_build(side):
     """The strided chain's first half queued when the submanifold map of the same rows is built
-    (what a U-Net's stem does): same coordinates and maps as without, a look-ahead nobody asks for
-    leaves no marks behind, and other rows or another geometry in between do not take it."""
+    (what a U-Net's stem does), on a second stream of the device or on the caller's: same
+    coordinates and maps as without, a look-ahead nobody asks for leaves no marks behind, and other
+    rows or another geometry in between do not take it."""
+    keep_side = backend.downsample_side_stream
+    backend.downsample_side_stream = side
+    try:
+        _chain_started_at_the_submanifold_build(side)
+    finally:
+        backend.downsample_side_stream = keep_side
+
+
+def _chain_started_at_the_submanifold_build(side):
     rng = np.random.default_rng(21)
     rows = lidar_like_coords(rng, 30000)
     rows = rows[np.lexsort((rows[:, 3], rows[:, 2], rows[:, 1], rows[:, 0]))]
@@ -510,6 +521,7 @@ def test_chain_started_at_the_submanifold_build():
             np.testing.assert_array_equal(km["out_in_map"].cpu().numpy(), m)
     state, = backend._stream_states.values()
     assert state.lookahead_hits == 2 and state.pending is None  # forwards three and four
+    assert (state.side is not None) == side
     # a forward that stops after the stem leaves a look-ahead behind; the next strided call of
     # other rows must not take it, and must find clean bitmaps
     F.build_kernel_map(coords, coords.shape[0], 3, 1, 1, mode="hashmap_on_the_fly")

@@ -647,9 +647,14 @@ def _strided_state(dev: torch.device) -> _StridedState:
 
 def release_scratch() -> None:
     """Drop the scratch bitmaps, the levels computed ahead and the chain history of every
-    stream (up to ~170 MB of device memory per stream that ran a large strided map)."""
+    stream (up to ~170 MB of device memory per stream that ran a large strided map), and the
+    buffers the convolutions of a stream share for partial sums and per-pair products (they
+    grow to the largest layer seen: K_vol * ceil128(N_out) * Cout elements for a layer over
+    pair segments)."""
     with _state_lock:
         _stream_states.clear()
+    with _scratch_lock:
+        _SCRATCH.clear()
 
 
 def _grid_layout(words0: int):
@@ -1235,28 +1240,31 @@ def pair_segments(out_in_map: torch.Tensor, n_rows: int) -> PairSegments:
         _check(_C.tsmi_pair_segments(stream, out_in_map.data_ptr(), n_rows, kvol, seg.seg_rows,
                                      pool.data_ptr() if kvol < 520 else None, seg.counts_ptr,
                                      seg.in_rows_ptr, seg.pos_ptr))
-    if len(_segments_of) >= 64:
-        for k in [k for k, v in _segments_of.items() if v[0]() is None]:
-            del _segments_of[k]
+    with _hint_lock:
         if len(_segments_of) >= 64:
-            _segments_of.clear()
-    _segments_of[id(out_in_map)] = (weakref.ref(out_in_map), out_in_map._version, out_in_map.data_ptr(),
-                                    stream, n_rows, seg)
+            for k in [k for k, v in _segments_of.items() if v[0]() is None]:
+                del _segments_of[k]
+            if len(_segments_of) >= 64:
+                _segments_of.clear()
+        _segments_of[id(out_in_map)] = (weakref.ref(out_in_map), out_in_map._version, out_in_map.data_ptr(),
+                                        stream, n_rows, seg)
     return seg
 
 
 _level_thinning = {}  # id(coords) -> (weak reference, rows kept per input row by the layer that made them)
 _sparse_maps = {}     # id(map) -> weak reference: maps over rows known to have few neighbours
+_hint_lock = threading.Lock()  # guards the two tables above and _segments_of
 
 
 def _note_level(out_coords: torch.Tensor, n_in: int) -> None:
     """``out_coords`` came out of a kernel size = stride, pad 0 layer over ``n_in`` rows."""
-    if len(_level_thinning) >= 256:
-        for key in [k for k, v in _level_thinning.items() if v[0]() is None]:
-            del _level_thinning[key]
+    with _hint_lock:
         if len(_level_thinning) >= 256:
-            _level_thinning.clear()
-    _level_thinning[id(out_coords)] = (weakref.ref(out_coords), out_coords.shape[0] / max(n_in, 1))
+            for key in [k for k, v in _level_thinning.items() if v[0]() is None]:
+                del _level_thinning[key]
+            if len(_level_thinning) >= 256:
+                _level_thinning.clear()
+        _level_thinning[id(out_coords)] = (weakref.ref(out_coords), out_coords.shape[0] / max(n_in, 1))
 
 
 def level_thinning(coords: torch.Tensor) -> Optional[float]:
@@ -1271,12 +1279,13 @@ def level_thinning(coords: torch.Tensor) -> Optional[float]:
 def hint_sparse_map(out_in_map: torch.Tensor) -> None:
     """Mark a kernel map as one over thin rows (few neighbours per row): the implicit-GEMM
     dataflow then runs its small, wide layers over pair segments."""
-    if len(_sparse_maps) >= 256:
-        for key in [k for k, v in _sparse_maps.items() if v() is None]:
-            del _sparse_maps[key]
+    with _hint_lock:
         if len(_sparse_maps) >= 256:
-            _sparse_maps.clear()
-    _sparse_maps[id(out_in_map)] = weakref.ref(out_in_map)
+            for key in [k for k, v in _sparse_maps.items() if v() is None]:
+                del _sparse_maps[key]
+            if len(_sparse_maps) >= 256:
+                _sparse_maps.clear()
+        _sparse_maps[id(out_in_map)] = weakref.ref(out_in_map)
 
 
 def _segments_pay(x, kvol, cin, cout, num_out_feats, out_in_map=None) -> bool:
