@@ -693,9 +693,12 @@ def main():
                                                      pmc_target=args.pmc_target)))
         return
 
-    ms_per_step = timed(model, args.steps, args.warmup)
+    # the secondary figures first: the clocks, the allocator and the library's own look-ahead
+    # state settle over the first few dozen forwards of a process (the headline loop measured
+    # first reads ~5 % higher than the same loop a moment later)
     ms_unfused = timed(unfused, max(args.steps // 2, 1), 2)
     ms_fresh = timed(model, args.steps, 2, fresh_coords=True)
+    ms_per_step = timed(model, args.steps, args.warmup)
 
     with torch.no_grad():
         inp = ts.SparseTensor(feats, coords)
