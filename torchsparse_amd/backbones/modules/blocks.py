@@ -22,14 +22,25 @@ def _conv_bn(cin: int, cout: int, kernel_size: _Size, act: bool, **conv_kwargs):
     return layers
 
 
-class SparseConvBlock(nn.Sequential):
+class _Chain(nn.Sequential):
+    """nn.Sequential that skips nn.Identity children (what nn.utils.fuse_inference leaves in
+    place of folded norms and activations) instead of calling them."""
+
+    def forward(self, x):
+        for m in self._modules.values():
+            if m.__class__ is not nn.Identity:
+                x = m(x)
+        return x
+
+
+class SparseConvBlock(_Chain):
     def __init__(self, in_channels: int, out_channels: int, kernel_size: _Size, stride: _Size = 1,
                  dilation: int = 1) -> None:
         super().__init__(*_conv_bn(in_channels, out_channels, kernel_size, True, stride=stride,
                                    dilation=dilation))
 
 
-class SparseConvTransposeBlock(nn.Sequential):
+class SparseConvTransposeBlock(_Chain):
     def __init__(self, in_channels: int, out_channels: int, kernel_size: _Size, stride: _Size = 1,
                  dilation: int = 1) -> None:
         super().__init__(*_conv_bn(in_channels, out_channels, kernel_size, True, stride=stride,
@@ -58,7 +69,11 @@ class SparseResBlock(nn.Module):
             # shortcut add + ReLU run in the epilogue of the block's last convolution
             shortcut = self.shortcut(x)
             y = x
-            for layer in list(self.main)[:-2]:
+            layers = self.__dict__.get("_fused_layers")
+            if layers is None:  # the convolutions of `main` (its folded norms are placeholders)
+                layers = self.__dict__["_fused_layers"] = tuple(
+                    m for m in list(self.main)[:-1] if not isinstance(m, nn.Identity))
+            for layer in layers[:-1]:
                 y = layer(y)
-            return self.main[-2](y, residual=shortcut.feats)
+            return layers[-1](y, residual=shortcut.feats)
         return self.relu(self.main(x) + self.shortcut(x))
