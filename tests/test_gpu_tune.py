@@ -16,9 +16,9 @@ def _net(spnn):
     return nn.Sequential(
         spnn.Conv3d(8, 16, 3), spnn.ReLU(True),
         spnn.Conv3d(16, 16, 3), spnn.ReLU(True),
-        spnn.Conv3d(16, 32, 2, stride=2), spnn.ReLU(True),
-        spnn.Conv3d(32, 32, 3), spnn.ReLU(True),
-        spnn.Conv3d(32, 16, 2, stride=2, transposed=True))
+        spnn.Conv3d(16, 128, 2, stride=2), spnn.ReLU(True),
+        spnn.Conv3d(128, 192, 3), spnn.ReLU(True),  # (wide enough for the pair-segment form)
+        spnn.Conv3d(192, 16, 2, stride=2, transposed=True))
 
 
 def _samples(ts, n_samples, seed=0):
@@ -49,7 +49,8 @@ def _oracle_net(model, spnn, feats, coords):
 
 
 def test_every_candidate_configuration_matches_the_oracle():
-    """Each configuration the tuner may time — unsorted, sorted with 1 to 4 mask splits,
+    """Each configuration the tuner may time — unsorted (as the library decides, and with the
+    pair-segment form of the wide layer forced on and off), sorted with 1 to 4 mask splits,
     fetch-on-demand, gather-scatter — set on every group at once, against the oracle."""
     import torchsparse_amd as ts
     from torchsparse_amd import nn as spnn
@@ -64,11 +65,15 @@ def test_every_candidate_configuration_matches_the_oracle():
     names = [name for name, _ in T._conv_modules(model)]
     flows = [F.Dataflow.ImplicitGEMM, F.Dataflow.FetchOnDemand, F.Dataflow.GatherScatter]
     cands = T._candidates(flows, tune_with_bwd=True)
-    assert len(cands) == 7
+    assert len(cands) == 9
+    from torchsparse_amd import backend
     for cand in cands:
         T._set_configs(model, names, cand)
+        backend._segments_of.clear()
         with torch.no_grad():
             got = model(ts.SparseTensor(x16.cuda(), probe.coords.cuda())).feats.float().cpu().numpy()
+        # the wide layer ran over pair segments exactly when the candidate forces that form
+        assert bool(backend._segments_of) == (cand.get("pair_segments") is True), cand
         assert rel_rms(got, want) < 2e-2, cand  # five fp16 layers deep: 1e-2 per layer does not compound past this
 
 

@@ -1164,14 +1164,14 @@ def _tile_counters(device, stream: int):
 
 def conv_forward_implicit_gemm_cuda(in_feats, kernel, out_in_map, num_out_feats, num_out_channels,
                                     allow_tf32=False, allow_fp16=True, bias=None, residual=None,
-                                    relu=False) -> torch.Tensor:
+                                    relu=False, segments=None) -> torch.Tensor:
     """convolution/convolution_forward_implicit_gemm_cuda.cu:1527-1986.  allow_tf32 /
     allow_fp16 are accepted and ignored: fp32 runs in true fp32, 16-bit types
     accumulate in fp32."""
     x, wp, (kvol, cin, cout) = _conv_common(in_feats, kernel)
     if cout != num_out_channels:
         raise ValueError("num_out_channels does not match the kernel")
-    return _implicit_gemm(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias, residual, relu)
+    return _implicit_gemm(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias, residual, relu, segments)
 
 
 # Small, wide layers of the implicit-GEMM dataflow run over pair segments (a per-offset
@@ -1288,7 +1288,7 @@ def hint_sparse_map(out_in_map: torch.Tensor) -> None:
         _sparse_maps[id(out_in_map)] = weakref.ref(out_in_map)
 
 
-def _segments_pay(x, kvol, cin, cout, num_out_feats, out_in_map=None) -> bool:
+def _segments_pay(x, kvol, cin, cout, num_out_feats, out_in_map=None, force=None) -> bool:
     """Whether a layer runs over pair segments: 16-bit features, a 3^3 or larger kernel, few rows
     and many channels (the regime in which the dense pass is bound by the weight slabs it streams
     per row tile) and a map with few pairs per row.  The cost of the pair form grows with the
@@ -1299,8 +1299,12 @@ def _segments_pay(x, kvol, cin, cout, num_out_feats, out_in_map=None) -> bool:
     dense); on a detection backbone's 55,578-row level (61 %): 128 -> 128 134 vs 85.  The number of
     pairs is not known on the host, so ``igemm_through_segments = True`` takes the pair form only
     for maps marked by hint_sparse_map (build_kernel_map marks those over rows that thin out like
-    surfaces, see level_thinning); "always" takes it wherever a variant exists."""
+    surfaces, see level_thinning); "always" takes it wherever a variant exists.  ``force`` (a
+    layer's conv_config "pair_segments": True / False) overrides the module-wide setting; the
+    row and channel limits hold either way."""
     mode = igemm_through_segments
+    if force is not None:  # a layer's own configuration (conv_config "pair_segments") decides
+        mode = "always" if force else False
     if not mode or not (kvol >= 27 and 0 < num_out_feats < 65536 and cout >= 128
                         and (cin * cout > 128 * 128 or num_out_feats >= 12000)
                         and _segments_supported(kvol, cin, cout, _dtype_code(x))):
@@ -1331,8 +1335,8 @@ def conv_implicit_gemm_segments(x, wp, kvol, cin, cout, out_in_map, num_out_feat
 
 
 def _implicit_gemm(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias=None, residual=None,
-                   relu=False) -> torch.Tensor:
-    if _segments_pay(x, kvol, cin, cout, num_out_feats, out_in_map):
+                   relu=False, segments=None) -> torch.Tensor:
+    if _segments_pay(x, kvol, cin, cout, num_out_feats, out_in_map, segments):
         return conv_implicit_gemm_segments(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias,
                                            residual, relu)
     y = torch.empty((num_out_feats, cout), dtype=x.dtype, device=x.device)

@@ -196,7 +196,7 @@ def conv3d_cached(input: SparseTensor, kernel: torch.Tensor, bias: Optional[torc
     if feats.shape[1] != cin:
         return None  # (conv3d raises the reference's error)
     out_feats = backend._implicit_gemm(feats, backend.pack_weights(kernel), kvol, cin, cout, omap, n_out,
-                                       bias, residual, activation == "relu")
+                                       bias, residual, activation == "relu", config.get("pair_segments"))
     output = SparseTensor._make(out_feats, out_coords, out_stride, out_range, caches)
     if out_stride not in caches.cmaps:
         caches.cmaps[out_stride] = (out_coords, out_range)

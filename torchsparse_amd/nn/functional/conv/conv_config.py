@@ -52,6 +52,9 @@ _DEFAULTS = (
     ("epsilon", 0.0),
     ("mm_thresh", 0),
     ("FOD_fusion", True),
+    # implicit GEMM over pair segments on small, wide layers: None = where the library knows the
+    # map to be thin, True = wherever the kernels have a variant, False = never (the tuner times both)
+    ("pair_segments", None),
 )
 
 _global_conv_config = None

@@ -40,7 +40,8 @@ class ImplicitGEMMConvolutionFuntion:
         if not config["ifsort"]:
             out = backend.conv_forward_implicit_gemm_cuda(
                 input, weight, kmap["out_in_map" + sfx], num_out_feats, weight.shape[-1],
-                backends.allow_tf32, backends.allow_fp16, bias=bias, residual=residual, relu=relu)
+                backends.allow_tf32, backends.allow_fp16, bias=bias, residual=residual, relu=relu,
+                segments=config.get("pair_segments"))
         else:
             out = backend.conv_forward_implicit_gemm_sorted_cuda(
                 input, weight, kmap["reorder_out_in_map" + sfx], kmap["reduced_sorted_mask" + sfx],

@@ -8,7 +8,9 @@ the fastest per group, writes the choice to ``save_dir/tune_tag`` and sets it on
 ``Conv3d`` modules.
 
 Candidates per dataflow:
-  ImplicitGEMM   unsorted, and sorted with 1 to 4 mask splits
+  ImplicitGEMM   unsorted (small wide layers over pair segments where the library knows the map
+                 to be thin; then the same with that form forced on and forced off), and sorted
+                 with 1 to 4 mask splits
   FetchOnDemand  one candidate (fusion does not change this implementation's kernels)
   GatherScatter  one candidate (epsilon / mm_thresh only steer grouping in the reference and
                  change neither results nor launches here, utils/tune.py:322-352 sweeps them)
@@ -34,7 +36,7 @@ from torchsparse_amd.utils import make_ntuple
 __all__ = ["tune"]
 
 _TUNED_KEYS = ("epsilon", "mm_thresh", "split_mask_num", "split_mask_num_bwd", "dataflow", "ifsort",
-               "FOD_fusion")
+               "FOD_fusion", "pair_segments")
 
 
 def _map_tensors(x, fn):
@@ -90,6 +92,11 @@ def _candidates(dataflow_range: List, tune_with_bwd: bool) -> List[Dict]:
     if F.Dataflow.ImplicitGEMM in dataflow_range:
         out.append(dict(dataflow=F.Dataflow.ImplicitGEMM, ifsort=False, split_mask_num=1,
                         split_mask_num_bwd=1))
+        # small, wide layers over pair segments, forced on and off (the default decides from what
+        # the library knows of the map; layers without a variant run the same either way)
+        for forced in (True, False):
+            out.append(dict(dataflow=F.Dataflow.ImplicitGEMM, ifsort=False, split_mask_num=1,
+                            split_mask_num_bwd=1, pair_segments=forced))
         for split in range(1, 5):
             out.append(dict(dataflow=F.Dataflow.ImplicitGEMM, ifsort=True, split_mask_num=split,
                             split_mask_num_bwd=split if tune_with_bwd else 1))
