@@ -461,3 +461,55 @@ def test_offset_split_sums_in_kernel_equal_second_launch(mods, cin, cout, dtype)
     assert int(counters.abs().sum().item()) == 0
     want = np.maximum(oracle.conv_implicit_gemm(_f32(x), _f32(w), omap.cpu().numpy(), n) + _f32(bias), 0)
     assert rel_rms(_f32(outs[1]), want) < TOL[dtype]
+
+
+def test_short_path_of_cached_map_layers_equals_conv3d(mods):
+    """Conv3d.forward takes a short host path (F.conv3d_cached) for inference calls whose map is
+    cached; it must return what F.conv3d returns, bit for bit (same kernels, same arguments), for
+    submanifold, strided, transposed and 1x1x1 layers with bias, residual and fused ReLU, and
+    must step aside whenever a gradient is wanted."""
+    ts, backend, spnn, F = mods
+    rng = np.random.default_rng(31)
+    coords = dev(random_coords(rng, 2500, (20, 20, 12)))
+    x = ts.SparseTensor(torch.randn(2500, 32, device="cuda", dtype=torch.float16), coords)
+    down = spnn.Conv3d(32, 64, 2, stride=2, bias=True).cuda().half().eval()
+    subm = spnn.Conv3d(64, 64, 3, bias=True).cuda().half().eval()
+    point = spnn.Conv3d(64, 48, 1, bias=True).cuda().half().eval()
+    up = spnn.Conv3d(48, 32, 2, stride=2, transposed=True).cuda().half().eval()
+    subm.activation = "relu"
+
+    def general(layer, inp, residual=None):
+        return F.conv3d(inp, weight=layer.kernel, kernel_size=layer.kernel_size, bias=layer.bias,
+                        stride=layer.stride, padding=layer.padding, dilation=layer.dilation,
+                        transposed=layer.transposed, generative=layer.generative, config=layer._config,
+                        training=False, residual=residual, activation=layer.activation)
+
+    with torch.no_grad():
+        mid = down(x)            # first call builds the map (general path) ...
+        res = torch.randn(mid.feats.shape[0], 64, device="cuda", dtype=torch.float16)
+        for layer, inp, r in ((down, x, None), (subm, mid, None), (subm, mid, res)):
+            general(layer, inp, r)  # ... and the maps are cached from here on
+            assert F.conv3d_cached(inp, layer.kernel, layer.bias, layer.kernel_size, layer.stride,
+                                   (1, 1, 1), layer.transposed, layer._config, r, layer.activation) is not None
+            a, b = layer(inp, residual=r) if r is not None else layer(inp), general(layer, inp, r)
+            assert torch.equal(a.feats, b.feats) and a.coords is b.coords and a.stride == b.stride
+            assert a._caches is inp._caches
+        p1, p2 = point(subm(mid)), general(point, general(subm, mid))
+        assert torch.equal(p1.feats, p2.feats) and p1.stride == (2, 2, 2)
+        general(up, p2)  # builds the transposed map
+        u1, u2 = up(p1), general(up, p2)
+        assert torch.equal(u1.feats, u2.feats) and u1.stride == (1, 1, 1) and u1.coords is x.coords
+    # a gradient is wanted: the short path declines and autograd gets its graph
+    xg = ts.SparseTensor(mid.feats.clone().requires_grad_(True), mid.coords, stride=mid.stride)
+    xg._caches = mid._caches
+    assert F.conv3d_cached(xg, subm.kernel, subm.bias, subm.kernel_size, subm.stride, (1, 1, 1), False,
+                           None, None, "relu") is None
+    out = subm(xg)
+    out.feats.float().sum().backward()
+    assert xg.feats.grad is not None and subm.kernel.grad is not None
+    # sorted mode and the other dataflows: not the short path's case
+    cfg = F.conv_config.get_default_conv_config()
+    cfg.dataflow = F.Dataflow.GatherScatter
+    with torch.no_grad():
+        assert F.conv3d_cached(mid, subm.kernel, subm.bias, subm.kernel_size, subm.stride, (1, 1, 1), False,
+                               cfg, None, "relu") is None
