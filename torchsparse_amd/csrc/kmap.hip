@@ -416,8 +416,9 @@ __global__ void grid_mark_kernel(const int4 *in_coords, int64_t total, Geom g, i
 // grid_mark_kernel for the strided-convolution rule (mode 0) with several candidates per
 // input, one thread per INPUT: the outputs along each axis (at most kMaxFanAxis) are worked out
 // once and the thread walks their combinations; candidates that share a bitmap word (neighbours
-// along z) are merged before the pre-checked atomic, and the block raises the maxima once per
-// input instead of once per candidate.  Marks exactly the bits grid_mark_kernel marks.
+// along z, of the thread itself and of the other lanes of its wavefront) are merged before the
+// pre-checked atomic, and the block raises the maxima once per input instead of once per
+// candidate.  Marks exactly the bits grid_mark_kernel marks.
 constexpr int kMaxFanAxis = 4;
 
 __global__ __launch_bounds__(kBlock) void grid_mark_fan_kernel(
@@ -431,13 +432,15 @@ __global__ __launch_bounds__(kBlock) void grid_mark_fan_kernel(
   output_ranges(g, out_max_host, has_host_max ? nullptr : in_max_dev, nullptr, 0, lo, hi);
   int mb = 0, m0 = 0, m1 = 0, m2 = 0;
   bool unpackable = false;
+  int4 c = make_int4(0, 0, 0, 0);
+  int cnt[3] = {0, 0, 0};
+  int ov[3][kMaxFanAxis];
+  bool live = false;
   if (i < n_in) {
-    const int4 c = in_coords[i];
+    c = in_coords[i];
     // an input the packed key cannot hold is missing from every table built from these rows
     if (!coords_packable(c.x, c.y, c.z, c.w)) unpackable = true;
     const int v[3] = {c.y, c.z, c.w};
-    int cnt[3] = {0, 0, 0};
-    int ov[3][kMaxFanAxis];
 #pragma unroll
     for (int a = 0; a < 3; ++a) {
       // o = (in + pad + digit - (ks-1)) / stride for the digits that make the division exact
@@ -451,35 +454,52 @@ __global__ __launch_bounds__(kBlock) void grid_mark_fan_kernel(
         if (o >= lo[a] && o <= hi[a]) ov[a][cnt[a]++] = o;
       }
     }
-    if (c.x <= in_max_dev[0]) {
-      for (int i0 = 0; i0 < cnt[0]; ++i0) {
-        for (int i1 = 0; i1 < cnt[1]; ++i1) {
-          int word = -1;
-          uint32_t bits = 0;
-          for (int i2 = 0; i2 < cnt[2]; ++i2) {
-            const int o0 = ov[0][i0], o1 = ov[1][i1], o2 = ov[2][i2];
-            if (!coords_packable(c.x, o0, o1, o2)) {
-              unpackable = true;
-              continue;
-            }
-            const uint32_t cell = (((uint32_t)c.x * d.e[0] + o0) * d.e[1] + o1) * d.e[2] + o2;
-            const int w = (int)(cell >> 5);
-            if (w != word) {
-              // bits are only ever set: a stale read of set bits is still right, a stale read
-              // of clear bits only costs the atomic
-              if (word >= 0 && (bitmap[word] & bits) != bits) atomicOr(&bitmap[word], bits);
-              word = w;
-              bits = 0;
-            }
-            bits |= 1u << (cell & 31);
-            mb = max(mb, c.x);
-            m0 = max(m0, o0);
-            m1 = max(m1, o1);
-            m2 = max(m2, o2);
+    live = c.x <= in_max_dev[0];
+  }
+  // Every lane walks the same (x, y) slots, so that the lanes of a wavefront - neighbours along
+  // z where the inputs are sorted - can merge the words they mark: lanes OR their bits into the
+  // last lane of each run of equal words and only that lane issues the pre-checked atomic.
+  const int lane = threadIdx.x & 63;
+  const int f0 = min(kMaxFanAxis, (g.ks[0] + g.stride[0] - 1) / g.stride[0]);
+  const int f1 = min(kMaxFanAxis, (g.ks[1] + g.stride[1] - 1) / g.stride[1]);
+  for (int i0 = 0; i0 < f0; ++i0) {
+    for (int i1 = 0; i1 < f1; ++i1) {
+      int word = -1;
+      uint32_t bits = 0;
+      if (live && i0 < cnt[0] && i1 < cnt[1]) {
+        for (int i2 = 0; i2 < cnt[2]; ++i2) {
+          const int o0 = ov[0][i0], o1 = ov[1][i1], o2 = ov[2][i2];
+          if (!coords_packable(c.x, o0, o1, o2)) {
+            unpackable = true;
+            continue;
           }
-          if (word >= 0 && (bitmap[word] & bits) != bits) atomicOr(&bitmap[word], bits);
+          const uint32_t cell = (((uint32_t)c.x * d.e[0] + o0) * d.e[1] + o1) * d.e[2] + o2;
+          const int w = (int)(cell >> 5);
+          if (w != word) {
+            // (the z run crosses into the next word: the earlier word goes out by itself)
+            // bits are only ever set: a stale read of set bits is still right, a stale read
+            // of clear bits only costs the atomic
+            if (word >= 0 && (bitmap[word] & bits) != bits) atomicOr(&bitmap[word], bits);
+            word = w;
+            bits = 0;
+          }
+          bits |= 1u << (cell & 31);
+          mb = max(mb, c.x);
+          m0 = max(m0, o0);
+          m1 = max(m1, o1);
+          m2 = max(m2, o2);
         }
       }
+      if (__ballot(word >= 0) == 0) continue;  // (the same for the whole wavefront)
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const int w = __shfl_up(word, off);
+        const uint32_t v = __shfl_up(bits, off);
+        if (lane >= off && w == word) bits |= v;
+      }
+      const int next = __shfl_down(word, 1);
+      if (word >= 0 && (lane == 63 || next != word) && (bitmap[word] & bits) != bits)
+        atomicOr(&bitmap[word], bits);
     }
   }
   if (unpackable) counters[3] = 1;
