@@ -153,9 +153,16 @@ __global__ void kmap_query_subm_kernel(TableView t, const int4 *coords, int64_t 
 
 __global__ void coords_max_kernel(const int4 *coords, int64_t n, int32_t *out_max) {
   __shared__ int smax[kBlock / 64][4];
-  int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  int4 c = i < n ? coords[i] : make_int4(0, 0, 0, 0);
-  int v[4] = {c.x, c.y, c.z, c.w};
+  // a bounded number of blocks strides over the rows: every block ends in atomics on the same
+  // four words, which the memory side works off one after the other
+  int v[4] = {0, 0, 0, 0};
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
+    const int4 c = coords[i];
+    v[0] = max(v[0], c.x);
+    v[1] = max(v[1], c.y);
+    v[2] = max(v[2], c.z);
+    v[3] = max(v[3], c.w);
+  }
 #pragma unroll
   for (int a = 0; a < 4; ++a) {
     int m = v[a];
@@ -167,7 +174,8 @@ __global__ void coords_max_kernel(const int4 *coords, int64_t n, int32_t *out_ma
   if (threadIdx.x < 4) {  // one atomic per block and column
     int m = max(max(smax[0][threadIdx.x], smax[1][threadIdx.x]),
                 max(smax[2][threadIdx.x], smax[3][threadIdx.x]));
-    if (m > 0) atomicMax(&out_max[threadIdx.x], m);
+    // the maxima only grow: a stale read that is already large enough spares the atomic
+    if (m > 0 && m > out_max[threadIdx.x]) atomicMax(&out_max[threadIdx.x], m);
   }
 }
 
@@ -1434,8 +1442,8 @@ extern "C" int tsmi_coords_max(tsmi_stream_t s, const int32_t *coords, int64_t n
                        (int64_t)4, 0);
   if (n > 0) {
     TSMI_GRID_CHECK(n);
-    hipLaunchKernelGGL(coords_max_kernel, grid_for(n), dim3(kBlock), 0, (hipStream_t)s,
-                       (const int4 *)coords, n, out_max);
+    hipLaunchKernelGGL(coords_max_kernel, dim3(std::min(grid_for(n).x, 512u)), dim3(kBlock), 0,
+                       (hipStream_t)s, (const int4 *)coords, n, out_max);
   }
   return check_launch("tsmi_coords_max");
 }
