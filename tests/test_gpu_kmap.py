@@ -539,6 +539,30 @@ def _chain_started_at_the_submanifold_build(side):
     m, c = oracle.kmap_downsample(rows, 3, 2, 1)
     np.testing.assert_array_equal(km["coords"].cpu().numpy(), c)
     np.testing.assert_array_equal(km["out_in_map"].cpu().numpy(), m)
+    # a network without that chain (submanifold maps of fresh rows, no strided call, or a strided
+    # call bounded by a spatial range) stops the queueing ahead after one miss
+    forward(coords)
+    assert state.root_chain is not None
+    F.build_kernel_map(coords, coords.shape[0], 3, 1, 1, mode="hashmap_on_the_fly")
+    assert state.pending is not None
+    fresh = dev(rows)
+    F.build_kernel_map(fresh, fresh.shape[0], 3, 1, 1, mode="hashmap_on_the_fly")
+    assert state.pending is None and state.root_chain is None
+    F.build_kernel_map(dev(rows), len(rows), 3, 1, 1, mode="hashmap_on_the_fly")
+    assert state.pending is None
+    forward(coords)
+    assert state.root_chain is not None  # learnt again from the strided call over the caller's rows
+    bounded = dev(rows)
+    F.build_kernel_map(bounded, len(rows), 3, 1, 1, mode="hashmap_on_the_fly")
+    extent = tuple(int(v) + 1 for v in rows[:, 1:].max(0))
+    km = F.build_kernel_map(bounded, len(rows), 2, 2, 0, mode="hashmap_on_the_fly",
+                            spatial_range=(int(rows[:, 0].max()) + 1,) + extent)
+    strided = (int(rows[:, 0].max()) + 1,) + tuple((e - 2) // 2 + 1 for e in extent)
+    m, c = oracle.kmap_downsample(rows, 2, 2, 0, spatial_range=strided)
+    np.testing.assert_array_equal(km["coords"].cpu().numpy(), c)
+    np.testing.assert_array_equal(km["out_in_map"].cpu().numpy(), m)
+    assert state.pending is None and state.root_chain is None
+    forward(coords)
     # and switched off, nothing is queued early
     backend.downsample_lookahead_at_subm = False
     try:

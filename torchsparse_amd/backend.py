@@ -490,8 +490,10 @@ def downsample_coords(coords: torch.Tensor, kernel_sizes, stride, padding, coord
                     tbl.insert_bxyz(ahead[0])
                     return ahead[0], tbl
                 return ahead
-            if chain is not None and _range_origin(coords) == "user":
-                state.root_chain = chain  # what strided_lookahead starts next time
+            if _range_origin(coords) == "user":
+                # what strided_lookahead starts next time (None: a call it cannot serve, e.g. one
+                # bounded by a spatial range - nothing is queued ahead for such rows any more)
+                state.root_chain = chain
             if (job is not None and job.coords is coords and job.geom == (ks, st, pd)
                     and job.coords_max_host is None and coords_max_host is None
                     and job.levels == 1 + ahead and state.pending_rsv == rsv_ratio):
@@ -910,7 +912,12 @@ def strided_lookahead(coords: torch.Tensor) -> None:
         if state.pending is not None:
             if state.pending.coords is coords:
                 return
-            state.pending = None  # never asked for; its marks are cleared by the next bitmap() call
+            # never asked for (its marks are cleared by the next bitmap() call): the network that
+            # runs now is not the one the chain was learnt from; queue nothing ahead until a
+            # strided call over a caller's own rows names a chain again
+            state.pending = None
+            state.root_chain = None
+            return
         ks, st, pd, rsv_ratio = root
         ahead = min(state.chain_len.get(root, 1) - 1, _GRID_LEVELS - 1)
         fan = _strided_fan(ks, st)
