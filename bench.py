@@ -325,6 +325,10 @@ def other_configs(ts, spnn, F, backend):
         "ms_maps_rebuilt": round(event_ms(lambda: run(ts.SparseTensor(feats, coords, spatial_range=spatial_range)),
                                           iters=10), 4),
         "ms_maps_cached": round(event_ms(lambda: run(warm), iters=10), 4)}
+    from torchsparse_amd.utils.graph import GraphedForward
+    runner = GraphedForward(net, warm)
+    out["detection_backbone"]["ms_maps_cached_graph_replay"] = round(event_ms(runner, iters=10), 4)
+    del runner
     del net, warm, feats, coords
     coords = torch.from_numpy(synthetic.sphere_shell_voxels(seed=3)).cuda()
     n = coords.shape[0]
@@ -704,6 +708,11 @@ def main():
         inp = ts.SparseTensor(feats, coords)
         records, outs = network_layers(model, inp)
         warm_ms = event_ms(lambda: model(inp), iters=10, warm=2)  # kernel maps cached
+        # the same forward (with the linear head) over cached maps, recorded as a HIP graph and replayed
+        from torchsparse_amd.utils.graph import GraphedForward
+        runner = GraphedForward(lambda t: head(model(t)[-1].feats), ts.SparseTensor(feats, coords))
+        graph_ms = event_ms(runner, iters=20, warm=3)
+        del runner
         roof = None if args.no_roofline else dominant_layer_roofline(ts, F, records, inp._caches)
         level_coords = {lvl: c[0].cpu().numpy() for lvl, c in inp._caches.cmaps.items()}
         layers = None if args.no_layers else layer_sweep(ts, spnn, F, backend, coords, n)
@@ -739,6 +748,7 @@ def main():
                                f"synthetic 64-beam scan seed 1, {n} voxels, 4 input channels, "
                                "kernel maps rebuilt every step",
                    "voxels": n, "warm_map_ms_per_step": round(warm_ms, 4),
+                   "warm_map_graph_replay_ms_per_step": round(graph_ms, 4),
                    "unfused_ms_per_step": round(ms_unfused, 4),
                    "fresh_coordinate_tensor_ms_per_step": round(ms_fresh, 4),
                    "conv_mode": F.get_conv_mode().value},

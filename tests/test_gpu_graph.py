@@ -1,0 +1,76 @@
+"""A forward over cached kernel maps recorded as a HIP graph (utils.graph.GraphedForward):
+every replay equals the eager forward of the same features, with eager work and
+synchronisations of the program's own between the replays, for the U-Net (pair-segment layers,
+offset splits with their shared scratch and counters, transposed layers, concatenations) and for
+the detection backbone (a spatial range, batches)."""
+import copy
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import random_coords
+
+pytestmark = pytest.mark.gpu
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def _stat_norms(model):
+    for m in model.modules():  # non-trivial norm statistics
+        if isinstance(m, torch.nn.BatchNorm1d):
+            m.running_mean.normal_(0, 0.3)
+            m.running_var.uniform_(0.5, 1.5)
+            m.weight.data.uniform_(0.5, 1.5)
+            m.bias.data.normal_(0, 0.2)
+
+
+def _check_replays(ts, model, coords, cin, spatial_range=None, pick=lambda out: out):
+    from torchsparse_amd.utils.graph import GraphedForward
+    n = coords.shape[0]
+    torch.manual_seed(5)
+    feats = [torch.randn(n, cin, device="cuda", dtype=torch.float16) for _ in range(4)]
+    x = ts.SparseTensor(feats[0], coords, spatial_range=spatial_range)
+    runner = GraphedForward(model, x)
+    for i in (1, 2, 3, 0, 2):
+        got = [t.clone() for t in pick(runner(feats[i]))]
+        # the program's own eager work between replays: a fresh tensor, maps rebuilt
+        with torch.no_grad():
+            want = pick(model(ts.SparseTensor(feats[i], coords.clone(), spatial_range=spatial_range)))
+        torch.cuda.synchronize()
+        assert len(got) == len(want) > 0
+        for g, w in zip(got, want):
+            assert g.shape == w.shape and torch.isfinite(w.float()).all()
+            assert torch.equal(g, w), (i, float((g.float() - w.float()).abs().max()))
+    with pytest.raises(ValueError):
+        runner(feats[0][:-1])
+
+
+def test_unet_replays_equal_eager_forwards():
+    import torchsparse_amd as ts
+    from torchsparse_amd.backbones import SparseResUNet42
+    from torchsparse_amd.nn.utils import fuse_inference
+    from torchsparse_amd.utils.synthetic import lidar_scan_voxels
+    torch.manual_seed(1)
+    coords = dev(lidar_scan_voxels(seed=1)[::3].copy())  # a thinned scan: deep levels over pair segments
+    model = SparseResUNet42(in_channels=4).cuda().eval()
+    _stat_norms(model)
+    model = fuse_inference(copy.deepcopy(model)).half()
+    _check_replays(ts, model, coords, 4, pick=lambda out: [o.feats for o in out])
+
+
+def test_detection_backbone_replays_equal_eager_forwards():
+    import torchsparse_amd as ts
+    from torchsparse_amd.backbones import VoxelResBackBone8x
+    from torchsparse_amd.nn.utils import fuse_inference
+    torch.manual_seed(2)
+    rng = np.random.default_rng(12)
+    coords = random_coords(rng, 9000, (41, 96, 96), batch=2)
+    coords = dev(coords[np.lexsort((coords[:, 3], coords[:, 2], coords[:, 1], coords[:, 0]))])
+    model = VoxelResBackBone8x(in_channels=5).cuda().eval()
+    _stat_norms(model)
+    model = fuse_inference(model).half()
+    _check_replays(ts, model, coords, 5, spatial_range=(2, 41, 96, 96),
+                   pick=lambda out: [v.feats for v in out.values()])
