@@ -267,6 +267,23 @@ int tsmi_downsample_grid_emit(tsmi_stream_t s, const int32_t ks[3], const int32_
                               int32_t *bitmap, int64_t bitmap_words, const int32_t *chunk_prefix, int64_t n_out, int64_t *keys,
                               int32_t *vals, int64_t cap, int32_t *out_coords, int32_t *counters);
 
+/* A whole chain of `levels` equal strided layers with one output per input (kernel size ==
+ * stride, no padding) queued by one call: tsmi_coords_max over coords, then per level
+ * tsmi_downsample_grid_count and tsmi_downsample_grid_emit with the count left on the device,
+ * each level marking from the rows of the one before.  scratch is the int32 buffer that holds
+ * every level's bitmap (at word bitmap_at[level], bitmap_words[level] words, all zero on entry
+ * and on completion) and chunk counts (at word chunks_at[level]); the three arrays are host
+ * int64[levels].  counters: zero-filled device int32[8 * levels], per level [n_out, -, grid too
+ * large, unpackable, maxima (b, x, y, z) of the level's INPUT rows]; rows: device
+ * int32[levels, n, 4], level i's first counters[8 i] rows are its output coordinates.  Nothing
+ * is read back.  No counterpart in the reference, which builds level after level with a
+ * read-back each (others/sparsemapping_cuda.cu:429-507, called once per strided layer). */
+int tsmi_downsample_chain_rows(tsmi_stream_t s, const int32_t *coords, int64_t n,
+                               const int32_t ks[3], const int32_t stride[3], const int32_t pad[3],
+                               int levels, int32_t *scratch, const int64_t *bitmap_at,
+                               const int64_t *bitmap_words, const int64_t *chunks_at,
+                               int32_t *counters, int32_t *rows);
+
 /* map_t[in,k] = out for every map[out,k] = in >= 0, out < n_rows; map_t
  * [n_rows_t, K_vol] is filled with -1 first.  Replaces
  * convert_transposed_out_in_map (others/query_cuda.cu:9-15,50-54) plus the

@@ -67,6 +67,7 @@ def _load():
         "tsmi_downsample_grid_count_next": [_vp, _I3, _I3, _I3, _vp, _vp, _i64, _vp, _vp, _i64, _vp, _vp, _vp],
         "tsmi_downsample_grid_emit": [_vp, _I3, _I3, _I3, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _vp,
                                       _i64, _vp, _vp],
+        "tsmi_downsample_chain_rows": [_vp, _vp, _i64, _I3, _I3, _I3, _i32, _vp, _vp, _vp, _vp, _vp, _vp],
         "tsmi_transpose_map": [_vp, _vp, _i64, _i32, _vp, _i64],
         "tsmi_derive_bitmask": [_vp, _vp, _i64, _i32, _i32, _i64, _vp],
         "tsmi_argsort_desc": [_vp, _vp, _vp, _vp, _i32, _i64, _vp, _i64],
@@ -159,7 +160,22 @@ def _need(t: torch.Tensor, dtype, name: str) -> torch.Tensor:
     return t if t.is_contiguous() else t.contiguous()
 
 
+@functools.lru_cache(maxsize=512)
+def _i3(t: Tuple[int, int, int]):
+    """int32[3] argument of a triple (one shared, read-only instance per value)."""
+    return _I3(*t)
+
+
+@functools.lru_cache(maxsize=512)
+def _triple_of_tuple(x: tuple) -> Tuple[int, int, int]:
+    x = tuple(int(v) for v in x)
+    assert len(x) == 3, x
+    return x
+
+
 def _triple(x) -> Tuple[int, int, int]:
+    if type(x) is tuple:
+        return _triple_of_tuple(x)
     if isinstance(x, torch.Tensor):
         x = x.view(-1).tolist()
     if isinstance(x, int):
@@ -255,8 +271,13 @@ def coords_ascending(coords: torch.Tensor) -> bool:
     return not (bits & 1)
 
 
+@functools.lru_cache(maxsize=256)
+def _sorted_supported(ks: Tuple[int, int, int]) -> bool:
+    return bool(_C.tsmi_kmap_sorted_supported(_I3(*ks)))
+
+
 def kmap_sorted_supported(kernel_size) -> bool:
-    return bool(kmap_through_sorted and _C.tsmi_kmap_sorted_supported(_I3(*_triple(kernel_size))))
+    return bool(kmap_through_sorted and _sorted_supported(_triple(kernel_size)))
 
 
 def kmap_sorted(in_coords: torch.Tensor, out_coords: torch.Tensor, kernel_size, stride, pad) -> torch.Tensor:
@@ -269,9 +290,14 @@ def kmap_sorted(in_coords: torch.Tensor, out_coords: torch.Tensor, kernel_size, 
     n_pad = make_divisible(n_out, 128)
     omap = torch.empty((n_pad, ks[0] * ks[1] * ks[2]), dtype=torch.int32, device=out_coords.device)
     samples = _sorted_samples(in_coords)
-    _check(_C.tsmi_kmap_sorted(_stream(), _ptr(in_coords), in_coords.shape[0], _ptr(out_coords), n_out,
-                               n_pad, _I3(*ks), _I3(*st), _I3(*pd), _ptr(samples), _ptr(omap)))
+    _check(_C.tsmi_kmap_sorted(_stream(), in_coords.data_ptr(), in_coords.shape[0], out_coords.data_ptr(),
+                               n_out, n_pad, _i3(ks), _i3(st), _i3(pd), _ptr(samples), omap.data_ptr()))
     return omap
+
+
+@functools.lru_cache(maxsize=1024)
+def _sample_elems(n: int) -> int:
+    return _C.tsmi_kmap_sorted_samples_elems(n)
 
 
 _samples_of = {}  # id(coords) -> (weak reference, version, address, stream, samples)
@@ -281,7 +307,7 @@ def _sorted_samples(coords: torch.Tensor) -> Optional[torch.Tensor]:
     """The search samples of a large input (None below 131073 rows), gathered once per
     coordinate tensor and stream: the submanifold and the strided map of a level share them."""
     n = coords.shape[0]
-    elems = _C.tsmi_kmap_sorted_samples_elems(n)
+    elems = _sample_elems(n)
     if elems == 0:
         return None
     stream = _stream()
@@ -700,16 +726,10 @@ def _grid_start(state, coords, ks, st, pd, coords_max_host, fan, ahead, early=Fa
     # per level 8 counters: [n_out, table overflow, grid too large, unpackable, max b, x, y, z of the INPUTS]
     ctr = torch.zeros(8 * levels, dtype=torch.int32, device=dev)
     s = _stream()
-    g = (_I3(*ks), _I3(*st), _I3(*pd))
+    g = (_i3(ks), _i3(st), _i3(pd))
     host_max = _I3(*[int(v) for v in coords_max_host]) if coords_max_host is not None else None
     buf_ptr, ctr_ptr = buf.data_ptr(), ctr.data_ptr()
     part = lambda level, what: _grid_part(buf_ptr, ctr_ptr, layout, levels, level, what)  # noqa: E731
-    _check(_C.tsmi_coords_max(s, _ptr(coords), n, part(0, "in_max"), 0))
-    state.grid_dirty = True  # marked bits stay behind unless the emit passes run
-    _check(_C.tsmi_downsample_grid_count(s, _ptr(coords), n, *g, host_max, part(0, "in_max"),
-                                         part(0, "bitmap"), layout[0][1], 0,
-                                         part(0, "chunks"), part(0, "counters"),
-                                         part(1, "in_max"), None))
     # One output per input (kernel size == stride, no padding: a level never has more rows than
     # the one before): every level's rows are emitted at once into a buffer of n rows while
     # their count is still on the device, and the next level marks from those rows.  Nothing is
@@ -719,22 +739,17 @@ def _grid_start(state, coords, ks, st, pd, coords_max_host, fan, ahead, early=Fa
     rows = None
     if (levels > 1 and fan == 1 and ks == st and pd == (0, 0, 0) and coords_max_host is None
             and downsample_emit_before_readback):
-        rows = []
-        src = coords
-        for level in range(levels):
-            if level > 0:
-                _check(_C.tsmi_downsample_grid_count(
-                    s, _ptr(src), n, *g, None, part(level, "in_max"), part(level, "bitmap"),
-                    layout[level][1], 0, part(level, "chunks"), part(level, "counters"),
-                    part(level + 1, "in_max"), part(level - 1, "counters")))
-            out = torch.empty((n, 4), dtype=torch.int32, device=dev)
-            _check(_C.tsmi_downsample_grid_emit(
-                s, *g, None, part(level, "in_max"), None, part(level, "bitmap"),
-                layout[level][1], part(level, "chunks"), -n, None, None, 0, _ptr(out),
-                part(level, "counters")))
-            rows.append(out)
-            src = out
+        rows = torch.empty((levels, n, 4), dtype=torch.int32, device=dev)  # level i: rows[i, :n_out_i]
+        state.grid_dirty = True
+        _check(_C.tsmi_downsample_chain_rows(s, _ptr(coords), n, *g, levels, buf_ptr, *_layout_arrays(layout),
+                                             ctr_ptr, rows.data_ptr()))
     else:
+        _check(_C.tsmi_coords_max(s, _ptr(coords), n, part(0, "in_max"), 0))
+        state.grid_dirty = True  # marked bits stay behind unless the emit passes run
+        _check(_C.tsmi_downsample_grid_count(s, _ptr(coords), n, *g, host_max, part(0, "in_max"),
+                                             part(0, "bitmap"), layout[0][1], 0,
+                                             part(0, "chunks"), part(0, "counters"),
+                                             part(1, "in_max"), None))
         for level in range(1, levels):
             _check(_C.tsmi_downsample_grid_count_next(
                 s, *g, part(level - 1, "in_max"), part(level - 1, "bitmap"), layout[level - 1][1],
@@ -763,6 +778,22 @@ def _grid_start(state, coords, ks, st, pd, coords_max_host, fan, ahead, early=Fa
     return job
 
 
+_LAYOUT_ARRAYS = {}
+
+
+def _layout_arrays(layout):
+    """(bitmap offsets, bitmap words, chunk-count offsets) of a scratch layout as int64 arrays."""
+    key = tuple(layout)
+    hit = _LAYOUT_ARRAYS.get(key)
+    if hit is None:
+        if len(_LAYOUT_ARRAYS) >= 64:
+            _LAYOUT_ARRAYS.clear()
+        arr = ctypes.c_int64 * len(layout)
+        hit = _LAYOUT_ARRAYS[key] = (arr(*[v[0] for v in layout]), arr(*[v[1] for v in layout]),
+                                     arr(*[v[2] for v in layout]))
+    return hit
+
+
 def _grid_part(buf_ptr, ctr_ptr, layout, levels, level, what):
     """Address of one part of the bitmap scratch (int32 words at ``buf_ptr``) or of the counters
     (8 int32 per level at ``ctr_ptr``): plain integers, no tensor views (a view costs more
@@ -789,7 +820,7 @@ def _grid_finish(state, job: _GridJob, rsv_ratio, cap, want_table):
     buf = state.grid_buf
     layout, _ = _grid_layout(state.grid_words)
     s = job.stream
-    g = (_I3(*ks), _I3(*st), _I3(*pd))
+    g = (_i3(ks), _i3(st), _i3(pd))
     host_max = _I3(*[int(v) for v in job.coords_max_host]) if job.coords_max_host is not None else None
     buf_ptr, ctr_ptr = buf.data_ptr(), ctr.data_ptr()
     part = lambda level, what: _grid_part(buf_ptr, ctr_ptr, layout, levels, level, what)  # noqa: E731
@@ -809,7 +840,7 @@ def _grid_finish(state, job: _GridJob, rsv_ratio, cap, want_table):
     def emit(level, n_in, capacity):
         n_out = host[8 * level]
         if job.rows is not None:  # emitted before the read-back: the level is a view of its buffer
-            out = job.rows[level][:n_out]
+            out = job.rows[level, :n_out]
             tbl = None
             if want_table:
                 _mark_range_ok(out, ascending=True)  # (known: the insert below does not read a flag back)
@@ -902,12 +933,12 @@ def strided_lookahead(coords: torch.Tensor) -> None:
     followed such rows last time on this stream, if any."""
     if not (downsample_lookahead_at_subm and downsample_through_grid and downsample_chain_ahead):
         return
-    if coords.shape[0] == 0:
+    if coords.shape[0] == 0 or _range_origin(coords) != "user":  # (most calls: a deeper level's rows)
         return
     with _state_lock:
         state = _strided_state(coords.device)
         root = state.root_chain  # geometry of the last chain that started from rows like these
-        if root is None or _range_origin(coords) != "user":
+        if root is None:
             return
         if state.pending is not None:
             if state.pending.coords is coords:
@@ -935,8 +966,8 @@ def strided_lookahead(coords: torch.Tensor) -> None:
                 state.side = torch.cuda.Stream(device=coords.device)
             with torch.cuda.stream(state.side):
                 job = _grid_start(state, coords, ks, st, pd, None, fan, ahead, early=True)
-            for rows in job.rows or ():
-                rows.record_stream(main)  # allocated on the side stream, read and freed on the caller's
+            if job.rows is not None:
+                job.rows.record_stream(main)  # allocated on the side stream, read and freed on the caller's
         else:
             job = _grid_start(state, coords, ks, st, pd, None, fan, ahead, early=True)
         state.pending = job

@@ -1660,6 +1660,38 @@ extern "C" int tsmi_downsample_grid_emit(tsmi_stream_t s, const int32_t ks[3], c
   return check_launch("tsmi_downsample_grid_emit");
 }
 
+extern "C" int tsmi_downsample_chain_rows(tsmi_stream_t s, const int32_t *coords, int64_t n,
+                                          const int32_t ks[3], const int32_t stride[3],
+                                          const int32_t pad[3], int levels, int32_t *scratch,
+                                          const int64_t *bitmap_at, const int64_t *bitmap_words,
+                                          const int64_t *chunks_at, int32_t *counters, int32_t *rows) {
+  TSMI_REQUIRE(levels >= 1 && levels <= 8 && n > 0 && coords && scratch && bitmap_at && bitmap_words &&
+                   chunks_at && counters && rows,
+               "downsample_chain_rows: bad arguments");
+  for (int a = 0; a < 3; ++a)
+    TSMI_REQUIRE(ks[a] == stride[a] && pad[a] == 0 && ks[a] >= 1,
+                 "downsample_chain_rows: one output per input needs kernel size == stride and no padding");
+  // counters: 8 per level, [4..8) of a level = the maxima of its INPUT rows
+  if (int e = tsmi_coords_max(s, coords, n, counters + 4, 0)) return e;
+  const int32_t *src = coords;
+  for (int level = 0; level < levels; ++level) {
+    int32_t *ctr = counters + 8 * level;
+    int32_t *bitmap = scratch + bitmap_at[level];
+    int32_t *chunks = scratch + chunks_at[level];
+    int32_t *next_max = level + 1 < levels ? ctr + 8 + 4 : nullptr;
+    if (int e = tsmi_downsample_grid_count(s, src, n, ks, stride, pad, nullptr, ctr + 4, bitmap,
+                                           bitmap_words[level], 0, chunks, ctr, next_max,
+                                           level > 0 ? ctr - 8 : nullptr))
+      return e;
+    int32_t *out = rows + (int64_t)level * n * 4;
+    if (int e = tsmi_downsample_grid_emit(s, ks, stride, pad, nullptr, ctr + 4, nullptr, bitmap,
+                                          bitmap_words[level], chunks, -n, nullptr, nullptr, 0, out, ctr))
+      return e;
+    src = out;
+  }
+  return TSMI_OK;
+}
+
 extern "C" int tsmi_transpose_map(tsmi_stream_t s, const int32_t *map, int64_t n_rows, int kvol,
                                   int32_t *map_t, int64_t n_rows_t) {
   TSMI_REQUIRE(kvol >= 1 && n_rows >= 0 && n_rows_t >= 0, "transpose_map: bad sizes");
