@@ -7,6 +7,7 @@ from typing import Dict
 from torch import nn
 
 from .. import nn as spnn
+from ..nn.utils.fuse import call_module
 from ..tensor import SparseTensor
 
 __all__ = ["SparseBasicBlock", "VoxelResBackBone8x"]
@@ -27,7 +28,8 @@ class SparseBasicBlock(nn.Module):
         if getattr(self, "_fused_tail", False):
             # after nn.utils.fuse_inference(): norms folded into the convolutions, ReLU and
             # the shortcut add in their epilogues
-            return self.conv2(self.conv1(x), residual=x.feats)
+            mods = self._modules
+            return call_module(mods["conv2"], call_module(mods["conv1"], x), residual=x.feats)
         out = self.bn2(self.conv2(self.relu(self.bn1(self.conv1(x)))))
         return self.relu(out + x)
 

@@ -8,6 +8,7 @@ import numpy as np
 from torch import nn
 
 from ... import nn as spnn
+from ...nn.utils.fuse import call_module
 from ...tensor import SparseTensor
 
 __all__ = ["SparseConvBlock", "SparseConvTransposeBlock", "SparseResBlock"]
@@ -29,7 +30,7 @@ class _Chain(nn.Sequential):
     def forward(self, x):
         for m in self._modules.values():
             if m.__class__ is not nn.Identity:
-                x = m(x)
+                x = call_module(m, x)
         return x
 
 
@@ -67,13 +68,14 @@ class SparseResBlock(nn.Module):
         if getattr(self, "_fused_tail", False):
             # after nn.utils.fuse_inference(): norms are folded into the convolutions and the
             # shortcut add + ReLU run in the epilogue of the block's last convolution
-            shortcut = self.shortcut(x)
-            y = x
             layers = self.__dict__.get("_fused_layers")
             if layers is None:  # the convolutions of `main` (its folded norms are placeholders)
                 layers = self.__dict__["_fused_layers"] = tuple(
                     m for m in list(self.main)[:-1] if not isinstance(m, nn.Identity))
+            shortcut = self._modules["shortcut"]
+            residual = x.feats if shortcut.__class__ is nn.Identity else call_module(shortcut, x).feats
+            y = x
             for layer in layers[:-1]:
-                y = layer(y)
-            return layers[-1](y, residual=shortcut.feats)
+                y = call_module(layer, y)
+            return call_module(layers[-1], y, residual=residual)
         return self.relu(self.main(x) + self.shortcut(x))

@@ -12,8 +12,21 @@ to the parameter dtype.
 """
 import torch
 from torch import nn
+from torch.nn.modules import module as _torch_module
 
-__all__ = ["fuse_inference"]
+__all__ = ["fuse_inference", "call_module"]
+
+
+def call_module(m: nn.Module, *args, **kwargs):
+    """``m(*args, **kwargs)`` without the two Python frames of nn.Module.__call__ when no hook
+    of any kind is registered (the test torch's own call path makes before it calls ``forward``
+    directly); with hooks, the ordinary call.  ~100 module calls per forward of a 42-layer U-Net
+    in inference form, 0.6 us each."""
+    if (m._forward_hooks or m._forward_pre_hooks or m._backward_hooks or m._backward_pre_hooks
+            or _torch_module._global_forward_hooks or _torch_module._global_forward_pre_hooks
+            or _torch_module._global_backward_hooks or _torch_module._global_backward_pre_hooks):
+        return m(*args, **kwargs)
+    return m.forward(*args, **kwargs)
 
 
 def _fold(conv, bn) -> None:
@@ -56,14 +69,14 @@ class FoldedSequential(nn.Sequential):
     def forward(self, x):
         for m in self._modules.values():
             if m.__class__ is not nn.Identity:
-                x = m(x)
+                x = call_module(m, x)
         return x
 
 
 def _skip_identities(seq: nn.Sequential) -> None:
-    """Plain nn.Sequential containers with placeholders become FoldedSequential (same children,
+    """Plain nn.Sequential containers of a fused model become FoldedSequential (same children,
     same names; copies and pickles like any module).  Subclasses keep their class."""
-    if type(seq) is nn.Sequential and any(isinstance(m, nn.Identity) for m in seq):
+    if type(seq) is nn.Sequential:
         seq.__class__ = FoldedSequential
 
 
