@@ -272,6 +272,9 @@ def test_minkunet_forward_on_the_scan(mods, scan):
     state, = backend._stream_states.values()
     assert state.ahead_hits == 6, state.ahead_hits  # per forward one strided call computed, three answered ahead
     assert state.lookahead_hits == 1 and state.pending is None  # bench.py's steady state
+    # ... and builds the four strided maps and the submanifold maps of levels 2 - 16 on the second
+    # stream as soon as the row counts are known (the maps compared below are those)
+    assert state.maps_ahead_hits == 8, state.maps_ahead_hits
 
     # --- the nine kernel maps and the coordinate levels, bit-exact
     caches = inp._caches

@@ -522,6 +522,10 @@ def _chain_started_at_the_submanifold_build(side):
     state, = backend._stream_states.values()
     assert state.lookahead_hits == 2 and state.pending is None  # forwards three and four
     assert (state.side is not None) == side
+    # the maps over the chain's levels (here the strided ones) that a forward asked for are queued
+    # on the second stream by the next forward that emits its rows there: forwards three and four
+    assert state.maps_ahead_hits == (6 if side else 0)
+    assert [r[:2] for r in state.map_plan if r[:2] != (0, 0)] == [(0, 1), (1, 2), (2, 3)]
     # a forward that stops after the stem leaves a look-ahead behind; the next strided call of
     # other rows must not take it, and must find clean bitmaps
     F.build_kernel_map(coords, coords.shape[0], 3, 1, 1, mode="hashmap_on_the_fly")

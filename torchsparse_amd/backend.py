@@ -286,9 +286,103 @@ def kmap_sorted(in_coords: torch.Tensor, out_coords: torch.Tensor, kernel_size, 
     in_coords = _need(in_coords, torch.int32, "coords")
     out_coords = _need(out_coords, torch.int32, "coords")
     ks, st, pd = _triple(kernel_size), _triple(stride), _triple(pad)
+    if kmap_queue_ahead:
+        ahead = _map_queued_ahead(in_coords, out_coords, ks, st, pd)
+        if ahead is not None:
+            return ahead
+    return _kmap_sorted_launch(in_coords, out_coords, ks, st, pd)
+
+
+# The maps a network builds over the levels of its strided chain (the submanifold map of every
+# level, the strided map to the next) depend on nothing but those levels' rows, which exist
+# - on the chain's second stream - long before the layers that ask for the maps are reached.
+# Once a forward has asked for such maps, the next forward queues the same builds on that
+# stream as soon as the row counts are on the host, beside the convolutions of the levels
+# above; the caller's stream waits once, for the end of that queue, when it takes the first
+# of them.  Maps queued and never asked for cost their kernels.
+kmap_queue_ahead = True
+
+
+def _map_queued_ahead(in_coords, out_coords, ks, st, pd) -> Optional[torch.Tensor]:
+    """The map of kmap_sorted(in_coords, out_coords, ...) if it was queued ahead on the second
+    stream; notes the request when both operands are levels of the chain in flight."""
+    dev = in_coords.device
+    with _state_lock:
+        state = _stream_states.get((dev.index if dev.index is not None else _cur_device(), _stream()))
+        if state is None or not state.level_index:
+            return None
+        a, b = state.level_index.get(id(in_coords)), state.level_index.get(id(out_coords))
+        if a is None or b is None or a[0]() is not in_coords or b[0]() is not out_coords:
+            return None
+        request = (a[1], b[1], ks, st, pd)
+        if request not in state.map_plan_seen:
+            state.map_plan_seen.append(request)
+        hit = state.maps_ahead.pop((id(in_coords), id(out_coords), ks, st, pd), None)
+        if (hit is None or hit[0]() is not in_coords or hit[1]() is not out_coords
+                or hit[3] != (in_coords._version, out_coords._version)):
+            return None
+        main = state.maps_main  # the caller's stream (this state belongs to it)
+        if state.maps_event is not None:
+            # usually the second stream is long done: then nothing has to wait on the device (a
+            # wait on a pending event costs the host 25 us, the query 2); later takers on this
+            # stream are ordered behind the wait
+            if not state.maps_event.query():
+                main.wait_event(state.maps_event)
+            state.maps_event = None
+        state.maps_ahead_hits += 1
+        return hit[2]
+
+
+def _queue_maps_ahead(state, chain_rows, on_side: bool) -> None:
+    """Called when the rows of a chain's levels (``chain_rows[0]``: its root) have become known
+    on the host: the requests of the forward before become this forward's plan, and - when the
+    rows were emitted on the second stream - the planned maps are queued there.  Runs with
+    _state_lock held, the caller's stream current."""
+    state.level_index = {id(t): (weakref.ref(t), i) for i, t in enumerate(chain_rows)}
+    plan, state.map_plan_seen = tuple(state.map_plan_seen), []
+    state.map_plan = plan
+    state.maps_ahead = {}
+    state.maps_event = None
+    if not (kmap_queue_ahead and on_side and plan and state.side is not None and kmap_through_sorted):
+        return
+    todo, rows_of = [], {}  # maps of one kernel volume share an allocation: one hand-over between the streams each
+    for i, o, ks, st, pd in plan:
+        if max(i, o) >= len(chain_rows) or max(i, o) == 0:  # (the root's own map is asked for before this point)
+            continue
+        a, b = chain_rows[i], chain_rows[o]
+        if a.shape[0] == 0 or b.shape[0] == 0:
+            continue
+        kvol = ks[0] * ks[1] * ks[2]
+        first = rows_of.get(kvol, 0)
+        rows_of[kvol] = first + make_divisible(b.shape[0], 128)
+        todo.append((a, b, ks, st, pd, kvol, first))
+    if not todo:
+        return
+    dev = chain_rows[0].device
+    main = state.maps_main = torch.cuda.current_stream(dev)
+    torch.cuda.set_stream(state.side)  # (the context manager costs 6 us, two switches 0.8)
+    try:
+        buffers = {kvol: torch.empty((rows, kvol), dtype=torch.int32, device=dev) for kvol, rows in rows_of.items()}
+        for a, b, ks, st, pd, kvol, first in todo:
+            omap = buffers[kvol][first:first + make_divisible(b.shape[0], 128)]
+            _kmap_sorted_launch(a, b, ks, st, pd, omap)
+            state.maps_ahead[(id(a), id(b), ks, st, pd)] = (weakref.ref(a), weakref.ref(b), omap,
+                                                            (a._version, b._version))
+        state.maps_event = torch.cuda.Event()
+        state.maps_event.record()
+    finally:
+        torch.cuda.set_stream(main)
+    for buf in buffers.values():
+        buf.record_stream(main)  # allocated on the second stream, read and freed on the caller's
+
+
+def _kmap_sorted_launch(in_coords, out_coords, ks, st, pd, omap=None) -> torch.Tensor:
+    """The launch of kmap_sorted on the current stream (operands checked by the caller), into
+    ``omap`` (int32 [ceil128(N_out), K_vol]) when given."""
     n_out = out_coords.shape[0]
     n_pad = make_divisible(n_out, 128)
-    omap = torch.empty((n_pad, ks[0] * ks[1] * ks[2]), dtype=torch.int32, device=out_coords.device)
+    if omap is None:
+        omap = torch.empty((n_pad, ks[0] * ks[1] * ks[2]), dtype=torch.int32, device=out_coords.device)
     samples = _sorted_samples(in_coords)
     _check(_C.tsmi_kmap_sorted(_stream(), in_coords.data_ptr(), in_coords.shape[0], out_coords.data_ptr(),
                                n_out, n_pad, _i3(ks), _i3(st), _i3(pd), _ptr(samples), omap.data_ptr()))
@@ -601,7 +695,8 @@ class _StridedState:
     stream (or device) get a state of their own and never see these tensors."""
     __slots__ = ("grid_buf", "grid_words", "grid_dirty", "chain_geom", "chain_last", "chain_count",
                  "chain_len", "ahead", "ahead_hits", "host_counters", "pending", "pending_rsv", "root_chain",
-                 "lookahead_hits", "side", "grid_event", "grid_old")
+                 "lookahead_hits", "side", "grid_event", "grid_old", "level_index", "map_plan",
+                 "map_plan_seen", "maps_ahead", "maps_event", "maps_ahead_hits", "maps_main")
 
     def __init__(self):
         self.grid_buf = None      # int32 scratch: bitmaps and chunk counts of every level
@@ -621,6 +716,13 @@ class _StridedState:
         self.side = None          # second stream of the device, for chains queued ahead of their use
         self.grid_event = None    # end of the last work queued on the bitmap scratch, on either stream
         self.grid_old = None      # the scratch before it last grew (kept until the next growth)
+        self.level_index = {}     # id(rows) -> (weak reference, position in the chain in flight; 0: its root)
+        self.map_plan = ()        # sorted-map builds the last forward asked for over its chain's levels
+        self.map_plan_seen = []   # ... the forward in flight has asked for so far
+        self.maps_ahead = {}      # (id(in), id(out), ks, st, pd) -> (refs, map) queued on the side stream
+        self.maps_event = None    # end of that queue; None once the caller's stream has waited for it
+        self.maps_ahead_hits = 0  # maps answered from `maps_ahead` (diagnostic)
+        self.maps_main = None     # the caller's stream object at the time of that queue
 
     def chain_step(self, coords, geom):
         """Book-keeping of chains of equal strided calls (each on the previous one's outputs).
@@ -872,6 +974,7 @@ def _grid_finish(state, job: _GridJob, rsv_ratio, cap, want_table):
     if thin:
         _note_level(first[0], n)
     prev = first[0]
+    chain_rows = [coords, prev]
     clean = True
     for level in range(1, levels):
         if prev.shape[0] == 0:
@@ -885,6 +988,7 @@ def _grid_finish(state, job: _GridJob, rsv_ratio, cap, want_table):
             clean = False  # this level's marks (and the later ones') are still in the bitmaps
             break
         state.ahead[id(prev)] = (weakref.ref(prev), (ks, st, pd, rsv_ratio), nxt[0], nxt[1])
+        chain_rows.append(nxt[0])
         if thin:
             _note_level(nxt[0], n_in)
         # the later levels are not flagged on the device; their inputs' maxima are on the host
@@ -894,6 +998,9 @@ def _grid_finish(state, job: _GridJob, rsv_ratio, cap, want_table):
         prev = nxt[0]
     # rows emitted before the read-back cleared every bitmap they read, asked for or not
     state.grid_dirty = (not clean) and job.rows is None
+    if levels > 1:
+        _queue_maps_ahead(state, chain_rows, job.rows is not None and state.side is not None
+                          and job.stream == state.side.cuda_stream)
     if state.side is not None and job.rows is None:  # emit passes ran on this stream just now
         state.grid_event = torch.cuda.Event()
         state.grid_event.record()
