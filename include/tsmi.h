@@ -139,6 +139,11 @@ int tsmi_kmap_sorted(tsmi_stream_t s, const int32_t *in_coords, int64_t n_in,
                      const int32_t *out_coords, int64_t n_out, int64_t n_out_pad,
                      const int32_t ks[3], const int32_t stride[3], const int32_t pad[3],
                      const int64_t *samples, int32_t *out_in_map);
+/* `count` calls of tsmi_kmap_sorted queued by one call (a network's maps over the levels of a
+ * strided chain, built ahead of their use).  args: host int64[16 * count], per map
+ * [in_coords, n_in, out_coords, n_out, n_out_pad, samples (0: none), out_in_map, ks[3],
+ * stride[3], pad[3]] with the pointers as integers.  No counterpart in the reference. */
+int tsmi_kmap_sorted_batch(tsmi_stream_t s, int count, const int64_t *args);
 /* Optional for tsmi_kmap_sorted, and only for inputs of more than 131072 rows (smaller ones
  * need none: tsmi_kmap_sorted_samples_elems returns 0): the keys every block of that kernel
  * searches before it stages its segment, gathered once per INPUT into

@@ -58,6 +58,7 @@ def _load():
         "tsmi_kmap_query": [_vp, _vp, _vp, _i64, _vp, _i64, _i64, _I3, _I3, _I3, _vp],
         "tsmi_kmap_query_subm": [_vp, _vp, _vp, _i64, _vp, _i64, _i64, _I3, _vp],
         "tsmi_coords_max": [_vp, _vp, _i64, _vp, _i32],
+        "tsmi_kmap_sorted_batch": [_vp, _i32, _vp],
         "tsmi_downsample_candidates": [_vp, _vp, _i64, _I3, _I3, _I3, _vp, _vp, _vp, _i32, _vp, _i64, _vp],
         "tsmi_hashtable_compact_keys": [_vp, _vp, _i64, _vp, _vp],
         "tsmi_sort_keys": [_vp, _vp, _vp, _i64, _i32, _vp, _i64],
@@ -306,13 +307,16 @@ kmap_queue_ahead = True
 def _map_queued_ahead(in_coords, out_coords, ks, st, pd) -> Optional[torch.Tensor]:
     """The map of kmap_sorted(in_coords, out_coords, ...) if it was queued ahead on the second
     stream; notes the request when both operands are levels of the chain in flight."""
-    dev = in_coords.device
+    index = in_coords.device.index
+    state = _stream_states.get((index if index is not None else _cur_device(), _stream()))
+    if state is None:
+        return None
+    a = state.level_index.get(id(in_coords))
+    if a is None:  # (the common miss, answered without the lock: neither table is changed here)
+        return None
     with _state_lock:
-        state = _stream_states.get((dev.index if dev.index is not None else _cur_device(), _stream()))
-        if state is None or not state.level_index:
-            return None
-        a, b = state.level_index.get(id(in_coords)), state.level_index.get(id(out_coords))
-        if a is None or b is None or a[0]() is not in_coords or b[0]() is not out_coords:
+        b = state.level_index.get(id(out_coords))
+        if b is None or a[0]() is not in_coords or b[0]() is not out_coords:
             return None
         request = (a[1], b[1], ks, st, pd)
         if request not in state.map_plan_seen:
@@ -363,11 +367,16 @@ def _queue_maps_ahead(state, chain_rows, on_side: bool) -> None:
     torch.cuda.set_stream(state.side)  # (the context manager costs 6 us, two switches 0.8)
     try:
         buffers = {kvol: torch.empty((rows, kvol), dtype=torch.int32, device=dev) for kvol, rows in rows_of.items()}
+        flat = []
         for a, b, ks, st, pd, kvol, first in todo:
-            omap = buffers[kvol][first:first + make_divisible(b.shape[0], 128)]
-            _kmap_sorted_launch(a, b, ks, st, pd, omap)
+            n_pad = make_divisible(b.shape[0], 128)
+            omap = buffers[kvol][first:first + n_pad]
+            samples = _sorted_samples(a)
+            flat += (a.data_ptr(), a.shape[0], b.data_ptr(), b.shape[0], n_pad,
+                     0 if samples is None else samples.data_ptr(), omap.data_ptr(), *ks, *st, *pd)
             state.maps_ahead[(id(a), id(b), ks, st, pd)] = (weakref.ref(a), weakref.ref(b), omap,
                                                             (a._version, b._version))
+        _check(_C.tsmi_kmap_sorted_batch(_stream(), len(todo), (ctypes.c_int64 * len(flat))(*flat)))
         state.maps_event = torch.cuda.Event()
         state.maps_event.record()
     finally:
@@ -695,7 +704,7 @@ class _StridedState:
     stream (or device) get a state of their own and never see these tensors."""
     __slots__ = ("grid_buf", "grid_words", "grid_dirty", "chain_geom", "chain_last", "chain_count",
                  "chain_len", "ahead", "ahead_hits", "host_counters", "pending", "pending_rsv", "root_chain",
-                 "lookahead_hits", "side", "grid_event", "grid_old", "level_index", "map_plan",
+                 "lookahead_hits", "side", "grid_event", "grid_event_stream", "grid_old", "level_index", "map_plan",
                  "map_plan_seen", "maps_ahead", "maps_event", "maps_ahead_hits", "maps_main")
 
     def __init__(self):
@@ -715,6 +724,7 @@ class _StridedState:
         self.lookahead_hits = 0   # chains whose first half was already queued (diagnostic)
         self.side = None          # second stream of the device, for chains queued ahead of their use
         self.grid_event = None    # end of the last work queued on the bitmap scratch, on either stream
+        self.grid_event_stream = 0  # ... and the stream it was queued on
         self.grid_old = None      # the scratch before it last grew (kept until the next growth)
         self.level_index = {}     # id(rows) -> (weak reference, position in the chain in flight; 0: its root)
         self.map_plan = ()        # sorted-map builds the last forward asked for over its chain's levels
@@ -819,7 +829,8 @@ def _grid_start(state, coords, ks, st, pd, coords_max_host, fan, ahead, early=Fa
     counters to the host; nothing waits.  Runs with _state_lock held."""
     n = coords.shape[0]
     dev = coords.device
-    if state.grid_event is not None:  # the scratch may last have been used on the other stream
+    if state.grid_event is not None and state.grid_event_stream != _stream():
+        # the scratch was last used on the other stream (work of the same stream is ordered anyway)
         torch.cuda.current_stream(dev).wait_event(state.grid_event)
     bits = min(max(1 << (n * fan * 2048 - 1).bit_length(), 1 << 20), 1 << 30)
     buf = state.bitmap(dev, bits // 32)
@@ -873,9 +884,9 @@ def _grid_start(state, coords, ks, st, pd, coords_max_host, fan, ahead, early=Fa
         job.host.copy_(ctr, non_blocking=True)
         job.event = torch.cuda.Event()
         job.event.record()
-        state.grid_event = job.event
+        state.grid_event, state.grid_event_stream = job.event, s
     elif state.side is not None:  # (a state that never used its side stream needs no events)
-        state.grid_event = torch.cuda.Event()
+        state.grid_event, state.grid_event_stream = torch.cuda.Event(), s
         state.grid_event.record()
     return job
 
@@ -1002,7 +1013,7 @@ def _grid_finish(state, job: _GridJob, rsv_ratio, cap, want_table):
         _queue_maps_ahead(state, chain_rows, job.rows is not None and state.side is not None
                           and job.stream == state.side.cuda_stream)
     if state.side is not None and job.rows is None:  # emit passes ran on this stream just now
-        state.grid_event = torch.cuda.Event()
+        state.grid_event, state.grid_event_stream = torch.cuda.Event(), _stream()
         state.grid_event.record()
     return first
 
@@ -1071,8 +1082,11 @@ def strided_lookahead(coords: torch.Tensor) -> None:
             main = torch.cuda.current_stream(coords.device)
             if state.side is None:
                 state.side = torch.cuda.Stream(device=coords.device)
-            with torch.cuda.stream(state.side):
+            torch.cuda.set_stream(state.side)  # (the context manager costs 6 us, two switches 0.8)
+            try:
                 job = _grid_start(state, coords, ks, st, pd, None, fan, ahead, early=True)
+            finally:
+                torch.cuda.set_stream(main)
             if job.rows is not None:
                 job.rows.record_stream(main)  # allocated on the side stream, read and freed on the caller's
         else:

@@ -1434,6 +1434,20 @@ extern "C" int tsmi_kmap_sorted(tsmi_stream_t s, const int32_t *in_coords, int64
   return check_launch("tsmi_kmap_sorted");
 }
 
+extern "C" int tsmi_kmap_sorted_batch(tsmi_stream_t s, int count, const int64_t *args) {
+  TSMI_REQUIRE(count >= 0 && (count == 0 || args), "kmap_sorted_batch: bad arguments");
+  for (int i = 0; i < count; ++i) {
+    const int64_t *a = args + 16 * i;
+    int32_t geom[9];
+    for (int j = 0; j < 9; ++j) geom[j] = (int32_t)a[7 + j];
+    if (int e = tsmi_kmap_sorted(s, (const int32_t *)(uintptr_t)a[0], a[1], (const int32_t *)(uintptr_t)a[2], a[3],
+                                 a[4], geom, geom + 3, geom + 6, (const int64_t *)(uintptr_t)a[5],
+                                 (int32_t *)(uintptr_t)a[6]))
+      return e;
+  }
+  return TSMI_OK;
+}
+
 extern "C" int tsmi_coords_max(tsmi_stream_t s, const int32_t *coords, int64_t n,
                                int32_t *out_max, int clear_first) {
   TSMI_REQUIRE(out_max && n >= 0 && (n == 0 || coords), "coords_max: bad arguments");
