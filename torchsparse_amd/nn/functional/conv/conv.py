@@ -102,7 +102,15 @@ def conv3d(input: SparseTensor, weight: torch.Tensor,
             for level, table in ((input.stride, kmap["in_hashmap"]), (out_stride, kmap["out_hashmap"])):
                 if table is not None and caches.hashmaps.get(level) is None:
                     caches.hashmaps[level] = table
-        out_feats = conv_fn.apply(feats, weight, kmap, config, False, bias, residual, relu)
+        if (weight.dim() == 3 and feats.shape[1] == weight.shape[1]
+                and _direct_ok(feats, weight, bias, residual, config)):
+            # (what conv_fn.apply comes down to for an inference call in the unsorted implicit GEMM)
+            from torchsparse_amd import backend
+            out_feats = backend._implicit_gemm(feats, backend.pack_weights(weight), *weight.shape,
+                                               kmap["out_in_map"], kmap["sizes"][1], bias, residual, relu,
+                                               config.get("pair_segments"))
+        else:
+            out_feats = conv_fn.apply(feats, weight, kmap, config, False, bias, residual, relu)
         output = SparseTensor._make(out_feats, kmap["coords"], out_stride, kmap["spatial_range"], caches)
     elif generative:
         # generative transposed convolution (conv.py:162-204): outputs are created around
@@ -125,13 +133,37 @@ def conv3d(input: SparseTensor, weight: torch.Tensor,
         kmap = transpose_kernel_map(kmap, config["ifsort"], training=training,
                                     split_mask_num=config["split_mask_num"],
                                     split_mask_num_bwd=config["split_mask_num_bwd"])
-        out_feats = conv_fn.apply(feats, weight, kmap, config, True, bias, residual, relu)
+        if (weight.dim() == 3 and feats.shape[1] == weight.shape[1]
+                and _direct_ok(feats, weight, bias, residual, config)):
+            from torchsparse_amd import backend
+            out_feats = backend._implicit_gemm(feats, backend.pack_weights(weight), *weight.shape,
+                                               kmap["out_in_map_t"], kmap["sizes"][0], bias, residual, relu,
+                                               config.get("pair_segments"))
+        else:
+            out_feats = conv_fn.apply(feats, weight, kmap, config, True, bias, residual, relu)
         fine_coords, fine_range = caches.cmaps[fine_stride]
         output = SparseTensor._make(out_feats, fine_coords, fine_stride, fine_range, caches)
 
     if output.stride not in caches.cmaps:
         caches.cmaps[output.stride] = (output.coords, output.spatial_range)
     return output
+
+
+def _direct_ok(feats, kernel, bias, residual, config) -> bool:
+    """Whether a call may go straight to the unsorted implicit-GEMM launch: that dataflow, no
+    gradient to record, operands that need no conversion."""
+    if config["dataflow"] != _cfg.Dataflow.ImplicitGEMM or config["ifsort"]:
+        return False
+    dtype = feats.dtype
+    if (not feats.is_cuda or dtype != kernel.dtype or not feats.is_contiguous()
+            or (bias is not None and bias.dtype != dtype)
+            or (residual is not None and (residual.dtype != dtype or not residual.is_contiguous()))):
+        return False
+    if torch.is_grad_enabled() and (feats.requires_grad or kernel.requires_grad
+                                    or (bias is not None and bias.requires_grad)
+                                    or (residual is not None and residual.requires_grad)):
+        return False
+    return True
 
 
 def conv3d_cached(input: SparseTensor, kernel: torch.Tensor, bias: Optional[torch.Tensor],
@@ -147,17 +179,8 @@ def conv3d_cached(input: SparseTensor, kernel: torch.Tensor, bias: Optional[torc
         config = _cfg.get_global_conv_config()
         if config is None:
             config = _cfg._shared_default_config(get_conv_mode())
-    if config["dataflow"] != _cfg.Dataflow.ImplicitGEMM or config["ifsort"]:
-        return None
     feats = input.feats
-    dtype = feats.dtype
-    if (not feats.is_cuda or dtype != kernel.dtype or not feats.is_contiguous()
-            or (bias is not None and bias.dtype != dtype)
-            or (residual is not None and (residual.dtype != dtype or not residual.is_contiguous()))):
-        return None
-    if torch.is_grad_enabled() and (feats.requires_grad or kernel.requires_grad
-                                    or (bias is not None and bias.requires_grad)
-                                    or (residual is not None and residual.requires_grad)):
+    if not _direct_ok(feats, kernel, bias, residual, config):
         return None
     caches = input._caches
     ist = input.stride
