@@ -531,6 +531,15 @@ int tsmi_conv_implicit_gemm_segments(tsmi_stream_t s, const void *x, const void 
                                      int cin, int cout, int dtype, const void *bias,
                                      const void *residual, int relu, void *products, void *y);
 
+/* tsmi_conv_implicit_gemm and tsmi_conv_implicit_gemm_segments with their arguments in one block
+ * of host int64, in the order of the declarations above (pointers and the stream as integers,
+ * 18 and 17 entries): the two calls a forward makes most often - about 60 per forward of a U-Net -
+ * for bindings that pay per argument (ctypes converts one in 0.1 us).  Same checks, same
+ * launches, same status.  No counterpart in the reference (pybind11 converts its arguments in
+ * compiled code). */
+int tsmi_conv_implicit_gemm_packed(const int64_t *args);
+int tsmi_conv_implicit_gemm_segments_packed(const int64_t *args);
+
 /* Gather-GEMM-scatter, step 1: buffer[nbaddrs[k] + p, :] = X[in(k,p), :].
  * Replaces gather_all_kernel_pad_sep_with_mask / gather_kernel
  * (convolution/convolution_gather_scatter_cuda.cu:17-40,70-112). */

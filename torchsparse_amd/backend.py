@@ -10,6 +10,7 @@ import collections
 import ctypes
 import functools
 import os
+import struct
 import threading
 import weakref
 from typing import List, Optional, Sequence, Tuple
@@ -101,6 +102,8 @@ def _load():
         "tsmi_pair_segments": [_vp, _vp, _i64, _i32, _i64, _vp, _vp, _vp, _vp],
         "tsmi_conv_implicit_gemm_segments": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _i32,
                                              _i32, _vp, _vp, _i32, _vp, _vp],
+        "tsmi_conv_implicit_gemm_packed": [ctypes.c_char_p],
+        "tsmi_conv_implicit_gemm_segments_packed": [ctypes.c_char_p],
         "tsmi_hash_coords": [_vp, _vp, _i64, _vp],
         "tsmi_kernel_hash": [_vp, _vp, _i64, _vp, _i32, _vp],
         "tsmi_count": [_vp, _vp, _i64, _vp, _i32],
@@ -1278,6 +1281,9 @@ def _epilogue_args(bias, residual, x, n_out, cout):
     return _ptr(bias), _ptr(residual)
 
 
+_PACK17 = struct.Struct("17q").pack
+_PACK18 = struct.Struct("18q").pack
+
 _SCRATCH = {}  # (device index, stream) -> uint8 tensor, grown on demand
 # held while a call that goes through the scratch buffer queues its launches: two host threads
 # that feed one stream must not interleave the launches of two such calls
@@ -1486,10 +1492,10 @@ def conv_implicit_gemm_segments(x, wp, kvol, cin, cout, out_in_map, num_out_feat
     pb, pr = _epilogue_args(bias, residual, x, num_out_feats, cout)
     with _scratch_lock:
         products = _scratch(x.device, stream, kvol * seg_rows * cout * x.element_size())
-        _check(_C.tsmi_conv_implicit_gemm_segments(stream, x.data_ptr(), wp.data_ptr(), seg.in_rows_ptr,
-                                                   seg.counts_ptr, seg.pos_ptr, seg_rows,
-                                                   num_out_feats, kvol, cin, cout, _dtype_code(x), pb, pr,
-                                                   int(relu), products, y.data_ptr()))
+        _check(_C.tsmi_conv_implicit_gemm_segments_packed(_PACK17(
+            stream, x.data_ptr(), wp.data_ptr(), seg.in_rows_ptr, seg.counts_ptr, seg.pos_ptr, seg_rows,
+            num_out_feats, kvol, cin, cout, _dtype_code(x), pb or 0, pr or 0, int(relu), products,
+            y.data_ptr())))
     return y
 
 
@@ -1502,16 +1508,19 @@ def _implicit_gemm(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias=None,
     code = _dtype_code(x)
     stream = _stream()
     pb, pr = _epilogue_args(bias, residual, x, num_out_feats, cout)
-    args = (stream, x.data_ptr(), wp.data_ptr(), out_in_map.data_ptr(), out_in_map.shape[0], num_out_feats,
-            kvol, cin, cout, code, pb, pr, int(relu))
+    # (the arguments of tsmi_conv_implicit_gemm in one block: one conversion instead of 18)
     ws_elems = _workspace_elems(num_out_feats, kvol, cin, cout, code) if num_out_feats < 65536 else 0
     if ws_elems > 0:  # (only maps with few row tiles use the offset split)
         with _scratch_lock:
-            _check(_C.tsmi_conv_implicit_gemm(*args, _scratch(x.device, stream, 4 * ws_elems), ws_elems,
-                                              _tile_counters(x.device, stream).data_ptr(),
-                                              _N_TILE_COUNTERS, y.data_ptr()))
+            _check(_C.tsmi_conv_implicit_gemm_packed(_PACK18(
+                stream, x.data_ptr(), wp.data_ptr(), out_in_map.data_ptr(), out_in_map.shape[0],
+                num_out_feats, kvol, cin, cout, code, pb or 0, pr or 0, int(relu),
+                _scratch(x.device, stream, 4 * ws_elems), ws_elems,
+                _tile_counters(x.device, stream).data_ptr(), _N_TILE_COUNTERS, y.data_ptr())))
     else:
-        _check(_C.tsmi_conv_implicit_gemm(*args, None, 0, None, _N_TILE_COUNTERS, y.data_ptr()))
+        _check(_C.tsmi_conv_implicit_gemm_packed(_PACK18(
+            stream, x.data_ptr(), wp.data_ptr(), out_in_map.data_ptr(), out_in_map.shape[0], num_out_feats,
+            kvol, cin, cout, code, pb or 0, pr or 0, int(relu), 0, 0, 0, _N_TILE_COUNTERS, y.data_ptr())))
     return y
 
 

@@ -233,3 +233,24 @@ extern "C" int tsmi_gs_scatter(tsmi_stream_t s, const void *out_buffer, const in
   return ops->scatter((hipStream_t)s, out_buffer, nbaddrs, row_mask, n_out, kvol, cout, center_k,
                       bias, residual, relu, y);
 }
+
+// The two calls a forward makes most often, with their arguments in one block: a binding that
+// converts arguments one by one (ctypes: 0.1 us each) passes one pointer instead of 17 or 18.
+static inline const void *as_ptr(int64_t v) { return (const void *)(uintptr_t)v; }
+
+extern "C" int tsmi_conv_implicit_gemm_packed(const int64_t *a) {
+  TSMI_REQUIRE(a, "conv_implicit_gemm_packed: null argument block");
+  return tsmi_conv_implicit_gemm((tsmi_stream_t)as_ptr(a[0]), as_ptr(a[1]), as_ptr(a[2]), (const int32_t *)as_ptr(a[3]),
+                                 a[4], a[5], (int)a[6], (int)a[7], (int)a[8], (int)a[9], as_ptr(a[10]),
+                                 as_ptr(a[11]), (int)a[12], (float *)as_ptr(a[13]), a[14],
+                                 (int32_t *)as_ptr(a[15]), a[16], (void *)as_ptr(a[17]));
+}
+
+extern "C" int tsmi_conv_implicit_gemm_segments_packed(const int64_t *a) {
+  TSMI_REQUIRE(a, "conv_implicit_gemm_segments_packed: null argument block");
+  return tsmi_conv_implicit_gemm_segments((tsmi_stream_t)as_ptr(a[0]), as_ptr(a[1]), as_ptr(a[2]),
+                                          (const int32_t *)as_ptr(a[3]), (const int32_t *)as_ptr(a[4]),
+                                          (const int32_t *)as_ptr(a[5]), a[6], a[7], (int)a[8], (int)a[9],
+                                          (int)a[10], (int)a[11], as_ptr(a[12]), as_ptr(a[13]), (int)a[14],
+                                          (void *)as_ptr(a[15]), (void *)as_ptr(a[16]));
+}
