@@ -1274,11 +1274,17 @@ def _conv_common(in_feats: torch.Tensor, kernel: torch.Tensor):
 
 
 def _epilogue_args(bias, residual, x, n_out, cout):
-    for name, t, shape in (("bias", bias, (cout,)), ("residual", residual, (n_out, cout))):
-        if t is not None:
-            if t.dtype != x.dtype or tuple(t.shape) != shape or not t.is_contiguous():
-                raise ValueError(f"{name} must be a contiguous {x.dtype} tensor of shape {shape}")
-    return _ptr(bias), _ptr(residual)
+    pb = pr = None
+    if bias is not None:
+        if bias.dtype != x.dtype or bias.dim() != 1 or bias.shape[0] != cout or not bias.is_contiguous():
+            raise ValueError(f"bias must be a contiguous {x.dtype} tensor of shape {(cout,)}")
+        pb = bias.data_ptr()
+    if residual is not None:
+        if (residual.dtype != x.dtype or residual.dim() != 2 or residual.shape[0] != n_out
+                or residual.shape[1] != cout or not residual.is_contiguous()):
+            raise ValueError(f"residual must be a contiguous {x.dtype} tensor of shape {(n_out, cout)}")
+        pr = residual.data_ptr()
+    return pb, pr
 
 
 _PACK17 = struct.Struct("17q").pack
