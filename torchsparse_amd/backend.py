@@ -370,22 +370,23 @@ def _queue_maps_ahead(state, chain_rows, on_side: bool) -> None:
     torch.cuda.set_stream(state.side)  # (the context manager costs 6 us, two switches 0.8)
     try:
         buffers = {kvol: torch.empty((rows, kvol), dtype=torch.int32, device=dev) for kvol, rows in rows_of.items()}
-        flat = []
+        flat, queued = [], {}
         for a, b, ks, st, pd, kvol, first in todo:
             n_pad = make_divisible(b.shape[0], 128)
             omap = buffers[kvol][first:first + n_pad]
             samples = _sorted_samples(a)
             flat += (a.data_ptr(), a.shape[0], b.data_ptr(), b.shape[0], n_pad,
                      0 if samples is None else samples.data_ptr(), omap.data_ptr(), *ks, *st, *pd)
-            state.maps_ahead[(id(a), id(b), ks, st, pd)] = (weakref.ref(a), weakref.ref(b), omap,
-                                                            (a._version, b._version))
+            queued[(id(a), id(b), ks, st, pd)] = (weakref.ref(a), weakref.ref(b), omap, (a._version, b._version))
         _check(_C.tsmi_kmap_sorted_batch(_stream(), len(todo), (ctypes.c_int64 * len(flat))(*flat)))
-        state.maps_event = torch.cuda.Event()
-        state.maps_event.record()
+        event = torch.cuda.Event()
+        event.record()
     finally:
         torch.cuda.set_stream(main)
     for buf in buffers.values():
         buf.record_stream(main)  # allocated on the second stream, read and freed on the caller's
+    # (only now: a call that failed above leaves no map behind that was never written)
+    state.maps_ahead, state.maps_event = queued, event
 
 
 def _kmap_sorted_launch(in_coords, out_coords, ks, st, pd, omap=None) -> torch.Tensor:
