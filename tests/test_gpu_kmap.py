@@ -578,3 +578,45 @@ def _chain_started_at_the_submanifold_build(side):
     finally:
         backend.downsample_lookahead_at_subm = True
     assert not any(st.grid_dirty for st in backend._stream_states.values())
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2, 3])
+def test_maps_queued_ahead_match_the_oracle(seed):
+    """Chains of kernel size = stride layers with a submanifold map per level, passed five times
+    (a new coordinate tensor on every other pass): from the third pass on the maps over the
+    chain's levels are built ahead on the second stream; every map of every pass equals the
+    oracle's, whatever the stride, the submanifold kernel of a level or the depth of the chain."""
+    rng = np.random.default_rng(400 + seed)
+    st = t3([(2, 2, 2), (2, 1, 2), (3, 3, 2), (2, 3, 2)][seed])
+    n = [3000, 30000, 60000, 500][seed]
+    ext = [(40, 100, 40), (100, 100, 40), (400, 40, 100), (40, 40, 40)][seed]
+    batch = 1 + seed % 2
+    cols = [rng.integers(0, batch, n)] + [rng.integers(0, e, n) for e in ext]
+    coords = np.unique(np.stack(cols, 1).astype(np.int32), axis=0)  # ascending rows
+    depth = [2, 3, 2, 3][seed]
+    sub_k = [t3(k) for k in [(3, 3, 3), (3, 1, 3), (1, 3, 3), (3, 3, 3)]][:depth + 1]
+    want, want_sub, c = [], [oracle.kmap_subm(coords, sub_k[0])], coords
+    for d in range(depth):
+        m, c2 = oracle.kmap_downsample(c, st, st, 0)
+        assert len(c2) > 0
+        want.append((m, c2))
+        want_sub.append(oracle.kmap_subm(c2, sub_k[d + 1]))
+        c = c2
+    backend.release_scratch()
+    x = None
+    for rep in range(5):
+        x = dev(coords) if rep % 2 == 0 else x
+        km = F.build_kernel_map(x, x.shape[0], sub_k[0], 1, 1, mode="hashmap_on_the_fly")
+        np.testing.assert_array_equal(km["out_in_map"].cpu().numpy(), want_sub[0])
+        lvl = x
+        for d, (m, c2) in enumerate(want):
+            km = F.build_kernel_map(lvl, lvl.shape[0], st, st, 0, mode="hashmap_on_the_fly")
+            np.testing.assert_array_equal(km["coords"].cpu().numpy(), c2)
+            np.testing.assert_array_equal(km["out_in_map"].cpu().numpy(), m)
+            lvl = km["coords"]
+            ks = sub_k[d + 1]
+            km = F.build_kernel_map(lvl, lvl.shape[0], ks, 1, tuple((k - 1) // 2 for k in ks),
+                                    mode="hashmap_on_the_fly")
+            np.testing.assert_array_equal(km["out_in_map"].cpu().numpy(), want_sub[d + 1])
+    state, = backend._stream_states.values()
+    assert state.maps_ahead_hits >= 2 * depth  # at least one pass took its maps from the queue
