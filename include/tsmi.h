@@ -531,6 +531,42 @@ int tsmi_conv_implicit_gemm_segments(tsmi_stream_t s, const void *x, const void 
                                      int cin, int cout, int dtype, const void *bias,
                                      const void *residual, int relu, void *products, void *y);
 
+/* Implicit GEMM over a 3x3x3 map whose rows are grouped by the kernel planes they use - the
+ * counterpart of the reference's mask-sorted dataflow (bitmask -> sort -> reordered map,
+ * nn/functional/conv/kmap/func/hashmap_on_the_fly.py:92-107, and
+ * convolution/convolution_forward_implicit_gemm_sorted_cuda.cu:94-95,341-342, which skips
+ * the offsets a 128-row tile does not use) without its device sort.
+ * tsmi_map_group_rows: inside windows of `window` consecutive rows (a multiple of 128, at
+ * most 8192) the rows of `map` (int32 [>= n_rows, 27], negative = none) are counting-sorted
+ * by the outer planes of the kernel that hold a neighbour (digit 0 or 2 along each axis: six
+ * bits; key = rank of the number of offsets those planes span << 6 | bits, ascending, so the
+ * rows with the most offsets end a window).  With P = tsmi_map_group_rows_padded(n_rows,
+ * window) = ceil(n_rows / window) * window positions (-1: bad sizes): grouped[p, :] =
+ * map[row_of[p], :] and row_of[p] = the row at position p (int32 [P, 27] and [P]; -1 and an
+ * all -1 map row for the padding positions behind n_rows); masks64[t] (int32 [P / 64]) = the
+ * union, bit k per kernel offset, of the offsets the rows at positions 64 t .. 64 t + 63 use;
+ * order64 (int32 [8 ceil(P / 512)]) / order128 (int32 [8 ceil(P / 1024)]) = the order in which a
+ * convolution starts the T = P / 64 (P / 128) tiles of 64 (128) rows: the tiles are cut into 8 runs
+ * of S = ceil(T / 8) consecutive ones, one per XCD (workgroup b runs on XCD b % 8), and
+ * order[8 j + c] = the tile of run c with the j-th most offsets (-1: the run has no such
+ * tile).  Two launches, no host read-back; the order of
+ * equal keys (and of tiles with equally many offsets) is not fixed, and what the convolution
+ * below computes is the same bit for bit whatever it is.
+ * tsmi_conv_implicit_gemm_grouped: Y[row_of[p], :] = sum over k of X[grouped[p, k], :] W[k]
+ * + bias + residual, optional ReLU - tsmi_conv_implicit_gemm's sums, row by row - with one
+ * workgroup per row tile, started in the listed order: on every XCD the long tiles first, the
+ * short ones fill the machine behind them.  n_grouped = P. */
+int64_t tsmi_map_group_rows_padded(int64_t n_rows, int window);
+int tsmi_map_group_rows(tsmi_stream_t s, const int32_t *map, int64_t n_rows, int kvol, int window,
+                        int32_t *grouped, int32_t *row_of, int32_t *masks64, int32_t *order64,
+                        int32_t *order128);
+int tsmi_conv_implicit_gemm_grouped(tsmi_stream_t s, const void *x, const void *w_packed,
+                                    const int32_t *grouped_map, const int32_t *row_of,
+                                    const int32_t *order64, const int32_t *order128,
+                                    int64_t n_grouped, int64_t n_out, int kvol, int cin, int cout,
+                                    int dtype, const void *bias, const void *residual, int relu,
+                                    void *y);
+
 /* tsmi_conv_implicit_gemm and tsmi_conv_implicit_gemm_segments with their arguments in one block
  * of host int64, in the order of the declarations above (pointers and the stream as integers,
  * 18 and 17 entries): the two calls a forward makes most often - about 60 per forward of a U-Net -
@@ -539,6 +575,7 @@ int tsmi_conv_implicit_gemm_segments(tsmi_stream_t s, const void *x, const void 
  * compiled code). */
 int tsmi_conv_implicit_gemm_packed(const int64_t *args);
 int tsmi_conv_implicit_gemm_segments_packed(const int64_t *args);
+int tsmi_conv_implicit_gemm_grouped_packed(const int64_t *args); /* 17 entries */
 
 /* Gather-GEMM-scatter, step 1: buffer[nbaddrs[k] + p, :] = X[in(k,p), :].
  * Replaces gather_all_kernel_pad_sep_with_mask / gather_kernel

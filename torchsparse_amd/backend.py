@@ -49,6 +49,8 @@ def _load():
     lib.tsmi_wgrad_pairs_capacity.argtypes = [_i64, _i32]
     lib.tsmi_conv_wgrad_pairs_workspace_elems.restype = _i64
     lib.tsmi_conv_wgrad_pairs_workspace_elems.argtypes = [_i64, _i32, _i32, _i32, _i32]
+    lib.tsmi_map_group_rows_padded.restype = _i64
+    lib.tsmi_map_group_rows_padded.argtypes = [_i64, _i32]
     lib.tsmi_kmap_sorted_samples_elems.restype = _i64
     lib.tsmi_kmap_sorted_samples_elems.argtypes = [_i64]
     sig = {
@@ -104,6 +106,10 @@ def _load():
                                              _i32, _vp, _vp, _i32, _vp, _vp],
         "tsmi_conv_implicit_gemm_packed": [ctypes.c_char_p],
         "tsmi_conv_implicit_gemm_segments_packed": [ctypes.c_char_p],
+        "tsmi_conv_implicit_gemm_grouped_packed": [ctypes.c_char_p],
+        "tsmi_conv_implicit_gemm_grouped": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _i32, _i32,
+                                            _vp, _vp, _i32, _vp],
+        "tsmi_map_group_rows": [_vp, _vp, _i64, _i32, _i32, _vp, _vp, _vp, _vp, _vp],
         "tsmi_hash_coords": [_vp, _vp, _i64, _vp],
         "tsmi_kernel_hash": [_vp, _vp, _i64, _vp, _i32, _vp],
         "tsmi_count": [_vp, _vp, _i64, _vp, _i32],
@@ -211,7 +217,25 @@ def hash_capacity(n: int, ratio: float = 2.0) -> int:
 # builders produce ascending rows in range and say so for their outputs.
 COORD_LIMIT = 1 << 17
 BATCH_LIMIT = 512
-_range_ok = {}  # id(tensor) -> (weak reference, version, address, ascending: True / False / None = not known)
+_range_ok = {}  # id(tensor) -> (weak reference, version, address, ascending: True / False / None = not known, origin)
+# A tensor the library has not seen is checked by one small kernel, and its verdict is read
+# back: that stops the host until everything queued on the stream has run (a quarter of a U-Net
+# forward when forwards follow each other).  The wait also stands for a fact the library
+# cannot see: rows produced by work queued on the caller's stream are complete only once that
+# work has run, and the strided chain that follows (whose row counts must reach the host
+# before anything can be sized) cannot start before.  A caller who knows that the rows are
+# complete - a data loader's own stream, a scan uploaded earlier - says so with
+# rows_ready(coords): the check then runs without a read-back (its verdict is copied to pinned
+# memory and picked up by a later call), the chain starts at once on the second stream, and
+# until the verdict is in the rows count as unordered (their own maps go through the hash
+# table, which takes any order).  A row outside the packed range of such a tensor raises its
+# ValueError from the call that picks the verdict up (settle_checks() picks up all of them).
+coords_check_deferred = True
+_rows_ready = {}  # id(tensor) -> (weak reference, version, address)
+_pending_verdicts = []  # (weak reference, version, address, pinned slot, event)
+_verdict_slots = None   # pinned int32 ring the verdicts are copied into
+_verdict_next = 0
+_VERDICT_SLOTS = 64
 # Kernel maps of ascending inputs are built by binary search over the coordinates themselves
 # (no hash table); False sends every map through the tables.
 kmap_through_sorted = True
@@ -236,8 +260,9 @@ def _range_known(coords: torch.Tensor) -> bool:
 
 
 def _range_origin(coords: torch.Tensor) -> Optional[str]:
-    """"user": a caller's tensor that coords_ascending looked at; "library": rows a strided
-    builder produced; None: not known."""
+    """"user": a caller's tensor that coords_ascending looked at (complete: its verdict was
+    read back, or the caller declared it so); "library": rows a strided builder produced; None:
+    not known."""
     hit = _range_entry(coords)
     return None if hit is None else hit[4]
 
@@ -258,16 +283,85 @@ def _mark_range_ok(coords: torch.Tensor, ascending: Optional[bool] = None, origi
     _range_ok[id(coords)] = (weakref.ref(coords), coords._version, coords.data_ptr(), ascending, origin)
 
 
+def settle_checks(block: bool = True) -> None:
+    """Pick up the verdicts of coordinate checks that were left on their way to the host
+    (coords_check_deferred): all of them, waiting for their copies, or with ``block=False``
+    those that have arrived.  Raises the ValueError of a tensor with a row outside the packed
+    range."""
+    global _pending_verdicts
+    if not _pending_verdicts:
+        return
+    bad = False
+    left = []
+    for item in _pending_verdicts:
+        ref, version, address, slot, event = item
+        if not block and not event.query():
+            left.append(item)
+            continue
+        if block:
+            event.synchronize()
+        bits = int(_verdict_slots[slot])
+        t = ref()
+        if bits & 2:
+            bad = True
+            if t is not None:
+                _range_ok.pop(id(t), None)
+            continue
+        hit = _range_ok.get(id(t)) if t is not None else None
+        if hit is not None and hit[0]() is t and hit[1] == version and hit[2] == address:
+            _range_ok[id(t)] = (hit[0], version, address, not (bits & 1), "user")
+    _pending_verdicts = left
+    if bad:
+        raise _range_error()
+
+
+def rows_ready(coords: torch.Tensor) -> torch.Tensor:
+    """Declare that the rows of ``coords`` are complete: no work still queued on any stream
+    writes them.  The library then neither waits for the caller's stream before it reads them
+    on its second stream nor reads the verdict of their first check back at once.  Returns
+    ``coords``.  Holds until the tensor is written in place."""
+    if len(_rows_ready) >= 256:
+        for key in [k for k, v in _rows_ready.items() if v[0]() is None]:
+            del _rows_ready[key]
+        if len(_rows_ready) >= 256:
+            _rows_ready.clear()
+    _rows_ready[id(coords)] = (weakref.ref(coords), coords._version, coords.data_ptr())
+    return coords
+
+
+def _declared_ready(coords: torch.Tensor) -> bool:
+    hit = _rows_ready.get(id(coords))
+    return (hit is not None and hit[0]() is coords and hit[1] == coords._version
+            and hit[2] == coords.data_ptr())
+
+
 def coords_ascending(coords: torch.Tensor) -> bool:
     """Whether the rows of ``coords`` ascend strictly in (b, x, y, z); raises ValueError for a
     row outside the packed key's range.  One kernel and one read-back the first time a tensor
-    is seen, nothing afterwards."""
+    is seen, nothing afterwards; for rows declared complete (rows_ready) the verdict is picked
+    up later and False is the answer until then."""
+    global _verdict_slots, _verdict_next
+    if _pending_verdicts:
+        settle_checks(block=False)
     hit = _range_entry(coords)
     if hit is not None and hit[3] is not None:
         return hit[3]
     rows = _need(coords, torch.int32, "coords")
     flags = torch.zeros(1, dtype=torch.int32, device=rows.device)
     _check(_C.tsmi_coords_check(_stream(), _ptr(rows), rows.shape[0], _ptr(flags)))
+    if coords_check_deferred and rows is coords and _declared_ready(coords):
+        if _verdict_slots is None:
+            _verdict_slots = torch.zeros(_VERDICT_SLOTS, dtype=torch.int32, pin_memory=True)
+        if len(_pending_verdicts) >= _VERDICT_SLOTS - 1:
+            settle_checks(block=True)  # (every slot is on its way: wait for them)
+        slot = _verdict_next
+        _verdict_next = (slot + 1) % _VERDICT_SLOTS
+        _verdict_slots[slot:slot + 1].copy_(flags, non_blocking=True)
+        event = torch.cuda.Event()
+        event.record()
+        _pending_verdicts.append((weakref.ref(coords), coords._version, coords.data_ptr(), slot, event))
+        _mark_range_ok(coords, ascending=False, origin="user")  # (complete: the caller said so)
+        return False
     bits = int(flags.item())
     if bits & 2:
         raise _range_error()
@@ -946,6 +1040,8 @@ def _grid_finish(state, job: _GridJob, rsv_ratio, cap, want_table):
         host = job.host.tolist()
     else:
         host = ctr.tolist()
+    if _pending_verdicts:
+        settle_checks(block=False)  # (checks queued before this chain have arrived with it)
     if host[2]:
         state.grid_dirty = False  # nothing was marked, at any level
         return None
@@ -1428,6 +1524,106 @@ _sparse_maps = {}     # id(map) -> weak reference: maps over rows known to have 
 _hint_lock = threading.Lock()  # guards the two tables above and _segments_of
 
 
+# Large 3x3x3 layers of the implicit-GEMM dataflow run over a copy of the map whose rows are
+# grouped, inside windows of consecutive rows, by the planes of the kernel they use
+# (tsmi_map_group_rows): a row tile then multiplies about half as many kernel offsets as a tile
+# of rows in coordinate order (a surface scan: 25 of 27 offsets per 128-row tile in coordinate
+# order, 14 grouped), and the tiles run heaviest first.  The copy is built by one launch the
+# first time a map is used that way and kept with it.  False: every layer in coordinate order.
+igemm_group_rows = True
+group_window = 8192      # rows per window (a multiple of 128, at most 8192)
+group_min_rows = 32768   # smaller maps have too few tiles for the order to matter
+
+_grouped_of = {}  # id(map) -> (weak reference, version, address, stream, rows, window, GroupedMap)
+
+
+class GroupedMap:
+    """What tsmi_map_group_rows leaves, in one int32 allocation: ``grouped`` [P, 27], ``row_of`` [P],
+    ``masks64`` [P / 64], ``order64`` [8 ceil(P / 512)], ``order128`` [8 ceil(P / 1024)] (views, made when asked for;
+    the convolution works from the addresses)."""
+    __slots__ = ("buffer", "padded", "window", "ptrs")
+
+    def __init__(self, padded: int, window: int, device):
+        self.padded, self.window = padded, window
+        sizes = self._sizes()
+        self.buffer = torch.empty(sum(sizes), dtype=torch.int32, device=device)
+        base, self.ptrs, off = self.buffer.data_ptr(), [], 0
+        for n in sizes:
+            self.ptrs.append(base + 4 * off)
+            off += n
+
+    def _sizes(self):
+        p = self.padded
+        return (p * 27, p, p // 64, 8 * -(-(p // 64) // 8), 8 * -(-(p // 128) // 8))
+
+    def _part(self, i):
+        sizes = self._sizes()
+        start = sum(sizes[:i])
+        return self.buffer[start:start + sizes[i]]
+
+    grouped = property(lambda self: self._part(0).view(self.padded, 27))
+    row_of = property(lambda self: self._part(1))
+    masks64 = property(lambda self: self._part(2))
+    order64 = property(lambda self: self._part(3))
+    order128 = property(lambda self: self._part(4))
+
+
+def grouped_map(out_in_map: torch.Tensor, n_rows: int, window: Optional[int] = None) -> GroupedMap:
+    """The grouped copy of a 3x3x3 kernel map's first ``n_rows`` rows: grouped[p] =
+    out_in_map[row_of[p]], positions sorted inside windows of ``window`` rows by the kernel
+    planes a row uses, padding positions (-1) last; and its row tiles listed heaviest first.
+    Two launches, once per map tensor and stream."""
+    window = group_window if window is None else int(window)
+    stream = _stream()
+    hit = _grouped_of.get(id(out_in_map))
+    if (hit is not None and hit[0]() is out_in_map and hit[1] == out_in_map._version
+            and hit[2] == out_in_map.data_ptr() and hit[3] == stream and hit[4] == n_rows and hit[5] == window):
+        return hit[6]
+    out_in_map = _need(out_in_map, torch.int32, "out_in_map")
+    if out_in_map.dim() != 2 or out_in_map.shape[1] != 27:
+        raise ValueError("rows are grouped for 3x3x3 maps only (27 kernel offsets)")
+    if n_rows > out_in_map.shape[0]:
+        raise ValueError(f"the map has {out_in_map.shape[0]} rows, fewer than the {n_rows} asked for")
+    padded = _C.tsmi_map_group_rows_padded(n_rows, window)
+    if padded < 0:
+        raise ValueError(f"bad window of {window} rows: a multiple of 128 between 128 and 8192")
+    if n_rows == 0:
+        raise ValueError("no rows to group")
+    g = GroupedMap(padded, window, out_in_map.device)
+    _check(_C.tsmi_map_group_rows(stream, out_in_map.data_ptr(), n_rows, 27, window, *g.ptrs))
+    with _scratch_lock:
+        if len(_grouped_of) >= 64:
+            for key in [k for k, v in _grouped_of.items() if v[0]() is None]:
+                del _grouped_of[key]
+            if len(_grouped_of) >= 64:
+                _grouped_of.clear()
+        _grouped_of[id(out_in_map)] = (weakref.ref(out_in_map), out_in_map._version, out_in_map.data_ptr(),
+                                       stream, n_rows, window, g)
+    return g
+
+
+def _grouping_pays(x, kvol: int, cin: int, cout: int, num_out_feats: int) -> bool:
+    """Layers that run over the grouped map: 3x3x3, enough rows for several hundred tiles, 16-bit
+    or 32-bit features in whole 16-byte pieces, and a channel count the one-column-tile kernels
+    cover (wider layers of fewer than 65536 rows run the tiled kernel, which keeps its order)."""
+    return bool(igemm_group_rows and kvol == 27 and num_out_feats >= group_min_rows
+                and cin > 8 and (cin * x.element_size()) % 16 == 0
+                and (cout < 128 or num_out_feats >= 65536))
+
+
+def conv_implicit_gemm_grouped(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias=None,
+                               residual=None, relu=False) -> torch.Tensor:
+    """The implicit-GEMM sums over the grouped copy of the map (same results bit for bit)."""
+    g = grouped_map(out_in_map, num_out_feats)
+    y = x.new_empty(num_out_feats, cout)
+    pb, pr = _epilogue_args(bias, residual, x, num_out_feats, cout)
+    ptrs = g.ptrs
+    _check(_C.tsmi_conv_implicit_gemm_grouped_packed(_PACK17(
+        _stream(), x.data_ptr(), wp.data_ptr(), ptrs[0], ptrs[1], ptrs[3], ptrs[4], g.padded,
+        num_out_feats, kvol, cin, cout, _dtype_code(x), pb or 0, pr or 0, int(relu), y.data_ptr())))
+    return y
+
+
 def _note_level(out_coords: torch.Tensor, n_in: int) -> None:
     """``out_coords`` came out of a kernel size = stride, pad 0 layer over ``n_in`` rows."""
     with _hint_lock:
@@ -1511,6 +1707,9 @@ def _implicit_gemm(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias=None,
     if _segments_pay(x, kvol, cin, cout, num_out_feats, out_in_map, segments):
         return conv_implicit_gemm_segments(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias,
                                            residual, relu)
+    if _grouping_pays(x, kvol, cin, cout, num_out_feats):
+        return conv_implicit_gemm_grouped(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias,
+                                          residual, relu)
     y = x.new_empty(num_out_feats, cout)  # (the cheapest form of the call: 1.2 us against 1.6)
     code = _dtype_code(x)
     stream = _stream()

@@ -63,7 +63,7 @@ extern "C" int tsmi_conv_implicit_gemm(tsmi_stream_t s, const void *x, const voi
                "conv_implicit_gemm: x, w_packed and y must be 16-byte aligned");
   return ops->igemm((hipStream_t)s, x, w_packed, map, n_map_rows, n_out, n_out, kvol, cin, cout,
                     bias, residual, relu, y, nullptr, 0, 1, workspace, workspace_elems,
-                    tile_counters, tile_counters ? n_tile_counters : 0);
+                    tile_counters, tile_counters ? n_tile_counters : 0, nullptr, nullptr);
 }
 
 extern "C" int tsmi_conv_implicit_gemm_sorted(tsmi_stream_t s, const void *x, const void *w_packed,
@@ -90,7 +90,28 @@ extern "C" int tsmi_conv_implicit_gemm_sorted(tsmi_stream_t s, const void *x, co
                "conv_implicit_gemm_sorted: x, w_packed and y must be 16-byte aligned");
   return ops->igemm((hipStream_t)s, x, w_packed, reorder_map, n_pad, n_pad, n_out, kvol, cin, cout,
                     bias, residual, relu, y, reorder_loc, n_pad, split, workspace, workspace_elems,
-                    tile_counters, tile_counters ? n_tile_counters : 0);
+                    tile_counters, tile_counters ? n_tile_counters : 0, nullptr, nullptr);
+}
+
+extern "C" int tsmi_conv_implicit_gemm_grouped(tsmi_stream_t s, const void *x, const void *w_packed,
+                                               const int32_t *grouped_map, const int32_t *row_of,
+                                               const int32_t *order64, const int32_t *order128,
+                                               int64_t n_grouped, int64_t n_out, int kvol, int cin,
+                                               int cout, int dtype, const void *bias,
+                                               const void *residual, int relu, void *y) {
+  const ConvOps *ops = ops_for(dtype);
+  if (int e = check_shapes("conv_implicit_gemm_grouped", ops, kvol, cin, cout)) return e;
+  TSMI_REQUIRE(n_out >= 0 && n_grouped >= n_out && n_grouped % 128 == 0,
+               "conv_implicit_gemm_grouped: bad sizes (%lld grouped rows for %lld outputs)",
+               (long long)n_grouped, (long long)n_out);
+  if (n_out == 0) return TSMI_OK;
+  TSMI_REQUIRE(x && w_packed && grouped_map && row_of && order64 && order128 && y,
+               "conv_implicit_gemm_grouped: null pointer");
+  TSMI_REQUIRE(aligned16(x) && aligned16(w_packed) && aligned16(y),
+               "conv_implicit_gemm_grouped: x, w_packed and y must be 16-byte aligned");
+  return ops->igemm((hipStream_t)s, x, w_packed, grouped_map, n_grouped, n_grouped, n_out, kvol, cin,
+                    cout, bias, residual, relu, y, row_of, n_grouped, 1, nullptr, 0, nullptr, 0, order64,
+                    order128);
 }
 
 extern "C" int64_t tsmi_conv_wgrad_workspace_elems(int64_t n_in, int kvol, int cin, int cout,
@@ -244,6 +265,15 @@ extern "C" int tsmi_conv_implicit_gemm_packed(const int64_t *a) {
                                  a[4], a[5], (int)a[6], (int)a[7], (int)a[8], (int)a[9], as_ptr(a[10]),
                                  as_ptr(a[11]), (int)a[12], (float *)as_ptr(a[13]), a[14],
                                  (int32_t *)as_ptr(a[15]), a[16], (void *)as_ptr(a[17]));
+}
+
+extern "C" int tsmi_conv_implicit_gemm_grouped_packed(const int64_t *a) {
+  TSMI_REQUIRE(a, "conv_implicit_gemm_grouped_packed: null argument block");
+  return tsmi_conv_implicit_gemm_grouped((tsmi_stream_t)as_ptr(a[0]), as_ptr(a[1]), as_ptr(a[2]),
+                                         (const int32_t *)as_ptr(a[3]), (const int32_t *)as_ptr(a[4]),
+                                         (const int32_t *)as_ptr(a[5]), (const int32_t *)as_ptr(a[6]), a[7], a[8],
+                                         (int)a[9], (int)a[10], (int)a[11], (int)a[12], as_ptr(a[13]),
+                                         as_ptr(a[14]), (int)a[15], (void *)as_ptr(a[16]));
 }
 
 extern "C" int tsmi_conv_implicit_gemm_segments_packed(const int64_t *a) {

@@ -16,12 +16,14 @@ struct ConvOps {
   // floats of scratch igemm wants for this problem (0 = none)
   int64_t (*workspace)(int64_t n_tile_rows, int64_t n_out, int kvol, int split, int cin, int cout,
                        int sorted);
-  // row_out == nullptr: plain implicit GEMM over `map`; otherwise sorted mode.
+  // row_out == nullptr: plain implicit GEMM over `map`; otherwise sorted mode.  order64 / order128
+  // (sorted mode, one split, n_tile_rows a multiple of 128): the 64-row / 128-row tiles of the map
+  // listed heaviest first (tsmi_map_group_rows); the tiles start in that order where the plan allows.
   int (*igemm)(hipStream_t s, const void *x, const void *wp, const int32_t *map,
                int64_t n_map_rows, int64_t n_tile_rows, int64_t n_out, int kvol, int cin, int cout,
                const void *bias, const void *residual, int relu, void *y, const int32_t *row_out,
                int64_t row_out_stride, int split, float *partial, int64_t partial_elems,
-               int32_t *counters, int64_t n_counters);
+               int32_t *counters, int64_t n_counters, const int32_t *order64, const int32_t *order128);
   // out[nbaddrs[k] + p, :] = X[rows[nbaddrs[k] + p], :] W[k] over 128-padded pair lists
   int (*pairs)(hipStream_t s, const void *x, const void *wp, const int32_t *rows,
                const int32_t *nbaddrs, const int32_t *qnbaddrs, int64_t qnnz, int kvol, int cin,

@@ -1851,6 +1851,179 @@ extern "C" int tsmi_pair_segments(tsmi_stream_t s, const int32_t *map, int64_t n
   return check_launch("tsmi_pair_segments");
 }
 
+// ---- rows of a 3x3x3 map grouped by the planes of the kernel they use ------------------------
+// An implicit-GEMM workgroup multiplies every kernel offset that ANY row of its tile uses; on a
+// surface scan in coordinate order four of five such products are for absent neighbours.  Rows
+// whose neighbours lie in the same outer planes of the kernel (digit 0 or 2 along each axis: six
+// planes) use nearly the same offsets, so inside windows of `window` consecutive rows (near
+// enough in space for the rows they gather to share an L2) the rows are counting-sorted by
+//   key = rank of (offsets the occupied planes span) << 6 | plane bits    (1024 bins, padding rows last)
+// where a row with neighbours in e_a of the three layers along axis a (the centre layer always
+// counts) spans e_0 * e_1 * e_2 offsets - one of 1, 2, 3, 4, 6, 8, 9, 12, 18, 27 -, and the map
+// is written out in that order together with the row each position came from and, per 64
+// positions, the union of the offsets their rows use.  A second launch (one workgroup) lists
+// the 64-row and the 128-row tiles by the size of that union, largest first: the order in which
+// the convolution starts them.  The order inside a bin (and among tiles of one size) depends on
+// the order in which threads draw their slots; what is computed through these arrays does not.
+constexpr int kGroupThreads = 1024;
+constexpr int kGroupMaxPerThread = 8;  // windows of at most 8192 rows
+
+__global__ __launch_bounds__(kGroupThreads) void map_group_rows_kernel(
+    const int32_t *__restrict__ map, int64_t n_rows, int window, int32_t *__restrict__ grouped,
+    int32_t *__restrict__ row_of, int32_t *__restrict__ masks64) {
+  __shared__ int hist[1024];
+  __shared__ int offs[1024];
+  __shared__ int lmask[kGroupThreads * kGroupMaxPerThread];
+  const int tid = threadIdx.x;
+  const int64_t base = (int64_t)blockIdx.x * window;
+  hist[tid] = 0;
+  __syncthreads();
+  int key[kGroupMaxPerThread], used[kGroupMaxPerThread];
+#pragma unroll
+  for (int j = 0; j < kGroupMaxPerThread; ++j) {
+    const int r = tid + j * kGroupThreads;
+    key[j] = -1;
+    used[j] = 0;
+    if (r >= window) continue;
+    const int64_t row = base + r;
+    int k = 1023;
+    if (row < n_rows) {
+      const int32_t *m = map + row * 27;
+      int planes = 0, mask = 0;
+#pragma unroll
+      for (int o = 0; o < 27; ++o) {
+        // digits of offset o (the first digit runs fastest): plane bits 0..5 = digit 0 / 2 per axis
+        constexpr int kBit[3] = {1, 0, 2};
+        const int d0 = o % 3, d1 = (o / 3) % 3, d2 = o / 9;
+        const int bits = (d0 != 1 ? kBit[d0] << 0 : 0) | (d1 != 1 ? kBit[d1] << 2 : 0) |
+                         (d2 != 1 ? kBit[d2] << 4 : 0);
+        if (m[o] >= 0) {
+          planes |= bits;
+          mask |= 1 << o;
+        }
+      }
+      const int span = (1 + __popc(planes & 3)) * (1 + __popc(planes & 12)) * (1 + __popc(planes & 48));
+      // rank of the span among 1, 2, 3, 4, 6, 8, 9, 12, 18, 27
+      const int rank = span <= 4 ? span - 1 : (span == 6 ? 4 : span == 8 ? 5 : span == 9 ? 6 : span == 12 ? 7 : span == 18 ? 8 : 9);
+      k = (rank << 6) | planes;
+      used[j] = mask;
+    }
+    key[j] = k;
+    atomicAdd(&hist[k], 1);
+  }
+  __syncthreads();
+  if (tid < 64) {  // exclusive scan of the 1024 bins: 16 per lane, then across the wavefront
+    int local[16], sum = 0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      local[i] = sum;
+      sum += hist[tid * 16 + i];
+    }
+    int incl = sum;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int up = __shfl_up(incl, d);
+      if (tid >= d) incl += up;
+    }
+    const int excl = incl - sum;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) offs[tid * 16 + i] = excl + local[i];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < kGroupMaxPerThread; ++j) {
+    if (key[j] < 0) continue;
+    const int64_t row = base + tid + j * kGroupThreads;
+    const int slot = atomicAdd(&offs[key[j]], 1);  // < window: the bins hold `window` rows in all
+    lmask[slot] = used[j];
+    int32_t *dst = grouped + (base + slot) * 27;
+    if (row < n_rows) {
+      const int32_t *m = map + row * 27;
+#pragma unroll
+      for (int o = 0; o < 27; ++o) dst[o] = m[o];
+      row_of[base + slot] = (int32_t)row;
+    } else {
+#pragma unroll
+      for (int o = 0; o < 27; ++o) dst[o] = -1;
+      row_of[base + slot] = -1;
+    }
+  }
+  __syncthreads();
+  // union of the offsets used by every 64 consecutive positions (window is a multiple of 128)
+  const int wave = tid >> 6, lane = tid & 63;
+  for (int g = wave; g < window / 64; g += kGroupThreads / 64) {
+    int v = lmask[g * 64 + lane];
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) v |= __shfl_xor(v, d);
+    if (lane == 0) masks64[base / 64 + g] = v;
+  }
+}
+
+// The order in which a convolution starts the T tiles of 64 (order64) or 128 (order128) rows:
+// workgroup b runs on XCD b % 8, so the tiles are cut into 8 runs of S = ceil(T / 8) consecutive
+// tiles (consecutive windows are neighbours in space: the rows a run gathers stay in one L2) and
+// order[8 j + c] = the tile of run c with the j-th most offsets, -1 when the run has fewer than
+// j + 1 tiles: every XCD starts its long tiles first, and the workgroups that share a CU are
+// a long, a middling and a short one.
+__global__ __launch_bounds__(kGroupThreads) void group_tile_order_kernel(
+    const int32_t *__restrict__ masks64, int n64, int32_t *__restrict__ order64,
+    int32_t *__restrict__ order128) {
+  __shared__ int hist[2][8][32];
+  __shared__ int offs[2][8][32];
+  const int tid = threadIdx.x;
+  const int n128 = n64 / 2;  // (n64 is even: the grouped map holds a multiple of 128 positions)
+  const int s64 = (n64 + 7) / 8, s128 = (n128 + 7) / 8;
+  if (tid < 512) (&hist[0][0][0])[tid] = 0;
+  for (int i = tid; i < 8 * s64; i += kGroupThreads) order64[i] = -1;
+  for (int i = tid; i < 8 * s128; i += kGroupThreads) order128[i] = -1;
+  __syncthreads();
+  for (int i = tid; i < n64; i += kGroupThreads) {
+    const int a = masks64[i];
+    atomicAdd(&hist[0][i / s64][27 - __popc(a)], 1);
+    if ((i & 1) == 0) atomicAdd(&hist[1][(i >> 1) / s128][27 - __popc(a | masks64[i + 1])], 1);
+  }
+  __syncthreads();
+  if (tid < 16) {
+    int sum = 0;
+    for (int c = 0; c < 28; ++c) {
+      offs[tid >> 3][tid & 7][c] = sum;
+      sum += hist[tid >> 3][tid & 7][c];
+    }
+  }
+  __syncthreads();
+  for (int i = tid; i < n64; i += kGroupThreads) {
+    const int a = masks64[i];
+    const int c64 = i / s64;
+    order64[8 * atomicAdd(&offs[0][c64][27 - __popc(a)], 1) + c64] = i;
+    if ((i & 1) == 0) {
+      const int c128 = (i >> 1) / s128;
+      order128[8 * atomicAdd(&offs[1][c128][27 - __popc(a | masks64[i + 1])], 1) + c128] = i >> 1;
+    }
+  }
+}
+
+extern "C" int64_t tsmi_map_group_rows_padded(int64_t n_rows, int window) {
+  if (n_rows < 0 || window < 128 || window > kGroupThreads * kGroupMaxPerThread || window % 128 != 0) return -1;
+  return ceil_div(n_rows, window) * window;
+}
+
+extern "C" int tsmi_map_group_rows(tsmi_stream_t s, const int32_t *map, int64_t n_rows, int kvol,
+                                   int window, int32_t *grouped, int32_t *row_of, int32_t *masks64,
+                                   int32_t *order64, int32_t *order128) {
+  TSMI_REQUIRE(kvol == 27, "map_group_rows: 3x3x3 maps only (kernel volume %d)", kvol);
+  const int64_t padded = tsmi_map_group_rows_padded(n_rows, window);
+  TSMI_REQUIRE(padded >= 0, "map_group_rows: bad sizes (%lld rows, windows of %d: a multiple of 128, at most %d)",
+               (long long)n_rows, window, kGroupThreads * kGroupMaxPerThread);
+  TSMI_REQUIRE(padded < (int64_t(1) << 31) / 27, "map_group_rows: too many map entries");
+  if (n_rows == 0) return TSMI_OK;
+  TSMI_REQUIRE(map && grouped && row_of && masks64 && order64 && order128, "map_group_rows: null pointer");
+  hipLaunchKernelGGL(map_group_rows_kernel, dim3((unsigned)(padded / window)), dim3(kGroupThreads), 0,
+                     (hipStream_t)s, map, n_rows, window, grouped, row_of, masks64);
+  hipLaunchKernelGGL(group_tile_order_kernel, dim3(1), dim3(kGroupThreads), 0, (hipStream_t)s, masks64,
+                     (int)(padded / 64), order64, order128);
+  return check_launch("tsmi_map_group_rows");
+}
+
 extern "C" int64_t tsmi_wgrad_pairs_capacity(int64_t n_rows, int kvol) {
   if (n_rows < 0 || kvol < 1) return 0;
   return n_rows * kvol + (int64_t)kvol * (kWgradPairStep - 1);

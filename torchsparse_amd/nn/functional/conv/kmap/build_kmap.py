@@ -194,6 +194,8 @@ def build_kernel_map(_coords: torch.Tensor, input_node_num: int,
             in_table = backend.GPUHashTable(hashmap_keys, hashmap_vals)
     else:
         # table over the input coordinates: reuse or build
+        if subm and mode == "hashmap_on_the_fly":
+            backend.strided_lookahead(_coords)  # (a caller's rows whose order is not known yet take this path)
         if fresh and subm and (mode == "hashmap_on_the_fly" or all(k % 2 == 1 for k in kernel_size)):
             # table and map in one call (an even kernel in "hashmap" mode is centred differently)
             in_table, out_in_map = backend.GPUHashTable.build_subm(coords, kernel_size, backends.hash_rsv_ratio)
