@@ -1,12 +1,16 @@
 """Benchmark of the sparse-convolution forward hot path on one MI355X.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-layers] [--no-backward] [--no-tune] [--no-pointops] [--no-configs]
+  python bench.py --summarize DIR     (no GPU: rocprofv3 output -> profiles/)
 
 One step = one MinkUNet (SparseResUNet42 + 19-class linear head) forward in fp16 on a
-synthetic 64-beam LiDAR scan (~90k voxels, 4 input channels), starting from a fresh
-SparseTensor, so every step rebuilds its 9 kernel maps.  Inputs and weights are
-resident in HBM before the timed region.  The network runs in inference form:
-eval-mode BatchNorm folded into the convolutions, ReLU and shortcut adds in the
+synthetic 64-beam LiDAR scan (~90k voxels, 4 input channels), starting from a coordinate
+tensor the library has not seen (a device copy of the resident scan, queued in the step) and a
+fresh SparseTensor: every step pays the first-sight check of the rows and rebuilds its 9 kernel
+maps.  Scan, features and weights are resident in HBM before the timed region.  The same loop
+over one and the same coordinate tensor, and over new tensors that were complete beforehand and
+are declared so (backend.rows_ready), is reported in `config`.  The network runs in inference
+form: eval-mode BatchNorm folded into the convolutions, ReLU and shortcut adds in the
 convolution epilogues (nn.utils.fuse_inference; same function, checked in the tests);
 the unfused module-by-module time is reported beside it.  Prints ONE JSON line.
 
@@ -65,6 +69,10 @@ def parse():
     ap.add_argument("--dense-deep", action="store_true",
                     help="run the small wide layers as a dense pass over the map instead of over pair "
                          "segments (for the counter passes that compare the two forms)")
+    ap.add_argument("--summarize", default=None, metavar="DIR",
+                    help="no GPU work: turn the rocprofv3 output of the passes listed in "
+                         "profiles/*.md (DIR/kt, DIR/pmc_fetch, DIR/pmc_write, DIR/pmc_sq, DIR/bench.json) "
+                         "into profiles/*.md and profiles/roofline_traffic.json")
     ap.add_argument("--sorted", type=int, default=-1,
                     help="1: run the implicit GEMM over row-sorted maps (conv_mode 1); 0: unsorted; "
                          "-1: the default of this benchmark")
@@ -106,12 +114,20 @@ def kmap_bytes_down(n, n_out, n_out_pad, cap, cand, kvol):
 
 # HBM bytes per launch of the roofline kernel from hardware counters (FETCH_SIZE and
 # WRITE_SIZE passes of `rocprofv3 --pmc ... -- python bench.py --pmc-target KERNEL`, each scaled
-# by what the same counter reads for the 256 MiB copy of that run), keyed by the kernel
-# description this script prints.  None when the kernel that dominates has not been
-# measured that way.
-PMC_TRAFFIC_BYTES = {
-    "igemm k(3, 3, 3) s(1, 1, 1) 96->96 level(1, 1, 1) n_out=89834 nnz=505724": 52499060,
-}
+# by what the same counter reads for the 256 MiB copy of that run): `bench.py --summarize DIR`
+# writes them, keyed by the kernel description this script prints, into this file next to the
+# summaries the figures come from.  No entry for the kernel that dominates: `traffic` is null.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "roofline_traffic.json")
+MARKER_ELEMS = 31337  # an int16 fill of this many elements brackets the timed loop in a kernel trace
+
+
+def pmc_traffic_bytes(desc):
+    try:
+        with open(TRAFFIC_FILE) as f:
+            entry = json.load(f).get(desc)
+    except (OSError, ValueError):
+        return None
+    return None if entry is None else int(entry["fetch_bytes"] + entry["write_bytes"])
 
 
 def roofline_of(flops, nbytes, ms):
@@ -339,14 +355,28 @@ def other_configs(ts, spnn, F, backend):
     nnz = int((km["out_in_map"][:n] >= 0).sum().item())
     x = torch.randn(n, 256, device="cuda", dtype=torch.float16)
     w = torch.randn(27, 256, 256, device="cuda", dtype=torch.float16) * 0.02
+    setting, backend.igemm_group_rows = backend.igemm_group_rows, False
     t = event_ms(lambda: backend.conv_forward_implicit_gemm_cuda(x, w, km["out_in_map"], n, 256), iters=5)
+    # the same layer over the grouped copy of the map (rows counting-sorted by kernel planes inside
+    # windows, tiles heaviest first), and what building that copy takes
+    backend.igemm_group_rows = "always"
+    omap = km["out_in_map"]
+
+    def regroup():
+        backend._grouped_of.pop(id(omap), None)
+        backend.grouped_map(omap, n)
+    t_group = event_ms(regroup, iters=5)
+    t_grouped = event_ms(lambda: backend.conv_forward_implicit_gemm_cuda(x, w, omap, n, 256), iters=5)
+    backend.igemm_group_rows = setting
     t_sorted = event_ms(lambda: backend.conv_forward_implicit_gemm_sorted_cuda(
         x, w, km["reorder_out_in_map"], km["reduced_sorted_mask"], km["reorder_loc"], n, 256), iters=5)
     flops = 2.0 * nnz * 256 * 256
     out["subm_k3_256_256_1M"] = {
         "voxels": n, "nnz": nnz, "kmap_ms": round(t_map, 4), "kmap_with_sort_products_ms": round(t_map_sorted, 4),
         "conv_ms": round(t, 4), "eff_TFLOPs": round(flops / (t * 1e-3) / 1e12, 1),
-        "conv_sorted_ms": round(t_sorted, 4), "sorted_eff_TFLOPs": round(flops / (t_sorted * 1e-3) / 1e12, 1)}
+        "conv_sorted_ms": round(t_sorted, 4), "sorted_eff_TFLOPs": round(flops / (t_sorted * 1e-3) / 1e12, 1),
+        "group_rows_ms": round(t_group, 4), "conv_grouped_ms": round(t_grouped, 4),
+        "grouped_eff_TFLOPs": round(flops / (t_grouped * 1e-3) / 1e12, 1)}
     return out
 
 
@@ -435,7 +465,11 @@ def dominant_layer_roofline(ts, F, records, caches, pmc_target=None):
         w = r["mod"].kernel.detach()
         run = (lambda x=x, w=w, omap=omap, n_out=r["n_out"], cout=cout:
                backend.conv_forward_implicit_gemm_cuda(x, w, omap, n_out, cout))
+        # as a step with rebuilt maps runs it: rows in coordinate order (a map's grouped copy is
+        # built only once the map has been used about ten times, see backend.igemm_group_rows)
+        setting, backend.igemm_group_rows = backend.igemm_group_rows, False
         ms = event_ms(run, iters=30, warm=5)
+        backend.igemm_group_rows = setting
         total = ms * len(rs)
         kvol = ks[0] * ks[1] * ks[2]
         nnz = int((omap[:r["n_out"]] >= 0).sum().item())
@@ -447,11 +481,19 @@ def dominant_layer_roofline(ts, F, records, caches, pmc_target=None):
         one = roofline_of(flops, nbytes, ms)
         form = ("pair segments (segment_products_kernel + segment_sum_kernel)"
                 if backend._segments_pay(x, kvol, cin, cout, r["n_out"], omap) else "dense pass over the map")
+        share = None
+        if form.startswith("dense") and backend._grouping_fits(x, kvol, cin, cout, r["n_out"]):
+            # the same layer over the grouped copy of its map (maps kept over several forwards)
+            backend.igemm_group_rows = "always"
+            share = tile_offset_share(backend, omap, r["n_out"], w)
+            share["launch_ms_over_grouped_map"] = round(event_ms(run, iters=30, warm=5), 5)
+            backend.igemm_group_rows = setting
         every.append({"kernel": desc, "form": form, "launches_per_step": len(rs), "launch_ms": round(ms, 5),
                       "step_ms": round(ms * len(rs), 4), "bound": one["bound"],
                       "achieved": round(one["achieved"], 2), "peak": one["peak"], "unit": one["unit"],
                       "frac": round(one["frac"], 4),
-                      "dense_map_TFLOPs": round(2.0 * omap.shape[0] * kvol * cin * cout / (ms * 1e-3) / 1e12, 1)})
+                      "dense_map_TFLOPs": round(2.0 * omap.shape[0] * kvol * cin * cout / (ms * 1e-3) / 1e12, 1),
+                      **({"rows_grouped_by_kernel_planes": share} if share else {})})
         if best is None or total > best["total_ms"]:
             best = {"total_ms": total, "ms": ms, "launches": len(rs), "flops": flops, "bytes": nbytes,
                     "run": run, "issued": 2.0 * omap.shape[0] * kvol * cin * cout,
@@ -467,7 +509,7 @@ def dominant_layer_roofline(ts, F, records, caches, pmc_target=None):
         torch.cuda.synchronize()
         return {"kernel": best["desc"]}
     roof = roofline_of(best["flops"], best["bytes"], best["ms"])
-    roof["traffic"] = PMC_TRAFFIC_BYTES.get(best["desc"])
+    roof["traffic"] = pmc_traffic_bytes(best["desc"])
     if roof["traffic"] is None:
         roof["traffic_note"] = "no FETCH_SIZE / WRITE_SIZE pass recorded for this kernel and shape"
     roof["kernel"] = best["desc"]
@@ -486,6 +528,22 @@ def dominant_layer_roofline(ts, F, records, caches, pmc_target=None):
     roof["frac"] = round(roof["frac"], 4)
     roof["measured_on_this_gpu"] = achievable_peaks()
     return roof
+
+
+def tile_offset_share(backend, omap, n_out, w):
+    """(wavefront of 32 rows, kernel offset) blocks a dense pass multiplies, as a share of all of
+    them: over the rows in coordinate order, and over the grouped copy of the map the layer
+    runs on."""
+    valid = (omap[:n_out] >= 0)
+    pad = (-n_out) % 32
+    if pad:
+        valid = torch.cat([valid, torch.zeros((pad, valid.shape[1]), dtype=torch.bool, device=valid.device)])
+    natural = float(valid.view(-1, 32, valid.shape[1]).any(1).float().mean())
+    g = backend.grouped_map(omap, n_out)
+    gv = g.grouped >= 0
+    grouped = float(gv.view(-1, 32, gv.shape[1]).any(1).float().sum() / (valid.shape[0] // 32 * valid.shape[1]))
+    return {"wavefront_offset_blocks_multiplied_coordinate_order": round(natural, 3),
+            "wavefront_offset_blocks_multiplied_grouped": round(grouped, 3)}
 
 
 def pmc_kernels(ts, spnn, F, backend, coords, n):
@@ -639,8 +697,168 @@ def cpu_baseline(records, level_coords):
             "kmap_ms": round(t_map * 1e3, 1), "conv_ms": round(t_conv * 1e3, 1)}
 
 
+def _short_kernel(name):
+    import re
+    n = name.replace("(anonymous namespace)::", "")
+    n = re.sub(r"\(.*", "", n)
+    n = n.replace("void ", "").replace("tsmi::f16::", "").replace("tsmi::", "")
+    n = n.replace("rocprim::ROCPRIM_400200_NS::detail::", "rocprim::")
+    m = re.match(r"_ZN4tsmi3f16\d+([a-z_0-9]+?)E", n)
+    if m:
+        n = m.group(1)
+    return n[:70]
+
+
+def summarize(meas):
+    """No GPU work: the rocprofv3 output under ``meas`` (written by the commands quoted in the
+    summaries) -> profiles/bench_minkunet_kernel_trace.md, profiles/igemm_roofline_kernel_pmc.md,
+    profiles/roofline_traffic.json."""
+    import collections
+    import csv
+    import re
+    prof = os.path.join(ROOT, "profiles")
+    bench = json.loads(open(os.path.join(meas, "bench.json")).read())
+    roof = bench["roofline"]
+    desc = roof["kernel"]
+    steps, warmup = bench["steps"], bench["warmup"]
+
+    # ---- kernel trace: stats, and the timed loop between the two marker fills ----
+    rows = list(csv.DictReader(open(os.path.join(meas, "kt", "kt_kernel_stats.csv"))))
+    out = ["# rocprofv3 kernel trace of bench.py (MinkUNet fp16 forward, %d-voxel synthetic scan)\n" % bench["config"]["voxels"],
+           "Command (from the repository root on one MI355X; `cd /tmp && export TMPDIR=/tmp` first), then "
+           "`python bench.py --summarize gpurun_out/meas` for this file:\n",
+           "```\nrocprofv3 --kernel-trace --stats --output-format csv -d gpurun_out/meas/kt -o kt -- python bench.py "
+           f"--steps {steps} --warmup {warmup} --no-cpu --no-layers --no-backward --no-tune --no-pointops --no-configs\n```\n",
+           "The process also runs the unfused network, the same-tensor and resident-tensor loops, warm-map forwards and the "
+           "per-group roofline timing, so `calls` mixes those phases; the second table isolates the timed loop "
+           "(the kernels between the two int16 marker fills that bracket it).\n",
+           "## Kernel stats of the whole process (top 24 by total time)\n",
+           "| kernel | calls | total µs | avg µs | % |\n|---|---:|---:|---:|---:|"]
+    for r in rows[:24]:
+        out.append(f"| `{_short_kernel(r['Name'])}` | {r['Calls']} | {float(r['TotalDurationNs']) / 1e3:.0f} | "
+                   f"{float(r['AverageNs']) / 1e3:.1f} | {float(r['Percentage']):.2f} |")
+    tr = list(csv.DictReader(open(os.path.join(meas, "kt", "kt_kernel_trace.csv"))))
+    tr.sort(key=lambda r: int(r["Start_Timestamp"]))
+    marks = [i for i, r in enumerate(tr) if "FillFunctor<short>" in r["Kernel_Name"]]
+    assert len(marks) == 2, f"expected the two marker fills around the timed loop, found {len(marks)}"
+    seg = tr[marks[0] + 1:marks[1]]
+    streams = collections.Counter(r["Stream_Id"] for r in seg)
+    main = streams.most_common(1)[0][0]
+    per = collections.defaultdict(lambda: [0, 0.0, 0.0])
+    busy = {True: 0.0, False: 0.0}
+    count = {True: 0, False: 0}
+    for r in seg:
+        n = _short_kernel(r["Kernel_Name"])
+        if n.startswith("Cijk"):
+            n = "hipBLASLt GEMM (linear head)"
+        elif n.startswith("rocprim"):
+            n = "rocprim (sort / select / scan)"
+        elif n.startswith("at::native") or n.startswith("__amd"):
+            n = "torch elementwise / copy / fill / cat"
+        dur = (int(r["End_Timestamp"]) - int(r["Start_Timestamp"])) / 1e3
+        on_main = r["Stream_Id"] == main
+        per[n][0] += 1
+        per[n][1 if on_main else 2] += dur
+        busy[on_main] += dur
+        count[on_main] += 1
+    wall = (int(seg[-1]["End_Timestamp"]) - int(seg[0]["Start_Timestamp"])) / 1e3
+    out.append(f"\n## The timed loop: {steps} steps (fused network, a new coordinate tensor and 9 kernel maps every step), per step\n")
+    out.append(f"{len(seg) / steps:.1f} kernels per step; kernel time {(busy[True] + busy[False]) / steps:.0f} µs per step, of it "
+               f"{busy[True] / steps:.0f} µs ({count[True] / steps:.1f} kernels) on the caller's stream and "
+               f"{busy[False] / steps:.0f} µs ({count[False] / steps:.1f} kernels) on the library's second stream; "
+               f"first kernel to last {wall / steps:.0f} µs per step; `ms_per_step` of this run "
+               f"{bench['ms_per_step'] * 1e3:.0f} µs.\n")
+    out.append("| kernel | launches / step | µs / step, caller's stream | µs / step, second stream |\n|---|---:|---:|---:|")
+    for k, v in sorted(per.items(), key=lambda kv: -(kv[1][1] + kv[1][2])):
+        out.append(f"| `{k}` | {v[0] / steps:.1f} | {v[1] / steps:.1f} | {v[2] / steps:.1f} |")
+    out.append("\n`igemm2_kernel<MF,NT,KS,OS>`: MF·64 output rows × NT·16 output channels per workgroup, KS·64 bytes of input "
+               "channels and OS kernel offsets per reduction step; `tile_kernel<..,WM,WN,KS,ST>`: 32·WM rows × 32·WN channels, "
+               "ST-stage LDS ring; `map_group_rows_kernel` / `group_tile_order_kernel`: the grouped copy of a level's 3×3×3 map.")
+    open(os.path.join(prof, "bench_minkunet_kernel_trace.md"), "w").write("\n".join(out) + "\n")
+
+    # ---- counters of the roofline kernel ----
+    def counter_rows(sub, stem):
+        path = os.path.join(meas, sub, stem + "_counter_collection.csv")
+        rs = list(csv.DictReader(open(path)))
+        rs.sort(key=lambda r: int(r["Dispatch_Id"]))
+        return rs
+
+    def last5(rs, ctr):
+        vals = [(r["Kernel_Name"], float(r["Counter_Value"]), int(r["Grid_Size"]),
+                 int(r["End_Timestamp"]) - int(r["Start_Timestamp"])) for r in rs if r["Counter_Name"] == ctr]
+        tgt = [v for v in vals if re.search(r"igemm2?_kernel|tile_kernel|segment_products", v[0])][-5:]
+        cp = [v for v in vals if "copyBuffer" in v[0] and v[2] == 131072][-5:]
+        return tgt, cp
+
+    avg = lambda v, i=1: sum(x[i] for x in v) / len(v)  # noqa: E731
+    ft, fc = last5(counter_rows("pmc_fetch", "f"), "FETCH_SIZE")
+    wt, wc = last5(counter_rows("pmc_write", "w"), "WRITE_SIZE")
+    kib = 256 * 1024
+    f_fac, w_fac = kib / avg(fc), kib / avg(wc)
+    fetch, write = avg(ft) * f_fac, avg(wt) * w_fac
+    kname = _short_kernel(ft[0][0])
+    o = ["# Hardware counters of the roofline kernel\n", f"Kernel: `{kname}` — {desc}\n",
+         "Commands (one pass per run; `bench.py --pmc-target KERNEL` launches a 256 MiB device-to-device copy five times "
+         "and then the kernel five times), then `python bench.py --summarize gpurun_out/meas`:\n",
+         f"```\nrocprofv3 --pmc FETCH_SIZE --output-format csv -d gpurun_out/meas/pmc_fetch -o f -- python bench.py --pmc-target \"{desc}\"\n"
+         f"rocprofv3 --pmc WRITE_SIZE --output-format csv -d gpurun_out/meas/pmc_write -o w -- python bench.py --pmc-target \"{desc}\"\n"
+         "rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES SQ_INSTS_VALU_MFMA_MOPS_F16 SQ_WAIT_INST_ANY SQ_ACTIVE_INST_LDS SQ_WAVE_CYCLES "
+         f"SQ_BUSY_CYCLES GRBM_GUI_ACTIVE --output-format csv -d gpurun_out/meas/pmc_sq -o q -- python bench.py --pmc-target \"{desc}\"\n```\n",
+         "## HBM traffic\n",
+         "| counter (KiB per dispatch) | 256 MiB copy reads | scale to true KiB | kernel reads | kernel, scaled |\n|---|---:|---:|---:|---:|",
+         f"| FETCH_SIZE | {avg(fc):.0f} | {f_fac:.3f} | {avg(ft):.0f} | {fetch:.0f} |",
+         f"| WRITE_SIZE | {avg(wc):.0f} | {w_fac:.3f} | {avg(wt):.0f} | {write:.0f} |"]
+    tot = (fetch + write) * 1024
+    o.append(f"\nHBM traffic per launch: {tot / 1e6:.1f} MB ({fetch * 1024 / 1e6:.1f} read + {write * 1024 / 1e6:.1f} written); "
+             f"algorithmic bytes {roof['algorithmic_bytes'] / 1e6:.1f} MB, algorithmic flops {roof['algorithmic_flops'] / 1e9:.2f} G; "
+             f"launch duration by HIP events in bench.py {roof['launch_ms'] * 1e3:.1f} µs "
+             f"({avg(ft, 3) / 1e3:.1f} µs under the counter pass).")
+    sq_path = os.path.join(meas, "pmc_sq", "q_counter_collection.csv")
+    if os.path.exists(sq_path):
+        rs = counter_rows("pmc_sq", "q")
+        names = ["SQ_VALU_MFMA_BUSY_CYCLES", "SQ_INSTS_VALU_MFMA_MOPS_F16", "SQ_WAIT_INST_ANY", "SQ_ACTIVE_INST_LDS",
+                 "SQ_WAVE_CYCLES", "SQ_BUSY_CYCLES", "GRBM_GUI_ACTIVE"]
+        got = {}
+        dur_ns = None
+        for nm in names:
+            tgt, _ = last5(rs, nm)
+            if tgt:
+                got[nm] = avg(tgt)
+                dur_ns = avg(tgt, 3)
+        o.append("\n## Matrix pipe, LDS and waiting (per launch, summed over the device)\n")
+        o.append("| counter | value |\n|---|---:|")
+        for nm in names:
+            if nm in got:
+                o.append(f"| {nm} | {got[nm]:.4g} |")
+        if "SQ_VALU_MFMA_BUSY_CYCLES" in got and "GRBM_GUI_ACTIVE" in got:
+            simd_cycles = got["GRBM_GUI_ACTIVE"] * 1024  # 256 CUs x 4 SIMDs
+            o.append(f"\nMatrix pipe busy {100 * got['SQ_VALU_MFMA_BUSY_CYCLES'] / simd_cycles:.1f} % of the SIMD cycles "
+                     f"(SQ_VALU_MFMA_BUSY_CYCLES ÷ (GRBM_GUI_ACTIVE × 1024 SIMDs)); kernel duration under this pass "
+                     f"{dur_ns / 1e3:.1f} µs.")
+        if "SQ_INSTS_VALU_MFMA_MOPS_F16" in got:
+            # one count = 512 multiply-adds... report raw and the flops it stands for (MOPS counts units of 512 flops)
+            o.append(f"fp16 matrix operations counted: {got['SQ_INSTS_VALU_MFMA_MOPS_F16']:.4g} × 512 flop = "
+                     f"{got['SQ_INSTS_VALU_MFMA_MOPS_F16'] * 512 / 1e9:.2f} GFLOP executed, against {roof['algorithmic_flops'] / 1e9:.2f} "
+                     f"GFLOP of pairs and {roof['dense_map_flops'] / 1e9:.2f} GFLOP of the whole map.")
+        if "SQ_WAIT_INST_ANY" in got and "SQ_WAVE_CYCLES" in got:
+            o.append(f"Wavefronts wait for an instruction {100 * got['SQ_WAIT_INST_ANY'] / got['SQ_WAVE_CYCLES']:.0f} % of "
+                     f"their cycles; LDS instructions are active {100 * got.get('SQ_ACTIVE_INST_LDS', 0) / got['SQ_WAVE_CYCLES']:.0f} %.")
+    open(os.path.join(prof, "igemm_roofline_kernel_pmc.md"), "w").write("\n".join(o) + "\n")
+    try:
+        table = json.load(open(TRAFFIC_FILE))
+    except (OSError, ValueError):
+        table = {}
+    table[desc] = {"fetch_bytes": int(fetch * 1024), "write_bytes": int(write * 1024), "kernel": kname,
+                   "copy_scale_fetch": round(f_fac, 4), "copy_scale_write": round(w_fac, 4)}
+    json.dump(table, open(TRAFFIC_FILE, "w"), indent=1, sort_keys=True)
+    print(desc, int(tot))
+
+
 def main():
     args = parse()
+    if args.summarize:
+        summarize(args.summarize)
+        return
     if args.gpus != 1:
         print(f"bench.py measures one GPU only (got --gpus {args.gpus}); nothing in this path "
               "communicates between GPUs", file=sys.stderr)
@@ -670,21 +888,43 @@ def main():
     if args.dense_deep:
         backend.igemm_through_segments = False
 
-    def timed(net, steps, warmup, fresh_coords=False):
+    def timed(net, steps, warmup, rows="new", mark=False):
+        """ms per forward.  rows = "new": a coordinate tensor the library has not seen, every step
+        (a device copy queued in the step: what a loader that hands over one scan after the
+        other amounts to; the library checks its range and row order - one small kernel and
+        one read-back - and every kernel map is rebuilt); "resident": a new tensor every step
+        that was complete before the loop and is declared so (backend.rows_ready), so its
+        check is not read back at once; "same": the same tensor every step (the check is
+        remembered, the strided chain runs ahead on the second stream; the maps are rebuilt)."""
+        pool = [coords.clone() for _ in range(steps + warmup)] if rows == "resident" else None
+        k = [0]
+
         def step():
             with torch.no_grad():
-                # a coordinate tensor is checked (range, row order: one small kernel and one
-                # read-back) the first time the library sees it; fresh_coords pays that every step
-                x = ts.SparseTensor(feats, coords.clone() if fresh_coords else coords)
-                return head(net(x)[-1].feats)
+                if rows == "new":
+                    c = coords.clone()
+                elif rows == "resident":
+                    c = backend.rows_ready(pool[k[0]])
+                    k[0] += 1
+                else:
+                    c = coords
+                return head(net(ts.SparseTensor(feats, c))[-1].feats)
         for _ in range(warmup):
             step()
         torch.cuda.synchronize()
+        marker = torch.empty(MARKER_ELEMS, dtype=torch.int16, device="cuda") if mark else None
+        if mark:
+            marker.fill_(1)  # (brackets the timed loop in a kernel trace)
         t0 = time.perf_counter()
         for _ in range(steps):
             step()
         torch.cuda.synchronize()
-        return (time.perf_counter() - t0) * 1e3 / steps
+        ms = (time.perf_counter() - t0) * 1e3 / steps
+        if mark:
+            marker.fill_(2)
+            torch.cuda.synchronize()
+        backend.settle_checks()
+        return ms
 
     if args.pmc_kernels:
         pmc_kernels(ts, spnn, F, backend, coords, n)
@@ -700,9 +940,10 @@ def main():
     # the secondary figures first: the clocks, the allocator and the library's own look-ahead
     # state settle over the first few dozen forwards of a process (the headline loop measured
     # first reads ~5 % higher than the same loop a moment later)
-    ms_unfused = timed(unfused, max(args.steps // 2, 1), 2)
-    ms_fresh = timed(model, args.steps, 2, fresh_coords=True)
-    ms_per_step = timed(model, args.steps, args.warmup)
+    ms_unfused = timed(unfused, max(args.steps // 2, 1), 2, rows="same")
+    ms_same = timed(model, args.steps, args.warmup, rows="same")
+    ms_resident = timed(model, args.steps, args.warmup, rows="resident")
+    ms_per_step = timed(model, args.steps, args.warmup, rows="new", mark=True)
 
     with torch.no_grad():
         inp = ts.SparseTensor(feats, coords)
@@ -732,8 +973,8 @@ def main():
                           save_dir=tmp, tune_tag="bench", verbose=False, skip_warning=True,
                           dataflow_range=[F.Dataflow.ImplicitGEMM, F.Dataflow.FetchOnDemand,
                                           F.Dataflow.GatherScatter])
-        tuned = {"ms_per_step": round(timed(tuned_model, args.steps, args.warmup), 4),
-                 "default_ms_per_step": round(timed(model, args.steps, args.warmup), 4),
+        tuned = {"ms_per_step": round(timed(tuned_model, args.steps, args.warmup, rows="same"), 4),
+                 "default_ms_per_step": round(timed(model, args.steps, args.warmup, rows="same"), 4),
                  "groups": [{"level": g[0], "kernel": g[1], "stride": g[2],
                              "dataflow": c["dataflow"].name, "ifsort": c["ifsort"],
                              "split_mask_num": c["split_mask_num"]} for g, c in chosen.items()]}
@@ -746,11 +987,12 @@ def main():
         "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": "MinkUNet (SparseResUNet42, cr=1.0) + Linear(96,19) forward, batch 1, "
                                f"synthetic 64-beam scan seed 1, {n} voxels, 4 input channels, "
-                               "kernel maps rebuilt every step",
+                               "a new coordinate tensor (checked on first sight) and 9 kernel maps every step",
                    "voxels": n, "warm_map_ms_per_step": round(warm_ms, 4),
                    "warm_map_graph_replay_ms_per_step": round(graph_ms, 4),
                    "unfused_ms_per_step": round(ms_unfused, 4),
-                   "fresh_coordinate_tensor_ms_per_step": round(ms_fresh, 4),
+                   "same_coordinate_tensor_ms_per_step": round(ms_same, 4),
+                   "resident_new_coordinate_tensor_declared_ready_ms_per_step": round(ms_resident, 4),
                    "conv_mode": F.get_conv_mode().value},
         "roofline": roof, "roofline_kmap": roof_kmap, "cpu_baseline": cpu, "layers": layers,
         "backward": backward,

@@ -130,7 +130,8 @@ def test_grouped_convolution_equals_the_plain_one_and_the_oracle(mods, cin, cout
     w = (torch.randn(27, cin, cout, device="cuda") * (2.0 / (27 * cin)) ** 0.5).to(dtype)
     bias = torch.randn(cout, device="cuda", dtype=dtype)
     res = torch.randn(n, cout, device="cuda", dtype=dtype)
-    assert backend._grouping_pays(x, 27, cin, cout, n)
+    monkeypatch.setattr(backend, "igemm_group_rows", "always")
+    assert backend._grouping_pays(x, 27, cin, cout, n, omap)
     got = backend.conv_forward_implicit_gemm_cuda(x, w, omap, n, cout, bias=bias, residual=res, relu=True)
     assert id(omap) in backend._grouped_of  # the grouped copy was built and kept with the map
     monkeypatch.setattr(backend, "igemm_group_rows", False)
@@ -154,6 +155,7 @@ def test_scan_layers_run_over_the_grouped_map(mods, monkeypatch):
     torch.manual_seed(3)
     layer = spnn.Conv3d(32, 48, 3).cuda().half()
     x = torch.randn(n, 32, device="cuda", dtype=torch.float16)
+    monkeypatch.setattr(backend, "igemm_group_rows", "always")
     with torch.no_grad():
         a = layer(ts.SparseTensor(x, coords))
         omap = a._caches.kmaps[((1, 1, 1), (3, 3, 3), (1, 1, 1), (1, 1, 1))]["out_in_map"]
@@ -169,3 +171,23 @@ def test_scan_layers_run_over_the_grouped_map(mods, monkeypatch):
     masks = g.masks64.cpu().numpy().astype(np.int64)
     grouped = np.array([bin(int(a | b)).count("1") for a, b in zip(masks[0::2], masks[1::2])]).mean()
     assert natural > 24 and grouped < 0.6 * natural
+
+
+def test_a_map_is_grouped_once_it_has_been_used_often_enough(mods, monkeypatch):
+    """With the default setting the copy is built at the group_after_uses-th eligible layer over the
+    same map tensor, not before; every call computes the same features."""
+    backend, F = mods
+    rng = np.random.default_rng(77)
+    coords = lidar_like_coords(rng, 36000, extent=(700, 700, 40))
+    n = len(coords)
+    omap = dev(oracle.kmap_subm(coords, 3))
+    x = torch.randn(n, 32, device="cuda", dtype=torch.float16)
+    w = torch.randn(27, 32, 32, device="cuda", dtype=torch.float16) * 0.05
+    monkeypatch.setattr(backend, "igemm_group_rows", True)
+    monkeypatch.setattr(backend, "group_after_uses", 4)
+    outs = []
+    for use in range(1, 7):
+        outs.append(backend.conv_forward_implicit_gemm_cuda(x, w, omap, n, 32))
+        assert (id(omap) in backend._grouped_of) == (use >= 4)
+    for y in outs[1:]:
+        assert torch.equal(y, outs[0])

@@ -1524,15 +1524,22 @@ _sparse_maps = {}     # id(map) -> weak reference: maps over rows known to have 
 _hint_lock = threading.Lock()  # guards the two tables above and _segments_of
 
 
-# Large 3x3x3 layers of the implicit-GEMM dataflow run over a copy of the map whose rows are
+# Large 3x3x3 layers of the implicit-GEMM dataflow can run over a copy of the map whose rows are
 # grouped, inside windows of consecutive rows, by the planes of the kernel they use
 # (tsmi_map_group_rows): a row tile then multiplies about half as many kernel offsets as a tile
 # of rows in coordinate order (a surface scan: 25 of 27 offsets per 128-row tile in coordinate
-# order, 14 grouped), and the tiles run heaviest first.  The copy is built by one launch the
-# first time a map is used that way and kept with it.  False: every layer in coordinate order.
+# order, 14 grouped), and the tiles run heaviest first.  Building the copy takes four launches
+# (about 20 us of kernels and 12 us of host time for a 90k-row map) and a layer gains 2 - 7 us
+# from it (96 -> 96 channels at 90k rows: 49 -> 42 us), so it pays from about the tenth layer
+# that runs over the same map tensor on: maps kept over several forwards (cached kernel maps, a
+# model applied again to the same SparseTensor), not the five to eight layers that share a map
+# inside one forward.  True: a map's copy is built at its group_after_uses-th eligible use and
+# used from then on; "always": at the first; False: never.
 igemm_group_rows = True
 group_window = 8192      # rows per window (a multiple of 128, at most 8192)
 group_min_rows = 32768   # smaller maps have too few tiles for the order to matter
+group_after_uses = 10
+_group_uses = {}  # id(map) -> [weak reference, version, address, eligible uses so far]
 
 _grouped_of = {}  # id(map) -> (weak reference, version, address, stream, rows, window, GroupedMap)
 
@@ -1602,13 +1609,36 @@ def grouped_map(out_in_map: torch.Tensor, n_rows: int, window: Optional[int] = N
     return g
 
 
-def _grouping_pays(x, kvol: int, cin: int, cout: int, num_out_feats: int) -> bool:
-    """Layers that run over the grouped map: 3x3x3, enough rows for several hundred tiles, 16-bit
-    or 32-bit features in whole 16-byte pieces, and a channel count the one-column-tile kernels
-    cover (wider layers of fewer than 65536 rows run the tiled kernel, which keeps its order)."""
+def _grouping_fits(x, kvol: int, cin: int, cout: int, num_out_feats: int) -> bool:
+    """Layers that can run over the grouped map: 3x3x3, enough rows for several hundred tiles,
+    features in whole 16-byte pieces, and a channel count the one-column-tile kernels cover
+    (wider layers of fewer than 65536 rows run the tiled kernel, which keeps its order)."""
     return bool(igemm_group_rows and kvol == 27 and num_out_feats >= group_min_rows
                 and cin > 8 and (cin * x.element_size()) % 16 == 0
                 and (cout < 128 or num_out_feats >= 65536))
+
+
+def _grouping_pays(x, kvol: int, cin: int, cout: int, num_out_feats: int, out_in_map=None) -> bool:
+    """Whether this call runs over the grouped copy of ``out_in_map``: an eligible layer, and a
+    map that has been used often enough for the copy to pay (or has its copy already)."""
+    if not _grouping_fits(x, kvol, cin, cout, num_out_feats):
+        return False
+    if igemm_group_rows == "always" or out_in_map is None:
+        return True
+    key = id(out_in_map)
+    if key in _grouped_of and _grouped_of[key][0]() is out_in_map:
+        return True
+    hit = _group_uses.get(key)
+    if (hit is None or hit[0]() is not out_in_map or hit[1] != out_in_map._version
+            or hit[2] != out_in_map.data_ptr()):
+        if len(_group_uses) >= 256:
+            for k in [k for k, v in _group_uses.items() if v[0]() is None]:
+                del _group_uses[k]
+            if len(_group_uses) >= 256:
+                _group_uses.clear()
+        hit = _group_uses[key] = [weakref.ref(out_in_map), out_in_map._version, out_in_map.data_ptr(), 0]
+    hit[3] += 1
+    return hit[3] >= group_after_uses
 
 
 def conv_implicit_gemm_grouped(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias=None,
@@ -1707,7 +1737,7 @@ def _implicit_gemm(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias=None,
     if _segments_pay(x, kvol, cin, cout, num_out_feats, out_in_map, segments):
         return conv_implicit_gemm_segments(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias,
                                            residual, relu)
-    if _grouping_pays(x, kvol, cin, cout, num_out_feats):
+    if _grouping_pays(x, kvol, cin, cout, num_out_feats, out_in_map):
         return conv_implicit_gemm_grouped(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias,
                                           residual, relu)
     y = x.new_empty(num_out_feats, cout)  # (the cheapest form of the call: 1.2 us against 1.6)

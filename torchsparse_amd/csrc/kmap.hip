@@ -1868,9 +1868,26 @@ extern "C" int tsmi_pair_segments(tsmi_stream_t s, const int32_t *map, int64_t n
 constexpr int kGroupThreads = 1024;
 constexpr int kGroupMaxPerThread = 8;  // windows of at most 8192 rows
 
+// used[row] = bit k per kernel offset the row has a neighbour at (thread per row, all CUs: a
+// workgroup per window reading whole rows would have a handful of CUs pull the map through
+// their load units row by row - 60 us for a 90k-row map, against 4 for this pass)
+__global__ __launch_bounds__(kBlock) void map_row_masks_kernel(const int32_t *__restrict__ map,
+                                                              int64_t n_rows, int32_t *__restrict__ used) {
+  const int64_t row = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (row >= n_rows) return;
+  const int32_t *m = map + row * 27;
+  int mask = 0;
+#pragma unroll
+  for (int o = 0; o < 27; ++o)
+    if (m[o] >= 0) mask |= 1 << o;
+  used[row] = mask;
+}
+
+// One workgroup per window: the counting sort of its rows by key (from their masks), row_of, and
+// the union of the masks of every 64 positions.
 __global__ __launch_bounds__(kGroupThreads) void map_group_rows_kernel(
-    const int32_t *__restrict__ map, int64_t n_rows, int window, int32_t *__restrict__ grouped,
-    int32_t *__restrict__ row_of, int32_t *__restrict__ masks64) {
+    const int32_t *__restrict__ used, int64_t n_rows, int window, int32_t *__restrict__ row_of,
+    int32_t *__restrict__ masks64) {
   __shared__ int hist[1024];
   __shared__ int offs[1024];
   __shared__ int lmask[kGroupThreads * kGroupMaxPerThread];
@@ -1878,35 +1895,29 @@ __global__ __launch_bounds__(kGroupThreads) void map_group_rows_kernel(
   const int64_t base = (int64_t)blockIdx.x * window;
   hist[tid] = 0;
   __syncthreads();
-  int key[kGroupMaxPerThread], used[kGroupMaxPerThread];
+  int key[kGroupMaxPerThread], mine[kGroupMaxPerThread];
 #pragma unroll
   for (int j = 0; j < kGroupMaxPerThread; ++j) {
     const int r = tid + j * kGroupThreads;
     key[j] = -1;
-    used[j] = 0;
+    mine[j] = 0;
     if (r >= window) continue;
     const int64_t row = base + r;
     int k = 1023;
     if (row < n_rows) {
-      const int32_t *m = map + row * 27;
-      int planes = 0, mask = 0;
-#pragma unroll
-      for (int o = 0; o < 27; ++o) {
-        // digits of offset o (the first digit runs fastest): plane bits 0..5 = digit 0 / 2 per axis
-        constexpr int kBit[3] = {1, 0, 2};
-        const int d0 = o % 3, d1 = (o / 3) % 3, d2 = o / 9;
-        const int bits = (d0 != 1 ? kBit[d0] << 0 : 0) | (d1 != 1 ? kBit[d1] << 2 : 0) |
-                         (d2 != 1 ? kBit[d2] << 4 : 0);
-        if (m[o] >= 0) {
-          planes |= bits;
-          mask |= 1 << o;
-        }
-      }
+      const int mask = used[row];
+      // plane bits 0..5: a neighbour with digit 0 / digit 2 along axis 0, 1, 2 (the first digit of
+      // an offset runs fastest: offset o has digits o % 3, o / 3 % 3, o / 9)
+      constexpr int kD0_0 = 0x1249249, kD0_2 = 0x4924924;  // offsets with first digit 0 / 2
+      constexpr int kD1_0 = 0x01C0E07, kD1_2 = 0x70381C0;  // second digit 0 / 2
+      constexpr int kD2_0 = 0x00001FF, kD2_2 = 0x7FC0000;  // third digit 0 / 2
+      const int planes = ((mask & kD0_0) ? 1 : 0) | ((mask & kD0_2) ? 2 : 0) | ((mask & kD1_0) ? 4 : 0) |
+                         ((mask & kD1_2) ? 8 : 0) | ((mask & kD2_0) ? 16 : 0) | ((mask & kD2_2) ? 32 : 0);
       const int span = (1 + __popc(planes & 3)) * (1 + __popc(planes & 12)) * (1 + __popc(planes & 48));
       // rank of the span among 1, 2, 3, 4, 6, 8, 9, 12, 18, 27
       const int rank = span <= 4 ? span - 1 : (span == 6 ? 4 : span == 8 ? 5 : span == 9 ? 6 : span == 12 ? 7 : span == 18 ? 8 : 9);
       k = (rank << 6) | planes;
-      used[j] = mask;
+      mine[j] = mask;
     }
     key[j] = k;
     atomicAdd(&hist[k], 1);
@@ -1935,18 +1946,8 @@ __global__ __launch_bounds__(kGroupThreads) void map_group_rows_kernel(
     if (key[j] < 0) continue;
     const int64_t row = base + tid + j * kGroupThreads;
     const int slot = atomicAdd(&offs[key[j]], 1);  // < window: the bins hold `window` rows in all
-    lmask[slot] = used[j];
-    int32_t *dst = grouped + (base + slot) * 27;
-    if (row < n_rows) {
-      const int32_t *m = map + row * 27;
-#pragma unroll
-      for (int o = 0; o < 27; ++o) dst[o] = m[o];
-      row_of[base + slot] = (int32_t)row;
-    } else {
-#pragma unroll
-      for (int o = 0; o < 27; ++o) dst[o] = -1;
-      row_of[base + slot] = -1;
-    }
+    lmask[slot] = mine[j];
+    row_of[base + slot] = row < n_rows ? (int32_t)row : -1;
   }
   __syncthreads();
   // union of the offsets used by every 64 consecutive positions (window is a multiple of 128)
@@ -1957,6 +1958,20 @@ __global__ __launch_bounds__(kGroupThreads) void map_group_rows_kernel(
     for (int d = 32; d >= 1; d >>= 1) v |= __shfl_xor(v, d);
     if (lane == 0) masks64[base / 64 + g] = v;
   }
+}
+
+// grouped[p, :] = map[row_of[p], :] (all -1 for a padding position): a thread per entry, so the
+// writes are contiguous and the reads walk whole rows of the window's part of the map
+__global__ __launch_bounds__(kBlock) void map_group_copy_kernel(const int32_t *__restrict__ map,
+                                                               const int32_t *__restrict__ row_of,
+                                                               int64_t n_entries,
+                                                               int32_t *__restrict__ grouped) {
+  const int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i >= n_entries) return;
+  const unsigned p = (unsigned)i / 27u;  // (fewer than 2^31 entries: checked by the host)
+  const int o = (int)((unsigned)i - p * 27u);
+  const int32_t row = row_of[p];
+  grouped[i] = row >= 0 ? map[(int64_t)row * 27 + o] : -1;
 }
 
 // The order in which a convolution starts the T tiles of 64 (order64) or 128 (order128) rows:
@@ -2017,10 +2032,16 @@ extern "C" int tsmi_map_group_rows(tsmi_stream_t s, const int32_t *map, int64_t 
   TSMI_REQUIRE(padded < (int64_t(1) << 31) / 27, "map_group_rows: too many map entries");
   if (n_rows == 0) return TSMI_OK;
   TSMI_REQUIRE(map && grouped && row_of && masks64 && order64 && order128, "map_group_rows: null pointer");
+  // the row masks go into the first n_rows ints of `grouped` (rewritten by the copy at the end,
+  // which reads row_of and map only)
+  int32_t *used = grouped;
+  hipLaunchKernelGGL(map_row_masks_kernel, grid_for(n_rows), dim3(kBlock), 0, (hipStream_t)s, map, n_rows, used);
   hipLaunchKernelGGL(map_group_rows_kernel, dim3((unsigned)(padded / window)), dim3(kGroupThreads), 0,
-                     (hipStream_t)s, map, n_rows, window, grouped, row_of, masks64);
+                     (hipStream_t)s, used, n_rows, window, row_of, masks64);
   hipLaunchKernelGGL(group_tile_order_kernel, dim3(1), dim3(kGroupThreads), 0, (hipStream_t)s, masks64,
                      (int)(padded / 64), order64, order128);
+  hipLaunchKernelGGL(map_group_copy_kernel, grid_for(padded * 27), dim3(kBlock), 0, (hipStream_t)s, map, row_of,
+                     padded * 27, grouped);
   return check_launch("tsmi_map_group_rows");
 }
 
