@@ -185,3 +185,109 @@ def test_million_voxel_256_channel_layer(mods):
         xi = ts.SparseTensor(x1, coords)
         y = F.conv3d(xi, w, kernel_size=3, padding=1, config=cfg).feats
         assert rel_rms(y[cfg_rows].float().cpu().numpy(), want) < 1e-2, flow
+
+
+def _strided(spatial_range, ks, st, pd):
+    return (spatial_range[0],) + tuple((spatial_range[a + 1] + 2 * pd[a] - (ks[a] - 1) - 1) // st[a] + 1
+                                       for a in range(3))
+
+
+def test_detection_backbone_every_layer_against_the_oracle(mods):
+    """The fused detection backbone on one multi-sweep sample cropped to at most 80k voxels: every
+    kernel map (the submanifold maps of the four levels, the three k3 s2 maps with paddings 1, 1
+    and (0, 1, 1), the (3, 1, 1) s(2, 1, 1) map) and every generated coordinate level bit for bit
+    against the oracle, and every convolution's output against oracle.conv_implicit_gemm fed that
+    layer's own fp16 input, bias, shortcut and ReLU included: 1e-2 of the RMS of the oracle's output
+    (fp16 storage, fp32 accumulation)."""
+    ts, backend, spnn, F, synthetic = mods
+    import copy
+    from torchsparse_amd.backbones import VoxelResBackBone8x
+    from torchsparse_amd.nn.utils import fuse_inference
+    coords_np, spatial_range = synthetic.multisweep_voxels(seed=2)
+    coords_np = coords_np[coords_np[:, 0] == 0]
+    half = 720
+    while True:  # a centred square window of the (y, x) plane holding at most 80k voxels
+        sel = (np.abs(coords_np[:, 2] - 720) < half) & (np.abs(coords_np[:, 3] - 720) < half)
+        if sel.sum() <= 80_000:
+            break
+        half -= 20
+    coords_np = np.ascontiguousarray(coords_np[sel])
+    n = coords_np.shape[0]
+    assert 40_000 <= n <= 80_000, n
+    spatial_range = (1,) + tuple(spatial_range[1:])
+    torch.manual_seed(4)
+    net = VoxelResBackBone8x(in_channels=5).eval()
+    g = torch.Generator().manual_seed(5)
+    for m in net.modules():
+        if isinstance(m, torch.nn.BatchNorm1d):
+            m.running_mean.copy_(torch.randn(m.num_features, generator=g) * 0.1)
+            m.running_var.copy_(torch.rand(m.num_features, generator=g) * 0.5 + 0.25)
+            m.weight.data.copy_(torch.rand(m.num_features, generator=g) + 0.75)
+            m.bias.data.copy_(torch.randn(m.num_features, generator=g) * 0.1)
+    net = fuse_inference(copy.deepcopy(net.cuda().half()))
+    assert not any(isinstance(m, torch.nn.BatchNorm1d) for m in net.modules())  # all folded
+    feats = torch.randn(n, 5, device="cuda", dtype=torch.float16)
+    coords = torch.from_numpy(coords_np).cuda()
+
+    records = []
+
+    def hook(mod, args, kwargs, output):
+        x = args[0]
+        res = kwargs.get("residual")
+        records.append({"mod": mod, "stride": x.stride, "range": x.spatial_range, "x": x.feats.clone(),
+                        "coords": x.coords, "res": None if res is None else res.clone(),
+                        "y": output.feats.clone(), "out_coords": output.coords,
+                        "out_range": output.spatial_range})
+
+    handles = [m.register_forward_hook(hook, with_kwargs=True)
+               for m in net.modules() if isinstance(m, spnn.Conv3d)]
+    with torch.no_grad():
+        inp = ts.SparseTensor(feats, coords, spatial_range=spatial_range)
+        outs = net(inp)
+    for h in handles:
+        h.remove()
+    # 1 stem + 2 blocks x 2, then three stages of (strided + 2 blocks x 2), then the output layer
+    assert len(records) == 1 + 4 + 3 * 5 + 1
+
+    f32 = lambda t: t.detach().float().cpu().numpy()  # noqa: E731
+    maps = {}  # (input level, kernel, stride) -> (oracle map, oracle output coordinates)
+    strided_seen = []
+    worst = 0.0
+    for i, r in enumerate(records):
+        mod = r["mod"]
+        ks, st, pd = mod.kernel_size, mod.stride, mod.padding
+        c_in = r["coords"].cpu().numpy()
+        key = (r["stride"], ks, st)
+        if key not in maps:
+            if st == (1, 1, 1):
+                maps[key] = (oracle.kmap_subm(c_in, ks), c_in)
+            else:
+                out_range = _strided(r["range"], ks, st, pd)
+                assert tuple(r["out_range"]) == out_range
+                maps[key] = oracle.kmap_downsample(c_in, ks, st, pd, spatial_range=out_range)
+                strided_seen.append((ks, st, pd))
+            want_map, want_coords = maps[key]
+            got = inp._caches.kmaps[(r["stride"], ks, st, (1, 1, 1))]
+            n_out = want_coords.shape[0]
+            got_map = got["out_in_map"].cpu().numpy()
+            np.testing.assert_array_equal(got_map[:n_out], want_map[:n_out])
+            assert (got_map[n_out:] == -1).all()
+            np.testing.assert_array_equal(r["out_coords"].cpu().numpy(), want_coords)
+        want_map, want_coords = maps[key]
+        n_out = want_coords.shape[0]
+        want = oracle.conv_implicit_gemm(f32(r["x"]), f32(mod.kernel), want_map, n_out)
+        if mod.bias is not None:
+            want = want + f32(mod.bias)
+        if r["res"] is not None:
+            want = want + f32(r["res"])
+        if mod.activation == "relu":
+            want = np.maximum(want, 0)
+        assert r["y"].shape == want.shape
+        err = rel_rms(f32(r["y"]), want)
+        worst = max(worst, err)
+        assert err < 1e-2, (i, ks, st, pd, err)
+    assert strided_seen == [((3, 3, 3), (2, 2, 2), (1, 1, 1)), ((3, 3, 3), (2, 2, 2), (1, 1, 1)),
+                            ((3, 3, 3), (2, 2, 2), (0, 1, 1)), ((3, 1, 1), (2, 1, 1), (0, 0, 0))]
+    assert len(maps) == 8  # four submanifold maps (levels 1, 2, 4, 8) and the four strided ones
+    assert outs["out"].coords.shape[0] == maps[((8, 8, 8), (3, 1, 1), (2, 1, 1))][1].shape[0]
+    print(f"{n} voxels, worst layer {worst:.2e}")

@@ -37,12 +37,8 @@ def mods():
     return ts, backend, spnn, F
 
 
-@pytest.fixture(scope="module")
-def scan():
-    """The scan's coordinate levels and kernel maps as the oracle builds them."""
-    from torchsparse_amd.utils.synthetic import lidar_scan_voxels
-    coords = lidar_scan_voxels(seed=1)
-    assert 85_000 < coords.shape[0] < 100_000
+def _scan_tables(coords):
+    """The coordinate levels and kernel maps of a scan as the oracle builds them."""
     levels = {1: coords}
     down = {}
     for s in (1, 2, 4, 8):
@@ -52,6 +48,14 @@ def scan():
     subm = {s: oracle.kmap_subm(c, 3) for s, c in levels.items()}
     up = {s: oracle.transpose_map(down[s], levels[s].shape[0]) for s in down}
     return {"levels": levels, "down": down, "subm": subm, "up": up}
+
+
+@pytest.fixture(scope="module")
+def scan():
+    from torchsparse_amd.utils.synthetic import lidar_scan_voxels
+    coords = lidar_scan_voxels(seed=1)
+    assert 85_000 < coords.shape[0] < 100_000
+    return _scan_tables(coords)
 
 
 def _f32(t):
@@ -321,3 +325,65 @@ def test_minkunet_forward_on_the_scan(mods, scan):
     # the forward measured by the benchmark is deterministic: a third run gives the same bits
     _, outs3, logits3 = step()
     assert torch.equal(logits3, logits) and torch.equal(outs3[-1].feats, outs[-1].feats)
+
+
+def _check_maps(caches, outs, tables):
+    """All nine kernel maps and the coordinate levels of one forward, bit for bit."""
+    assert len(caches.kmaps) == 9
+    for s in (1, 2, 4, 8, 16):
+        np.testing.assert_array_equal(caches.kmaps[_key(s, 3, 1)]["out_in_map"].cpu().numpy(), tables["subm"][s])
+        np.testing.assert_array_equal(caches.cmaps[(s,) * 3][0].cpu().numpy(), tables["levels"][s])
+    for s in (1, 2, 4, 8):
+        got = caches.kmaps[_key(s, 2, 2)]
+        np.testing.assert_array_equal(got["out_in_map"].cpu().numpy(), tables["down"][s])
+        np.testing.assert_array_equal(got["coords"].cpu().numpy(), tables["levels"][2 * s])
+        np.testing.assert_array_equal(got["out_in_map_t"].cpu().numpy(), tables["up"][s])
+    for i, out in enumerate(outs):
+        level = (1, 2, 4, 8, 16, 8, 4, 2, 1)[i]
+        np.testing.assert_array_equal(out.coords.cpu().numpy(), tables["levels"][level])
+
+
+def test_minkunet_over_alternating_scans(mods, scan):
+    """One fused model over scan A, scan B (another scene, other row counts at every level), scan A
+    again, each as a new coordinate tensor: what the first scan left behind (the levels computed
+    ahead, the maps queued ahead, the learnt chain of strided layers, cached buffers sized for A)
+    must not reach B's result, nor B's reach A's.  Every forward: the nine maps and five levels bit
+    for bit against the oracle's for THAT scan, and the output against the whole network evaluated
+    on the CPU (3e-2 of RMS end to end, as in the test above); A's output after B equals A's
+    output before B bit for bit."""
+    ts, backend, spnn, F = mods
+    from torchsparse_amd.backbones import SparseResUNet42
+    from torchsparse_amd.nn.utils import fuse_inference
+    from torchsparse_amd.utils.synthetic import lidar_scan_voxels
+    tables = {"A": scan, "B": _scan_tables(lidar_scan_voxels(seed=7, n_azimuth=1500, n_boxes=18))}
+    sizes = {k: [t["levels"][s].shape[0] for s in (1, 2, 4, 8, 16)] for k, t in tables.items()}
+    assert all(a != b for a, b in zip(sizes["A"], sizes["B"])), sizes
+    assert sizes["B"][0] > 40_000
+    unfused = SparseResUNet42(in_channels=4).eval()
+    _randomise_norms(unfused, 3)
+    unfused = unfused.cuda().half()
+    model = fuse_inference(copy.deepcopy(unfused))
+    head = torch.nn.Linear(96, 19).cuda().half().eval()
+    torch.manual_seed(11)
+    feats = {k: torch.randn(sizes[k][0], 4, device="cuda", dtype=torch.float16) for k in tables}
+    want = {}
+    for k, t in tables.items():
+        want[k] = _OracleNet(t, spnn).forward(unfused, head, _f32(feats[k]))[0]
+
+    def step(k):
+        with torch.no_grad():
+            x = ts.SparseTensor(feats[k], torch.from_numpy(tables[k]["levels"][1]).cuda())
+            outs = model(x)
+            return x, outs, head(outs[-1].feats)
+
+    backend.release_scratch()
+    logits = {}
+    for turn, k in enumerate("AAABABBA"):
+        x, outs, got = step(k)
+        _check_maps(x._caches, outs, tables[k])
+        assert got.shape == (sizes[k][0], 19)
+        err = rel_rms(_f32(got), want[k])
+        assert err < 3e-2, (turn, k, err)
+        if k in logits:
+            assert torch.equal(got, logits[k]), (turn, k)
+        logits[k] = got

@@ -91,6 +91,50 @@ def test_unsorted_or_repeated_rows_take_the_tables():
     assert backend.coords_ascending(dev(coords[:1])) and backend.coords_ascending(dev(coords[:0]))
 
 
+def test_rows_declared_ready_are_checked_without_waiting_for_the_verdict():
+    """rows_ready(): the first map over such a tensor is built through the tables (the verdict of
+    the ordering check is still on its way), equals the oracle's, and later maps take the
+    table-free builder once the verdict has been picked up; unsorted rows keep the tables; a row
+    outside the packed range raises at the latest when settle_checks() is called."""
+    rng = np.random.default_rng(303)
+    coords = ascending(random_coords(rng, 3000, (30, 30, 12)))
+    t = backend.rows_ready(dev(coords))
+    assert backend._declared_ready(t)
+    assert not backend.coords_ascending(t)  # the verdict has not been read
+    kmap = F.build_kernel_map(t, len(coords), 3, 1, 0, mode="hashmap_on_the_fly")
+    np.testing.assert_array_equal(kmap["out_in_map"].cpu().numpy(), oracle.kmap_subm(coords, 3))
+    backend.settle_checks()
+    assert not backend._pending_verdicts and backend.coords_ascending(t)
+    kmap = F.build_kernel_map(t, len(coords), 3, 2, 1, mode="hashmap_on_the_fly")
+    assert kmap["in_hashmap"] is None  # (the table-free builder)
+    want_map, want_coords = oracle.kmap_downsample(coords, 3, 2, 1)
+    np.testing.assert_array_equal(kmap["coords"].cpu().numpy(), want_coords)
+    np.testing.assert_array_equal(kmap["out_in_map"].cpu().numpy(), want_map)
+
+    swapped = coords.copy()
+    swapped[[100, 101]] = swapped[[101, 100]]
+    u = backend.rows_ready(dev(swapped))
+    assert not backend.coords_ascending(u)
+    backend.settle_checks()
+    assert not backend.coords_ascending(u)
+    kmap = F.build_kernel_map(u, len(swapped), 3, 1, 0, mode="hashmap_on_the_fly")
+    assert kmap["in_hashmap"] is not None
+    np.testing.assert_array_equal(kmap["out_in_map"].cpu().numpy(), oracle.kmap_subm(swapped, 3))
+
+    # written in place afterwards: the declaration no longer holds
+    t.add_(0)
+    assert not backend._declared_ready(t)
+
+    far = coords.copy()
+    far[-1, 2] = 1 << 20  # beyond the 18 bits a packed key holds per axis
+    v = backend.rows_ready(dev(far))
+    backend.coords_ascending(v)
+    with pytest.raises(ValueError, match="range"):
+        backend.settle_checks()
+    assert not backend._pending_verdicts
+    backend.settle_checks()  # raised once
+
+
 def test_segments_longer_than_the_staging_area_are_searched_in_memory():
     """A thin slab next to a dense one: the block that holds the thin slab's rows needs the
     whole dense slab as its segment for the x-digit that points there."""
