@@ -206,3 +206,42 @@ def test_coordinate_range_bookkeeping_on_the_host():
     msg = str(backend._range_error())
     assert "-131072" in msg and "131072)" in msg and "512" in msg
     assert backend.COORD_LIMIT == 1 << 17 and backend.BATCH_LIMIT == 512
+
+
+def test_buffers_collected_while_recording_outlive_the_tables():
+    """backend.pinned(): every library-owned buffer an accessor returns inside the block is
+    collected once; dropping the scratch of every stream and pushing seventeen other sizes
+    through the identity-map table (it keeps sixteen) leaves the collected tensors where they
+    were, with their contents (host tensors stand in for device memory here)."""
+    from torchsparse_amd import backend
+    cpu = torch.device("cpu", 0)
+    with backend.pinned() as held:
+        at = backend._scratch(cpu, 1234, 4096)
+        assert backend._scratch(cpu, 1234, 100) == at  # same buffer: collected once
+        counters = backend._tile_counters(cpu, 1234)
+        ident = backend._identity_map(300, cpu)
+        w = torch.randn(27, 8, 8)
+        w._tsmi_packed = (w._version, w.data_ptr(), torch.zeros(5))
+        packed = backend.pack_weights(w)
+        with backend.pinned() as inner:  # recordings may nest: both collect
+            assert backend._identity_map(300, cpu) is ident
+        assert len(inner) == 1 and inner[0] is ident
+    assert not backend._pin_sinks
+    assert [t.data_ptr() for t in held] == [at, counters.data_ptr(), ident.data_ptr(), packed.data_ptr()]
+    backend._identity_map(301, cpu)  # outside the block: not collected
+    assert len(held) == 4
+    recorded = [t.data_ptr() for t in held]
+    backend.release_scratch()
+    assert (cpu.index, 1234) not in backend._SCRATCH
+    for n in range(1000, 1017):
+        backend._identity_map(n, cpu)
+    assert (0, 300) not in backend._IDENTITY_MAPS and len(backend._IDENTITY_MAPS) == 16
+    w.add_(1)  # a new version of the weights: the cached packing is replaced on the next use
+    assert [t.data_ptr() for t in held] == recorded
+    assert held[0].numel() >= 4096
+    np.testing.assert_array_equal(ident[:300, 0].numpy(), np.arange(300))
+    assert (ident[300:] == -1).all() and ident.shape == (384, 1)
+    assert backend._scratch(cpu, 1234, 4096) != at  # the table allocates anew; the old block is still held
+    backend.release_scratch()
+    backend._IDENTITY_MAPS.clear()
+    backend._TILE_COUNTERS.pop((0, 1234), None)

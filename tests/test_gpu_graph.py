@@ -74,3 +74,64 @@ def test_detection_backbone_replays_equal_eager_forwards():
     model = fuse_inference(model).half()
     _check_replays(ts, model, coords, 5, spatial_range=(2, 41, 96, 96),
                    pick=lambda out: [v.feats for v in out.values()])
+
+
+def test_replays_survive_the_eviction_of_every_library_table():
+    """After the recording: release_scratch(), 1x1x1 layers over seventeen other row counts (the
+    identity-map table keeps sixteen), pair segments of seventy other maps (that table is cleared
+    at sixty-four), and eager forwards of a larger input on
+    the recording's own stream (its scratch regrown).  The recording keeps the buffers it was
+    made over: they are still where they were, and the replay still equals the eager forward."""
+    import torchsparse_amd as ts
+    from torchsparse_amd import backend
+    from torchsparse_amd.backbones import SparseResUNet42
+    from torchsparse_amd.nn.utils import fuse_inference
+    from torchsparse_amd.utils.graph import GraphedForward
+    from torchsparse_amd.utils.synthetic import lidar_scan_voxels
+    import oracle
+    torch.manual_seed(1)
+    scan = lidar_scan_voxels(seed=1)
+    coords = dev(scan[::3].copy())
+    n = coords.shape[0]
+    model = SparseResUNet42(in_channels=4).cuda().eval()
+    _stat_norms(model)
+    model = fuse_inference(copy.deepcopy(model)).half()
+    pick = lambda out: [o.feats for o in out]  # noqa: E731
+    feats = [torch.randn(n, 4, device="cuda", dtype=torch.float16) for _ in range(2)]
+    runner = GraphedForward(model, ts.SparseTensor(feats[0], coords))
+    assert len(runner.pinned) >= 40  # the packed weights of 49 layers, scratch, counters, segments ...
+    recorded = [t.data_ptr() for t in runner.pinned]
+    sizes = {t.numel() * t.element_size() for t in runner.pinned}
+    assert max(sizes) >= 1 << 20  # the stream's scratch is among them
+    with torch.no_grad():
+        want = [[t.clone() for t in pick(model(ts.SparseTensor(f, coords.clone())))] for f in feats]
+
+    backend.release_scratch()
+    w1 = torch.randn(16, 16, device="cuda", dtype=torch.float16)
+    for m in range(2000, 2017):
+        backend.conv_pointwise_cuda(torch.randn(m, 16, device="cuda", dtype=torch.float16), w1)
+    rng = np.random.default_rng(3)
+    small = oracle.kmap_subm(random_coords(rng, 200, (8, 8, 8)), 3)
+    keep = [dev(small.copy()) for _ in range(70)]
+    for m in keep:
+        backend.pair_segments(m, 200)
+    assert len(backend._segments_of) < 64  # (cleared on the way)
+    big = dev(scan)
+    fb = torch.randn(big.shape[0], 4, device="cuda", dtype=torch.float16)
+    torch.cuda.synchronize()
+    with torch.no_grad(), torch.cuda.stream(runner.stream):
+        model(ts.SparseTensor(fb, big))
+    runner.stream.synchronize()
+    junk = [torch.full((1 << 22,), 7, dtype=torch.int32, device="cuda") for _ in range(8)]  # reuse freed blocks
+    torch.cuda.synchronize()
+    assert [t.data_ptr() for t in runner.pinned] == recorded
+    for i in (1, 0, 1):
+        got = pick(runner(feats[i]))
+        torch.cuda.synchronize()
+        for g, w in zip(got, want[i]):
+            assert torch.equal(g, w), i
+    del junk
+    # a moved buffer is refused
+    runner.pinned[0].resize_(runner.pinned[0].numel() * 4 + (1 << 24))
+    with pytest.raises(RuntimeError, match="moved"):
+        runner(feats[0])

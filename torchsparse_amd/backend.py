@@ -1343,6 +1343,8 @@ def pack_weights(kernel: torch.Tensor) -> torch.Tensor:
     Cached on the tensor object and refreshed when its version counter moves."""
     cached = getattr(kernel, "_tsmi_packed", None)
     if cached is not None and cached[0] == kernel._version and cached[1] == kernel.data_ptr():
+        if _pin_sinks:
+            _pin(cached[2])
         return cached[2]
     w = kernel.detach()
     if w.dim() == 2:
@@ -1355,6 +1357,8 @@ def pack_weights(kernel: torch.Tensor) -> torch.Tensor:
         kernel._tsmi_packed = (kernel._version, kernel.data_ptr(), packed)
     except AttributeError:
         pass
+    if _pin_sinks:
+        _pin(packed)
     return packed
 
 
@@ -1387,6 +1391,39 @@ def _epilogue_args(bias, residual, x, n_out, cout):
 _PACK17 = struct.Struct("17q").pack
 _PACK18 = struct.Struct("18q").pack
 
+# Buffers the library owns (the scratch of a stream, its tile counters, identity maps, pair
+# segments, grouped maps, packed weights) live in tables that drop or replace their entries.  A
+# caller that keeps their ADDRESSES beyond the call - a recorded HIP graph - collects the tensors
+# themselves while it records: every accessor below hands each buffer it returns to the open
+# collectors, and a tensor that is referenced is not freed whatever the tables do.
+_pin_sinks = []
+
+
+class pinned:
+    """``with pinned() as held:`` - ``held`` (a list) receives every library-owned tensor whose
+    address is handed to a launch inside the block, once per tensor."""
+
+    def __enter__(self):
+        self.held, self._seen = [], set()
+        _pin_sinks.append(self)
+        return self.held
+
+    def __exit__(self, *exc):
+        _pin_sinks.remove(self)
+        return False
+
+    def add(self, t):
+        if id(t) not in self._seen:
+            self._seen.add(id(t))
+            self.held.append(t)
+
+
+def _pin(t):
+    for sink in _pin_sinks:
+        sink.add(t)
+    return t
+
+
 _SCRATCH = {}  # (device index, stream) -> uint8 tensor, grown on demand
 # held while a call that goes through the scratch buffer queues its launches: two host threads
 # that feed one stream must not interleave the launches of two such calls
@@ -1403,6 +1440,8 @@ def _scratch(device, stream: int, nbytes: int) -> int:
     t = _SCRATCH.get(key)
     if t is None or t.numel() < nbytes:
         t = _SCRATCH[key] = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+    if _pin_sinks:
+        _pin(t)
     return t.data_ptr()
 
 
@@ -1427,6 +1466,8 @@ def _tile_counters(device, stream: int):
     t = _TILE_COUNTERS.get(key)
     if t is None:
         t = _TILE_COUNTERS[key] = torch.zeros(_N_TILE_COUNTERS, dtype=torch.int32, device=device)
+    if _pin_sinks:
+        _pin(t)
     return t
 
 
@@ -1493,6 +1534,8 @@ def pair_segments(out_in_map: torch.Tensor, n_rows: int) -> PairSegments:
     hit = _segments_of.get(id(out_in_map))
     if (hit is not None and hit[0]() is out_in_map and hit[1] == out_in_map._version
             and hit[2] == out_in_map.data_ptr() and hit[3] == stream and hit[4] == n_rows):
+        if _pin_sinks:
+            _pin(hit[5].buffer)
         return hit[5]
     out_in_map = _need(out_in_map, torch.int32, "out_in_map")
     kvol = out_in_map.shape[1]
@@ -1504,10 +1547,15 @@ def pair_segments(out_in_map: torch.Tensor, n_rows: int) -> PairSegments:
     pool = _SEGMENT_POOLS.get(key)
     if pool is None:
         pool = _SEGMENT_POOLS[key] = torch.zeros(520, dtype=torch.int32, device=dev)
+    if _pin_sinks:
+        _pin(pool)
+        _pin(seg.buffer)
     with _scratch_lock:  # (the pool is shared by the builds of one stream)
         _check(_C.tsmi_pair_segments(stream, out_in_map.data_ptr(), n_rows, kvol, seg.seg_rows,
                                      pool.data_ptr() if kvol < 520 else None, seg.counts_ptr,
                                      seg.in_rows_ptr, seg.pos_ptr))
+    if torch.cuda.is_current_stream_capturing():
+        return seg  # filled by the recording's replays only: not for the table
     with _hint_lock:
         if len(_segments_of) >= 64:
             for k in [k for k, v in _segments_of.items() if v[0]() is None]:
@@ -1585,6 +1633,8 @@ def grouped_map(out_in_map: torch.Tensor, n_rows: int, window: Optional[int] = N
     hit = _grouped_of.get(id(out_in_map))
     if (hit is not None and hit[0]() is out_in_map and hit[1] == out_in_map._version
             and hit[2] == out_in_map.data_ptr() and hit[3] == stream and hit[4] == n_rows and hit[5] == window):
+        if _pin_sinks:
+            _pin(hit[6].buffer)
         return hit[6]
     out_in_map = _need(out_in_map, torch.int32, "out_in_map")
     if out_in_map.dim() != 2 or out_in_map.shape[1] != 27:
@@ -1597,7 +1647,11 @@ def grouped_map(out_in_map: torch.Tensor, n_rows: int, window: Optional[int] = N
     if n_rows == 0:
         raise ValueError("no rows to group")
     g = GroupedMap(padded, window, out_in_map.device)
+    if _pin_sinks:
+        _pin(g.buffer)
     _check(_C.tsmi_map_group_rows(stream, out_in_map.data_ptr(), n_rows, 27, window, *g.ptrs))
+    if torch.cuda.is_current_stream_capturing():
+        return g  # filled by the recording's replays only: not for the table
     with _scratch_lock:
         if len(_grouped_of) >= 64:
             for key in [k for k, v in _grouped_of.items() if v[0]() is None]:
@@ -1638,7 +1692,8 @@ def _grouping_pays(x, kvol: int, cin: int, cout: int, num_out_feats: int, out_in
                 _group_uses.clear()
         hit = _group_uses[key] = [weakref.ref(out_in_map), out_in_map._version, out_in_map.data_ptr(), 0]
     hit[3] += 1
-    return hit[3] >= group_after_uses
+    # (a copy built while a graph is being recorded would hold nothing until the first replay)
+    return hit[3] >= group_after_uses and not torch.cuda.is_current_stream_capturing()
 
 
 def conv_implicit_gemm_grouped(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias=None,
@@ -1774,6 +1829,8 @@ def _identity_map(n: int, device) -> torch.Tensor:
         m = torch.full((make_divisible(n, 128), 1), -1, dtype=torch.int32, device=device)
         m[:n, 0] = torch.arange(n, dtype=torch.int32, device=device)
         _IDENTITY_MAPS[key] = m
+    if _pin_sinks:
+        _pin(m)
     return m
 
 

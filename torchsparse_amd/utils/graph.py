@@ -15,11 +15,20 @@ library keeps its scratch buffers and per-map products per stream, and the warm-
 where the recording finds them (nothing is allocated for them while recording).  Replays are
 ordered after the work queued on the caller's current stream and the caller's stream after the
 replay.  The output tensors are the graph's own: a replay overwrites them, so copy what must
-outlive the next call."""
+outlive the next call.
+
+The recording holds ADDRESSES.  Those of the kernel maps stay valid because the input's caches
+are kept here; those of buffers the library owns (a stream's scratch and tile counters, identity
+maps, pair segments, grouped maps, packed weights) because every such tensor handed to a launch
+during warm-up and recording is collected (``backend.pinned``) and referenced by this object:
+``backend.release_scratch()`` and the eviction of the library's tables drop THEIR references, the
+memory stays.  A replay first checks that the collected tensors still sit where they were
+recorded (``resize_`` or ``set_`` on one of them would move it) and raises otherwise."""
 from typing import Any, Callable, Optional
 
 import torch
 
+from torchsparse_amd import backend
 from torchsparse_amd.tensor import SparseTensor
 
 __all__ = ["GraphedForward"]
@@ -57,15 +66,19 @@ class GraphedForward:
         caller = torch.cuda.current_stream(dev)
         self.stream = torch.cuda.Stream(device=dev)
         self.stream.wait_stream(caller)
-        with torch.no_grad(), torch.cuda.stream(self.stream):
-            for _ in range(warmup):
-                fn(self.x)
-        self.stream.synchronize()
-        self.graph = torch.cuda.CUDAGraph()
-        with torch.no_grad(), torch.cuda.graph(self.graph, stream=self.stream):
-            self.out = fn(self.x)
+        with backend.pinned() as held:
+            with torch.no_grad(), torch.cuda.stream(self.stream):
+                for _ in range(warmup):
+                    fn(self.x)
+            self.stream.synchronize()
+            self.graph = torch.cuda.CUDAGraph()
+            with torch.no_grad(), torch.cuda.graph(self.graph, stream=self.stream):
+                self.out = fn(self.x)
         caller.wait_stream(self.stream)
         self._outputs = _tensors_of(self.out)
+        # the library's buffers the recorded launches read and write, and where they were
+        self.pinned = tuple(held)
+        self._pinned_at = tuple(t.data_ptr() for t in held)
 
     def __call__(self, feats: Optional[torch.Tensor] = None):
         """Replay with ``feats`` (same shape and dtype as the recorded input; None: whatever the
@@ -76,5 +89,9 @@ class GraphedForward:
                 raise ValueError(f"the graph was recorded for features of shape {tuple(self.feats.shape)} "
                                  f"and dtype {self.feats.dtype}")
             self.feats.copy_(feats)
+        for t, at in zip(self.pinned, self._pinned_at):
+            if t.data_ptr() != at:
+                raise RuntimeError("a buffer this graph was recorded over has been moved (resize_/set_ on a "
+                                   "tensor of the library): record a new GraphedForward")
         self.graph.replay()
         return self.out
