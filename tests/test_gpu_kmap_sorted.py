@@ -223,6 +223,32 @@ def test_negative_coordinates_and_the_edge_of_the_packed_range():
     np.testing.assert_array_equal(kmap["out_in_map"].cpu().numpy(), want_map)
 
 
+@pytest.mark.parametrize("edge", ["low", "high"])
+def test_blocks_that_start_inside_a_plane_at_the_edge_of_the_packed_range(edge):
+    """Runs of 300 rows per (x, y) line, lines at the first (last) packable x and y: the blocks of
+    256 rows start and end inside the edge lines, where the targets one step outside clamp.  The
+    bounds of a block's segment must still hold the neighbours of its rows in the next line."""
+    xs = np.arange(2) + (-131072 if edge == "low" else 131070)
+    ys = np.arange(3) + (-131072 if edge == "low" else 131069)
+    zs = np.arange(300) + (-131072 if edge == "low" else 131072 - 300)
+    x, y, z = np.meshgrid(xs, ys, zs, indexing="ij")
+    coords = np.stack([np.zeros(x.size), x.ravel(), y.ravel(), z.ravel()], 1).astype(np.int32)
+    rng = np.random.default_rng(7)
+    coords = ascending(coords[rng.random(len(coords)) < 0.9])  # (a few holes: not every target exists)
+    lo, hi = coords.min(0), coords.max(0)
+    for ks in (3, (3, 5, 3), (5, 3, 3)):
+        kmap = build(coords, ks, 1, 0)
+        want = oracle.kmap_subm(coords, ks, coords_min=lo, coords_max=hi)
+        np.testing.assert_array_equal(kmap["out_in_map"].cpu().numpy(), want)
+        assert (want[:len(coords)] >= 0).mean() > 0.2
+    if edge == "high":
+        for ks, st, pd in ((3, 2, 1), (2, 2, 0), ((3, 3, 3), (1, 2, 2), (1, 1, 1))):
+            kmap = build(coords, ks, st, pd)
+            want_map, want_coords = oracle.kmap_downsample(coords, ks, st, pd)
+            np.testing.assert_array_equal(kmap["coords"].cpu().numpy(), want_coords)
+            np.testing.assert_array_equal(kmap["out_in_map"].cpu().numpy(), want_map)
+
+
 def test_scan_like_surface_and_switch():
     rng = np.random.default_rng(205)
     coords = ascending(lidar_like_coords(rng, 60000))
