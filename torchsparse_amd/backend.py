@@ -241,6 +241,22 @@ _VERDICT_SLOTS = 64
 kmap_through_sorted = True
 
 
+_tables_lock = threading.Lock()  # guards the insertions and prunings of the module's tables
+
+
+def _remember(table: dict, key, value, limit: int) -> None:
+    """``table[key] = value``; a table that holds ``limit`` entries first drops those whose
+    tensor (``entry[0]``, a weak reference) is gone, and everything if none is.  One host thread
+    at a time: a second one would otherwise iterate a table the first is resizing."""
+    with _tables_lock:
+        if len(table) >= limit:
+            for k in [k for k, v in table.items() if v[0]() is None]:
+                del table[k]
+            if len(table) >= limit:
+                table.clear()
+        table[key] = value
+
+
 def _range_error() -> ValueError:
     return ValueError(
         f"coordinates outside the range of the packed hash key: x, y, z must lie in "
@@ -275,12 +291,8 @@ def _mark_range_ok(coords: torch.Tensor, ascending: Optional[bool] = None, origi
         if hit is not None:
             return
         origin = "user"  # vouched for by a flag read-back over a caller's rows
-    if len(_range_ok) >= 512:
-        for key in [k for k, v in _range_ok.items() if v[0]() is None]:
-            del _range_ok[key]
-        if len(_range_ok) >= 512:
-            _range_ok.clear()
-    _range_ok[id(coords)] = (weakref.ref(coords), coords._version, coords.data_ptr(), ascending, origin)
+    _remember(_range_ok, id(coords), (weakref.ref(coords), coords._version, coords.data_ptr(), ascending, origin),
+              512)
 
 
 def settle_checks(block: bool = True) -> None:
@@ -320,12 +332,7 @@ def rows_ready(coords: torch.Tensor) -> torch.Tensor:
     writes them.  The library then neither waits for the caller's stream before it reads them
     on its second stream nor reads the verdict of their first check back at once.  Returns
     ``coords``.  Holds until the tensor is written in place."""
-    if len(_rows_ready) >= 256:
-        for key in [k for k, v in _rows_ready.items() if v[0]() is None]:
-            del _rows_ready[key]
-        if len(_rows_ready) >= 256:
-            _rows_ready.clear()
-    _rows_ready[id(coords)] = (weakref.ref(coords), coords._version, coords.data_ptr())
+    _remember(_rows_ready, id(coords), (weakref.ref(coords), coords._version, coords.data_ptr()), 256)
     return coords
 
 
@@ -518,12 +525,8 @@ def _sorted_samples(coords: torch.Tensor) -> Optional[torch.Tensor]:
         return hit[4]
     samples = torch.empty(elems, dtype=torch.int64, device=coords.device)
     _check(_C.tsmi_kmap_sorted_samples(stream, _ptr(coords), n, _ptr(samples)))
-    if len(_samples_of) >= 64:
-        for key in [k for k, v in _samples_of.items() if v[0]() is None]:
-            del _samples_of[key]
-        if len(_samples_of) >= 64:
-            _samples_of.clear()
-    _samples_of[id(coords)] = (weakref.ref(coords), coords._version, coords.data_ptr(), stream, samples)
+    _remember(_samples_of, id(coords), (weakref.ref(coords), coords._version, coords.data_ptr(), stream, samples),
+              64)
     return samples
 
 
@@ -1439,7 +1442,10 @@ def _scratch(device, stream: int, nbytes: int) -> int:
     key = (device.index, stream)
     t = _SCRATCH.get(key)
     if t is None or t.numel() < nbytes:
-        t = _SCRATCH[key] = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        with _tables_lock:  # (two host threads that miss together must end with one buffer)
+            t = _SCRATCH.get(key)
+            if t is None or t.numel() < nbytes:
+                t = _SCRATCH[key] = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
     if _pin_sinks:
         _pin(t)
     return t.data_ptr()
@@ -1465,7 +1471,10 @@ def _tile_counters(device, stream: int):
     key = (device.index, stream)
     t = _TILE_COUNTERS.get(key)
     if t is None:
-        t = _TILE_COUNTERS[key] = torch.zeros(_N_TILE_COUNTERS, dtype=torch.int32, device=device)
+        with _tables_lock:
+            t = _TILE_COUNTERS.get(key)
+            if t is None:
+                t = _TILE_COUNTERS[key] = torch.zeros(_N_TILE_COUNTERS, dtype=torch.int32, device=device)
     if _pin_sinks:
         _pin(t)
     return t
@@ -1546,7 +1555,10 @@ def pair_segments(out_in_map: torch.Tensor, n_rows: int) -> PairSegments:
     key = (dev.index, stream)
     pool = _SEGMENT_POOLS.get(key)
     if pool is None:
-        pool = _SEGMENT_POOLS[key] = torch.zeros(520, dtype=torch.int32, device=dev)
+        with _tables_lock:
+            pool = _SEGMENT_POOLS.get(key)
+            if pool is None:
+                pool = _SEGMENT_POOLS[key] = torch.zeros(520, dtype=torch.int32, device=dev)
     if _pin_sinks:
         _pin(pool)
         _pin(seg.buffer)
@@ -1556,20 +1568,14 @@ def pair_segments(out_in_map: torch.Tensor, n_rows: int) -> PairSegments:
                                      seg.in_rows_ptr, seg.pos_ptr))
     if torch.cuda.is_current_stream_capturing():
         return seg  # filled by the recording's replays only: not for the table
-    with _hint_lock:
-        if len(_segments_of) >= 64:
-            for k in [k for k, v in _segments_of.items() if v[0]() is None]:
-                del _segments_of[k]
-            if len(_segments_of) >= 64:
-                _segments_of.clear()
-        _segments_of[id(out_in_map)] = (weakref.ref(out_in_map), out_in_map._version, out_in_map.data_ptr(),
-                                        stream, n_rows, seg)
+    _remember(_segments_of, id(out_in_map), (weakref.ref(out_in_map), out_in_map._version, out_in_map.data_ptr(),
+                                             stream, n_rows, seg), 64)
     return seg
 
 
 _level_thinning = {}  # id(coords) -> (weak reference, rows kept per input row by the layer that made them)
 _sparse_maps = {}     # id(map) -> weak reference: maps over rows known to have few neighbours
-_hint_lock = threading.Lock()  # guards the two tables above and _segments_of
+_hint_lock = threading.Lock()  # guards the two tables above
 
 
 # Large 3x3x3 layers of the implicit-GEMM dataflow can run over a copy of the map whose rows are
@@ -1652,14 +1658,8 @@ def grouped_map(out_in_map: torch.Tensor, n_rows: int, window: Optional[int] = N
     _check(_C.tsmi_map_group_rows(stream, out_in_map.data_ptr(), n_rows, 27, window, *g.ptrs))
     if torch.cuda.is_current_stream_capturing():
         return g  # filled by the recording's replays only: not for the table
-    with _scratch_lock:
-        if len(_grouped_of) >= 64:
-            for key in [k for k, v in _grouped_of.items() if v[0]() is None]:
-                del _grouped_of[key]
-            if len(_grouped_of) >= 64:
-                _grouped_of.clear()
-        _grouped_of[id(out_in_map)] = (weakref.ref(out_in_map), out_in_map._version, out_in_map.data_ptr(),
-                                       stream, n_rows, window, g)
+    _remember(_grouped_of, id(out_in_map), (weakref.ref(out_in_map), out_in_map._version, out_in_map.data_ptr(),
+                                            stream, n_rows, window, g), 64)
     return g
 
 
@@ -1685,12 +1685,8 @@ def _grouping_pays(x, kvol: int, cin: int, cout: int, num_out_feats: int, out_in
     hit = _group_uses.get(key)
     if (hit is None or hit[0]() is not out_in_map or hit[1] != out_in_map._version
             or hit[2] != out_in_map.data_ptr()):
-        if len(_group_uses) >= 256:
-            for k in [k for k, v in _group_uses.items() if v[0]() is None]:
-                del _group_uses[k]
-            if len(_group_uses) >= 256:
-                _group_uses.clear()
-        hit = _group_uses[key] = [weakref.ref(out_in_map), out_in_map._version, out_in_map.data_ptr(), 0]
+        hit = [weakref.ref(out_in_map), out_in_map._version, out_in_map.data_ptr(), 0]
+        _remember(_group_uses, key, hit, 256)
     hit[3] += 1
     # (a copy built while a graph is being recorded would hold nothing until the first replay)
     return hit[3] >= group_after_uses and not torch.cuda.is_current_stream_capturing()
@@ -1824,11 +1820,12 @@ def _identity_map(n: int, device) -> torch.Tensor:
     key = (device.index if device.index is not None else _cur_device(), n)
     m = _IDENTITY_MAPS.get(key)
     if m is None:
-        if len(_IDENTITY_MAPS) >= 16:
-            _IDENTITY_MAPS.pop(next(iter(_IDENTITY_MAPS)))
         m = torch.full((make_divisible(n, 128), 1), -1, dtype=torch.int32, device=device)
         m[:n, 0] = torch.arange(n, dtype=torch.int32, device=device)
-        _IDENTITY_MAPS[key] = m
+        with _tables_lock:
+            if len(_IDENTITY_MAPS) >= 16:
+                _IDENTITY_MAPS.pop(next(iter(_IDENTITY_MAPS)), None)
+            _IDENTITY_MAPS[key] = m
     if _pin_sinks:
         _pin(m)
     return m
