@@ -78,10 +78,11 @@ def lib():
     """Load (building on first use when absent) oracle/liboracle.so."""
     global _LIB
     if _LIB is None:
-        path = os.path.join(_HERE, "liboracle.so")
-        if not os.path.exists(path):
-            from . import build as _build
+        from . import build as _build
 
+        # (ASAN=1: the build with the host sanitizers, see build.py)
+        path = os.path.join(_HERE, "liboracle_asan.so" if _build.SANITIZE else "liboracle.so")
+        if not os.path.exists(path):
             _build.build_oracle()
         _LIB = ctypes.CDLL(path)
         _LIB.tso_pair_lists.restype = ctypes.c_int64

@@ -14,10 +14,32 @@ REFERENCE_BACKEND = "/root/reference/torchsparse/backend"
 REF_MODULE = "tsref_cpu"
 
 
+# ASAN=1 (or SANITIZE=address) in the environment: the oracle is built with AddressSanitizer and
+# UndefinedBehaviorSanitizer into liboracle_asan.so, by the clang that also builds the host side
+# of libtsmi_asan.so (one process can hold one sanitizer runtime), and oracle.lib() loads that
+# file.  Host code only.  To run the CPU tests under it:
+#   ASAN=1 python oracle/build.py && ASAN=1 python torchsparse_amd/csrc/build.py
+#   ASAN=1 ASAN_OPTIONS=detect_leaks=0 LD_PRELOAD=$(python oracle/build.py --asan-runtime) \
+#       python -m pytest tests -q -m "not gpu"
+SANITIZE = os.environ.get("ASAN", "0") not in ("", "0") or os.environ.get("SANITIZE") == "address"
+CLANG = os.environ.get("HOST_CLANG", "/opt/rocm/lib/llvm/bin/clang")
+
+
+def asan_runtime() -> str:
+    """Path of the shared sanitizer runtime that has to be loaded before python itself."""
+    return subprocess.check_output([CLANG, "-print-file-name=libclang_rt.asan-x86_64.so"], text=True).strip()
+
+
 def build_oracle(verbose: bool = False) -> str:
-    out = os.path.join(HERE, "liboracle.so")
-    cmd = ["gcc", "-O3", "-march=native", "-fopenmp", "-fPIC", "-shared", "-std=c11",
-           "-fvisibility=hidden", os.path.join(HERE, "oracle.c"), "-o", out, "-lm"]
+    src = os.path.join(HERE, "oracle.c")
+    if SANITIZE:
+        out = os.path.join(HERE, "liboracle_asan.so")
+        cmd = [CLANG, "-O1", "-g", "-fno-omit-frame-pointer", "-fsanitize=address,undefined", "-shared-libasan",
+               "-fopenmp", "-fPIC", "-shared", "-std=c11", "-fvisibility=hidden", src, "-o", out, "-lm"]
+    else:
+        out = os.path.join(HERE, "liboracle.so")
+        cmd = ["gcc", "-O3", "-march=native", "-fopenmp", "-fPIC", "-shared", "-std=c11",
+               "-fvisibility=hidden", src, "-o", out, "-lm"]
     if verbose:
         print(" ".join(cmd))
     subprocess.check_call(cmd)
@@ -59,6 +81,9 @@ def build_ref(verbose: bool = False):
 
 
 if __name__ == "__main__":
+    if "--asan-runtime" in sys.argv:
+        print(asan_runtime())
+        sys.exit(0)
     print(build_oracle(verbose=True))
     if "--ref" in sys.argv:
         print(build_ref(verbose=True))

@@ -18,7 +18,10 @@ from typing import List, Optional, Sequence, Tuple
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB_PATH = os.path.join(_HERE, "libtsmi.so")
+# (ASAN=1 / SANITIZE=address: the build whose host code carries AddressSanitizer, for CPU runs of
+# the host logic under a preloaded sanitizer runtime; csrc/build.py makes it under the same switch)
+_SANITIZE = os.environ.get("ASAN", "0") not in ("", "0") or os.environ.get("SANITIZE") == "address"
+_LIB_PATH = os.path.join(_HERE, "libtsmi_asan.so" if _SANITIZE else "libtsmi.so")
 
 F32, F16, BF16 = 0, 1, 2
 _DTYPE_CODE = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}

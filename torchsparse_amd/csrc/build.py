@@ -34,9 +34,23 @@ FLAGS = [
 ]
 
 
+# ASAN=1 (or SANITIZE=address) in the environment: the host passes of the sources without device
+# code (argument checks, plans, dispatch) are compiled with AddressSanitizer into libtsmi_asan.so,
+# which the package then loads; device code is never instrumented.  For CPU runs of the host
+# logic (python started with the sanitizer runtime preloaded), not for the GPU.
+SANITIZE = os.environ.get("ASAN", "0") not in ("", "0") or os.environ.get("SANITIZE") == "address"
+HOST_ONLY = ("common.cpp", "conv_api.cpp")
+HOST_SANITIZE = ["-Xarch_host", "-fsanitize=address", "-Xarch_host", "-shared-libasan",
+                 "-Xarch_host", "-fno-omit-frame-pointer", "-Xarch_host", "-g"]
+if SANITIZE:
+    OUT = os.path.join(PKG, "libtsmi_asan.so")
+    OBJ_DIR = os.path.join(HERE, "build_asan")
+
+
 def _compile(src, verbose):
     obj = os.path.join(OBJ_DIR, src.rsplit(".", 1)[0] + ".o")
-    cmd = [HIPCC] + FLAGS + ["-x", "hip", "-c", os.path.join(HERE, src), "-o", obj]
+    flags = FLAGS + (HOST_SANITIZE if SANITIZE and src in HOST_ONLY else [])
+    cmd = [HIPCC] + flags + ["-x", "hip", "-c", os.path.join(HERE, src), "-o", obj]
     if verbose:
         print(" ".join(cmd), flush=True)
     r = subprocess.run(cmd, capture_output=True, text=True)
@@ -53,6 +67,8 @@ def build(verbose: bool = False, jobs: int = 8) -> str:
     with ThreadPoolExecutor(max_workers=jobs) as ex:
         objs = list(ex.map(lambda s: _compile(s, verbose), SOURCES))
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", OUT] + objs
+    if SANITIZE:
+        cmd += ["-fno-gpu-sanitize", "-fsanitize=address", "-shared-libasan"]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)
