@@ -139,10 +139,19 @@ int tsmi_kmap_sorted(tsmi_stream_t s, const int32_t *in_coords, int64_t n_in,
                      const int32_t *out_coords, int64_t n_out, int64_t n_out_pad,
                      const int32_t ks[3], const int32_t stride[3], const int32_t pad[3],
                      const int64_t *samples, int32_t *out_in_map);
-/* `count` calls of tsmi_kmap_sorted queued by one call (a network's maps over the levels of a
- * strided chain, built ahead of their use).  args: host int64[16 * count], per map
+/* `count` builds of tsmi_kmap_sorted queued by one call (a network's maps over the levels of a
+ * strided chain, built ahead of their use): maps with 2^3 and 3^3 kernels share one launch, up to
+ * eight at a time; others get a launch each.  args: host int64[20 * count], per map
  * [in_coords, n_in, out_coords, n_out, n_out_pad, samples (0: none), out_in_map, ks[3],
- * stride[3], pad[3]] with the pointers as integers.  No counterpart in the reference. */
+ * stride[3], pad[3], map_t, n_t_pad, pair_words, pair_out] with the pointers as integers.  The last
+ * four are optional products of the same launch (0: not wanted):
+ *   map_t int32[n_t_pad * K_vol] (n_t_pad >= n_in), filled with -1 by the caller beforehand:
+ *     receives map_t[in, k] = out for every pair found, which makes it the transposed map
+ *     (tsmi_transpose_map's result; the reference's others/query_cuda.cu:9-15 after the fill of
+ *     conv/hash/query.py:47-55).
+ *   pair_words int64[2], zero before the first use and left zero by every launch, and pair_out
+ *     int64[1]: receives the number of entries >= 0 of the whole map.
+ * No counterpart in the reference. */
 int tsmi_kmap_sorted_batch(tsmi_stream_t s, int count, const int64_t *args);
 /* Optional for tsmi_kmap_sorted, and only for inputs of more than 131072 rows (smaller ones
  * need none: tsmi_kmap_sorted_samples_elems returns 0): the keys every block of that kernel

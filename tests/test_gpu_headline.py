@@ -279,6 +279,7 @@ def test_minkunet_forward_on_the_scan(mods, scan):
     # ... and builds the four strided maps and the submanifold maps of levels 2 - 16 on the second
     # stream as soon as the row counts are known (the maps compared below are those)
     assert state.maps_ahead_hits == 8, state.maps_ahead_hits
+    assert state.transposed_hits == 0  # (asked for in this forward for the first time: see the end)
 
     # --- the nine kernel maps and the coordinate levels, bit-exact
     caches = inp._caches
@@ -293,6 +294,11 @@ def test_minkunet_forward_on_the_scan(mods, scan):
         np.testing.assert_array_equal(got["coords"].cpu().numpy(), scan["levels"][2 * s])
         np.testing.assert_array_equal(got["out_in_map_t"].cpu().numpy(), scan["up"][s])
         assert got["sizes"] == (scan["levels"][s].shape[0], scan["levels"][2 * s].shape[0])
+    torch.cuda.synchronize()
+    for s in (2, 4, 8, 16):
+        want = scan["subm"][s][:scan["levels"][s].shape[0]]
+        assert backend.map_density(caches.kmaps[_key(s, 3, 1)]["out_in_map"]) == (want >= 0).mean()
+    assert backend.map_density(caches.kmaps[_key(1, 3, 1)]["out_in_map"]) is None  # (built before the chain is known)
     for i, out in enumerate(outs):
         level = (1, 2, 4, 8, 16, 8, 4, 2, 1)[i]
         assert out.stride == (level,) * 3
@@ -323,8 +329,13 @@ def test_minkunet_forward_on_the_scan(mods, scan):
     print(f"per-layer worst {worst:.2e}, last features {e_last:.2e}, logits {e_logits:.2e}")
     assert e_last < 3e-2 and e_logits < 3e-2, (e_last, e_logits)
     # the forward measured by the benchmark is deterministic: a third run gives the same bits
-    _, outs3, logits3 = step()
+    inp3, outs3, logits3 = step()
     assert torch.equal(logits3, logits) and torch.equal(outs3[-1].feats, outs[-1].feats)
+    # ... in which the launch of the maps queued ahead has also stored the transposed maps of the
+    # four strided ones (the forward before asked for them): still the oracle's
+    assert state.transposed_hits == 4, state.transposed_hits
+    for s in (1, 2, 4, 8):
+        np.testing.assert_array_equal(inp3._caches.kmaps[_key(s, 2, 2)]["out_in_map_t"].cpu().numpy(), scan["up"][s])
 
 
 def _check_maps(caches, outs, tables):

@@ -261,3 +261,57 @@ def test_scan_like_surface_and_switch():
         backend.kmap_through_sorted = True
     assert hashed["in_hashmap"] is not None
     assert torch.equal(hashed["out_in_map"], kmap["out_in_map"])
+
+
+def test_batch_of_maps_in_one_call_with_transposed_maps_and_pair_counts():
+    """tsmi_kmap_sorted_batch over the levels of a strided chain: submanifold 3^3 maps and 2^3
+    stride-2 maps in one launch, a (3, 1, 1) map beside them in its own; every map bit for bit
+    the oracle's, the transposed maps whose entries the same launch stores (into buffers filled
+    with -1) equal to the oracle's transposition, the pair counts equal to the number of entries >= 0, and
+    the two words the blocks add up in zero again (the call is repeated over them)."""
+    import ctypes
+    rng = np.random.default_rng(404)
+    c1 = ascending(lidar_like_coords(rng, 30000))
+    d1, c2 = oracle.kmap_downsample(c1, 2, 2, 0)
+    d2, c3 = oracle.kmap_downsample(c2, 2, 2, 0)
+    t1, t2, t3 = dev(c1), dev(c2), dev(c3)
+    jobs = [  # (inputs, outputs, ks, st, pd, transposed?, oracle map)
+        (t1, t1, (3, 3, 3), (1, 1, 1), (1, 1, 1), True, oracle.kmap_subm(c1, 3)),
+        (t1, t2, (2, 2, 2), (2, 2, 2), (0, 0, 0), True, d1),
+        (t2, t2, (3, 3, 3), (1, 1, 1), (1, 1, 1), False, oracle.kmap_subm(c2, 3)),
+        (t2, t2, (3, 1, 1), (1, 1, 1), (1, 0, 0), False, oracle.kmap_subm(c2, (3, 1, 1))),
+        (t2, t3, (2, 2, 2), (2, 2, 2), (0, 0, 0), True, d2),
+        (t3, t3, (3, 3, 3), (1, 1, 1), (1, 1, 1), False, oracle.kmap_subm(c3, 3)),
+    ]
+    words = torch.zeros(3 * len(jobs), dtype=torch.int64, device="cuda")
+    for attempt in range(2):
+        flat, outs = [], []
+        for slot, (a, b, ks, st, pd, tr, want) in enumerate(jobs):
+            kvol = ks[0] * ks[1] * ks[2]
+            n_pad = -(-b.shape[0] // 128) * 128
+            t_pad = -(-a.shape[0] // 128) * 128
+            omap = torch.full((n_pad, kvol), -9, dtype=torch.int32, device="cuda")
+            omap_t = torch.full((t_pad, kvol), -1, dtype=torch.int32, device="cuda") if tr else None
+            flat += [a.data_ptr(), a.shape[0], b.data_ptr(), b.shape[0], n_pad, 0, omap.data_ptr(), *ks, *st, *pd,
+                     omap_t.data_ptr() if tr else 0, t_pad, words.data_ptr() + 16 * slot,
+                     words.data_ptr() + 8 * (2 * len(jobs) + slot)]
+            outs.append((omap, omap_t))
+        status = backend._C.tsmi_kmap_sorted_batch(backend._stream(), len(jobs), (ctypes.c_int64 * len(flat))(*flat))
+        assert status == 0, backend._C.tsmi_last_error()
+        torch.cuda.synchronize()
+        host = words.cpu().numpy()
+        assert (host[:2 * len(jobs)] == 0).all()
+        for slot, ((a, b, ks, st, pd, tr, want), (omap, omap_t)) in enumerate(zip(jobs, outs)):
+            np.testing.assert_array_equal(omap.cpu().numpy(), want)
+            assert host[2 * len(jobs) + slot] == (want >= 0).sum()
+            if tr:
+                n_in = a.shape[0]
+                want_t = oracle.transpose_map(want, n_in)
+                got_t = omap_t.cpu().numpy()
+                np.testing.assert_array_equal(got_t[:n_in], want_t[:n_in])
+                assert (got_t[n_in:] == -1).all()
+    # a transposed map with fewer rows than there are inputs is refused
+    bad = list(flat[20:40])
+    bad[17] = jobs[1][0].shape[0] - 1
+    status = backend._C.tsmi_kmap_sorted_batch(backend._stream(), 1, (ctypes.c_int64 * 20)(*bad))
+    assert status != 0 and b"transposed" in backend._C.tsmi_last_error()

@@ -221,3 +221,69 @@ def test_maps_over_thinned_rows_are_marked_sparse_and_solid_ones_are_not(mods):
         want = oracle.conv_implicit_gemm(_f32(mid.feats), _f32(deep.kernel), omap.cpu().numpy(), mid.feats.shape[0])
         assert rel_rms(_f32(out.feats), want) < 1e-2
     assert backend.level_thinning(dev(scattered)) is None  # a caller's own rows: nothing known
+
+
+def test_the_form_of_a_wide_layer_follows_the_measured_density_of_its_map(mods):
+    """Maps queued ahead of their use count their pairs; once the count is on the host the
+    implicit-GEMM dataflow takes the pair form for a wide, small layer where at most
+    segments_max_density of the map's entries are pairs.  A solid volume (more than half of the
+    entries) and a surface scan (a quarter or less): the measured density equals the oracle's,
+    decides the form, and the form taken is the quicker of the two on the device (medians of
+    20 timed calls each; the slower form is slower by 25 % and more on both, the test allows
+    the taken one 15 %)."""
+    backend, F = mods
+    import torchsparse_amd as ts
+    from torchsparse_amd import nn as spnn
+    from torchsparse_amd.utils.synthetic import lidar_scan_voxels
+    g = np.stack(np.meshgrid(np.arange(64), np.arange(64), np.arange(32), indexing="ij"), -1).reshape(-1, 3)
+    solid = np.concatenate([np.zeros((len(g), 1), np.int64), g], 1).astype(np.int32)
+    thin = lidar_scan_voxels(seed=1)[::2].copy()  # (every other voxel of the benchmark's scan)
+    torch.manual_seed(9)
+    net = torch.nn.ModuleList([spnn.Conv3d(16, 128, 2, stride=2), spnn.Conv3d(128, 256, 3),
+                               spnn.Conv3d(256, 256, 2, stride=2), spnn.Conv3d(256, 256, 3),
+                               spnn.Conv3d(4, 16, 3)]).cuda().half().eval()
+    key2 = ((2, 2, 2), (3, 3, 3), (1, 1, 1), (1, 1, 1))
+
+    def median_us(fn):
+        ts_ = []
+        for _ in range(20):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            fn()
+            b.record()
+            b.synchronize()
+            ts_.append(a.elapsed_time(b) * 1e3)
+        return float(np.median(ts_))
+
+    for coords_np, dense in ((solid, True), (thin, False)):
+        coords_np = coords_np[np.lexsort((coords_np[:, 3], coords_np[:, 2], coords_np[:, 1], coords_np[:, 0]))]
+        base = dev(coords_np)
+        feats = torch.randn(len(coords_np), 4, device="cuda", dtype=torch.float16)
+        backend.release_scratch()
+        with torch.no_grad():
+            # (a submanifold layer first, as in a network: the chain of the two strided layers starts
+            # beside it once it has been learnt, and the maps over its levels are queued ahead)
+            for _ in range(5):
+                x = ts.SparseTensor(feats, base.clone())
+                mid = net[1](net[0](net[4](x)))
+                net[3](net[2](mid))
+        torch.cuda.synchronize()
+        omap = x._caches.kmaps[key2]["out_in_map"]
+        n2 = mid.feats.shape[0]
+        want = oracle.kmap_subm(mid.coords.cpu().numpy(), 3)[:n2]
+        density = backend.map_density(omap)
+        assert density is not None and density == (want >= 0).mean()
+        assert (density >= 0.5) if dense else (density <= 0.25), density
+        assert 4000 < n2 < 65536
+        assert backend._segments_pay(mid.feats, 27, 128, 256, n2, omap) == (not dense)
+        xin = torch.randn(n2, 128, device="cuda", dtype=torch.float16)
+        wp = backend.pack_weights(net[1].kernel)
+        pair = median_us(lambda: backend.conv_implicit_gemm_segments(xin, wp, 27, 128, 256, omap, n2))
+        try:
+            backend.igemm_through_segments = False
+            plain = median_us(lambda: backend._implicit_gemm(xin, wp, 27, 128, 256, omap, n2))
+        finally:
+            backend.igemm_through_segments = True
+        taken, other = (plain, pair) if dense else (pair, plain)
+        print(f"density {density:.3f}: pair form {pair:.1f} us, dense pass {plain:.1f} us")
+        assert taken <= 1.15 * other, (density, pair, plain)

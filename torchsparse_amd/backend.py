@@ -409,6 +409,29 @@ def kmap_sorted(in_coords: torch.Tensor, out_coords: torch.Tensor, kernel_size, 
 # above; the caller's stream waits once, for the end of that queue, when it takes the first
 # of them.  Maps queued and never asked for cost their kernels.
 kmap_queue_ahead = True
+# The launch that builds the maps queued ahead also counts their pairs (entries >= 0); the counts
+# travel to pinned memory behind it and tell the convolutions how dense each map is.
+map_pairs_counted = True
+_PAIR_SLOTS = 16
+_map_requests = {}  # id(map) -> (weak reference, stream state, request, transposed map or None)
+
+
+def map_density(out_in_map: torch.Tensor) -> Optional[float]:
+    """Pairs per entry of a kernel map that was queued ahead of its use, once its count has
+    reached the host (None: not such a map, or not yet).  Never waits."""
+    index = out_in_map.device.index
+    state = _stream_states.get((index if index is not None else _cur_device(), _stream()))
+    if state is None:
+        return None
+    hit = state.pairs_of.get(id(out_in_map))
+    if hit is None or hit[0]() is not out_in_map:
+        return None
+    if state.pair_vals is None:
+        event = state.pair_event
+        if event is None or not event.query():
+            return None
+        state.pair_vals, state.pair_event = state.pair_host.tolist(), None
+    return state.pair_vals[hit[1]] / max(hit[2], 1)
 
 
 def _map_queued_ahead(in_coords, out_coords, ks, st, pd) -> Optional[torch.Tensor]:
@@ -441,6 +464,7 @@ def _map_queued_ahead(in_coords, out_coords, ks, st, pd) -> Optional[torch.Tenso
                 main.wait_event(state.maps_event)
             state.maps_event = None
         state.maps_ahead_hits += 1
+        _remember(_map_requests, id(hit[2]), (weakref.ref(hit[2]), state, request, hit[4]), 64)
         return hit[2]
 
 
@@ -452,12 +476,17 @@ def _queue_maps_ahead(state, chain_rows, on_side: bool) -> None:
     state.level_index = {id(t): (weakref.ref(t), i) for i, t in enumerate(chain_rows)}
     plan, state.map_plan_seen = tuple(state.map_plan_seen), []
     state.map_plan = plan
+    state.transposed_plan, state.transposed_seen = frozenset(state.transposed_seen), set()
     state.maps_ahead = {}
     state.maps_event = None
+    state.pairs_of, state.pair_event, state.pair_vals = {}, None, None
     if not (kmap_queue_ahead and on_side and plan and state.side is not None and kmap_through_sorted):
         return
-    todo, rows_of = [], {}  # maps of one kernel volume share an allocation: one hand-over between the streams each
-    for i, o, ks, st, pd in plan:
+    # maps of one kernel volume share an allocation, the transposed maps another: one hand-over
+    # between the streams each
+    todo, rows_of, t_ints = [], {}, 0
+    for request in plan:
+        i, o, ks, st, pd = request
         if max(i, o) >= len(chain_rows) or max(i, o) == 0:  # (the root's own map is asked for before this point)
             continue
         a, b = chain_rows[i], chain_rows[o]
@@ -466,7 +495,12 @@ def _queue_maps_ahead(state, chain_rows, on_side: bool) -> None:
         kvol = ks[0] * ks[1] * ks[2]
         first = rows_of.get(kvol, 0)
         rows_of[kvol] = first + make_divisible(b.shape[0], 128)
-        todo.append((a, b, ks, st, pd, kvol, first))
+        # the transposed map comes out of the same launch where the forward before asked for it
+        t_first = -1
+        if request in state.transposed_plan:
+            t_first = t_ints
+            t_ints += make_divisible(a.shape[0], 128) * kvol
+        todo.append((a, b, ks, st, pd, kvol, first, t_first))
     if not todo:
         return
     dev = chain_rows[0].device
@@ -474,23 +508,44 @@ def _queue_maps_ahead(state, chain_rows, on_side: bool) -> None:
     torch.cuda.set_stream(state.side)  # (the context manager costs 6 us, two switches 0.8)
     try:
         buffers = {kvol: torch.empty((rows, kvol), dtype=torch.int32, device=dev) for kvol, rows in rows_of.items()}
-        flat, queued = [], {}
-        for a, b, ks, st, pd, kvol, first in todo:
+        # (one fill for the transposed maps of all levels; the map launch stores their entries)
+        t_buffer = torch.full((t_ints,), -1, dtype=torch.int32, device=dev) if t_ints else None
+        counted = map_pairs_counted and len(todo) <= _PAIR_SLOTS
+        if counted and state.pair_dev is None:
+            state.pair_dev = torch.zeros(3 * _PAIR_SLOTS, dtype=torch.int64, device=dev)
+            state.pair_host = torch.zeros(_PAIR_SLOTS, dtype=torch.int64, pin_memory=True)
+        pair_ptr = state.pair_dev.data_ptr() if counted else 0
+        flat, queued, pairs_of = [], {}, {}
+        for slot, (a, b, ks, st, pd, kvol, first, t_first) in enumerate(todo):
             n_pad = make_divisible(b.shape[0], 128)
             omap = buffers[kvol][first:first + n_pad]
             samples = _sorted_samples(a)
+            omap_t, t_pad = None, make_divisible(a.shape[0], 128)
+            if t_first >= 0:
+                omap_t = t_buffer[t_first:t_first + t_pad * kvol].view(t_pad, kvol)
             flat += (a.data_ptr(), a.shape[0], b.data_ptr(), b.shape[0], n_pad,
-                     0 if samples is None else samples.data_ptr(), omap.data_ptr(), *ks, *st, *pd)
-            queued[(id(a), id(b), ks, st, pd)] = (weakref.ref(a), weakref.ref(b), omap, (a._version, b._version))
+                     0 if samples is None else samples.data_ptr(), omap.data_ptr(), *ks, *st, *pd,
+                     0 if omap_t is None else omap_t.data_ptr(), t_pad,
+                     pair_ptr + 16 * slot if counted else 0, pair_ptr + 8 * (2 * _PAIR_SLOTS + slot) if counted else 0)
+            queued[(id(a), id(b), ks, st, pd)] = (weakref.ref(a), weakref.ref(b), omap, (a._version, b._version),
+                                                  omap_t)
+            if counted:
+                pairs_of[id(omap)] = (weakref.ref(omap), slot, b.shape[0] * kvol)
         _check(_C.tsmi_kmap_sorted_batch(_stream(), len(todo), (ctypes.c_int64 * len(flat))(*flat)))
+        if counted:
+            state.pair_host.copy_(state.pair_dev[2 * _PAIR_SLOTS:], non_blocking=True)
         event = torch.cuda.Event()
         event.record()
     finally:
         torch.cuda.set_stream(main)
     for buf in buffers.values():
         buf.record_stream(main)  # allocated on the second stream, read and freed on the caller's
+    if t_buffer is not None:
+        t_buffer.record_stream(main)
     # (only now: a call that failed above leaves no map behind that was never written)
     state.maps_ahead, state.maps_event = queued, event
+    if counted:
+        state.pairs_of, state.pair_event = pairs_of, event
 
 
 def _kmap_sorted_launch(in_coords, out_coords, ks, st, pd, omap=None) -> torch.Tensor:
@@ -809,7 +864,8 @@ class _StridedState:
     __slots__ = ("grid_buf", "grid_words", "grid_dirty", "chain_geom", "chain_last", "chain_count",
                  "chain_len", "ahead", "ahead_hits", "host_counters", "pending", "pending_rsv", "root_chain",
                  "lookahead_hits", "side", "grid_event", "grid_event_stream", "grid_old", "level_index", "map_plan",
-                 "map_plan_seen", "maps_ahead", "maps_event", "maps_ahead_hits", "maps_main")
+                 "map_plan_seen", "maps_ahead", "maps_event", "maps_ahead_hits", "maps_main", "transposed_plan",
+                 "transposed_seen", "transposed_hits", "pair_dev", "pair_host", "pair_event", "pair_vals", "pairs_of")
 
     def __init__(self):
         self.grid_buf = None      # int32 scratch: bitmaps and chunk counts of every level
@@ -837,6 +893,17 @@ class _StridedState:
         self.maps_event = None    # end of that queue; None once the caller's stream has waited for it
         self.maps_ahead_hits = 0  # maps answered from `maps_ahead` (diagnostic)
         self.maps_main = None     # the caller's stream object at the time of that queue
+        self.transposed_plan = frozenset()  # requests of map_plan whose transposed map was asked for too
+        self.transposed_seen = set()
+        self.transposed_hits = 0  # transposed maps answered by the launch of their strided map (diagnostic)
+        # pair counts of the maps queued ahead: int64 [3 * 16] on the device (two words the blocks add
+        # up in and take tickets from, then the count, per map), pinned copy of the counts, the event
+        # behind that copy (None once it was seen done), the counts as a list, id(map) -> (ref, slot, entries)
+        self.pair_dev = None
+        self.pair_host = None
+        self.pair_event = None
+        self.pair_vals = None
+        self.pairs_of = {}
 
     def chain_step(self, coords, geom):
         """Book-keeping of chains of equal strided calls (each on the previous one's outputs).
@@ -1230,6 +1297,16 @@ def convert_transposed_out_in_map(out_in_map: torch.Tensor, n_rows_t: int, n_row
     out_in_map = _need(out_in_map, torch.int32, "out_in_map")
     kvol = out_in_map.shape[1]
     n_rows = out_in_map.shape[0] if n_rows is None else n_rows
+    hit = _map_requests.get(id(out_in_map))
+    if hit is not None and hit[0]() is out_in_map:
+        # a map of the chain in flight: the next forward's launch of this map writes the transposed
+        # one too; this forward's did if the forward before asked
+        hit[1].transposed_seen.add(hit[2])
+        ready = hit[3]
+        if ready is not None and ready.shape[0] == n_rows_t:
+            _map_requests[id(out_in_map)] = hit[:3] + (None,)
+            hit[1].transposed_hits += 1
+            return ready
     map_t = out_in_map.new_empty(n_rows_t, kvol)
     _check(_C.tsmi_transpose_map(_stream(), _ptr(out_in_map), n_rows, kvol, _ptr(map_t), n_rows_t))
     return map_t
@@ -1500,6 +1577,11 @@ def conv_forward_implicit_gemm_cuda(in_feats, kernel, out_in_map, num_out_feats,
 # all offsets of every row tile, where the map is known to have few pairs per row (True), wherever
 # the kernels have a variant ("always"), or never (False).
 igemm_through_segments = True
+# The pair form costs about 0.2 + 2.3 d of the dense pass on the layers it is made for (d: pairs
+# per map entry; fitted to 0.74 at d = 0.24 and 1.58 at d = 0.61, the two workloads measured in
+# _segments_pay's note): it is the cheaper one below d = 0.35.  Used where the density of the map
+# is known (map_density); other maps go by the hint of the level's thinning.
+segments_max_density = 0.35
 
 _segments_of = {}  # id(map) -> (weak reference, version, address, stream, rows, segments)
 _SEGMENT_POOLS = {}  # (device index, stream) -> zero int32 tensor the builder's blocks add up in
@@ -1748,10 +1830,12 @@ def _segments_pay(x, kvol, cin, cout, num_out_feats, out_in_map=None, force=None
     registers: measured on the levels of an 89,834-voxel scan (24 % of the map entries are pairs):
     8,045 rows 256 -> 256 32 vs 43 us, 384 -> 256 39 vs 57, 19,815 rows 128 -> 128 30 vs 36,
     192 -> 128 33 vs 47, 3,105 rows 256 -> 256 22 vs 28 (8,045 rows 128 -> 128, 21 vs 20, stays
-    dense); on a detection backbone's 55,578-row level (61 %): 128 -> 128 134 vs 85.  The number of
-    pairs is not known on the host, so ``igemm_through_segments = True`` takes the pair form only
-    for maps marked by hint_sparse_map (build_kernel_map marks those over rows that thin out like
-    surfaces, see level_thinning); "always" takes it wherever a variant exists.  ``force`` (a
+    dense); on a detection backbone's 55,578-row level (61 %): 128 -> 128 134 vs 85.  With
+    ``igemm_through_segments = True`` the pair form is taken where the map's measured density
+    (map_density: maps built ahead of their use count their pairs) is at most
+    ``segments_max_density``; a map without a count goes by hint_sparse_map (build_kernel_map marks
+    the maps over rows that thin out like surfaces, see level_thinning); "always" takes the pair
+    form wherever a variant exists.  ``force`` (a
     layer's conv_config "pair_segments": True / False) overrides the module-wide setting; the
     row and channel limits hold either way."""
     mode = igemm_through_segments
@@ -1763,7 +1847,12 @@ def _segments_pay(x, kvol, cin, cout, num_out_feats, out_in_map=None, force=None
         return False
     if mode == "always":
         return True
-    hit = _sparse_maps.get(id(out_in_map)) if out_in_map is not None else None
+    if out_in_map is None:
+        return False
+    density = map_density(out_in_map)  # measured, where the map's build counted its pairs
+    if density is not None:
+        return density <= segments_max_density
+    hit = _sparse_maps.get(id(out_in_map))
     return hit is not None and hit() is out_in_map
 
 

@@ -1398,52 +1398,133 @@ extern "C" int tsmi_kmap_sorted_samples(tsmi_stream_t s, const int32_t *in_coord
   return check_launch("tsmi_kmap_sorted_samples");
 }
 
-extern "C" int tsmi_kmap_sorted(tsmi_stream_t s, const int32_t *in_coords, int64_t n_in,
-                                const int32_t *out_coords, int64_t n_out, int64_t n_out_pad,
-                                const int32_t ks[3], const int32_t stride[3], const int32_t pad[3],
-                                const int64_t *samples, int32_t *out_in_map) {
-  SortedArgs a;
-  if (int e = make_geom(&a.g, ks, stride, pad)) return e;
+// Checks the operands of one sorted-map build and fills its kernel arguments.  *cube: the
+// compile-time kernel size that serves it (2, 3) or 0; *blocks: its workgroups (0: nothing to do).
+static int sorted_args(SortedArgs *a, int *cube, int64_t *blocks, const int32_t *in_coords, int64_t n_in,
+                       const int32_t *out_coords, int64_t n_out, int64_t n_out_pad, const int32_t ks[3],
+                       const int32_t stride[3], const int32_t pad[3], const int64_t *samples,
+                       int32_t *out_in_map, int32_t *map_t, int64_t n_t_pad, int64_t *pair_words,
+                       int64_t *pair_out) {
+  if (int e = make_geom(&a->g, ks, stride, pad)) return e;
   TSMI_REQUIRE(tsmi_kmap_sorted_supported(ks), "kmap_sorted: kernel size (%d, %d, %d) not supported",
                ks[0], ks[1], ks[2]);
   TSMI_REQUIRE(n_in >= 0 && n_in < (int64_t(1) << 31) && (n_in == 0 || in_coords), "kmap_sorted: bad in_coords");
   TSMI_REQUIRE(n_out >= 0 && n_out_pad >= n_out && n_out_pad < (int64_t(1) << 31),
                "kmap_sorted: n_out_pad < n_out");
   TSMI_REQUIRE(n_out == 0 || out_coords, "kmap_sorted: null out_coords");
+  *blocks = 0;
+  *cube = 0;
+  TSMI_REQUIRE(!map_t || (n_t_pad >= n_in && n_t_pad < (int64_t(1) << 31)),
+               "kmap_sorted: the transposed map needs n_t_pad >= n_in rows");
+  TSMI_REQUIRE((pair_words == nullptr) == (pair_out == nullptr), "kmap_sorted: pair_words and pair_out go together");
+  TSMI_REQUIRE(!pair_out || n_out_pad > 0, "kmap_sorted: a map without rows has no pairs to count");
   if (n_out_pad == 0) return TSMI_OK;
   TSMI_REQUIRE(out_in_map, "kmap_sorted: null out_in_map");
-  a.in_coords = (const int4 *)in_coords;
-  a.out_coords = (const int4 *)out_coords;
-  a.map = out_in_map;
-  a.n_in = n_in;
-  a.n_out = n_out;
-  a.n_out_pad = n_out_pad;
-  a.rows = std::min(kBlock, kSortedTileInts / a.g.kvol);
+  a->in_coords = (const int4 *)in_coords;
+  a->out_coords = (const int4 *)out_coords;
+  a->map = out_in_map;
+  a->n_in = n_in;
+  a->n_out = n_out;
+  a->n_out_pad = n_out_pad;
+  a->rows = std::min(kBlock, kSortedTileInts / a->g.kvol);
   const bool sampled = samples != nullptr && tsmi_kmap_sorted_samples_elems(n_in) > 0;
-  a.first = sampled ? (const unsigned long long *)samples : nullptr;
-  a.cell = sampled ? (const unsigned long long *)samples + kSortedSamples : nullptr;
-  const int64_t blocks = ceil_div(n_out_pad, a.rows);
-  TSMI_REQUIRE(grid_fits(blocks), "kmap_sorted: too many rows for one launch");
+  a->first = sampled ? (const unsigned long long *)samples : nullptr;
+  a->cell = sampled ? (const unsigned long long *)samples + kSortedSamples : nullptr;
+  a->map_t = map_t;
+  a->n_t_pad = n_t_pad;
+  a->pair_acc = (unsigned long long *)pair_words;
+  a->pair_ticket = pair_words ? (unsigned int *)(pair_words + 1) : nullptr;
+  a->pair_out = (long long *)pair_out;
+  *blocks = ceil_div(n_out_pad, a->rows);
+  TSMI_REQUIRE(grid_fits(*blocks), "kmap_sorted: too many rows for one launch");
+  a->n_blocks = (unsigned)*blocks;
+  *cube = (ks[0] == ks[1] && ks[1] == ks[2] && a->rows == kBlock) ? ks[0] : 0;
+  if (*cube != 2 && *cube != 3) *cube = 0;
+  return TSMI_OK;
+}
+
+static int sorted_launch(hipStream_t s, const SortedArgs &a, int cube, int64_t blocks) {
+  if (blocks == 0) return TSMI_OK;
   const dim3 grid((unsigned)blocks), block(kBlock);
-  const int cube = (ks[0] == ks[1] && ks[1] == ks[2] && a.rows == kBlock) ? ks[0] : 0;
   switch (cube) {
-    case 2: hipLaunchKernelGGL(kmap_sorted_kernel<2>, grid, block, 0, (hipStream_t)s, a); break;
-    case 3: hipLaunchKernelGGL(kmap_sorted_kernel<3>, grid, block, 0, (hipStream_t)s, a); break;
-    default: hipLaunchKernelGGL(kmap_sorted_kernel<0>, grid, block, 0, (hipStream_t)s, a); break;
+    case 2: hipLaunchKernelGGL(kmap_sorted_kernel<2>, grid, block, 0, s, a); break;
+    case 3: hipLaunchKernelGGL(kmap_sorted_kernel<3>, grid, block, 0, s, a); break;
+    default: hipLaunchKernelGGL(kmap_sorted_kernel<0>, grid, block, 0, s, a); break;
   }
   return check_launch("tsmi_kmap_sorted");
 }
 
+extern "C" int tsmi_kmap_sorted(tsmi_stream_t s, const int32_t *in_coords, int64_t n_in,
+                                const int32_t *out_coords, int64_t n_out, int64_t n_out_pad,
+                                const int32_t ks[3], const int32_t stride[3], const int32_t pad[3],
+                                const int64_t *samples, int32_t *out_in_map) {
+  SortedArgs a;
+  int cube;
+  int64_t blocks;
+  if (int e = sorted_args(&a, &cube, &blocks, in_coords, n_in, out_coords, n_out, n_out_pad, ks, stride, pad,
+                          samples, out_in_map, nullptr, 0, nullptr, nullptr))
+    return e;
+  return sorted_launch((hipStream_t)s, a, cube, blocks);
+}
+
 extern "C" int tsmi_kmap_sorted_batch(tsmi_stream_t s, int count, const int64_t *args) {
   TSMI_REQUIRE(count >= 0 && (count == 0 || args), "kmap_sorted_batch: bad arguments");
-  for (int i = 0; i < count; ++i) {
-    const int64_t *a = args + 16 * i;
-    int32_t geom[9];
-    for (int j = 0; j < 9; ++j) geom[j] = (int32_t)a[7 + j];
-    if (int e = tsmi_kmap_sorted(s, (const int32_t *)(uintptr_t)a[0], a[1], (const int32_t *)(uintptr_t)a[2], a[3],
-                                 a[4], geom, geom + 3, geom + 6, (const int64_t *)(uintptr_t)a[5],
-                                 (int32_t *)(uintptr_t)a[6]))
-      return e;
+  constexpr int kWords = 20;  // int64 words per map
+  int done = 0;
+  while (done < count) {
+    // as many of the next maps as one launch takes: 2^3 and 3^3 kernels, up to kSortedBatchMax
+    SortedBatch b;
+    b.count = 0;
+    b.first_block[0] = 0;
+    SortedArgs single;
+    int single_cube = 0;
+    int64_t single_blocks = 0;
+    bool have_single = false;
+    while (done < count && b.count < kSortedBatchMax) {
+      const int64_t *a = args + (int64_t)kWords * done;
+      int32_t geom[9];
+      for (int j = 0; j < 9; ++j) geom[j] = (int32_t)a[7 + j];
+      SortedArgs one;
+      int cube;
+      int64_t blocks;
+      if (int e = sorted_args(&one, &cube, &blocks, (const int32_t *)(uintptr_t)a[0], a[1],
+                              (const int32_t *)(uintptr_t)a[2], a[3], a[4], geom, geom + 3, geom + 6,
+                              (const int64_t *)(uintptr_t)a[5], (int32_t *)(uintptr_t)a[6],
+                              (int32_t *)(uintptr_t)a[16], a[17], (int64_t *)(uintptr_t)a[18],
+                              (int64_t *)(uintptr_t)a[19]))
+        return e;
+      if (blocks == 0) {
+        ++done;
+        continue;
+      }
+      if (cube == 0 || !grid_fits((int64_t)b.first_block[b.count] + blocks)) {
+        if (b.count > 0) break;  // launch what has been gathered first
+        single = one;
+        single_cube = cube;
+        single_blocks = blocks;
+        have_single = true;
+        ++done;
+        break;
+      }
+      b.a[b.count] = one;
+      b.kc[b.count] = cube;
+      b.first_block[b.count + 1] = b.first_block[b.count] + (unsigned)blocks;
+      ++b.count;
+      ++done;
+    }
+    if (have_single) {
+      if (int e = sorted_launch((hipStream_t)s, single, single_cube, single_blocks)) return e;
+    } else if (b.count == 1) {
+      if (int e = sorted_launch((hipStream_t)s, b.a[0], b.kc[0], b.first_block[1])) return e;
+    } else if (b.count > 1) {
+      for (int i = b.count; i < kSortedBatchMax; ++i) {
+        b.a[i] = b.a[0];
+        b.kc[i] = b.kc[0];
+        b.first_block[i + 1] = b.first_block[b.count];
+      }
+      hipLaunchKernelGGL(kmap_sorted_batch_kernel, dim3(b.first_block[b.count]), dim3(kBlock), 0, (hipStream_t)s, b);
+      if (int e = check_launch("tsmi_kmap_sorted_batch")) return e;
+    }
   }
   return TSMI_OK;
 }
