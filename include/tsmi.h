@@ -576,15 +576,22 @@ int tsmi_conv_implicit_gemm_grouped(tsmi_stream_t s, const void *x, const void *
                                     int dtype, const void *bias, const void *residual, int relu,
                                     void *y);
 
-/* tsmi_conv_implicit_gemm and tsmi_conv_implicit_gemm_segments with their arguments in one block
- * of host int64, in the order of the declarations above (pointers and the stream as integers,
- * 18 and 17 entries): the two calls a forward makes most often - about 60 per forward of a U-Net -
- * for bindings that pay per argument (ctypes converts one in 0.1 us).  Same checks, same
- * launches, same status.  No counterpart in the reference (pybind11 converts its arguments in
- * compiled code). */
-int tsmi_conv_implicit_gemm_packed(const int64_t *args);
-int tsmi_conv_implicit_gemm_segments_packed(const int64_t *args);
-int tsmi_conv_implicit_gemm_grouped_packed(const int64_t *args); /* 17 entries */
+/* tsmi_conv_implicit_gemm, tsmi_conv_implicit_gemm_segments and tsmi_conv_implicit_gemm_grouped
+ * with their arguments in one block of host int64, in the order of the declarations above
+ * (pointers and the stream as integers: 18, 17 and 17 entries) followed by three entries that
+ * place the result: [ldy, y2, ldy2] - the calls a forward makes most often, about 60 per forward
+ * of a U-Net, for bindings that pay per argument (ctypes converts one in 0.1 us).
+ *   ldy   row pitch of y in elements (0: cout, a dense result); a multiple of 8 that holds a row
+ *   y2    optional second destination of the same rows (0: none), 16-byte aligned, row pitch ldy2
+ * With them a layer writes into a column slice of a wider buffer, and a layer whose result a
+ * later concatenation would copy writes it there as well: torch.cat([a, b], 1) of two layers'
+ * results (the decoder of a U-Net, the reference's backbones/unet.py:99-103) costs no launch.
+ * All three zero: same checks, same launches, same status as the unpacked call.  Calls that would
+ * finish their rows in a second launch (the offset split without tile counters) refuse a placed
+ * result.  No counterpart in the reference (pybind11 converts its arguments in compiled code). */
+int tsmi_conv_implicit_gemm_packed(const int64_t *args);          /* 21 entries */
+int tsmi_conv_implicit_gemm_segments_packed(const int64_t *args); /* 20 entries */
+int tsmi_conv_implicit_gemm_grouped_packed(const int64_t *args);  /* 20 entries */
 
 /* Gather-GEMM-scatter, step 1: buffer[nbaddrs[k] + p, :] = X[in(k,p), :].
  * Replaces gather_all_kernel_pad_sep_with_mask / gather_kernel

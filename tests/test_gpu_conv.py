@@ -11,7 +11,7 @@ import pytest
 import torch
 
 import oracle
-from helpers import random_coords, rel_rms
+from helpers import lidar_like_coords, random_coords, rel_rms
 
 pytestmark = pytest.mark.gpu
 
@@ -513,3 +513,55 @@ def test_short_path_of_cached_map_layers_equals_conv3d(mods):
     with torch.no_grad():
         assert F.conv3d_cached(mid, subm.kernel, subm.bias, subm.kernel_size, subm.stride, (1, 1, 1), False,
                                cfg, None, "relu") is None
+
+
+@pytest.mark.parametrize("n,cin,cout,dtype,how", [
+    (40000, 32, 32, torch.float16, "plain"), (5000, 64, 64, torch.float16, "plain"),
+    (3000, 256, 256, torch.float16, "plain"), (3000, 256, 256, torch.float16, "segments"),
+    (40000, 96, 96, torch.bfloat16, "grouped"), (9000, 16, 24, torch.float32, "plain"),
+    (2000, 4, 32, torch.float16, "plain"), (6000, 128, 96, torch.float16, "transposed")])
+def test_results_placed_into_column_slices_equal_the_dense_ones(n, cin, cout, dtype, how, monkeypatch):
+    """out= / also=: the launch writes its rows into a column slice of a wider buffer (and a
+    second time into another) - bit for bit the rows of the dense result, nothing outside the
+    slices touched; bias, residual and ReLU included."""
+    import torchsparse_amd as ts
+    from torchsparse_amd import backend
+    from torchsparse_amd import nn as spnn
+    rng = np.random.default_rng(n + cin)
+    coords_np = lidar_like_coords(rng, n)
+    coords_np = coords_np[np.lexsort((coords_np[:, 3], coords_np[:, 2], coords_np[:, 1], coords_np[:, 0]))]
+    coords = torch.from_numpy(coords_np).cuda()
+    n = coords.shape[0]
+    torch.manual_seed(n)
+    if how == "grouped":
+        monkeypatch.setattr(backend, "igemm_group_rows", "always")
+        monkeypatch.setattr(backend, "group_min_rows", 1024)
+    if how == "transposed":
+        down = spnn.Conv3d(8, cin, 2, stride=2).cuda().to(dtype).eval()
+        layer = spnn.Conv3d(cin, cout, 2, stride=2, transposed=True, bias=True).cuda().to(dtype).eval()
+        with torch.no_grad():
+            x = down(ts.SparseTensor(torch.randn(n, 8, device="cuda", dtype=dtype), coords))
+        n_out = n
+    else:
+        layer = spnn.Conv3d(cin, cout, 3, bias=True).cuda().to(dtype).eval()
+        if how == "segments":
+            monkeypatch.setattr(backend, "igemm_through_segments", "always")
+        x = ts.SparseTensor(torch.randn(n, cin, device="cuda", dtype=dtype), coords)
+        n_out = n
+    layer.activation = "relu"
+    res = torch.randn(n_out, cout, device="cuda", dtype=dtype)
+    with torch.no_grad():
+        want = layer(x, residual=res).feats
+        wide = torch.full((n_out, 8 + cout + 16), 7.0, device="cuda", dtype=dtype)
+        second = torch.full((n_out, cout + 8), 5.0, device="cuda", dtype=dtype)
+        got = layer(x, residual=res, out=wide[:, 8:8 + cout], also=second[:, :cout])
+    assert got.feats.data_ptr() == wide[:, 8:].data_ptr() and got.feats.shape == (n_out, cout)
+    assert torch.equal(got.feats, want) and torch.equal(second[:, :cout], want)
+    assert (wide[:, :8] == 7).all() and (wide[:, 8 + cout:] == 7).all() and (second[:, cout:] == 5).all()
+    assert torch.equal(got.coords, x.coords if how != "transposed" else coords)
+    # other dataflows copy; misplaced views are refused
+    with torch.no_grad():
+        with pytest.raises(ValueError, match="placed"):
+            layer(x, out=wide[:, 3:3 + cout])
+        with pytest.raises(ValueError, match="placed"):
+            layer(x, also=second[:-1, :cout])

@@ -64,7 +64,9 @@ class SparseResBlock(nn.Module):
             self.shortcut = nn.Identity()
         self.relu = spnn.ReLU(True)
 
-    def forward(self, x: SparseTensor) -> SparseTensor:
+    def forward(self, x: SparseTensor, also=None) -> SparseTensor:
+        """``also``: a [N, out_channels] view the block's result is written into as well (the
+        place a later concatenation wants it)."""
         if getattr(self, "_fused_tail", False):
             # after nn.utils.fuse_inference(): norms are folded into the convolutions and the
             # shortcut add + ReLU run in the epilogue of the block's last convolution
@@ -77,5 +79,10 @@ class SparseResBlock(nn.Module):
             y = x
             for layer in layers[:-1]:
                 y = call_module(layer, y)
-            return call_module(layers[-1], y, residual=residual)
-        return self.relu(self.main(x) + self.shortcut(x))
+            if also is None:
+                return call_module(layers[-1], y, residual=residual)
+            return call_module(layers[-1], y, residual=residual, also=also)
+        out = self.relu(self.main(x) + self.shortcut(x))
+        if also is not None:
+            also.copy_(out.feats)
+        return out

@@ -43,6 +43,11 @@ class SparseResUNet(nn.Module):
             }) for i in range(4))
 
     def forward(self, x: SparseTensor) -> List[SparseTensor]:
+        plan = self.__dict__.get("_placed_plan")
+        if plan is None:
+            plan = self.__dict__["_placed_plan"] = self._plan_placement()
+        if plan and not self.training and x.feats.is_cuda:
+            return self._forward_placed(x, plan)
         skips = [self.stem(x)]
         for enc in self.encoders:
             skips.append(enc(skips[-1]))
@@ -50,6 +55,64 @@ class SparseResUNet(nn.Module):
         y = skips[-1]
         for i, dec in enumerate(self.decoders):
             y = dec["fuse"](cat([dec["upsample"](y), skips[3 - i]]))
+            outputs.append(y)
+        return outputs
+
+    # In inference form (nn.utils.fuse_inference: norms folded, activations in the convolutions'
+    # epilogues) the concatenations of the decoder cost nothing: the buffer [N, C_up + C_skip] of
+    # a level is allocated when the level's skip is produced, the layer that produces the skip
+    # writes it into the right-hand columns as well, and the transposed convolution of the decoder
+    # writes its rows into the left-hand ones.
+
+    def _plan_placement(self):
+        """Per skip level (stem, encoders 0-2): (layers before the last, the last layer, the
+        transposed convolution that returns to the level, its channels, the skip's channels);
+        () when the model is not in inference form or a channel count does not fit."""
+        from .modules.blocks import SparseResBlock
+        stages = [self.stem] + list(self.encoders)[:3]
+        plan = []
+        for j, stage in enumerate(stages):
+            layers = [m for m in stage if not isinstance(m, nn.Identity)]
+            up = [m for m in self.decoders[3 - j]["upsample"] if not isinstance(m, nn.Identity)]
+            last = layers[-1]
+            if len(up) != 1 or not isinstance(up[0], spnn.Conv3d):
+                return ()
+            if isinstance(last, SparseResBlock):
+                if not getattr(last, "_fused_tail", False):
+                    return ()
+                c_skip = last.main[0].out_channels
+            elif isinstance(last, spnn.Conv3d):
+                c_skip = last.out_channels
+            else:
+                return ()
+            if any(isinstance(m, spnn.BatchNorm) for m in stage.modules()):
+                return ()
+            c_up = up[0].out_channels
+            if c_up % 8 or c_skip % 8:
+                return ()
+            plan.append((tuple(layers[:-1]), last, up[0], c_up, c_skip))
+        return tuple(plan)
+
+    def _forward_placed(self, x: SparseTensor, plan) -> List[SparseTensor]:
+        from ..nn.utils.fuse import call_module
+        skips, buffers = [], []
+        y = x
+        for before, last, _, c_up, c_skip in plan:
+            for m in before:
+                y = call_module(m, y)
+            buf = y.feats.new_empty(y.feats.shape[0], c_up + c_skip)
+            y = call_module(last, y, also=buf[:, c_up:])
+            skips.append(y)
+            buffers.append(buf)
+        y = call_module(self.encoders[3], y)
+        outputs = skips + [y]
+        for i, dec in enumerate(self.decoders):
+            _, _, up, c_up, _ = plan[3 - i]
+            buf = buffers[3 - i]
+            u = call_module(up, y, out=buf[:, :c_up])
+            if u.feats.shape[0] != buf.shape[0]:  # (cannot happen: the level's rows are its skip's)
+                raise RuntimeError("the transposed convolution did not return to the rows of its skip")
+            y = call_module(dec["fuse"], SparseTensor._make(buf, u.coords, u.stride, u.spatial_range, u._caches))
             outputs.append(y)
         return outputs
 

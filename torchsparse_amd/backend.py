@@ -1471,8 +1471,31 @@ def _epilogue_args(bias, residual, x, n_out, cout):
     return pb, pr
 
 
-_PACK17 = struct.Struct("17q").pack
-_PACK18 = struct.Struct("18q").pack
+_PACK20 = struct.Struct("20q").pack
+_PACK21 = struct.Struct("21q").pack
+
+
+def _placed(x, num_out_feats: int, cout: int, out, also):
+    """(y, row pitch of y or 0, address of the second destination or 0, its row pitch) of a
+    convolution whose result goes into ``out`` (None: a new dense tensor) and, a second time, into
+    ``also``: [num_out_feats, cout] views of the features' dtype with unit column stride, rows a
+    multiple of 8 elements apart and 16-byte aligned (column slices of wider buffers)."""
+    ldy = a2 = ld2 = 0
+    for t in (out, also):
+        if t is None:
+            continue
+        if (t.dtype != x.dtype or t.dim() != 2 or t.shape[0] != num_out_feats or t.shape[1] != cout
+                or t.stride(1) != 1 or t.stride(0) % 8 or t.stride(0) < cout or t.data_ptr() % 16
+                or t.device != x.device):
+            raise ValueError(f"a placed result needs a {x.dtype} [{num_out_feats}, {cout}] view with unit column "
+                             "stride, rows a multiple of 8 elements apart and 16-byte aligned")
+    if out is None:
+        y = x.new_empty(num_out_feats, cout)
+    else:
+        y, ldy = out, out.stride(0)
+    if also is not None:
+        a2, ld2 = also.data_ptr(), also.stride(0)
+    return y, ldy, a2, ld2
 
 # Buffers the library owns (the scratch of a stream, its tile counters, identity maps, pair
 # segments, grouped maps, packed weights) live in tables that drop or replace their entries.  A
@@ -1778,15 +1801,19 @@ def _grouping_pays(x, kvol: int, cin: int, cout: int, num_out_feats: int, out_in
 
 
 def conv_implicit_gemm_grouped(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias=None,
-                               residual=None, relu=False) -> torch.Tensor:
+                               residual=None, relu=False, out=None, also=None) -> torch.Tensor:
     """The implicit-GEMM sums over the grouped copy of the map (same results bit for bit)."""
     g = grouped_map(out_in_map, num_out_feats)
-    y = x.new_empty(num_out_feats, cout)
+    if out is None and also is None:
+        y, ldy, a2, ld2 = x.new_empty(num_out_feats, cout), 0, 0, 0
+    else:
+        y, ldy, a2, ld2 = _placed(x, num_out_feats, cout, out, also)
     pb, pr = _epilogue_args(bias, residual, x, num_out_feats, cout)
     ptrs = g.ptrs
-    _check(_C.tsmi_conv_implicit_gemm_grouped_packed(_PACK17(
+    _check(_C.tsmi_conv_implicit_gemm_grouped_packed(_PACK20(
         _stream(), x.data_ptr(), wp.data_ptr(), ptrs[0], ptrs[1], ptrs[3], ptrs[4], g.padded,
-        num_out_feats, kvol, cin, cout, _dtype_code(x), pb or 0, pr or 0, int(relu), y.data_ptr())))
+        num_out_feats, kvol, cin, cout, _dtype_code(x), pb or 0, pr or 0, int(relu), y.data_ptr(),
+        ldy, a2, ld2)))
     return y
 
 
@@ -1857,33 +1884,42 @@ def _segments_pay(x, kvol, cin, cout, num_out_feats, out_in_map=None, force=None
 
 
 def conv_implicit_gemm_segments(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias=None,
-                                residual=None, relu=False) -> torch.Tensor:
+                                residual=None, relu=False, out=None, also=None) -> torch.Tensor:
     """The implicit-GEMM sums over pair segments: one launch multiplies every pair's input row
     by its offset's weights (a workgroup reads one offset's weights only), a second adds each
     output row's products."""
     seg = pair_segments(out_in_map, num_out_feats)
     seg_rows = seg.seg_rows
-    y = x.new_empty(num_out_feats, cout)  # (the cheapest form of the call: 1.2 us against 1.6)
+    if out is None and also is None:
+        y, ldy, a2, ld2 = x.new_empty(num_out_feats, cout), 0, 0, 0  # (the cheapest form of the call: 1.2 us against 1.6)
+    else:
+        y, ldy, a2, ld2 = _placed(x, num_out_feats, cout, out, also)
     stream = _stream()
     pb, pr = _epilogue_args(bias, residual, x, num_out_feats, cout)
     with _scratch_lock:
         products = _scratch(x.device, stream, kvol * seg_rows * cout * x.element_size())
-        _check(_C.tsmi_conv_implicit_gemm_segments_packed(_PACK17(
+        _check(_C.tsmi_conv_implicit_gemm_segments_packed(_PACK20(
             stream, x.data_ptr(), wp.data_ptr(), seg.in_rows_ptr, seg.counts_ptr, seg.pos_ptr, seg_rows,
             num_out_feats, kvol, cin, cout, _dtype_code(x), pb or 0, pr or 0, int(relu), products,
-            y.data_ptr())))
+            y.data_ptr(), ldy, a2, ld2)))
     return y
 
 
 def _implicit_gemm(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias=None, residual=None,
-                   relu=False, segments=None) -> torch.Tensor:
+                   relu=False, segments=None, out=None, also=None) -> torch.Tensor:
+    """``out`` / ``also``: the result goes into ``out`` instead of a new tensor, and a second time
+    into ``also`` (see _placed: column slices of wider buffers, which spares the copy of a later
+    concatenation)."""
     if _segments_pay(x, kvol, cin, cout, num_out_feats, out_in_map, segments):
         return conv_implicit_gemm_segments(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias,
-                                           residual, relu)
+                                           residual, relu, out, also)
     if _grouping_pays(x, kvol, cin, cout, num_out_feats, out_in_map):
         return conv_implicit_gemm_grouped(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias,
-                                          residual, relu)
-    y = x.new_empty(num_out_feats, cout)  # (the cheapest form of the call: 1.2 us against 1.6)
+                                          residual, relu, out, also)
+    if out is None and also is None:
+        y, ldy, a2, ld2 = x.new_empty(num_out_feats, cout), 0, 0, 0  # (the cheapest form of the call: 1.2 us against 1.6)
+    else:
+        y, ldy, a2, ld2 = _placed(x, num_out_feats, cout, out, also)
     code = _dtype_code(x)
     stream = _stream()
     pb, pr = _epilogue_args(bias, residual, x, num_out_feats, cout)
@@ -1891,15 +1927,16 @@ def _implicit_gemm(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias=None,
     ws_elems = _workspace_elems(num_out_feats, kvol, cin, cout, code) if num_out_feats < 65536 else 0
     if ws_elems > 0:  # (only maps with few row tiles use the offset split)
         with _scratch_lock:
-            _check(_C.tsmi_conv_implicit_gemm_packed(_PACK18(
+            _check(_C.tsmi_conv_implicit_gemm_packed(_PACK21(
                 stream, x.data_ptr(), wp.data_ptr(), out_in_map.data_ptr(), out_in_map.shape[0],
                 num_out_feats, kvol, cin, cout, code, pb or 0, pr or 0, int(relu),
                 _scratch(x.device, stream, 4 * ws_elems), ws_elems,
-                _tile_counters(x.device, stream).data_ptr(), _N_TILE_COUNTERS, y.data_ptr())))
+                _tile_counters(x.device, stream).data_ptr(), _N_TILE_COUNTERS, y.data_ptr(), ldy, a2, ld2)))
     else:
-        _check(_C.tsmi_conv_implicit_gemm_packed(_PACK18(
+        _check(_C.tsmi_conv_implicit_gemm_packed(_PACK21(
             stream, x.data_ptr(), wp.data_ptr(), out_in_map.data_ptr(), out_in_map.shape[0], num_out_feats,
-            kvol, cin, cout, code, pb or 0, pr or 0, int(relu), 0, 0, 0, _N_TILE_COUNTERS, y.data_ptr())))
+            kvol, cin, cout, code, pb or 0, pr or 0, int(relu), 0, 0, 0, _N_TILE_COUNTERS, y.data_ptr(),
+            ldy, a2, ld2)))
     return y
 
 

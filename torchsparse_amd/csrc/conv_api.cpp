@@ -47,14 +47,27 @@ extern "C" int64_t tsmi_conv_workspace_elems(int64_t n_tile_rows, int64_t n_out,
   return ops->workspace(n_tile_rows, n_out, kvol, split, cin, cout, sorted);
 }
 
-extern "C" int tsmi_conv_implicit_gemm(tsmi_stream_t s, const void *x, const void *w_packed,
-                                       const int32_t *map, int64_t n_map_rows, int64_t n_out,
-                                       int kvol, int cin, int cout, int dtype, const void *bias,
-                                       const void *residual, int relu, float *workspace,
-                                       int64_t workspace_elems, int32_t *tile_counters,
-                                       int64_t n_tile_counters, void *y) {
+// A placed result (tsmi.h: the *_packed entry points): pitches in whole 16-byte pieces that hold
+// a row, the second destination aligned like the first.
+static int check_place(const char *who, const OutPlace *place, int cout) {
+  if (!place) return TSMI_OK;
+  TSMI_REQUIRE(place->ldy == 0 || (place->ldy >= cout && place->ldy % 8 == 0),
+               "%s: the row pitch of y (%lld) must be a multiple of 8 elements that holds %d channels", who,
+               (long long)place->ldy, cout);
+  TSMI_REQUIRE(!place->y2 || (aligned16(place->y2) && place->ldy2 >= cout && place->ldy2 % 8 == 0),
+               "%s: the second destination must be 16-byte aligned, its row pitch (%lld) a multiple of 8 "
+               "elements that holds %d channels", who, (long long)place->ldy2, cout);
+  return TSMI_OK;
+}
+
+static int implicit_gemm(tsmi_stream_t s, const void *x, const void *w_packed, const int32_t *map,
+                         int64_t n_map_rows, int64_t n_out, int kvol, int cin, int cout, int dtype,
+                         const void *bias, const void *residual, int relu, float *workspace,
+                         int64_t workspace_elems, int32_t *tile_counters, int64_t n_tile_counters, void *y,
+                         const OutPlace *place) {
   const ConvOps *ops = ops_for(dtype);
   if (int e = check_shapes("conv_implicit_gemm", ops, kvol, cin, cout)) return e;
+  if (int e = check_place("conv_implicit_gemm", place, cout)) return e;
   TSMI_REQUIRE(n_out >= 0 && n_map_rows >= n_out, "conv_implicit_gemm: map has %lld rows, need %lld",
                (long long)n_map_rows, (long long)n_out);
   if (n_out == 0) return TSMI_OK;
@@ -63,7 +76,17 @@ extern "C" int tsmi_conv_implicit_gemm(tsmi_stream_t s, const void *x, const voi
                "conv_implicit_gemm: x, w_packed and y must be 16-byte aligned");
   return ops->igemm((hipStream_t)s, x, w_packed, map, n_map_rows, n_out, n_out, kvol, cin, cout,
                     bias, residual, relu, y, nullptr, 0, 1, workspace, workspace_elems,
-                    tile_counters, tile_counters ? n_tile_counters : 0, nullptr, nullptr);
+                    tile_counters, tile_counters ? n_tile_counters : 0, nullptr, nullptr, place);
+}
+
+extern "C" int tsmi_conv_implicit_gemm(tsmi_stream_t s, const void *x, const void *w_packed,
+                                       const int32_t *map, int64_t n_map_rows, int64_t n_out,
+                                       int kvol, int cin, int cout, int dtype, const void *bias,
+                                       const void *residual, int relu, float *workspace,
+                                       int64_t workspace_elems, int32_t *tile_counters,
+                                       int64_t n_tile_counters, void *y) {
+  return implicit_gemm(s, x, w_packed, map, n_map_rows, n_out, kvol, cin, cout, dtype, bias, residual, relu,
+                       workspace, workspace_elems, tile_counters, n_tile_counters, y, nullptr);
 }
 
 extern "C" int tsmi_conv_implicit_gemm_sorted(tsmi_stream_t s, const void *x, const void *w_packed,
@@ -90,17 +113,18 @@ extern "C" int tsmi_conv_implicit_gemm_sorted(tsmi_stream_t s, const void *x, co
                "conv_implicit_gemm_sorted: x, w_packed and y must be 16-byte aligned");
   return ops->igemm((hipStream_t)s, x, w_packed, reorder_map, n_pad, n_pad, n_out, kvol, cin, cout,
                     bias, residual, relu, y, reorder_loc, n_pad, split, workspace, workspace_elems,
-                    tile_counters, tile_counters ? n_tile_counters : 0, nullptr, nullptr);
+                    tile_counters, tile_counters ? n_tile_counters : 0, nullptr, nullptr, nullptr);
 }
 
-extern "C" int tsmi_conv_implicit_gemm_grouped(tsmi_stream_t s, const void *x, const void *w_packed,
+static int implicit_gemm_grouped(tsmi_stream_t s, const void *x, const void *w_packed,
                                                const int32_t *grouped_map, const int32_t *row_of,
                                                const int32_t *order64, const int32_t *order128,
                                                int64_t n_grouped, int64_t n_out, int kvol, int cin,
                                                int cout, int dtype, const void *bias,
-                                               const void *residual, int relu, void *y) {
+                                               const void *residual, int relu, void *y, const OutPlace *place) {
   const ConvOps *ops = ops_for(dtype);
   if (int e = check_shapes("conv_implicit_gemm_grouped", ops, kvol, cin, cout)) return e;
+  if (int e = check_place("conv_implicit_gemm_grouped", place, cout)) return e;
   TSMI_REQUIRE(n_out >= 0 && n_grouped >= n_out && n_grouped % 128 == 0,
                "conv_implicit_gemm_grouped: bad sizes (%lld grouped rows for %lld outputs)",
                (long long)n_grouped, (long long)n_out);
@@ -111,7 +135,17 @@ extern "C" int tsmi_conv_implicit_gemm_grouped(tsmi_stream_t s, const void *x, c
                "conv_implicit_gemm_grouped: x, w_packed and y must be 16-byte aligned");
   return ops->igemm((hipStream_t)s, x, w_packed, grouped_map, n_grouped, n_grouped, n_out, kvol, cin,
                     cout, bias, residual, relu, y, row_of, n_grouped, 1, nullptr, 0, nullptr, 0, order64,
-                    order128);
+                    order128, place);
+}
+
+extern "C" int tsmi_conv_implicit_gemm_grouped(tsmi_stream_t s, const void *x, const void *w_packed,
+                                               const int32_t *grouped_map, const int32_t *row_of,
+                                               const int32_t *order64, const int32_t *order128,
+                                               int64_t n_grouped, int64_t n_out, int kvol, int cin,
+                                               int cout, int dtype, const void *bias,
+                                               const void *residual, int relu, void *y) {
+  return implicit_gemm_grouped(s, x, w_packed, grouped_map, row_of, order64, order128, n_grouped, n_out, kvol,
+                               cin, cout, dtype, bias, residual, relu, y, nullptr);
 }
 
 extern "C" int64_t tsmi_conv_wgrad_workspace_elems(int64_t n_in, int kvol, int cin, int cout,
@@ -193,14 +227,14 @@ extern "C" int tsmi_conv_segments_supported(int kvol, int cin, int cout, int dty
   return ops->segments_supported(kvol, cin, cout);
 }
 
-extern "C" int tsmi_conv_implicit_gemm_segments(tsmi_stream_t s, const void *x, const void *w_packed,
-                                               const int32_t *in_rows, const int32_t *counts,
-                                               const int32_t *pos, int64_t seg_rows, int64_t n_out,
-                                               int kvol, int cin, int cout, int dtype,
-                                               const void *bias, const void *residual, int relu,
-                                               void *products, void *y) {
+static int implicit_gemm_segments(tsmi_stream_t s, const void *x, const void *w_packed,
+                                  const int32_t *in_rows, const int32_t *counts, const int32_t *pos,
+                                  int64_t seg_rows, int64_t n_out, int kvol, int cin, int cout, int dtype,
+                                  const void *bias, const void *residual, int relu, void *products, void *y,
+                                  const OutPlace *place) {
   const ConvOps *ops = ops_for(dtype);
   if (int e = check_shapes("conv_implicit_gemm_segments", ops, kvol, cin, cout)) return e;
+  if (int e = check_place("conv_implicit_gemm_segments", place, cout)) return e;
   TSMI_REQUIRE(n_out >= 0 && seg_rows >= n_out && seg_rows % 64 == 0,
                "conv_implicit_gemm_segments: bad sizes (n_out %lld, seg_rows %lld)", (long long)n_out,
                (long long)seg_rows);
@@ -213,7 +247,17 @@ extern "C" int tsmi_conv_implicit_gemm_segments(tsmi_stream_t s, const void *x, 
                             products))
     return e;
   return ops->segment_sum((hipStream_t)s, products, pos, n_out, kvol, seg_rows, cout, bias, residual,
-                          relu, y);
+                          relu, y, place);
+}
+
+extern "C" int tsmi_conv_implicit_gemm_segments(tsmi_stream_t s, const void *x, const void *w_packed,
+                                               const int32_t *in_rows, const int32_t *counts,
+                                               const int32_t *pos, int64_t seg_rows, int64_t n_out,
+                                               int kvol, int cin, int cout, int dtype,
+                                               const void *bias, const void *residual, int relu,
+                                               void *products, void *y) {
+  return implicit_gemm_segments(s, x, w_packed, in_rows, counts, pos, seg_rows, n_out, kvol, cin, cout, dtype,
+                                bias, residual, relu, products, y, nullptr);
 }
 
 extern "C" int tsmi_gs_gather(tsmi_stream_t s, const void *x, const int32_t *nbmaps_inter,
@@ -259,28 +303,41 @@ extern "C" int tsmi_gs_scatter(tsmi_stream_t s, const void *out_buffer, const in
 // converts arguments one by one (ctypes: 0.1 us each) passes one pointer instead of 17 or 18.
 static inline const void *as_ptr(int64_t v) { return (const void *)(uintptr_t)v; }
 
+// The placement of a packed call's result: three more entries (row pitch of y, second destination,
+// its row pitch); all zero: a dense y and nothing else.
+static const OutPlace *place_of(const int64_t *w, OutPlace *place) {
+  if (w[0] == 0 && w[1] == 0) return nullptr;
+  place->ldy = w[0];
+  place->y2 = (void *)as_ptr(w[1]);
+  place->ldy2 = w[2];
+  return place;
+}
+
 extern "C" int tsmi_conv_implicit_gemm_packed(const int64_t *a) {
   TSMI_REQUIRE(a, "conv_implicit_gemm_packed: null argument block");
-  return tsmi_conv_implicit_gemm((tsmi_stream_t)as_ptr(a[0]), as_ptr(a[1]), as_ptr(a[2]), (const int32_t *)as_ptr(a[3]),
-                                 a[4], a[5], (int)a[6], (int)a[7], (int)a[8], (int)a[9], as_ptr(a[10]),
-                                 as_ptr(a[11]), (int)a[12], (float *)as_ptr(a[13]), a[14],
-                                 (int32_t *)as_ptr(a[15]), a[16], (void *)as_ptr(a[17]));
+  OutPlace place;
+  return implicit_gemm((tsmi_stream_t)as_ptr(a[0]), as_ptr(a[1]), as_ptr(a[2]), (const int32_t *)as_ptr(a[3]),
+                       a[4], a[5], (int)a[6], (int)a[7], (int)a[8], (int)a[9], as_ptr(a[10]),
+                       as_ptr(a[11]), (int)a[12], (float *)as_ptr(a[13]), a[14],
+                       (int32_t *)as_ptr(a[15]), a[16], (void *)as_ptr(a[17]), place_of(a + 18, &place));
 }
 
 extern "C" int tsmi_conv_implicit_gemm_grouped_packed(const int64_t *a) {
   TSMI_REQUIRE(a, "conv_implicit_gemm_grouped_packed: null argument block");
-  return tsmi_conv_implicit_gemm_grouped((tsmi_stream_t)as_ptr(a[0]), as_ptr(a[1]), as_ptr(a[2]),
-                                         (const int32_t *)as_ptr(a[3]), (const int32_t *)as_ptr(a[4]),
-                                         (const int32_t *)as_ptr(a[5]), (const int32_t *)as_ptr(a[6]), a[7], a[8],
-                                         (int)a[9], (int)a[10], (int)a[11], (int)a[12], as_ptr(a[13]),
-                                         as_ptr(a[14]), (int)a[15], (void *)as_ptr(a[16]));
+  OutPlace place;
+  return implicit_gemm_grouped((tsmi_stream_t)as_ptr(a[0]), as_ptr(a[1]), as_ptr(a[2]),
+                               (const int32_t *)as_ptr(a[3]), (const int32_t *)as_ptr(a[4]),
+                               (const int32_t *)as_ptr(a[5]), (const int32_t *)as_ptr(a[6]), a[7], a[8],
+                               (int)a[9], (int)a[10], (int)a[11], (int)a[12], as_ptr(a[13]),
+                               as_ptr(a[14]), (int)a[15], (void *)as_ptr(a[16]), place_of(a + 17, &place));
 }
 
 extern "C" int tsmi_conv_implicit_gemm_segments_packed(const int64_t *a) {
   TSMI_REQUIRE(a, "conv_implicit_gemm_segments_packed: null argument block");
-  return tsmi_conv_implicit_gemm_segments((tsmi_stream_t)as_ptr(a[0]), as_ptr(a[1]), as_ptr(a[2]),
-                                          (const int32_t *)as_ptr(a[3]), (const int32_t *)as_ptr(a[4]),
-                                          (const int32_t *)as_ptr(a[5]), a[6], a[7], (int)a[8], (int)a[9],
-                                          (int)a[10], (int)a[11], as_ptr(a[12]), as_ptr(a[13]), (int)a[14],
-                                          (void *)as_ptr(a[15]), (void *)as_ptr(a[16]));
+  OutPlace place;
+  return implicit_gemm_segments((tsmi_stream_t)as_ptr(a[0]), as_ptr(a[1]), as_ptr(a[2]),
+                                (const int32_t *)as_ptr(a[3]), (const int32_t *)as_ptr(a[4]),
+                                (const int32_t *)as_ptr(a[5]), a[6], a[7], (int)a[8], (int)a[9],
+                                (int)a[10], (int)a[11], as_ptr(a[12]), as_ptr(a[13]), (int)a[14],
+                                (void *)as_ptr(a[15]), (void *)as_ptr(a[16]), place_of(a + 17, &place));
 }

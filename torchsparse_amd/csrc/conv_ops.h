@@ -10,6 +10,16 @@
 
 namespace tsmi {
 
+// Where a convolution's result rows go when not into a dense [n_out, cout] tensor: row pitch of y
+// in elements (0: cout), and an optional second destination that receives the same values (a
+// column slice of a wider buffer, say).  Honoured by the launches that finish their rows
+// themselves (igemm with its in-kernel epilogue, segment_sum).
+struct OutPlace {
+  int64_t ldy;
+  void *y2;
+  int64_t ldy2;
+};
+
 struct ConvOps {
   int step;  // reduction elements per MFMA step (Cin is padded to a multiple)
   int (*pack)(hipStream_t s, const void *w, void *wp, int kvol, int cin, int cout);
@@ -23,7 +33,8 @@ struct ConvOps {
                int64_t n_map_rows, int64_t n_tile_rows, int64_t n_out, int kvol, int cin, int cout,
                const void *bias, const void *residual, int relu, void *y, const int32_t *row_out,
                int64_t row_out_stride, int split, float *partial, int64_t partial_elems,
-               int32_t *counters, int64_t n_counters, const int32_t *order64, const int32_t *order128);
+               int32_t *counters, int64_t n_counters, const int32_t *order64, const int32_t *order128,
+               const OutPlace *place);
   // out[nbaddrs[k] + p, :] = X[rows[nbaddrs[k] + p], :] W[k] over 128-padded pair lists
   int (*pairs)(hipStream_t s, const void *x, const void *wp, const int32_t *rows,
                const int32_t *nbaddrs, const int32_t *qnbaddrs, int64_t qnnz, int kvol, int cin,
@@ -53,7 +64,7 @@ struct ConvOps {
   // y[o, :] = sum over k of products[k * seg_rows + pos[k * n_out + o], :] where pos >= 0
   int (*segment_sum)(hipStream_t s, const void *products, const int32_t *pos, int64_t n_out, int kvol,
                      int64_t seg_rows, int cout, const void *bias, const void *residual, int relu,
-                     void *y);
+                     void *y, const OutPlace *place);
 };
 
 const ConvOps &conv_ops_f16();

@@ -27,7 +27,8 @@ def conv3d(input: SparseTensor, weight: torch.Tensor,
            dilation: Union[int, Tuple[int, ...]] = 1, config: Dict = None,
            transposed: bool = False, generative: bool = False,
            training: bool = False, residual: Optional[torch.Tensor] = None,
-           activation: Optional[str] = None) -> SparseTensor:
+           activation: Optional[str] = None, out: Optional[torch.Tensor] = None,
+           also: Optional[torch.Tensor] = None) -> SparseTensor:
     """Sparse convolution on a SparseTensor (the reference's
     nn/functional/conv/conv.py:15-210): config resolution (per call -> global ->
     default), 1x1x1 fast path, kernel-map cache lookup / build, dataflow dispatch,
@@ -39,7 +40,13 @@ def conv3d(input: SparseTensor, weight: torch.Tensor,
 
     Two optional extras fuse what usually follows a convolution into its epilogue:
     ``residual`` (a [N_out, Cout] tensor added to the result) and ``activation``
-    (None or "relu"): output = act(conv(input) + bias + residual)."""
+    (None or "relu"): output = act(conv(input) + bias + residual).
+
+    ``out`` / ``also`` place the result: it is written into ``out`` (a [N_out, Cout] view with
+    unit column stride, e.g. a column slice of a wider buffer) instead of a new tensor, and a
+    second time into ``also``.  A layer whose result a later ``cat`` would copy writes it where
+    the concatenation wants it; the implicit-GEMM inference launch stores there directly, any
+    other path copies."""
     if activation not in (None, "relu"):
         raise ValueError(f"unsupported fused activation: {activation}")
     relu = activation == "relu"
@@ -108,7 +115,8 @@ def conv3d(input: SparseTensor, weight: torch.Tensor,
             from torchsparse_amd import backend
             out_feats = backend._implicit_gemm(feats, backend.pack_weights(weight), *weight.shape,
                                                kmap["out_in_map"], kmap["sizes"][1], bias, residual, relu,
-                                               config.get("pair_segments"))
+                                               config.get("pair_segments"), out, also)
+            out = also = None  # (placed by the launch)
         else:
             out_feats = conv_fn.apply(feats, weight, kmap, config, False, bias, residual, relu)
         output = SparseTensor._make(out_feats, kmap["coords"], out_stride, kmap["spatial_range"], caches)
@@ -138,12 +146,18 @@ def conv3d(input: SparseTensor, weight: torch.Tensor,
             from torchsparse_amd import backend
             out_feats = backend._implicit_gemm(feats, backend.pack_weights(weight), *weight.shape,
                                                kmap["out_in_map_t"], kmap["sizes"][0], bias, residual, relu,
-                                               config.get("pair_segments"))
+                                               config.get("pair_segments"), out, also)
+            out = also = None  # (placed by the launch)
         else:
             out_feats = conv_fn.apply(feats, weight, kmap, config, True, bias, residual, relu)
         fine_coords, fine_range = caches.cmaps[fine_stride]
         output = SparseTensor._make(out_feats, fine_coords, fine_stride, fine_range, caches)
 
+    if also is not None:  # (a path that does not place its result itself)
+        also.copy_(output.feats)
+    if out is not None:
+        out.copy_(output.feats)
+        output = SparseTensor._make(out, output.coords, output.stride, output.spatial_range, caches)
     if output.stride not in caches.cmaps:
         caches.cmaps[output.stride] = (output.coords, output.spatial_range)
     return output
@@ -169,7 +183,8 @@ def _direct_ok(feats, kernel, bias, residual, config) -> bool:
 def conv3d_cached(input: SparseTensor, kernel: torch.Tensor, bias: Optional[torch.Tensor],
                   kernel_size: Tuple[int, int, int], stride: Tuple[int, int, int],
                   dilation: Tuple[int, int, int], transposed: bool, config: Optional[Dict],
-                  residual: Optional[torch.Tensor], activation: Optional[str]) -> Optional[SparseTensor]:
+                  residual: Optional[torch.Tensor], activation: Optional[str],
+                  out: Optional[torch.Tensor] = None, also: Optional[torch.Tensor] = None) -> Optional[SparseTensor]:
     """The hot case of ``conv3d`` with most of its bookkeeping left out: an inference call
     (no gradient flows) of a real-kernel, non-generative layer in the unsorted implicit-GEMM
     dataflow whose kernel map is already in the tensor's cache and whose operands need no
@@ -186,7 +201,7 @@ def conv3d_cached(input: SparseTensor, kernel: torch.Tensor, bias: Optional[torc
     ist = input.stride
     if kernel.dim() != 3:  # a 1x1x1 stride-1 layer: no map, the outputs are the inputs
         if kernel_size != (1, 1, 1) or stride != (1, 1, 1) or dilation != (1, 1, 1) or feats.shape[0] == 0 \
-                or feats.shape[1] != kernel.shape[0]:
+                or feats.shape[1] != kernel.shape[0] or out is not None or also is not None:
             return None
         from torchsparse_amd import backend
         if ist not in caches.cmaps:
@@ -219,7 +234,8 @@ def conv3d_cached(input: SparseTensor, kernel: torch.Tensor, bias: Optional[torc
     if feats.shape[1] != cin:
         return None  # (conv3d raises the reference's error)
     out_feats = backend._implicit_gemm(feats, backend.pack_weights(kernel), kvol, cin, cout, omap, n_out,
-                                       bias, residual, activation == "relu", config.get("pair_segments"))
+                                       bias, residual, activation == "relu", config.get("pair_segments"),
+                                       out, also)
     output = SparseTensor._make(out_feats, out_coords, out_stride, out_range, caches)
     if out_stride not in caches.cmaps:
         caches.cmaps[out_stride] = (out_coords, out_range)

@@ -71,17 +71,20 @@ class Conv3d(nn.Module):
             parts.append("generative=True")
         return ", ".join(parts)
 
-    def forward(self, input: SparseTensor, residual: torch.Tensor = None) -> SparseTensor:
+    def forward(self, input: SparseTensor, residual: torch.Tensor = None, out: torch.Tensor = None,
+                also: torch.Tensor = None) -> SparseTensor:
+        """``residual``: added before the activation; ``out`` / ``also``: where the result is
+        written instead of a new tensor / a second time (functional.conv3d)."""
         if not self.training and not self.generative and self.activation in (None, "relu"):
             # a layer whose map is already cached, in inference: the short way (None: not that case)
             dilation = getattr(self, "_dilation3", None) or make_ntuple(self.dilation, ndim=3)
             params = self._parameters  # (plain dictionary look-ups: Module.__getattr__ costs 0.4 us each)
-            out = F.conv3d_cached(input, params["kernel"], params["bias"], self.kernel_size, self.stride,
-                                  dilation, self.transposed, self._config, residual, self.activation)
-            if out is not None:
-                return out
+            done = F.conv3d_cached(input, params["kernel"], params["bias"], self.kernel_size, self.stride,
+                                   dilation, self.transposed, self._config, residual, self.activation, out, also)
+            if done is not None:
+                return done
         return F.conv3d(input, weight=self.kernel, kernel_size=self.kernel_size, bias=self.bias,
                         stride=self.stride, padding=self.padding, dilation=self.dilation,
                         transposed=self.transposed, generative=self.generative,
                         config=self._config, training=self.training, residual=residual,
-                        activation=self.activation)
+                        activation=self.activation, out=out, also=also)

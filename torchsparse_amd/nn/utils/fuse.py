@@ -110,4 +110,5 @@ def fuse_inference(model: nn.Module) -> nn.Module:
     for m in model.modules():
         if isinstance(m, nn.Sequential):
             _skip_identities(m)
+        m.__dict__.pop("_placed_plan", None)  # (what a network derived from its unfused layers)
     return model
