@@ -559,7 +559,15 @@ def test_results_placed_into_column_slices_equal_the_dense_ones(n, cin, cout, dt
     assert torch.equal(got.feats, want) and torch.equal(second[:, :cout], want)
     assert (wide[:, :8] == 7).all() and (wide[:, 8 + cout:] == 7).all() and (second[:, cout:] == 5).all()
     assert torch.equal(got.coords, x.coords if how != "transposed" else coords)
-    # other dataflows copy; misplaced views are refused
+    # the same through column slices named without a view
+    with torch.no_grad():
+        wide2 = torch.full((n_out, 8 + cout + 16), 7.0, device="cuda", dtype=dtype)
+        second2 = torch.full((n_out, cout + 8), 5.0, device="cuda", dtype=dtype)
+        got2 = layer(x, residual=res, out=backend.ColumnSlice(wide2, 8, cout), also=backend.ColumnSlice(second2, 0, cout))
+    assert got2.feats is wide2 and torch.equal(wide2, wide) and torch.equal(second2, second)
+    with pytest.raises(ValueError):
+        backend.ColumnSlice(wide2, 3, cout)
+    # misplaced views are refused
     with torch.no_grad():
         with pytest.raises(ValueError, match="placed"):
             layer(x, out=wide[:, 3:3 + cout])

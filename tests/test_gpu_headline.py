@@ -316,7 +316,11 @@ def test_minkunet_forward_on_the_scan(mods, scan):
             want = want + _f32(r["res"])
         if mod.activation == "relu":
             want = np.maximum(want, 0)
-        err = rel_rms(_f32(r["y"]), want)
+        got = _f32(r["y"])
+        if mod.transposed:  # placed into the left-hand columns of the buffer its level concatenates in
+            assert got.shape[1] > want.shape[1]
+            got = got[:, :want.shape[1]]
+        err = rel_rms(got, want)
         worst = max(worst, err)
         assert err < FP16_TOL, (i, mod, r["level"], err)
 

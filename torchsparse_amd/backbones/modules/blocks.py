@@ -84,5 +84,8 @@ class SparseResBlock(nn.Module):
             return call_module(layers[-1], y, residual=residual, also=also)
         out = self.relu(self.main(x) + self.shortcut(x))
         if also is not None:
+            if not hasattr(also, "copy_"):  # a backend.ColumnSlice
+                first = (also.ptr - also.buffer.data_ptr()) // also.buffer.element_size()
+                also = also.buffer[:, first:first + also.cols]
             also.copy_(out.feats)
         return out

@@ -94,6 +94,7 @@ class SparseResUNet(nn.Module):
         return tuple(plan)
 
     def _forward_placed(self, x: SparseTensor, plan) -> List[SparseTensor]:
+        from ..backend import ColumnSlice
         from ..nn.utils.fuse import call_module
         skips, buffers = [], []
         y = x
@@ -101,7 +102,7 @@ class SparseResUNet(nn.Module):
             for m in before:
                 y = call_module(m, y)
             buf = y.feats.new_empty(y.feats.shape[0], c_up + c_skip)
-            y = call_module(last, y, also=buf[:, c_up:])
+            y = call_module(last, y, also=ColumnSlice(buf, c_up, c_skip))
             skips.append(y)
             buffers.append(buf)
         y = call_module(self.encoders[3], y)
@@ -109,10 +110,8 @@ class SparseResUNet(nn.Module):
         for i, dec in enumerate(self.decoders):
             _, _, up, c_up, _ = plan[3 - i]
             buf = buffers[3 - i]
-            u = call_module(up, y, out=buf[:, :c_up])
-            if u.feats.shape[0] != buf.shape[0]:  # (cannot happen: the level's rows are its skip's)
-                raise RuntimeError("the transposed convolution did not return to the rows of its skip")
-            y = call_module(dec["fuse"], SparseTensor._make(buf, u.coords, u.stride, u.spatial_range, u._caches))
+            # (the result tensor of a call placed through a ColumnSlice is the whole buffer)
+            y = call_module(dec["fuse"], call_module(up, y, out=ColumnSlice(buf, 0, c_up)))
             outputs.append(y)
         return outputs
 

@@ -1475,14 +1475,35 @@ _PACK20 = struct.Struct("20q").pack
 _PACK21 = struct.Struct("21q").pack
 
 
+class ColumnSlice:
+    """Columns [first, first + cols) of a contiguous 2-D ``buffer``, for ``out=`` / ``also=`` of a
+    convolution: the same as the view ``buffer[:, first:first + cols]`` without making one (a
+    view costs 2 us, a forward of a U-Net places eight results).  A call placed through
+    ``out=ColumnSlice(...)`` returns the whole buffer as its result tensor."""
+    __slots__ = ("buffer", "ptr", "pitch", "rows", "cols")
+
+    def __init__(self, buffer: torch.Tensor, first: int, cols: int):
+        if buffer.dim() != 2 or not buffer.is_contiguous() or first < 0 or cols < 1 or first + cols > buffer.shape[1]:
+            raise ValueError("a column slice needs a contiguous 2-D buffer that holds its columns")
+        self.buffer, self.rows, self.cols, self.pitch = buffer, buffer.shape[0], cols, buffer.shape[1]
+        self.ptr = buffer.data_ptr() + first * buffer.element_size()
+        if self.pitch % 8 or self.ptr % 16:
+            raise ValueError("a placed result needs rows a multiple of 8 elements apart and 16-byte aligned")
+
+
 def _placed(x, num_out_feats: int, cout: int, out, also):
-    """(y, row pitch of y or 0, address of the second destination or 0, its row pitch) of a
+    """(result tensor, address of y, row pitch of y or 0, address of the second destination or 0,
+    its row pitch) of a
     convolution whose result goes into ``out`` (None: a new dense tensor) and, a second time, into
     ``also``: [num_out_feats, cout] views of the features' dtype with unit column stride, rows a
     multiple of 8 elements apart and 16-byte aligned (column slices of wider buffers)."""
     ldy = a2 = ld2 = 0
     for t in (out, also):
         if t is None:
+            continue
+        if t.__class__ is ColumnSlice:
+            if t.rows != num_out_feats or t.cols != cout or t.buffer.dtype != x.dtype or t.buffer.device != x.device:
+                raise ValueError(f"a placed result needs {x.dtype} columns for [{num_out_feats}, {cout}] values")
             continue
         if (t.dtype != x.dtype or t.dim() != 2 or t.shape[0] != num_out_feats or t.shape[1] != cout
                 or t.stride(1) != 1 or t.stride(0) % 8 or t.stride(0) < cout or t.data_ptr() % 16
@@ -1491,11 +1512,14 @@ def _placed(x, num_out_feats: int, cout: int, out, also):
                              "stride, rows a multiple of 8 elements apart and 16-byte aligned")
     if out is None:
         y = x.new_empty(num_out_feats, cout)
+        at = y.data_ptr()
+    elif out.__class__ is ColumnSlice:
+        y, at, ldy = out.buffer, out.ptr, out.pitch
     else:
-        y, ldy = out, out.stride(0)
+        y, at, ldy = out, out.data_ptr(), out.stride(0)
     if also is not None:
-        a2, ld2 = also.data_ptr(), also.stride(0)
-    return y, ldy, a2, ld2
+        a2, ld2 = (also.ptr, also.pitch) if also.__class__ is ColumnSlice else (also.data_ptr(), also.stride(0))
+    return y, at, ldy, a2, ld2
 
 # Buffers the library owns (the scratch of a stream, its tile counters, identity maps, pair
 # segments, grouped maps, packed weights) live in tables that drop or replace their entries.  A
@@ -1805,15 +1829,15 @@ def conv_implicit_gemm_grouped(x, wp, kvol, cin, cout, out_in_map, num_out_feats
     """The implicit-GEMM sums over the grouped copy of the map (same results bit for bit)."""
     g = grouped_map(out_in_map, num_out_feats)
     if out is None and also is None:
-        y, ldy, a2, ld2 = x.new_empty(num_out_feats, cout), 0, 0, 0
+        y = x.new_empty(num_out_feats, cout)
+        at, ldy, a2, ld2 = y.data_ptr(), 0, 0, 0
     else:
-        y, ldy, a2, ld2 = _placed(x, num_out_feats, cout, out, also)
+        y, at, ldy, a2, ld2 = _placed(x, num_out_feats, cout, out, also)
     pb, pr = _epilogue_args(bias, residual, x, num_out_feats, cout)
     ptrs = g.ptrs
     _check(_C.tsmi_conv_implicit_gemm_grouped_packed(_PACK20(
         _stream(), x.data_ptr(), wp.data_ptr(), ptrs[0], ptrs[1], ptrs[3], ptrs[4], g.padded,
-        num_out_feats, kvol, cin, cout, _dtype_code(x), pb or 0, pr or 0, int(relu), y.data_ptr(),
-        ldy, a2, ld2)))
+        num_out_feats, kvol, cin, cout, _dtype_code(x), pb or 0, pr or 0, int(relu), at, ldy, a2, ld2)))
     return y
 
 
@@ -1891,9 +1915,10 @@ def conv_implicit_gemm_segments(x, wp, kvol, cin, cout, out_in_map, num_out_feat
     seg = pair_segments(out_in_map, num_out_feats)
     seg_rows = seg.seg_rows
     if out is None and also is None:
-        y, ldy, a2, ld2 = x.new_empty(num_out_feats, cout), 0, 0, 0  # (the cheapest form of the call: 1.2 us against 1.6)
+        y = x.new_empty(num_out_feats, cout)  # (the cheapest form of the call: 1.2 us against 1.6)
+        at, ldy, a2, ld2 = y.data_ptr(), 0, 0, 0
     else:
-        y, ldy, a2, ld2 = _placed(x, num_out_feats, cout, out, also)
+        y, at, ldy, a2, ld2 = _placed(x, num_out_feats, cout, out, also)
     stream = _stream()
     pb, pr = _epilogue_args(bias, residual, x, num_out_feats, cout)
     with _scratch_lock:
@@ -1901,7 +1926,7 @@ def conv_implicit_gemm_segments(x, wp, kvol, cin, cout, out_in_map, num_out_feat
         _check(_C.tsmi_conv_implicit_gemm_segments_packed(_PACK20(
             stream, x.data_ptr(), wp.data_ptr(), seg.in_rows_ptr, seg.counts_ptr, seg.pos_ptr, seg_rows,
             num_out_feats, kvol, cin, cout, _dtype_code(x), pb or 0, pr or 0, int(relu), products,
-            y.data_ptr(), ldy, a2, ld2)))
+            at, ldy, a2, ld2)))
     return y
 
 
@@ -1917,9 +1942,10 @@ def _implicit_gemm(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias=None,
         return conv_implicit_gemm_grouped(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias,
                                           residual, relu, out, also)
     if out is None and also is None:
-        y, ldy, a2, ld2 = x.new_empty(num_out_feats, cout), 0, 0, 0  # (the cheapest form of the call: 1.2 us against 1.6)
+        y = x.new_empty(num_out_feats, cout)  # (the cheapest form of the call: 1.2 us against 1.6)
+        at, ldy, a2, ld2 = y.data_ptr(), 0, 0, 0
     else:
-        y, ldy, a2, ld2 = _placed(x, num_out_feats, cout, out, also)
+        y, at, ldy, a2, ld2 = _placed(x, num_out_feats, cout, out, also)
     code = _dtype_code(x)
     stream = _stream()
     pb, pr = _epilogue_args(bias, residual, x, num_out_feats, cout)
@@ -1931,12 +1957,11 @@ def _implicit_gemm(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias=None,
                 stream, x.data_ptr(), wp.data_ptr(), out_in_map.data_ptr(), out_in_map.shape[0],
                 num_out_feats, kvol, cin, cout, code, pb or 0, pr or 0, int(relu),
                 _scratch(x.device, stream, 4 * ws_elems), ws_elems,
-                _tile_counters(x.device, stream).data_ptr(), _N_TILE_COUNTERS, y.data_ptr(), ldy, a2, ld2)))
+                _tile_counters(x.device, stream).data_ptr(), _N_TILE_COUNTERS, at, ldy, a2, ld2)))
     else:
         _check(_C.tsmi_conv_implicit_gemm_packed(_PACK21(
             stream, x.data_ptr(), wp.data_ptr(), out_in_map.data_ptr(), out_in_map.shape[0], num_out_feats,
-            kvol, cin, cout, code, pb or 0, pr or 0, int(relu), 0, 0, 0, _N_TILE_COUNTERS, y.data_ptr(),
-            ldy, a2, ld2)))
+            kvol, cin, cout, code, pb or 0, pr or 0, int(relu), 0, 0, 0, _N_TILE_COUNTERS, at, ldy, a2, ld2)))
     return y
 
 

@@ -153,11 +153,20 @@ def conv3d(input: SparseTensor, weight: torch.Tensor,
         fine_coords, fine_range = caches.cmaps[fine_stride]
         output = SparseTensor._make(out_feats, fine_coords, fine_stride, fine_range, caches)
 
-    if also is not None:  # (a path that does not place its result itself)
-        also.copy_(output.feats)
-    if out is not None:
-        out.copy_(output.feats)
-        output = SparseTensor._make(out, output.coords, output.stride, output.spatial_range, caches)
+    if also is not None or out is not None:  # (a path that does not place its result itself)
+        from torchsparse_amd.backend import ColumnSlice
+
+        def view(t):
+            if t.__class__ is not ColumnSlice:
+                return t
+            first = (t.ptr - t.buffer.data_ptr()) // t.buffer.element_size()
+            return t.buffer[:, first:first + t.cols]
+        if also is not None:
+            view(also).copy_(output.feats)
+        if out is not None:
+            view(out).copy_(output.feats)
+            output = SparseTensor._make(out.buffer if out.__class__ is ColumnSlice else out, output.coords,
+                                        output.stride, output.spatial_range, caches)
     if output.stride not in caches.cmaps:
         caches.cmaps[output.stride] = (output.coords, output.spatial_range)
     return output
