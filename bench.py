@@ -831,15 +831,20 @@ def summarize(meas):
             if nm in got:
                 o.append(f"| {nm} | {got[nm]:.4g} |")
         if "SQ_VALU_MFMA_BUSY_CYCLES" in got and "GRBM_GUI_ACTIVE" in got:
-            simd_cycles = got["GRBM_GUI_ACTIVE"] * 1024  # 256 CUs x 4 SIMDs
+            # GRBM_GUI_ACTIVE comes back summed over the 8 XCDs; one XCD's count is the kernel's cycles
+            cycles = got["GRBM_GUI_ACTIVE"] / 8
+            simd_cycles = cycles * 1024  # 256 CUs x 4 SIMDs
             o.append(f"\nMatrix pipe busy {100 * got['SQ_VALU_MFMA_BUSY_CYCLES'] / simd_cycles:.1f} % of the SIMD cycles "
-                     f"(SQ_VALU_MFMA_BUSY_CYCLES ÷ (GRBM_GUI_ACTIVE × 1024 SIMDs)); kernel duration under this pass "
-                     f"{dur_ns / 1e3:.1f} µs.")
+                     f"(SQ_VALU_MFMA_BUSY_CYCLES ÷ (GRBM_GUI_ACTIVE ÷ 8 XCDs × 1024 SIMDs)); kernel duration under "
+                     f"this pass {dur_ns / 1e3:.1f} µs = {cycles / (dur_ns * 1e-9) / 1e9:.2f} GHz × {cycles:.4g} cycles.")
         if "SQ_INSTS_VALU_MFMA_MOPS_F16" in got:
             # one count = 512 multiply-adds... report raw and the flops it stands for (MOPS counts units of 512 flops)
             o.append(f"fp16 matrix operations counted: {got['SQ_INSTS_VALU_MFMA_MOPS_F16']:.4g} × 512 flop = "
                      f"{got['SQ_INSTS_VALU_MFMA_MOPS_F16'] * 512 / 1e9:.2f} GFLOP executed, against {roof['algorithmic_flops'] / 1e9:.2f} "
-                     f"GFLOP of pairs and {roof['dense_map_flops'] / 1e9:.2f} GFLOP of the whole map.")
+                     f"GFLOP of pairs and {roof['dense_map_flops'] / 1e9:.2f} GFLOP of the whole map"
+                     + (f" ({got['SQ_INSTS_VALU_MFMA_MOPS_F16'] * 512 / (dur_ns * 1e-9) / 1e12:.0f} TFLOP/s executed, "
+                        f"{100 * got['SQ_INSTS_VALU_MFMA_MOPS_F16'] * 512 / (dur_ns * 1e-9) / 2.5e15:.1f} % of the dense "
+                        "fp16 peak)." if dur_ns else "."))
         if "SQ_WAIT_INST_ANY" in got and "SQ_WAVE_CYCLES" in got:
             o.append(f"Wavefronts wait for an instruction {100 * got['SQ_WAIT_INST_ANY'] / got['SQ_WAVE_CYCLES']:.0f} % of "
                      f"their cycles; LDS instructions are active {100 * got.get('SQ_ACTIVE_INST_LDS', 0) / got['SQ_WAVE_CYCLES']:.0f} %.")
