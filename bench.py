@@ -831,12 +831,12 @@ def summarize(meas):
             if nm in got:
                 o.append(f"| {nm} | {got[nm]:.4g} |")
         if "SQ_VALU_MFMA_BUSY_CYCLES" in got and "GRBM_GUI_ACTIVE" in got:
-            # GRBM_GUI_ACTIVE comes back summed over the 8 XCDs; one XCD's count is the kernel's cycles
-            cycles = got["GRBM_GUI_ACTIVE"] / 8
-            simd_cycles = cycles * 1024  # 256 CUs x 4 SIMDs
+            # SIMD cycles of the launch: its duration at the 2.4 GHz peak engine clock x 256 CUs x 4 SIMDs
+            # (GRBM_GUI_ACTIVE is summed over the XCDs' instances and is listed as read)
+            simd_cycles = dur_ns * 1e-9 * 2.4e9 * 1024
             o.append(f"\nMatrix pipe busy {100 * got['SQ_VALU_MFMA_BUSY_CYCLES'] / simd_cycles:.1f} % of the SIMD cycles "
-                     f"(SQ_VALU_MFMA_BUSY_CYCLES ÷ (GRBM_GUI_ACTIVE ÷ 8 XCDs × 1024 SIMDs)); kernel duration under "
-                     f"this pass {dur_ns / 1e3:.1f} µs = {cycles / (dur_ns * 1e-9) / 1e9:.2f} GHz × {cycles:.4g} cycles.")
+                     f"(SQ_VALU_MFMA_BUSY_CYCLES ÷ (duration × 2.4 GHz × 1024 SIMDs)); kernel duration under this "
+                     f"pass {dur_ns / 1e3:.1f} µs.")
         if "SQ_INSTS_VALU_MFMA_MOPS_F16" in got:
             # one count = 512 multiply-adds... report raw and the flops it stands for (MOPS counts units of 512 flops)
             o.append(f"fp16 matrix operations counted: {got['SQ_INSTS_VALU_MFMA_MOPS_F16']:.4g} × 512 flop = "
