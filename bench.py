@@ -725,9 +725,10 @@ def summarize(meas):
     # ---- kernel trace: stats, and the timed loop between the two marker fills ----
     rows = list(csv.DictReader(open(os.path.join(meas, "kt", "kt_kernel_stats.csv"))))
     out = ["# rocprofv3 kernel trace of bench.py (MinkUNet fp16 forward, %d-voxel synthetic scan)\n" % bench["config"]["voxels"],
-           "Command (from the repository root on one MI355X; `cd /tmp && export TMPDIR=/tmp` first), then "
-           "`python bench.py --summarize gpurun_out/meas` for this file:\n",
-           "```\nrocprofv3 --kernel-trace --stats --output-format csv -d gpurun_out/meas/kt -o kt -- python bench.py "
+           "Command (from the repository root on one MI355X; `cd /tmp && export TMPDIR=/tmp` first; OUT: a scratch "
+           "directory that also holds the output of a plain `python bench.py > OUT/bench.json`), then "
+           "`python bench.py --summarize OUT` for this file:\n",
+           "```\nrocprofv3 --kernel-trace --stats --output-format csv -d OUT/kt -o kt -- python bench.py "
            f"--steps {steps} --warmup {warmup} --no-cpu --no-layers --no-backward --no-tune --no-pointops --no-configs\n```\n",
            "The process also runs the unfused network, the same-tensor and resident-tensor loops, warm-map forwards and the "
            "per-group roofline timing, so `calls` mixes those phases; the second table isolates the timed loop "
@@ -799,11 +800,11 @@ def summarize(meas):
     kname = _short_kernel(ft[0][0])
     o = ["# Hardware counters of the roofline kernel\n", f"Kernel: `{kname}` — {desc}\n",
          "Commands (one pass per run; `bench.py --pmc-target KERNEL` launches a 256 MiB device-to-device copy five times "
-         "and then the kernel five times), then `python bench.py --summarize gpurun_out/meas`:\n",
-         f"```\nrocprofv3 --pmc FETCH_SIZE --output-format csv -d gpurun_out/meas/pmc_fetch -o f -- python bench.py --pmc-target \"{desc}\"\n"
-         f"rocprofv3 --pmc WRITE_SIZE --output-format csv -d gpurun_out/meas/pmc_write -o w -- python bench.py --pmc-target \"{desc}\"\n"
+         "and then the kernel five times), then `python bench.py --summarize OUT`:\n",
+         f"```\nrocprofv3 --pmc FETCH_SIZE --output-format csv -d OUT/pmc_fetch -o f -- python bench.py --pmc-target \"{desc}\"\n"
+         f"rocprofv3 --pmc WRITE_SIZE --output-format csv -d OUT/pmc_write -o w -- python bench.py --pmc-target \"{desc}\"\n"
          "rocprofv3 --pmc SQ_VALU_MFMA_BUSY_CYCLES SQ_INSTS_VALU_MFMA_MOPS_F16 SQ_WAIT_INST_ANY SQ_ACTIVE_INST_LDS SQ_WAVE_CYCLES "
-         f"SQ_BUSY_CYCLES GRBM_GUI_ACTIVE --output-format csv -d gpurun_out/meas/pmc_sq -o q -- python bench.py --pmc-target \"{desc}\"\n```\n",
+         f"SQ_BUSY_CYCLES GRBM_GUI_ACTIVE --output-format csv -d OUT/pmc_sq -o q -- python bench.py --pmc-target \"{desc}\"\n```\n",
          "## HBM traffic\n",
          "| counter (KiB per dispatch) | 256 MiB copy reads | scale to true KiB | kernel reads | kernel, scaled |\n|---|---:|---:|---:|---:|",
          f"| FETCH_SIZE | {avg(fc):.0f} | {f_fac:.3f} | {avg(ft):.0f} | {fetch:.0f} |",
