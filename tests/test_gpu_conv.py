@@ -573,3 +573,56 @@ def test_results_placed_into_column_slices_equal_the_dense_ones(n, cin, cout, dt
             layer(x, out=wide[:, 3:3 + cout])
         with pytest.raises(ValueError, match="placed"):
             layer(x, also=second[:-1, :cout])
+
+
+def test_placed_results_through_paths_that_copy():
+    """out= / also= where the launch does not place its rows itself: another dataflow, a call
+    that records gradients, a 1x1x1 layer, the unfused residual block.  The values are copied into
+    the slices and the returned tensor is the slice (or the slice's buffer)."""
+    import torchsparse_amd as ts
+    from torchsparse_amd import backend
+    from torchsparse_amd import nn as spnn
+    from torchsparse_amd.backbones.modules.blocks import SparseResBlock
+    from torchsparse_amd.nn import functional as F
+    rng = np.random.default_rng(5)
+    coords_np = lidar_like_coords(rng, 3000)
+    coords_np = coords_np[np.lexsort((coords_np[:, 3], coords_np[:, 2], coords_np[:, 1], coords_np[:, 0]))]
+    coords = torch.from_numpy(coords_np).cuda()
+    n = coords.shape[0]
+    torch.manual_seed(5)
+    feats = torch.randn(n, 16, device="cuda", dtype=torch.float16)
+
+    def slices():
+        wide = torch.full((n, 48), 7.0, device="cuda", dtype=torch.float16)
+        second = torch.full((n, 40), 5.0, device="cuda", dtype=torch.float16)
+        return wide, second
+
+    cfg = F.conv_config.get_default_conv_config()
+    cfg.dataflow = F.Dataflow.GatherScatter
+    layer = spnn.Conv3d(16, 32, 3, bias=True, config=cfg).cuda().half().eval()
+    with torch.no_grad():
+        want = layer(ts.SparseTensor(feats, coords)).feats
+        wide, second = slices()
+        got = layer(ts.SparseTensor(feats, coords), out=wide[:, 8:40], also=backend.ColumnSlice(second, 8, 32))
+    assert torch.equal(got.feats, want) and torch.equal(second[:, 8:], want) and (wide[:, :8] == 7).all()
+    # gradients recorded: the autograd function computes, the slices receive copies
+    layer2 = spnn.Conv3d(16, 32, 3).cuda().half()
+    x = ts.SparseTensor(feats.clone().requires_grad_(True), coords)
+    want = layer2(x).feats.detach()
+    wide, second = slices()
+    got = layer2(ts.SparseTensor(feats.clone().requires_grad_(True), coords), out=backend.ColumnSlice(wide, 16, 32))
+    assert got.feats is wide and torch.equal(wide[:, 16:], want)
+    # a 1x1x1 layer
+    point = spnn.Conv3d(16, 32, 1).cuda().half().eval()
+    with torch.no_grad():
+        want = point(ts.SparseTensor(feats, coords)).feats
+        wide, second = slices()
+        got = point(ts.SparseTensor(feats, coords), also=second[:, :32])
+    assert torch.equal(got.feats, want) and torch.equal(second[:, :32], want) and (second[:, 32:] == 5).all()
+    # the residual block before fuse_inference
+    block = SparseResBlock(16, 32, 3).cuda().half().eval()
+    with torch.no_grad():
+        want = block(ts.SparseTensor(feats, coords)).feats
+        wide, second = slices()
+        got = block(ts.SparseTensor(feats, coords), also=backend.ColumnSlice(wide, 8, 32))
+    assert torch.equal(got.feats, want) and torch.equal(wide[:, 8:40], want) and (wide[:, 40:] == 7).all()
