@@ -135,3 +135,68 @@ def test_replays_survive_the_eviction_of_every_library_table():
     runner.pinned[0].resize_(runner.pinned[0].numel() * 4 + (1 << 24))
     with pytest.raises(RuntimeError, match="moved"):
         runner(feats[0])
+
+
+def test_convolution_calls_through_the_launch_thread():
+    """Inside backend.launch_region() the convolution calls are carried out by the library's launch
+    thread: same results bit for bit, in order with the calls this thread makes itself once
+    flush_launches() has returned, nothing handed over while hooks are registered or outside a
+    region, and a call the library refuses raises at the flush."""
+    import torchsparse_amd as ts
+    from torchsparse_amd import backend
+    from torchsparse_amd import nn as spnn
+    from torchsparse_amd.backbones import SparseResUNet42
+    from torchsparse_amd.nn.utils import fuse_inference
+    from torchsparse_amd.utils.synthetic import lidar_scan_voxels
+    assert backend.launch_thread
+    torch.manual_seed(2)
+    coords = dev(lidar_scan_voxels(seed=1)[::2].copy())
+    n = coords.shape[0]
+    model = SparseResUNet42(in_channels=4).cuda().eval()
+    _stat_norms(model)
+    model = fuse_inference(copy.deepcopy(model)).half()
+    feats = torch.randn(n, 4, device="cuda", dtype=torch.float16)
+    done = backend._C.tsmi_launch_thread_completed().contents
+    with torch.no_grad():
+        before = done.value
+        threaded = [o.feats.clone() for o in model(ts.SparseTensor(feats, coords.clone()))]
+        handed = done.value - before
+        assert handed >= 49 and not backend._region_calls and backend._region_depth == 0
+        backend.launch_thread = False
+        try:
+            before = done.value
+            direct = [o.feats.clone() for o in model(ts.SparseTensor(feats, coords.clone()))]
+            assert done.value == before
+        finally:
+            backend.launch_thread = True
+        for a, b in zip(threaded, direct):
+            assert torch.equal(a, b)
+        # layers called one by one inside a region: torch reads a result only after the flush
+        layer = spnn.Conv3d(4, 32, 3).cuda().half().eval()
+        x = ts.SparseTensor(feats, coords)
+        want = layer(x).feats.clone()
+        with backend.launch_region():
+            for _ in range(20):
+                y = layer(x)
+            assert backend._region_calls  # (handed over, possibly not launched yet)
+            backend.flush_launches()
+            assert not backend._region_calls
+            assert torch.equal(y.feats, want)
+            # a forward hook looks at the result as soon as the layer returns
+            seen = []
+            handle = layer.register_forward_hook(lambda m, a, out: seen.append(out.feats.clone()))
+            from torchsparse_amd.nn.utils.fuse import call_module
+            before = done.value
+            call_module(layer, x)
+            handle.remove()
+            assert done.value == before and torch.equal(seen[0], want)
+        # a call the library refuses (a null map pointer) surfaces when the region flushes
+        with pytest.raises(ValueError, match="null pointer"):
+            with backend.launch_region():
+                bad = backend._PACK21(backend._stream(), feats.data_ptr(), feats.data_ptr(), 0, n, n, 27, 4, 32, 1,
+                                      0, 0, 0, 0, 0, 0, 0, feats.data_ptr(), 0, 0, 0)
+                assert backend._hand_over(0, bad, 21, (feats,))
+        assert backend._region_depth == 0
+        assert backend._C.tsmi_launch_thread_submit(0, bad, 21) == -1  # no region open: nothing is taken
+        y = layer(x)
+        assert torch.equal(y.feats, want)

@@ -4,6 +4,7 @@ examples/openpcdet/pcdet_plugin/models/backbones_3d/backbone3d.py:39-80 and
 backbone_voxel_next.py:57-138).  Coordinates are (b, z, y, x)."""
 from typing import Dict
 
+import torch
 from torch import nn
 
 from .. import nn as spnn
@@ -51,6 +52,14 @@ class VoxelResBackBone8x(nn.Module):
         self.conv_out = _block(128, 128, (3, 1, 1), (2, 1, 1), 0)
 
     def forward(self, x: SparseTensor) -> Dict[str, SparseTensor]:
+        if not self.training and x.feats.is_cuda and not torch.is_grad_enabled():
+            # inference: the convolution calls go through the library's launch thread
+            from .. import backend
+            with backend.launch_region():
+                return self._forward(x)
+        return self._forward(x)
+
+    def _forward(self, x: SparseTensor) -> Dict[str, SparseTensor]:
         x = self.conv_input(x)
         c1 = self.conv1(x)
         c2 = self.conv2(c1)

@@ -3,6 +3,7 @@ backbones/unet.py).  Module names (stem, encoders.N, decoders.N.upsample / .fuse
 match the reference so its checkpoints load."""
 from typing import List
 
+import torch
 from torch import nn
 
 from .. import nn as spnn
@@ -43,6 +44,14 @@ class SparseResUNet(nn.Module):
             }) for i in range(4))
 
     def forward(self, x: SparseTensor) -> List[SparseTensor]:
+        if not self.training and x.feats.is_cuda and not torch.is_grad_enabled():
+            # inference: the convolution calls go through the library's launch thread
+            from .. import backend
+            with backend.launch_region():
+                return self._forward(x)
+        return self._forward(x)
+
+    def _forward(self, x: SparseTensor) -> List[SparseTensor]:
         plan = self.__dict__.get("_placed_plan")
         if plan is None:
             plan = self.__dict__["_placed_plan"] = self._plan_placement()

@@ -38,6 +38,10 @@ def _load():
             "(python torchsparse_amd/csrc/build.py, or __graft_entry__.build())")
     lib = ctypes.CDLL(_LIB_PATH)
     lib.tsmi_last_error.restype = ctypes.c_char_p
+    lib.tsmi_launch_thread_submit.restype = _i64
+    lib.tsmi_launch_thread_submit.argtypes = [_i32, ctypes.c_char_p, _i32]
+    lib.tsmi_launch_thread_completed.restype = ctypes.POINTER(ctypes.c_int64)
+    lib.tsmi_launch_thread_completed.argtypes = []
     lib.tsmi_sort_temp_bytes.restype = _i64
     lib.tsmi_sort_temp_bytes.argtypes = [_i64]
     lib.tsmi_packed_weight_elems.restype = _i64
@@ -107,6 +111,9 @@ def _load():
         "tsmi_pair_segments": [_vp, _vp, _i64, _i32, _i64, _vp, _vp, _vp, _vp],
         "tsmi_conv_implicit_gemm_segments": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _i32,
                                              _i32, _vp, _vp, _i32, _vp, _vp],
+        "tsmi_launch_thread_open": [],
+        "tsmi_launch_thread_flush": [],
+        "tsmi_launch_thread_close": [],
         "tsmi_conv_implicit_gemm_packed": [ctypes.c_char_p],
         "tsmi_conv_implicit_gemm_segments_packed": [ctypes.c_char_p],
         "tsmi_conv_implicit_gemm_grouped_packed": [ctypes.c_char_p],
@@ -138,7 +145,34 @@ def _load():
     return lib
 
 
-_C = _load()
+class _Library:
+    """The entry points of the loaded library.  Every call that can queue work first waits for
+    the convolution calls that were handed to the library's launch thread (launch_region below):
+    whatever is queued from this thread then comes after them on the stream.  The packed
+    convolution calls, which go to that thread inside a region, the thread's own entry points and
+    the entry points that only answer a question are passed through as they are."""
+
+    _ASIS = ("tsmi_conv_implicit_gemm_packed", "tsmi_conv_implicit_gemm_segments_packed",
+             "tsmi_conv_implicit_gemm_grouped_packed", "tsmi_last_error", "tsmi_version")
+    _ASIS_ENDINGS = ("_elems", "_supported", "_bytes", "_capacity", "_padded")
+
+    def __init__(self, lib):
+        self._lib = lib
+
+    def __getattr__(self, name):  # (once per name: the result becomes an attribute)
+        fn = getattr(self._lib, name)
+        if not (name in self._ASIS or name.startswith("tsmi_launch_thread_") or name.endswith(self._ASIS_ENDINGS)):
+            raw = fn
+
+            def fn(*args, _raw=raw):
+                if _region_calls:
+                    flush_launches()
+                return _raw(*args)
+        setattr(self, name, fn)
+        return fn
+
+
+_C = _Library(_load())
 
 
 def _check(status: int) -> None:
@@ -1471,6 +1505,92 @@ def _epilogue_args(bias, residual, x, n_out, cout):
     return pb, pr
 
 
+# ---- a launch thread for the convolution calls of a forward --------------------------------
+#
+# Inside ``with launch_region():`` the convolution calls of this module hand their packed
+# argument block to the library's launch thread (tsmi_launch_thread_submit) instead of launching
+# themselves: the ~5 us a call spends inside the library (checks, plan, hipLaunchKernel) run beside
+# the ~5 us Python spends on the next call.  The launch thread keeps the order of the calls; what
+# this thread queues itself - other library calls, torch's kernels, event records - is ordered
+# against them only by flush_launches(), which every function here that consumes a convolution's
+# result or reuses its operands calls first (and which the region calls when it ends).  The
+# tensors of a handed-over call are kept referenced until the launch thread has carried it out.
+# The networks in ``backbones`` open a region around their inference forward when
+# ``launch_thread = True``.
+launch_thread = True
+_region_depth = 0
+_region_calls = collections.deque()  # (ticket, tensors the call reads and writes)
+_completed = None                    # the launch thread's counter of calls carried out (a ctypes int64)
+
+
+class launch_region:
+    """Context: convolution calls inside are carried out by the library's launch thread (see
+    above).  A no-op where ``launch_thread`` is False, while a graph is being recorded, and on
+    CPU-only builds."""
+    __slots__ = ("opened",)
+
+    def __enter__(self):
+        global _region_depth, _completed
+        self.opened = False
+        if launch_thread and torch.cuda.is_available() and not torch.cuda.is_current_stream_capturing():
+            if _completed is None:
+                _completed = _C.tsmi_launch_thread_completed().contents
+            _check(_C.tsmi_launch_thread_open())
+            _region_depth += 1
+            self.opened = True
+        return self
+
+    def __exit__(self, *exc):
+        global _region_depth
+        if self.opened:
+            _region_depth -= 1
+            status = _C.tsmi_launch_thread_close()  # (waits for every call handed over)
+            _region_calls.clear()
+            if exc[0] is None:
+                _check(status)
+        return False
+
+
+class direct_launches:
+    """Context inside a launch_region in which convolution calls launch themselves again (after
+    waiting for those handed over): for code that looks at results as soon as a layer returns -
+    forward hooks, debugging."""
+    __slots__ = ("depth",)
+
+    def __enter__(self):
+        global _region_depth
+        flush_launches()
+        self.depth, _region_depth = _region_depth, 0
+        return self
+
+    def __exit__(self, *exc):
+        global _region_depth
+        _region_depth = self.depth
+        return False
+
+
+def flush_launches() -> None:
+    """Returns once every convolution call handed to the launch thread has been launched; raises
+    the error of the first that failed.  Cheap when no region is open or nothing is pending."""
+    if _region_depth and _region_calls:
+        status = _C.tsmi_launch_thread_flush()
+        _region_calls.clear()
+        _check(status)
+
+
+def _hand_over(kind: int, block: bytes, words: int, keep) -> bool:
+    """Hands a packed convolution call to the launch thread; False: no region, make the call."""
+    ticket = _C.tsmi_launch_thread_submit(kind, block, words)
+    if ticket < 0:
+        return False
+    calls = _region_calls
+    done = _completed.value
+    while calls and calls[0][0] <= done:
+        calls.popleft()
+    calls.append((ticket, keep))
+    return True
+
+
 _PACK20 = struct.Struct("20q").pack
 _PACK21 = struct.Struct("21q").pack
 
@@ -1835,9 +1955,10 @@ def conv_implicit_gemm_grouped(x, wp, kvol, cin, cout, out_in_map, num_out_feats
         y, at, ldy, a2, ld2 = _placed(x, num_out_feats, cout, out, also)
     pb, pr = _epilogue_args(bias, residual, x, num_out_feats, cout)
     ptrs = g.ptrs
-    _check(_C.tsmi_conv_implicit_gemm_grouped_packed(_PACK20(
-        _stream(), x.data_ptr(), wp.data_ptr(), ptrs[0], ptrs[1], ptrs[3], ptrs[4], g.padded,
-        num_out_feats, kvol, cin, cout, _dtype_code(x), pb or 0, pr or 0, int(relu), at, ldy, a2, ld2)))
+    block = _PACK20(_stream(), x.data_ptr(), wp.data_ptr(), ptrs[0], ptrs[1], ptrs[3], ptrs[4], g.padded,
+                    num_out_feats, kvol, cin, cout, _dtype_code(x), pb or 0, pr or 0, int(relu), at, ldy, a2, ld2)
+    if not (_region_depth and _hand_over(2, block, 20, (x, wp, g, bias, residual, y, also))):
+        _check(_C.tsmi_conv_implicit_gemm_grouped_packed(block))
     return y
 
 
@@ -1923,10 +2044,12 @@ def conv_implicit_gemm_segments(x, wp, kvol, cin, cout, out_in_map, num_out_feat
     pb, pr = _epilogue_args(bias, residual, x, num_out_feats, cout)
     with _scratch_lock:
         products = _scratch(x.device, stream, kvol * seg_rows * cout * x.element_size())
-        _check(_C.tsmi_conv_implicit_gemm_segments_packed(_PACK20(
-            stream, x.data_ptr(), wp.data_ptr(), seg.in_rows_ptr, seg.counts_ptr, seg.pos_ptr, seg_rows,
-            num_out_feats, kvol, cin, cout, _dtype_code(x), pb or 0, pr or 0, int(relu), products,
-            at, ldy, a2, ld2)))
+        block = _PACK20(stream, x.data_ptr(), wp.data_ptr(), seg.in_rows_ptr, seg.counts_ptr, seg.pos_ptr, seg_rows,
+                        num_out_feats, kvol, cin, cout, _dtype_code(x), pb or 0, pr or 0, int(relu), products,
+                        at, ldy, a2, ld2)
+        if not (_region_depth and _hand_over(1, block, 20, (x, wp, seg, bias, residual, y, also,
+                                                            _SCRATCH.get((x.device.index, stream))))):
+            _check(_C.tsmi_conv_implicit_gemm_segments_packed(block))
     return y
 
 
@@ -1953,15 +2076,18 @@ def _implicit_gemm(x, wp, kvol, cin, cout, out_in_map, num_out_feats, bias=None,
     ws_elems = _workspace_elems(num_out_feats, kvol, cin, cout, code) if num_out_feats < 65536 else 0
     if ws_elems > 0:  # (only maps with few row tiles use the offset split)
         with _scratch_lock:
-            _check(_C.tsmi_conv_implicit_gemm_packed(_PACK21(
-                stream, x.data_ptr(), wp.data_ptr(), out_in_map.data_ptr(), out_in_map.shape[0],
-                num_out_feats, kvol, cin, cout, code, pb or 0, pr or 0, int(relu),
-                _scratch(x.device, stream, 4 * ws_elems), ws_elems,
-                _tile_counters(x.device, stream).data_ptr(), _N_TILE_COUNTERS, at, ldy, a2, ld2)))
+            block = _PACK21(stream, x.data_ptr(), wp.data_ptr(), out_in_map.data_ptr(), out_in_map.shape[0],
+                            num_out_feats, kvol, cin, cout, code, pb or 0, pr or 0, int(relu),
+                            _scratch(x.device, stream, 4 * ws_elems), ws_elems,
+                            _tile_counters(x.device, stream).data_ptr(), _N_TILE_COUNTERS, at, ldy, a2, ld2)
+            if not (_region_depth and _hand_over(0, block, 21, (x, wp, out_in_map, bias, residual, y, also,
+                                                                _SCRATCH.get((x.device.index, stream))))):
+                _check(_C.tsmi_conv_implicit_gemm_packed(block))
     else:
-        _check(_C.tsmi_conv_implicit_gemm_packed(_PACK21(
-            stream, x.data_ptr(), wp.data_ptr(), out_in_map.data_ptr(), out_in_map.shape[0], num_out_feats,
-            kvol, cin, cout, code, pb or 0, pr or 0, int(relu), 0, 0, 0, _N_TILE_COUNTERS, at, ldy, a2, ld2)))
+        block = _PACK21(stream, x.data_ptr(), wp.data_ptr(), out_in_map.data_ptr(), out_in_map.shape[0], num_out_feats,
+                        kvol, cin, cout, code, pb or 0, pr or 0, int(relu), 0, 0, 0, _N_TILE_COUNTERS, at, ldy, a2, ld2)
+        if not (_region_depth and _hand_over(0, block, 21, (x, wp, out_in_map, bias, residual, y, also))):
+            _check(_C.tsmi_conv_implicit_gemm_packed(block))
     return y
 
 

@@ -21,6 +21,7 @@ SOURCES = [
     "pointops.hip",
     "norm.hip",
     "conv_api.cpp",
+    "launch_thread.cpp",
     "conv_igemm_f16.hip",
     "conv_igemm_bf16.hip",
     "conv_igemm_f32.hip",
@@ -39,7 +40,7 @@ FLAGS = [
 # which the package then loads; device code is never instrumented.  For CPU runs of the host
 # logic (python started with the sanitizer runtime preloaded), not for the GPU.
 SANITIZE = os.environ.get("ASAN", "0") not in ("", "0") or os.environ.get("SANITIZE") == "address"
-HOST_ONLY = ("common.cpp", "conv_api.cpp")
+HOST_ONLY = ("common.cpp", "conv_api.cpp", "launch_thread.cpp")
 HOST_SANITIZE = ["-Xarch_host", "-fsanitize=address", "-Xarch_host", "-shared-libasan",
                  "-Xarch_host", "-fno-omit-frame-pointer", "-Xarch_host", "-g"]
 if SANITIZE:

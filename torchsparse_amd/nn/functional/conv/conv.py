@@ -84,6 +84,9 @@ def conv3d(input: SparseTensor, weight: torch.Tensor,
                 feats, weight, None if bias is None else bias.to(feats.dtype),
                 None if residual is None else residual.contiguous(), relu)
         else:
+            if feats.is_cuda:
+                from torchsparse_amd import backend
+                backend.flush_launches()
             out_feats = feats.matmul(weight) if bias is None else torch.addmm(bias, feats, weight)
             if residual is not None:
                 out_feats += residual
@@ -154,7 +157,8 @@ def conv3d(input: SparseTensor, weight: torch.Tensor,
         output = SparseTensor._make(out_feats, fine_coords, fine_stride, fine_range, caches)
 
     if also is not None or out is not None:  # (a path that does not place its result itself)
-        from torchsparse_amd.backend import ColumnSlice
+        from torchsparse_amd.backend import ColumnSlice, flush_launches
+        flush_launches()
 
         def view(t):
             if t.__class__ is not ColumnSlice:

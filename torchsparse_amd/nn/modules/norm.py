@@ -59,6 +59,9 @@ class GroupNorm(nn.GroupNorm):
 
     def forward(self, input: SparseTensor) -> SparseTensor:
         feats, batch_col = input.feats, input.coords[:, 0]
+        if feats.is_cuda:
+            from ... import backend
+            backend.flush_launches()
         out = torch.zeros_like(feats)
         for b in range(int(batch_col.max().item()) + 1):
             rows = batch_col == b

@@ -25,6 +25,10 @@ def call_module(m: nn.Module, *args, **kwargs):
     if (m._forward_hooks or m._forward_pre_hooks or m._backward_hooks or m._backward_pre_hooks
             or _torch_module._global_forward_hooks or _torch_module._global_forward_pre_hooks
             or _torch_module._global_backward_hooks or _torch_module._global_backward_pre_hooks):
+        from torchsparse_amd import backend
+        if backend._region_depth:  # hooks look at the result: nothing stays with the launch thread
+            with backend.direct_launches():
+                return m(*args, **kwargs)
         return m(*args, **kwargs)
     return m.forward(*args, **kwargs)
 

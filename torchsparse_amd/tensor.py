@@ -94,6 +94,9 @@ class SparseTensor:
         return to_dense(self.feats, self.coords, self.spatial_range)
 
     def __add__(self, other: "SparseTensor") -> "SparseTensor":
+        if self.feats.is_cuda:
+            from . import backend
+            backend.flush_launches()  # (either operand may still be with the launch thread)
         return self._like(self.feats + other.feats)
 
 
