@@ -511,6 +511,7 @@ def _queue_maps_ahead(state, chain_rows, on_side: bool) -> None:
     plan, state.map_plan_seen = tuple(state.map_plan_seen), []
     state.map_plan = plan
     state.transposed_plan, state.transposed_seen = frozenset(state.transposed_seen), set()
+    state.segments_plan, state.segments_seen = frozenset(state.segments_seen), set()
     state.maps_ahead = {}
     state.maps_event = None
     state.pairs_of, state.pair_event, state.pair_vals = {}, None, None
@@ -534,7 +535,7 @@ def _queue_maps_ahead(state, chain_rows, on_side: bool) -> None:
         if request in state.transposed_plan:
             t_first = t_ints
             t_ints += make_divisible(a.shape[0], 128) * kvol
-        todo.append((a, b, ks, st, pd, kvol, first, t_first))
+        todo.append((a, b, ks, st, pd, kvol, first, t_first, request in state.segments_plan))
     if not todo:
         return
     dev = chain_rows[0].device
@@ -550,7 +551,8 @@ def _queue_maps_ahead(state, chain_rows, on_side: bool) -> None:
             state.pair_host = torch.zeros(_PAIR_SLOTS, dtype=torch.int64, pin_memory=True)
         pair_ptr = state.pair_dev.data_ptr() if counted else 0
         flat, queued, pairs_of = [], {}, {}
-        for slot, (a, b, ks, st, pd, kvol, first, t_first) in enumerate(todo):
+        segment_jobs = []
+        for slot, (a, b, ks, st, pd, kvol, first, t_first, with_segments) in enumerate(todo):
             n_pad = make_divisible(b.shape[0], 128)
             omap = buffers[kvol][first:first + n_pad]
             samples = _sorted_samples(a)
@@ -565,7 +567,17 @@ def _queue_maps_ahead(state, chain_rows, on_side: bool) -> None:
                                                   omap_t)
             if counted:
                 pairs_of[id(omap)] = (weakref.ref(omap), slot, b.shape[0] * kvol)
+            if with_segments:
+                segment_jobs.append((omap, b.shape[0], kvol))
         _check(_C.tsmi_kmap_sorted_batch(_stream(), len(todo), (ctypes.c_int64 * len(flat))(*flat)))
+        # the pair segments the forward before built over these maps, behind the maps on this
+        # stream instead of in front of their first layer on the caller's
+        for omap, n_rows, kvol in segment_jobs:
+            seg = _build_pair_segments(omap, n_rows, kvol, dev)
+            seg.buffer.record_stream(main)
+            _remember(_segments_of, id(omap), (weakref.ref(omap), omap._version, omap.data_ptr(),
+                                               main.cuda_stream, n_rows, seg), 64)
+            state.segments_hits += 1
         if counted:
             state.pair_host.copy_(state.pair_dev[2 * _PAIR_SLOTS:], non_blocking=True)
         event = torch.cuda.Event()
@@ -899,7 +911,8 @@ class _StridedState:
                  "chain_len", "ahead", "ahead_hits", "host_counters", "pending", "pending_rsv", "root_chain",
                  "lookahead_hits", "side", "grid_event", "grid_event_stream", "grid_old", "level_index", "map_plan",
                  "map_plan_seen", "maps_ahead", "maps_event", "maps_ahead_hits", "maps_main", "transposed_plan",
-                 "transposed_seen", "transposed_hits", "pair_dev", "pair_host", "pair_event", "pair_vals", "pairs_of")
+                 "transposed_seen", "transposed_hits", "pair_dev", "pair_host", "pair_event", "pair_vals", "pairs_of",
+                 "segments_plan", "segments_seen", "segments_hits")
 
     def __init__(self):
         self.grid_buf = None      # int32 scratch: bitmaps and chunk counts of every level
@@ -933,6 +946,9 @@ class _StridedState:
         # pair counts of the maps queued ahead: int64 [3 * 16] on the device (two words the blocks add
         # up in and take tickets from, then the count, per map), pinned copy of the counts, the event
         # behind that copy (None once it was seen done), the counts as a list, id(map) -> (ref, slot, entries)
+        self.segments_plan = frozenset()  # requests of map_plan whose pair segments were asked for too
+        self.segments_seen = set()
+        self.segments_hits = 0     # pair segments that were built on the second stream (diagnostic)
         self.pair_dev = None
         self.pair_host = None
         self.pair_event = None
@@ -1786,6 +1802,27 @@ class PairSegments:
         return iter((self.counts, self.in_rows, self.pos, self.seg_rows))
 
 
+def _build_pair_segments(out_in_map: torch.Tensor, n_rows: int, kvol: int, dev) -> PairSegments:
+    """One launch on the current stream (operands checked by the caller)."""
+    stream = _stream()
+    seg = PairSegments(kvol, n_rows, make_divisible(max(n_rows, 1), 128), dev)
+    key = (dev.index, stream)
+    pool = _SEGMENT_POOLS.get(key)
+    if pool is None:
+        with _tables_lock:
+            pool = _SEGMENT_POOLS.get(key)
+            if pool is None:
+                pool = _SEGMENT_POOLS[key] = torch.zeros(520, dtype=torch.int32, device=dev)
+    if _pin_sinks:
+        _pin(pool)
+        _pin(seg.buffer)
+    with _scratch_lock:  # (the pool is shared by the builds of one stream)
+        _check(_C.tsmi_pair_segments(stream, out_in_map.data_ptr(), n_rows, kvol, seg.seg_rows,
+                                     pool.data_ptr() if kvol < 520 else None, seg.counts_ptr,
+                                     seg.in_rows_ptr, seg.pos_ptr))
+    return seg
+
+
 def pair_segments(out_in_map: torch.Tensor, n_rows: int) -> PairSegments:
     """The pair segments of a kernel map's first ``n_rows`` rows: per kernel offset the input
     rows of its pairs, compacted (``in_rows``), their number (``counts``) and for every (offset,
@@ -1802,22 +1839,10 @@ def pair_segments(out_in_map: torch.Tensor, n_rows: int) -> PairSegments:
     kvol = out_in_map.shape[1]
     if n_rows > out_in_map.shape[0]:
         raise ValueError(f"the map has {out_in_map.shape[0]} rows, fewer than the {n_rows} asked for")
-    dev = out_in_map.device
-    seg = PairSegments(kvol, n_rows, make_divisible(max(n_rows, 1), 128), dev)
-    key = (dev.index, stream)
-    pool = _SEGMENT_POOLS.get(key)
-    if pool is None:
-        with _tables_lock:
-            pool = _SEGMENT_POOLS.get(key)
-            if pool is None:
-                pool = _SEGMENT_POOLS[key] = torch.zeros(520, dtype=torch.int32, device=dev)
-    if _pin_sinks:
-        _pin(pool)
-        _pin(seg.buffer)
-    with _scratch_lock:  # (the pool is shared by the builds of one stream)
-        _check(_C.tsmi_pair_segments(stream, out_in_map.data_ptr(), n_rows, kvol, seg.seg_rows,
-                                     pool.data_ptr() if kvol < 520 else None, seg.counts_ptr,
-                                     seg.in_rows_ptr, seg.pos_ptr))
+    request = _map_requests.get(id(out_in_map))
+    if request is not None and request[0]() is out_in_map:
+        request[1].segments_seen.add(request[2])  # a map of the chain in flight: built ahead next time
+    seg = _build_pair_segments(out_in_map, n_rows, kvol, out_in_map.device)
     if torch.cuda.is_current_stream_capturing():
         return seg  # filled by the recording's replays only: not for the table
     _remember(_segments_of, id(out_in_map), (weakref.ref(out_in_map), out_in_map._version, out_in_map.data_ptr(),
