@@ -949,6 +949,23 @@ def main():
     ms_unfused = timed(unfused, max(args.steps // 2, 1), 2, rows="same")
     ms_same = timed(model, args.steps, args.warmup, rows="same")
     ms_resident = timed(model, args.steps, args.warmup, rows="resident")
+    # the same new-tensor loop with the convolution calls launched by this thread instead of the
+    # library's launch thread, and what queuing one forward costs the host (device idle at its start)
+    backend.launch_thread = False
+    ms_direct = timed(model, args.steps, args.warmup, rows="new")
+    backend.launch_thread = True
+
+    def host_ms(iters=20):
+        total = 0.0
+        with torch.no_grad():
+            for _ in range(iters):
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                head(model(ts.SparseTensor(feats, coords))[-1].feats)
+                total += time.perf_counter() - t0
+        torch.cuda.synchronize()
+        return total * 1e3 / iters
+    ms_host = host_ms()
     ms_per_step = timed(model, args.steps, args.warmup, rows="new", mark=True)
 
     with torch.no_grad():
@@ -999,6 +1016,8 @@ def main():
                    "unfused_ms_per_step": round(ms_unfused, 4),
                    "same_coordinate_tensor_ms_per_step": round(ms_same, 4),
                    "resident_new_coordinate_tensor_declared_ready_ms_per_step": round(ms_resident, 4),
+                   "host_ms_to_queue_one_forward": round(ms_host, 4),
+                   "new_tensor_ms_per_step_without_launch_thread": round(ms_direct, 4),
                    "conv_mode": F.get_conv_mode().value},
         "roofline": roof, "roofline_kmap": roof_kmap, "cpu_baseline": cpu, "layers": layers,
         "backward": backward,
