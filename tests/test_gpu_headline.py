@@ -340,6 +340,8 @@ def test_minkunet_forward_on_the_scan(mods, scan):
     assert state.transposed_hits == 4, state.transposed_hits
     # ... and the pair segments of the three deep maps behind them, on the second stream
     assert state.segments_hits == 3, state.segments_hits
+    step()
+    assert state.segments_hits == 6 and state.transposed_hits == 8  # ... in every forward from then on
     for s in (1, 2, 4, 8):
         np.testing.assert_array_equal(inp3._caches.kmaps[_key(s, 2, 2)]["out_in_map_t"].cpu().numpy(), scan["up"][s])
 

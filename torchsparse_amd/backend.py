@@ -535,7 +535,12 @@ def _queue_maps_ahead(state, chain_rows, on_side: bool) -> None:
         if request in state.transposed_plan:
             t_first = t_ints
             t_ints += make_divisible(a.shape[0], 128) * kvol
-        todo.append((a, b, ks, st, pd, kvol, first, t_first, request in state.segments_plan))
+        with_segments = request in state.segments_plan
+        if with_segments:
+            # (a layer that finds its segments built asks no builder: the plan carries itself over;
+            # segments no layer uses any more cost their launch until the stream's state is reset)
+            state.segments_seen.add(request)
+        todo.append((a, b, ks, st, pd, kvol, first, t_first, with_segments))
     if not todo:
         return
     dev = chain_rows[0].device
