@@ -1915,7 +1915,7 @@ def grouped_map(out_in_map: torch.Tensor, n_rows: int, window: Optional[int] = N
     """The grouped copy of a 3x3x3 kernel map's first ``n_rows`` rows: grouped[p] =
     out_in_map[row_of[p]], positions sorted inside windows of ``window`` rows by the kernel
     planes a row uses, padding positions (-1) last; and its row tiles listed heaviest first.
-    Two launches, once per map tensor and stream."""
+    Four launches, once per map tensor and stream."""
     window = group_window if window is None else int(window)
     stream = _stream()
     hit = _grouped_of.get(id(out_in_map))
