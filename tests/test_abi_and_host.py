@@ -245,3 +245,26 @@ def test_buffers_collected_while_recording_outlive_the_tables():
     backend.release_scratch()
     backend._IDENTITY_MAPS.clear()
     backend._TILE_COUNTERS.pop((0, 1234), None)
+
+
+def test_launch_thread_without_a_device():
+    """The launch thread starts, takes nothing while no device can be asked for its index (or no
+    region is open), and flushing and closing return at once."""
+    import struct
+    from torchsparse_amd import backend
+    C = backend._C
+    block = struct.pack("21q", *([0] * 21))
+    assert C.tsmi_launch_thread_submit(0, block, 21) == -1  # no region open
+    assert C.tsmi_launch_thread_open() == 0
+    done = C.tsmi_launch_thread_completed().contents.value
+    assert C.tsmi_launch_thread_submit(3, block, 21) == -1 and C.tsmi_launch_thread_submit(0, block, 22) == -1
+    if not torch.cuda.is_available():
+        assert C.tsmi_launch_thread_submit(0, block, 21) == -1  # (no device: the caller makes the call itself)
+    assert C.tsmi_launch_thread_flush() == 0
+    assert C.tsmi_launch_thread_close() == 0
+    assert C.tsmi_launch_thread_completed().contents.value == done
+    assert C.tsmi_launch_thread_submit(0, block, 21) == -1
+    # the Python region is a no-op without a GPU
+    with backend.launch_region() as region:
+        assert region.opened == torch.cuda.is_available()
+    assert backend._region_depth == 0
