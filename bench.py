@@ -47,8 +47,8 @@ MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-layers", action="store_true", help="skip the single-layer sweep")
     ap.add_argument("--no-roofline", action="store_true", help="skip the per-kernel roofline timing")
