@@ -141,10 +141,15 @@ int tsmi_kmap_sorted(tsmi_stream_t s, const int32_t *in_coords, int64_t n_in,
                      const int64_t *samples, int32_t *out_in_map);
 /* `count` builds of tsmi_kmap_sorted queued by one call (a network's maps over the levels of a
  * strided chain, built ahead of their use): maps with 2^3 and 3^3 kernels share one launch, up to
- * eight at a time; others get a launch each.  args: host int64[20 * count], per map
+ * eight at a time; others get a launch each.  args: host int64[22 * count], per map
  * [in_coords, n_in, out_coords, n_out, n_out_pad, samples (0: none), out_in_map, ks[3],
- * stride[3], pad[3], map_t, n_t_pad, pair_words, pair_out] with the pointers as integers.  The last
- * four are optional products of the same launch (0: not wanted):
+ * stride[3], pad[3], map_t, n_t_pad, pair_words, pair_out, n_in_dev, n_out_dev] with the pointers as
+ * integers.  n_in_dev / n_out_dev (0: none): device int32 that hold the row counts when these are
+ * not on the host yet (the rows come out of launches queued just before, tsmi_downsample_chain_rows):
+ * n_in, n_out and n_out_pad are then upper bounds that size the launch and the buffers, the kernel
+ * works on min(count, bound) rows and pads the map to the next multiple of 128 of the count; only for
+ * inputs of at most 131,072 rows (no samples).  map_t .. pair_out are optional products of the same
+ * launch (0: not wanted):
  *   map_t int32[n_t_pad * K_vol] (n_t_pad >= n_in), filled with -1 by the caller beforehand:
  *     receives map_t[in, k] = out for every pair found, which makes it the transposed map
  *     (tsmi_transpose_map's result; the reference's others/query_cuda.cu:9-15 after the fill of

@@ -280,6 +280,8 @@ def test_minkunet_forward_on_the_scan(mods, scan):
     # stream as soon as the row counts are known (the maps compared below are those)
     assert state.maps_ahead_hits == 8, state.maps_ahead_hits
     assert state.transposed_hits == 0  # (asked for in this forward for the first time: see the end)
+    # ... queued behind the chain before its counts had reached the host (the counts stay on the device)
+    assert state.maps_early_hits == 1, state.maps_early_hits
 
     # --- the nine kernel maps and the coordinate levels, bit-exact
     caches = inp._caches
@@ -406,3 +408,10 @@ def test_minkunet_over_alternating_scans(mods, scan):
         if k in logits:
             assert torch.equal(got, logits[k]), (turn, k)
         logits[k] = got
+    state, = backend._stream_states.values()
+    # from the third forward on the maps are queued before the counts of their levels are known on
+    # the host, with room for an eighth more rows than the forward before had: enough for A after
+    # A, B after B and B (the smaller scan) after A; A after B outgrows it, twice, and has its
+    # maps queued once the counts are there
+    assert all(a > b + b // 8 + 1024 for a, b in zip(sizes["A"][1:3], sizes["B"][1:3])), sizes
+    assert state.maps_early_hits == 4, state.maps_early_hits

@@ -294,7 +294,7 @@ def test_batch_of_maps_in_one_call_with_transposed_maps_and_pair_counts():
             omap_t = torch.full((t_pad, kvol), -1, dtype=torch.int32, device="cuda") if tr else None
             flat += [a.data_ptr(), a.shape[0], b.data_ptr(), b.shape[0], n_pad, 0, omap.data_ptr(), *ks, *st, *pd,
                      omap_t.data_ptr() if tr else 0, t_pad, words.data_ptr() + 16 * slot,
-                     words.data_ptr() + 8 * (2 * len(jobs) + slot)]
+                     words.data_ptr() + 8 * (2 * len(jobs) + slot), 0, 0]
             outs.append((omap, omap_t))
         status = backend._C.tsmi_kmap_sorted_batch(backend._stream(), len(jobs), (ctypes.c_int64 * len(flat))(*flat))
         assert status == 0, backend._C.tsmi_last_error()
@@ -311,7 +311,88 @@ def test_batch_of_maps_in_one_call_with_transposed_maps_and_pair_counts():
                 np.testing.assert_array_equal(got_t[:n_in], want_t[:n_in])
                 assert (got_t[n_in:] == -1).all()
     # a transposed map with fewer rows than there are inputs is refused
-    bad = list(flat[20:40])
+    bad = list(flat[22:44])
     bad[17] = jobs[1][0].shape[0] - 1
-    status = backend._C.tsmi_kmap_sorted_batch(backend._stream(), 1, (ctypes.c_int64 * 20)(*bad))
+    status = backend._C.tsmi_kmap_sorted_batch(backend._stream(), 1, (ctypes.c_int64 * 22)(*bad))
     assert status != 0 and b"transposed" in backend._C.tsmi_last_error()
+
+
+@pytest.mark.parametrize("rows", [30000, 700, 0])
+def test_batch_of_maps_whose_row_counts_are_on_the_device(rows):
+    """tsmi_kmap_sorted_batch with the counts of the levels left on the device: the call gets only
+    a bound (the root's rows) for every level, buffers sized by it, and pointers to the counts.
+    The rows of each map up to ceil128 of its real count equal the oracle's map, rows beyond stay
+    untouched, transposed maps and pair counts are those of the real counts; a level without rows
+    (count 0 on the device) writes nothing and counts no pairs."""
+    import ctypes
+    rng = np.random.default_rng(405)
+    c1 = ascending(lidar_like_coords(rng, 30000))
+    d1, c2 = oracle.kmap_downsample(c1, 2, 2, 0)
+    d2, c3 = oracle.kmap_downsample(c2, 2, 2, 0)
+    sub2, sub3 = oracle.kmap_subm(c2, 3), oracle.kmap_subm(c3, 3)
+    if rows < 30000:
+        # the later levels hold fewer rows than the chain found (down to none): a prefix of the
+        # ascending rows keeps its indices, so the maps are the full ones cut to the prefix, with
+        # the entries that pointed beyond the inputs' prefix gone
+        def cut(full, n_out, n_in):
+            m = full[:n_out].copy()
+            m[m >= n_in] = -1
+            return m
+        n2, n3 = rows, min(rows, len(c3)) // 2
+        d1, d2 = cut(d1, n2, len(c1)), cut(d2, n3, n2)
+        sub2, sub3 = cut(sub2, n2, n2), cut(sub3, n3, n3)
+        c2, c3 = c2[:n2], c3[:n3]
+    n = c1.shape[0]
+    n_pad = -(-n // 128) * 128
+    # the levels in one buffer of n rows each (what a chain that emits before the read-back leaves)
+    levels = torch.full((2, n, 4), 0x7fffffff, dtype=torch.int32, device="cuda")
+    if len(c2):
+        levels[0, :len(c2)] = dev(c2)
+    if len(c3):
+        levels[1, :len(c3)] = dev(c3)
+    counts = torch.zeros(16, dtype=torch.int32, device="cuda")
+    counts[0], counts[8] = len(c2), len(c3)
+    t1 = dev(c1)
+    jobs = [  # (input level, output level, ks, st, pd, transposed?, oracle map)
+        (0, 1, (2, 2, 2), (2, 2, 2), (0, 0, 0), True, d1),
+        (1, 1, (3, 3, 3), (1, 1, 1), (1, 1, 1), False, sub2),
+        (1, 2, (2, 2, 2), (2, 2, 2), (0, 0, 0), True, d2),
+        (2, 2, (3, 3, 3), (1, 1, 1), (1, 1, 1), True, sub3),
+    ]
+    real = [n, len(c2), len(c3)]
+    rows_ptr = lambda l: t1.data_ptr() if l == 0 else levels.data_ptr() + (l - 1) * n * 16  # noqa: E731
+    count_ptr = lambda l: 0 if l == 0 else counts.data_ptr() + 32 * (l - 1)  # noqa: E731
+    words = torch.zeros(3 * len(jobs), dtype=torch.int64, device="cuda")
+    for attempt in range(2):
+        flat, outs = [], []
+        for slot, (i, o, ks, st, pd, tr, want) in enumerate(jobs):
+            kvol = ks[0] * ks[1] * ks[2]
+            omap = torch.full((n_pad, kvol), -9, dtype=torch.int32, device="cuda")
+            omap_t = torch.full((n_pad, kvol), -1, dtype=torch.int32, device="cuda") if tr else None
+            flat += [rows_ptr(i), n, rows_ptr(o), n, n_pad, 0, omap.data_ptr(), *ks, *st, *pd,
+                     omap_t.data_ptr() if tr else 0, n_pad, words.data_ptr() + 16 * slot,
+                     words.data_ptr() + 8 * (2 * len(jobs) + slot), count_ptr(i), count_ptr(o)]
+            outs.append((omap, omap_t))
+        status = backend._C.tsmi_kmap_sorted_batch(backend._stream(), len(jobs), (ctypes.c_int64 * len(flat))(*flat))
+        assert status == 0, backend._C.tsmi_last_error()
+        torch.cuda.synchronize()
+        host = words.cpu().numpy()
+        assert (host[:2 * len(jobs)] == 0).all()
+        for slot, ((i, o, ks, st, pd, tr, want), (omap, omap_t)) in enumerate(zip(jobs, outs)):
+            n_out, n_in = real[o], real[i]
+            pad = -(-n_out // 128) * 128
+            got = omap.cpu().numpy()
+            np.testing.assert_array_equal(got[:n_out], want[:n_out])
+            assert (got[n_out:pad] == -1).all() and (got[pad:] == -9).all()
+            assert host[2 * len(jobs) + slot] == (want[:n_out] >= 0).sum()
+            if tr:
+                want_t = (oracle.transpose_map(want[:n_out], n_in) if n_out and n_in
+                          else np.full((n_in, got.shape[1]), -1))
+                got_t = omap_t.cpu().numpy()
+                np.testing.assert_array_equal(got_t[:n_in], want_t[:n_in])
+                assert (got_t[n_in:] == -1).all()
+    # counts on the device go with inputs small enough to be searched without samples
+    big = list(flat[22:44])
+    big[1] = 200000
+    status = backend._C.tsmi_kmap_sorted_batch(backend._stream(), 1, (ctypes.c_int64 * 22)(*big))
+    assert status != 0 and b"samples" in backend._C.tsmi_last_error()

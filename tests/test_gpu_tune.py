@@ -70,6 +70,8 @@ def test_every_candidate_configuration_matches_the_oracle():
     for cand in cands:
         T._set_configs(model, names, cand)
         backend._segments_of.clear()
+        torch.cuda.synchronize()
+        backend.release_scratch()  # (and what the forward before asked to be built ahead of this one)
         with torch.no_grad():
             got = model(ts.SparseTensor(x16.cuda(), probe.coords.cuda())).feats.float().cpu().numpy()
         # the wide layer ran over pair segments exactly when the candidate forces that form

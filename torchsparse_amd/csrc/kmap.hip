@@ -1404,7 +1404,7 @@ static int sorted_args(SortedArgs *a, int *cube, int64_t *blocks, const int32_t 
                        const int32_t *out_coords, int64_t n_out, int64_t n_out_pad, const int32_t ks[3],
                        const int32_t stride[3], const int32_t pad[3], const int64_t *samples,
                        int32_t *out_in_map, int32_t *map_t, int64_t n_t_pad, int64_t *pair_words,
-                       int64_t *pair_out) {
+                       int64_t *pair_out, const int32_t *n_in_dev = nullptr, const int32_t *n_out_dev = nullptr) {
   if (int e = make_geom(&a->g, ks, stride, pad)) return e;
   TSMI_REQUIRE(tsmi_kmap_sorted_supported(ks), "kmap_sorted: kernel size (%d, %d, %d) not supported",
                ks[0], ks[1], ks[2]);
@@ -1427,6 +1427,8 @@ static int sorted_args(SortedArgs *a, int *cube, int64_t *blocks, const int32_t 
   a->n_out = n_out;
   a->n_out_pad = n_out_pad;
   a->rows = std::min(kBlock, kSortedTileInts / a->g.kvol);
+  TSMI_REQUIRE(!n_in_dev || tsmi_kmap_sorted_samples_elems(n_in) == 0,
+               "kmap_sorted: inputs whose count is on the device must be small enough to need no samples");
   const bool sampled = samples != nullptr && tsmi_kmap_sorted_samples_elems(n_in) > 0;
   a->first = sampled ? (const unsigned long long *)samples : nullptr;
   a->cell = sampled ? (const unsigned long long *)samples + kSortedSamples : nullptr;
@@ -1435,6 +1437,8 @@ static int sorted_args(SortedArgs *a, int *cube, int64_t *blocks, const int32_t 
   a->pair_acc = (unsigned long long *)pair_words;
   a->pair_ticket = pair_words ? (unsigned int *)(pair_words + 1) : nullptr;
   a->pair_out = (long long *)pair_out;
+  a->n_in_dev = n_in_dev;
+  a->n_out_dev = n_out_dev;
   *blocks = ceil_div(n_out_pad, a->rows);
   TSMI_REQUIRE(grid_fits(*blocks), "kmap_sorted: too many rows for one launch");
   a->n_blocks = (unsigned)*blocks;
@@ -1469,7 +1473,7 @@ extern "C" int tsmi_kmap_sorted(tsmi_stream_t s, const int32_t *in_coords, int64
 
 extern "C" int tsmi_kmap_sorted_batch(tsmi_stream_t s, int count, const int64_t *args) {
   TSMI_REQUIRE(count >= 0 && (count == 0 || args), "kmap_sorted_batch: bad arguments");
-  constexpr int kWords = 20;  // int64 words per map
+  constexpr int kWords = 22;  // int64 words per map
   int done = 0;
   while (done < count) {
     // as many of the next maps as one launch takes: 2^3 and 3^3 kernels, up to kSortedBatchMax
@@ -1491,7 +1495,8 @@ extern "C" int tsmi_kmap_sorted_batch(tsmi_stream_t s, int count, const int64_t 
                               (const int32_t *)(uintptr_t)a[2], a[3], a[4], geom, geom + 3, geom + 6,
                               (const int64_t *)(uintptr_t)a[5], (int32_t *)(uintptr_t)a[6],
                               (int32_t *)(uintptr_t)a[16], a[17], (int64_t *)(uintptr_t)a[18],
-                              (int64_t *)(uintptr_t)a[19]))
+                              (int64_t *)(uintptr_t)a[19], (const int32_t *)(uintptr_t)a[20],
+                              (const int32_t *)(uintptr_t)a[21]))
         return e;
       if (blocks == 0) {
         ++done;
