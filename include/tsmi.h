@@ -287,21 +287,29 @@ int tsmi_downsample_grid_emit(tsmi_stream_t s, const int32_t ks[3], const int32_
                               int32_t *vals, int64_t cap, int32_t *out_coords, int32_t *counters);
 
 /* A whole chain of `levels` equal strided layers with one output per input (kernel size ==
- * stride, no padding) queued by one call: tsmi_coords_max over coords, then per level
- * tsmi_downsample_grid_count and tsmi_downsample_grid_emit with the count left on the device,
- * each level marking from the rows of the one before.  scratch is the int32 buffer that holds
- * every level's bitmap (at word bitmap_at[level], bitmap_words[level] words, all zero on entry
- * and on completion) and chunk counts (at word chunks_at[level]); the three arrays are host
- * int64[levels].  counters: zero-filled device int32[8 * levels], per level [n_out, -, grid too
- * large, unpackable, maxima (b, x, y, z) of the level's INPUT rows]; rows: device
- * int32[levels, n, 4], level i's first counters[8 i] rows are its output coordinates.  Nothing
- * is read back.  No counterpart in the reference, which builds level after level with a
- * read-back each (others/sparsemapping_cuda.cu:429-507, called once per strided layer). */
+ * stride, no padding) queued by one call.  The outputs of level l are the cells of the ROOT's
+ * rows carried down l + 1 layers (a row drops out where a layer's rule leaves its output out:
+ * beyond floor((max - (ks - 1)) / stride) of that layer's inputs), so no level needs the rows
+ * of the one before, only the maxima of its inputs: tsmi_coords_max over coords, one launch per
+ * level that marks its bitmap from the root's rows and raises the maxima of the next level, then
+ * one launch that counts the chunks of every level, one that scans them (the counters are
+ * complete), one that emits every level's rows and clears the bitmaps: levels + 4 launches.
+ * phase 0: all of them; 1: up to the counters (what a caller copies to the host); 2: the rows
+ * (after phase 1 with the same arguments, on the same stream).  scratch is the int32 buffer that
+ * holds every level's bitmap (at word bitmap_at[level], a multiple of 4, bitmap_words[level]
+ * words, all zero on entry and after phase 2) and chunk counts (at word chunks_at[level]); the
+ * three arrays are host int64[levels].  counters: zero-filled device int32[8 * levels], per level
+ * [n_out, -, grid too large, unpackable, maxima (b, x, y, z) of the level's INPUT rows]; rows:
+ * device int32[levels, n, 4], level i's first counters[8 i] rows are its output coordinates in
+ * ascending order.  A level whose grid does not fit its bitmap is flagged and leaves no rows, nor
+ * do the levels after it.  Nothing is read back.  No counterpart in the reference, which builds
+ * level after level with a read-back each (others/sparsemapping_cuda.cu:429-507, called once per
+ * strided layer). */
 int tsmi_downsample_chain_rows(tsmi_stream_t s, const int32_t *coords, int64_t n,
                                const int32_t ks[3], const int32_t stride[3], const int32_t pad[3],
                                int levels, int32_t *scratch, const int64_t *bitmap_at,
                                const int64_t *bitmap_words, const int64_t *chunks_at,
-                               int32_t *counters, int32_t *rows);
+                               int32_t *counters, int32_t *rows, int phase);
 
 /* map_t[in,k] = out for every map[out,k] = in >= 0, out < n_rows; map_t
  * [n_rows_t, K_vol] is filled with -1 first.  Replaces

@@ -620,3 +620,69 @@ def test_maps_queued_ahead_match_the_oracle(seed):
             np.testing.assert_array_equal(km["out_in_map"].cpu().numpy(), want_sub[d + 1])
     state, = backend._stream_states.values()
     assert state.maps_ahead_hits >= 2 * depth  # at least one pass took its maps from the queue
+
+
+def _chain_cases():
+    rng = np.random.default_rng(321)
+    scan = lidar_like_coords(rng, 30000)
+    # a cloud whose largest coordinates are lone rows: the row with the largest x has an even y
+    # at the largest y (the layer's rule leaves its output out), so the maxima of the next level
+    # come from other rows than the maxima of this one; the same again one level further down
+    cloud = random_coords(rng, 3000, (200, 180, 40), 1)
+    lone = np.array([[0, 260, 250, 17], [0, 259, 3, 77], [0, 4, 249, 76], [0, 258, 7, 2], [0, 131, 125, 39]], np.int32)
+    spiky = np.concatenate([cloud, lone])
+    # ... and one whose largest row is alone far out: the next level's largest x is not half of it
+    gap = np.concatenate([random_coords(rng, 3000, (198, 180, 40), 1), np.array([[0, 260, 250, 17]], np.int32)])
+    batches = random_coords(rng, 5000, (60, 50, 30), 3)
+    few = np.array([[0, 1, 1, 0], [0, 0, 1, 1], [0, 1, 0, 0]], np.int32)  # gone after two layers
+    below = np.concatenate([random_coords(rng, 500, (40, 40, 20), 1), np.array([[0, -3, 5, 5], [0, 7, -1, 2]], np.int32)])
+    return [("scan", scan, 2, 4), ("spiky", spiky, 2, 4), ("gap", gap, 2, 4), ("batches", batches, 2, 3),
+            ("threes", scan, 3, 3),
+            ("flat", spiky, (2, 2, 1), 4), ("few", few, 2, 4), ("one", few[:1], 2, 2), ("below", below, 2, 3),
+            ("shuffled", scan[rng.permutation(len(scan))], 2, 4)]
+
+
+@pytest.mark.parametrize("name,coords,ks,levels", _chain_cases(), ids=[c[0] for c in _chain_cases()])
+def test_chain_of_strided_levels_from_the_root_rows(name, coords, ks, levels):
+    """tsmi_downsample_chain_rows marks every level from the chain's root: the rows of each level
+    equal the oracle's strided layer applied to the level before (whose outputs and extents
+    follow from the largest coordinates of ITS inputs), the counters hold the counts and those
+    maxima, the bitmaps are clear again; in one call and in the two phases a caller puts its copy
+    of the counters between."""
+    import ctypes
+    ks = t3(ks)
+    want, c = [], coords
+    while len(want) < levels and len(c):
+        c = oracle.kmap_downsample(c, ks, ks, 0)[1]
+        want.append(c)
+    n = len(coords)
+    words = max(1 << 15, (1 << (n * 2048 - 1).bit_length()) // 32)
+    layout, total = backend._grid_layout(words)
+    arrays = backend._layout_arrays(layout)
+    g = (backend._i3(ks), backend._i3(ks), backend._i3((0, 0, 0)))
+    root = dev(coords)
+    for phases in ((0,), (1, 2)):
+        scratch = torch.zeros(total, dtype=torch.int32, device="cuda")
+        ctr = torch.zeros(8 * levels, dtype=torch.int32, device="cuda")
+        rows = torch.full((levels, n, 4), -7, dtype=torch.int32, device="cuda")
+        for phase in phases:
+            status = backend._C.tsmi_downsample_chain_rows(backend._stream(), root.data_ptr(), n, *g, levels,
+                                                           scratch.data_ptr(), *arrays, ctr.data_ptr(),
+                                                           rows.data_ptr(), phase)
+            assert status == 0, backend._C.tsmi_last_error()
+            if phase == 1:
+                counts_first = ctr.cpu().numpy().copy()
+        host, got = ctr.cpu().numpy().reshape(levels, 8), rows.cpu().numpy()
+        if phases == (1, 2):
+            np.testing.assert_array_equal(counts_first, host.reshape(-1))  # complete before the rows
+        assert not any(scratch[at:at + w].any() for at, w, _ in layout[:levels])  # (the chunk counts stay)
+        inputs = coords
+        for level in range(levels):
+            out = want[level] if level < len(want) else np.zeros((0, 4), np.int32)
+            assert host[level, 0] == len(out), (name, level)
+            assert host[level, 2] == 0 and host[level, 3] == 0
+            np.testing.assert_array_equal(got[level, :len(out)], out)
+            assert (got[level, len(out):] == -7).all()
+            if len(inputs):
+                np.testing.assert_array_equal(host[level, 4:], np.maximum(inputs.max(0), 0))
+            inputs = out

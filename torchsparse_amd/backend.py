@@ -78,7 +78,7 @@ def _load():
         "tsmi_downsample_grid_count_next": [_vp, _I3, _I3, _I3, _vp, _vp, _i64, _vp, _vp, _i64, _vp, _vp, _vp],
         "tsmi_downsample_grid_emit": [_vp, _I3, _I3, _I3, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _vp,
                                       _i64, _vp, _vp],
-        "tsmi_downsample_chain_rows": [_vp, _vp, _i64, _I3, _I3, _I3, _i32, _vp, _vp, _vp, _vp, _vp, _vp],
+        "tsmi_downsample_chain_rows": [_vp, _vp, _i64, _I3, _I3, _I3, _i32, _vp, _vp, _vp, _vp, _vp, _vp, _i32],
         "tsmi_transpose_map": [_vp, _vp, _i64, _i32, _vp, _i64],
         "tsmi_derive_bitmask": [_vp, _vp, _i64, _i32, _i32, _i64, _vp],
         "tsmi_argsort_desc": [_vp, _vp, _vp, _vp, _i32, _i64, _vp, _i64],
@@ -268,6 +268,9 @@ _range_ok = {}  # id(tensor) -> (weak reference, version, address, ascending: Tr
 # table, which takes any order).  A row outside the packed range of such a tensor raises its
 # ValueError from the call that picks the verdict up (settle_checks() picks up all of them).
 coords_check_deferred = True
+# The first check of any other tensor is read back at once; the strided chain that followed such
+# rows last time is queued before the host waits for the verdict (False: after it).
+coords_check_overlap = True
 _rows_ready = {}  # id(tensor) -> (weak reference, version, address)
 _pending_verdicts = []  # (weak reference, version, address, pinned slot, event)
 _verdict_slots = None   # pinned int32 ring the verdicts are copied into
@@ -406,7 +409,28 @@ def coords_ascending(coords: torch.Tensor) -> bool:
         _pending_verdicts.append((weakref.ref(coords), coords._version, coords.data_ptr(), slot, event))
         _mark_range_ok(coords, ascending=False, origin="user")  # (complete: the caller said so)
         return False
-    bits = int(flags.item())
+    if coords_check_overlap and rows is coords:
+        # The read-back below waits for everything the stream has queued - the whole forward
+        # before, in a loop over new tensors - and until it returns the device gets nothing new.
+        # What does not depend on the verdict is therefore queued first: the strided chain that
+        # followed rows like these last time (any order of rows will do for it, and rows it cannot
+        # take are flagged, not followed), on the second stream behind the check.
+        if _verdict_slots is None:
+            _verdict_slots = torch.zeros(_VERDICT_SLOTS, dtype=torch.int32, pin_memory=True)
+        if len(_pending_verdicts) >= _VERDICT_SLOTS - 1:
+            settle_checks(block=True)
+        slot = _verdict_next
+        while any(item[3] == slot for item in _pending_verdicts):  # (a verdict still on its way keeps its slot)
+            slot = (slot + 1) % _VERDICT_SLOTS
+        _verdict_next = (slot + 1) % _VERDICT_SLOTS
+        _verdict_slots[slot:slot + 1].copy_(flags, non_blocking=True)
+        event = torch.cuda.Event()
+        event.record()
+        strided_lookahead(coords, behind=event)
+        event.synchronize()
+        bits = int(_verdict_slots[slot])
+    else:
+        bits = int(flags.item())
     if bits & 2:
         raise _range_error()
     _mark_range_ok(coords, ascending=not (bits & 1), origin="user")
@@ -1124,7 +1148,7 @@ class _GridJob:
     marks and counts of every level queued, the counters on their way to pinned host memory —
     whose second half (emit) needs the counts on the host."""
     __slots__ = ("coords", "geom", "coords_max_host", "fan", "levels", "ctr", "host", "event", "stream", "rows",
-                 "early")
+                 "early", "rows_event")
 
 
 def _strided_fan(ks, st) -> int:
@@ -1164,8 +1188,9 @@ def _grid_start(state, coords, ks, st, pd, coords_max_host, fan, ahead, early=Fa
             and downsample_emit_before_readback):
         rows = torch.empty((levels, n, 4), dtype=torch.int32, device=dev)  # level i: rows[i, :n_out_i]
         state.grid_dirty = True
-        _check(_C.tsmi_downsample_chain_rows(s, _ptr(coords), n, *g, levels, buf_ptr, *_layout_arrays(layout),
-                                             ctr_ptr, rows.data_ptr()))
+        # (first what the counters need; the rows follow behind the copy of the counters)
+        chain_args = (s, _ptr(coords), n, *g, levels, buf_ptr, *_layout_arrays(layout), ctr_ptr, rows.data_ptr())
+        _check(_C.tsmi_downsample_chain_rows(*chain_args, 1))
     else:
         _check(_C.tsmi_coords_max(s, _ptr(coords), n, part(0, "in_max"), 0))
         state.grid_dirty = True  # marked bits stay behind unless the emit passes run
@@ -1179,7 +1204,7 @@ def _grid_start(state, coords, ks, st, pd, coords_max_host, fan, ahead, early=Fa
                 part(level, "in_max"), part(level, "bitmap"), layout[level][1],
                 part(level, "chunks"), part(level, "counters"), part(level + 1, "in_max")))
     job = _GridJob()
-    job.early = None
+    job.early = job.rows_event = None
     job.rows = rows
     job.coords, job.geom, job.coords_max_host, job.fan = coords, (ks, st, pd), coords_max_host, fan
     job.levels, job.ctr, job.stream = levels, ctr, s
@@ -1195,13 +1220,23 @@ def _grid_start(state, coords, ks, st, pd, coords_max_host, fan, ahead, early=Fa
         job.host.copy_(ctr, non_blocking=True)
         job.event = torch.cuda.Event()
         job.event.record()
-        state.grid_event, state.grid_event_stream = job.event, s
+        if rows is not None:
+            _check(_C.tsmi_downsample_chain_rows(*chain_args, 2))
+            # (the scratch is free again behind the rows, not behind the counters)
+            job.rows_event = state.grid_event = torch.cuda.Event()
+            state.grid_event.record()
+            state.grid_event_stream = s
+        else:
+            state.grid_event, state.grid_event_stream = job.event, s
         if (rows is not None and kmap_queue_before_counts and kmap_queue_ahead and kmap_through_sorted
                 and state.side is not None and s == state.side.cuda_stream):
             _launch_maps_early(state, job, coords)  # (behind the counters' copy: the host gets those first)
-    elif state.side is not None:  # (a state that never used its side stream needs no events)
-        state.grid_event, state.grid_event_stream = torch.cuda.Event(), s
-        state.grid_event.record()
+    else:
+        if rows is not None:
+            _check(_C.tsmi_downsample_chain_rows(*chain_args, 2))
+        if state.side is not None:  # (a state that never used its side stream needs no events)
+            state.grid_event, state.grid_event_stream = torch.cuda.Event(), s
+            state.grid_event.record()
     return job
 
 
@@ -1254,6 +1289,10 @@ def _grid_finish(state, job: _GridJob, rsv_ratio, cap, want_table):
     if job.event is not None:
         job.event.synchronize()
         host = job.host.tolist()
+        # the rows were emitted behind the counters' copy: a launch or two that the caller's stream,
+        # if it is another one, has to be behind as well (usually they are over by now)
+        if job.rows_event is not None and s != _stream() and not job.rows_event.query():
+            torch.cuda.current_stream(dev).wait_event(job.rows_event)
     else:
         host = ctr.tolist()
     if _pending_verdicts:
@@ -1363,12 +1402,16 @@ downsample_emit_before_readback = True
 downsample_side_stream = True
 
 
-def strided_lookahead(coords: torch.Tensor) -> None:
+def strided_lookahead(coords: torch.Tensor, behind=None) -> None:
     """Called when a submanifold map is built over ``coords``: start the strided chain that
-    followed such rows last time on this stream, if any."""
+    followed such rows last time on this stream, if any.  ``behind``: an event on the caller's
+    stream that the rows are complete behind - for a caller's rows whose check is still on its
+    way (no verdict yet: the chain takes rows in any order and flags those it cannot take)."""
     if not (downsample_lookahead_at_subm and downsample_through_grid and downsample_chain_ahead):
         return
-    if coords.shape[0] == 0 or _range_origin(coords) != "user":  # (most calls: a deeper level's rows)
+    if coords.shape[0] == 0:
+        return
+    if behind is None and _range_origin(coords) != "user":  # (most calls: a deeper level's rows)
         return
     with _state_lock:
         state = _strided_state(coords.device)
@@ -1401,6 +1444,8 @@ def strided_lookahead(coords: torch.Tensor) -> None:
                 state.side = torch.cuda.Stream(device=coords.device)
             torch.cuda.set_stream(state.side)  # (the context manager costs 6 us, two switches 0.8)
             try:
+                if behind is not None:
+                    state.side.wait_event(behind)
                 job = _grid_start(state, coords, ks, st, pd, None, fan, ahead, early=True)
             finally:
                 torch.cuda.set_stream(main)

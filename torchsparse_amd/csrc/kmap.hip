@@ -607,17 +607,18 @@ __device__ __forceinline__ int grid_thread_words(const uint32_t *bitmap, int64_t
   return __popc(v.x) + __popc(v.y);
 }
 
-__global__ __launch_bounds__(kBlock) void grid_count_kernel(const uint32_t *bitmap, int64_t cap_words,
-                                                            Geom g, int3 out_max_host, int has_host_max,
-                                                            const int32_t *in_max_dev,
-                                                            int32_t *chunk_counts) {
+// Set bits of every chunk -> chunk_counts; the blocks `first`, `first + step`, ... share the chunks.
+__device__ __forceinline__ void grid_count_chunks(const uint32_t *bitmap, int64_t cap_words, const Geom &g,
+                                                  int3 out_max_host, int has_host_max,
+                                                  const int32_t *in_max_dev, int32_t *chunk_counts,
+                                                  unsigned first, unsigned step) {
   // The extents live on the device, so the launch cannot be sized to the grid; a block that
   // only learns it has nothing to do still waits ~2 us for them, and thousands of such blocks
   // queue up behind each other.  A bounded number of blocks stride over the chunks instead.
   __shared__ int wave_sum[kBlock / 64];
   const GridDims d = grid_dims(g, out_max_host, has_host_max, in_max_dev, cap_words);
   const int64_t chunks = d.used_words / kGridChunkWords;
-  for (int64_t chunk = blockIdx.x; chunk < chunks; chunk += gridDim.x) {
+  for (int64_t chunk = first; chunk < chunks; chunk += step) {
     uint32_t w[2];
     int c = grid_thread_words(bitmap, chunk, w);
 #pragma unroll
@@ -629,10 +630,18 @@ __global__ __launch_bounds__(kBlock) void grid_count_kernel(const uint32_t *bitm
   }
 }
 
+__global__ __launch_bounds__(kBlock) void grid_count_kernel(const uint32_t *bitmap, int64_t cap_words,
+                                                            Geom g, int3 out_max_host, int has_host_max,
+                                                            const int32_t *in_max_dev,
+                                                            int32_t *chunk_counts) {
+  grid_count_chunks(bitmap, cap_words, g, out_max_host, has_host_max, in_max_dev, chunk_counts, blockIdx.x,
+                    gridDim.x);
+}
+
 // One block: chunk_counts[0 .. used chunks) -> exclusive prefix in place, total -> counters[0].
-__global__ __launch_bounds__(1024) void grid_scan_kernel(int32_t *chunk_counts, int64_t cap_words, Geom g,
-                                                         int3 out_max_host, int has_host_max,
-                                                         const int32_t *in_max_dev, int32_t *counters) {
+__device__ __forceinline__ void grid_scan_chunks(int32_t *chunk_counts, int64_t cap_words, const Geom &g,
+                                                 int3 out_max_host, int has_host_max,
+                                                 const int32_t *in_max_dev, int32_t *counters) {
   __shared__ int wave_sum[16];
   const GridDims d = grid_dims(g, out_max_host, has_host_max, in_max_dev, cap_words);
   const int n = (int)(d.used_words / kGridChunkWords);
@@ -663,18 +672,24 @@ __global__ __launch_bounds__(1024) void grid_scan_kernel(int32_t *chunk_counts, 
   }
 }
 
+__global__ __launch_bounds__(1024) void grid_scan_kernel(int32_t *chunk_counts, int64_t cap_words, Geom g,
+                                                         int3 out_max_host, int has_host_max,
+                                                         const int32_t *in_max_dev, int32_t *counters) {
+  grid_scan_chunks(chunk_counts, cap_words, g, out_max_host, has_host_max, in_max_dev, counters);
+}
+
 // Set bits in ascending order -> out_coords rows; every word read is cleared again.
 // Occupied cells cluster (surfaces): a few words of a chunk can hold most of its outputs, so
 // the block does not walk bits word by word.  It keeps the chunk's words and the exclusive
 // prefix of their bit counts in LDS, and thread i takes output rank i, i + 256, ...: a binary
 // search of the prefix finds the word, five halvings find the bit.  The table entries
 // (coordinate -> row + 1) are a separate launch of one thread per row.
-__global__ __launch_bounds__(kBlock) void grid_emit_kernel(uint32_t *bitmap, int64_t cap_words,
-                                                           const int32_t *chunk_prefix, Geom g,
-                                                           int3 out_max_host, int has_host_max,
-                                                           const int32_t *in_max_dev, GridDims host_dims,
-                                                           int have_host_dims, int4 *out_coords,
-                                                           int64_t n_out) {
+__device__ __forceinline__ void grid_emit_chunks(uint32_t *bitmap, int64_t cap_words,
+                                                 const int32_t *chunk_prefix, const Geom &g,
+                                                 int3 out_max_host, int has_host_max,
+                                                 const int32_t *in_max_dev, const GridDims &host_dims,
+                                                 int have_host_dims, int4 *out_coords, int64_t n_out,
+                                                 unsigned first_chunk, unsigned step) {
   __shared__ int wave_sum[kBlock / 64];
   __shared__ uint32_t words[kGridChunkWords];
   __shared__ int before[kGridChunkWords];  // set bits of the chunk before each word
@@ -683,7 +698,7 @@ __global__ __launch_bounds__(kBlock) void grid_emit_kernel(uint32_t *bitmap, int
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   // one block per chunk when the host knows the extents; otherwise a bounded number of blocks
   // strides over the chunks the device-side extents cover
-  for (int64_t chunk = blockIdx.x; chunk * kGridChunkWords < d.used_words; chunk += gridDim.x) {
+  for (int64_t chunk = first_chunk; chunk * kGridChunkWords < d.used_words; chunk += step) {
   uint32_t w[2];
   const int mine = grid_thread_words(bitmap, chunk, w);
   if (mine)  // leave the bitmap all clear for the next call
@@ -736,6 +751,114 @@ __global__ __launch_bounds__(kBlock) void grid_emit_kernel(uint32_t *bitmap, int
   }
   __syncthreads();  // the LDS arrays are rewritten by the next chunk
   }
+}
+
+__global__ __launch_bounds__(kBlock) void grid_emit_kernel(uint32_t *bitmap, int64_t cap_words,
+                                                           const int32_t *chunk_prefix, Geom g,
+                                                           int3 out_max_host, int has_host_max,
+                                                           const int32_t *in_max_dev, GridDims host_dims,
+                                                           int have_host_dims, int4 *out_coords,
+                                                           int64_t n_out) {
+  grid_emit_chunks(bitmap, cap_words, chunk_prefix, g, out_max_host, has_host_max, in_max_dev, host_dims,
+                   have_host_dims, out_coords, n_out, blockIdx.x, gridDim.x);
+}
+
+// ---- a chain of equal strided layers with one output per input, every level marked from the
+// chain's ROOT rows.  Level l's cells are those of the root's rows carried down l + 1 layers, so
+// the marks of level l need the maxima of its inputs (the extents of its grid, and which outputs
+// the rule keeps) but not the rows of level l - 1: one launch per level marks it and raises the
+// maxima of the next, and then ONE launch counts the chunks of every level, one scans them, one
+// emits every level's rows.  levels + 3 launches (and tsmi_coords_max before them) where level
+// after level takes 4 each.
+constexpr int kChainMaxLevels = 8;
+struct ChainLayout {
+  int64_t bitmap_at[kChainMaxLevels];   // word of `scratch` where the level's bitmap starts
+  int64_t words[kChainMaxLevels];       // ... and its capacity
+  int64_t chunks_at[kChainMaxLevels];   // ... and where its chunk counts start
+  unsigned first_block[kChainMaxLevels + 1];  // blocks of the counting / emitting launch per level
+  int levels;
+};
+
+// One thread per root row: follow it down to `level` (dropped where the rule leaves a layer's
+// output out: beyond floor((max - (ks - 1)) / stride) of that layer's inputs, or unpackable) and
+// mark its cell there.  counters: 8 per level, [4..8) the maxima of the level's inputs - complete
+// for the levels up to `level`, raised here for `level + 1`.
+__global__ __launch_bounds__(kBlock) void chain_mark_kernel(const int4 *coords, int64_t n, Geom g, int level,
+                                                            ChainLayout lay, int32_t *scratch,
+                                                            int32_t *counters) {
+  const int3 none = make_int3(0, 0, 0);
+  GridDims d;
+  for (int j = 0; j <= level; ++j) {  // (the same for every thread)
+    d = grid_dims(g, none, 0, counters + 8 * j + 4, lay.words[j]);
+    if (!d.fits || d.used_words == 0) return;  // a level without outputs leaves none to the later ones
+  }
+  const int64_t tid = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  bool have = tid < n;
+  int4 c = have ? coords[tid] : make_int4(0, 0, 0, 0);
+  // an input the packed key cannot hold is missing from every table built from these rows
+  if (have && level == 0 && !coords_packable(c.x, c.y, c.z, c.w)) counters[3] = 1;
+  for (int j = 0; j <= level && have; ++j) {
+    const int32_t *in_max = counters + 8 * j + 4;
+    int lo[3], hi[3], b, o[3];
+    output_ranges(g, none, in_max, nullptr, 2, lo, hi);
+    bool unpackable = false;
+    have = strided_candidate_in(c, 0, g, lo, hi, 2, &b, o, &unpackable) && b <= in_max[0];
+    if (unpackable && j == level) counters[8 * level + 3] = 1;
+    c = make_int4(b, o[0], o[1], o[2]);
+  }
+  int word = -1;
+  uint32_t bits = 0;
+  if (have) {
+    const uint32_t cell = (((uint32_t)c.x * d.e[0] + c.y) * d.e[1] + c.z) * d.e[2] + c.w;
+    word = (int)(cell >> 5);
+    bits = 1u << (cell & 31);
+  }
+  if (level + 1 < lay.levels)
+    block_raise_max(have ? c.x : 0, have ? c.y : 0, have ? c.z : 0, have ? c.w : 0, counters + 8 * (level + 1) + 4);
+  uint32_t *bitmap = (uint32_t *)scratch + lay.bitmap_at[level];
+  const int lane = threadIdx.x & 63;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int w = __shfl_up(word, off);
+    const uint32_t v = __shfl_up(bits, off);
+    if (lane >= off && w == word) bits |= v;
+  }
+  const int next = __shfl_down(word, 1);
+  if (word >= 0 && (lane == 63 || next != word)) {
+    if ((bitmap[word] & bits) != bits) atomicOr(&bitmap[word], bits);
+  }
+}
+
+__device__ __forceinline__ int chain_level_of_block(const ChainLayout &lay, unsigned *first, unsigned *step) {
+  int level = 0;
+  while (level + 1 < lay.levels && blockIdx.x >= lay.first_block[level + 1]) ++level;
+  *first = blockIdx.x - lay.first_block[level];
+  *step = lay.first_block[level + 1] - lay.first_block[level];
+  return level;
+}
+
+__global__ __launch_bounds__(kBlock) void chain_count_kernel(Geom g, ChainLayout lay, const int32_t *scratch,
+                                                             int32_t *chunk_scratch, const int32_t *counters) {
+  unsigned first, step;
+  const int level = chain_level_of_block(lay, &first, &step);
+  grid_count_chunks((const uint32_t *)scratch + lay.bitmap_at[level], lay.words[level], g, make_int3(0, 0, 0), 0,
+                    counters + 8 * level + 4, chunk_scratch + lay.chunks_at[level], first, step);
+}
+
+__global__ __launch_bounds__(1024) void chain_scan_kernel(Geom g, ChainLayout lay, int32_t *scratch,
+                                                          int32_t *counters) {
+  const int level = blockIdx.x;
+  grid_scan_chunks(scratch + lay.chunks_at[level], lay.words[level], g, make_int3(0, 0, 0), 0,
+                   counters + 8 * level + 4, counters + 8 * level);
+}
+
+__global__ __launch_bounds__(kBlock) void chain_emit_kernel(Geom g, ChainLayout lay, int32_t *scratch,
+                                                            const int32_t *counters, int4 *rows, int64_t n) {
+  unsigned first, step;
+  const int level = chain_level_of_block(lay, &first, &step);
+  grid_emit_chunks((uint32_t *)scratch + lay.bitmap_at[level], lay.words[level], scratch + lay.chunks_at[level], g,
+                   make_int3(0, 0, 0), 0, counters + 8 * level + 4, GridDims{}, 0, rows + (int64_t)level * n, n,
+                   first, step);
 }
 
 // Occupied slots of a table, gathered in arbitrary order: one atomic per workgroup
@@ -1764,32 +1887,52 @@ extern "C" int tsmi_downsample_chain_rows(tsmi_stream_t s, const int32_t *coords
                                           const int32_t ks[3], const int32_t stride[3],
                                           const int32_t pad[3], int levels, int32_t *scratch,
                                           const int64_t *bitmap_at, const int64_t *bitmap_words,
-                                          const int64_t *chunks_at, int32_t *counters, int32_t *rows) {
-  TSMI_REQUIRE(levels >= 1 && levels <= 8 && n > 0 && coords && scratch && bitmap_at && bitmap_words &&
-                   chunks_at && counters && rows,
+                                          const int64_t *chunks_at, int32_t *counters, int32_t *rows,
+                                          int phase) {
+  TSMI_REQUIRE(levels >= 1 && levels <= kChainMaxLevels && n > 0 && coords && scratch && bitmap_at &&
+                   bitmap_words && chunks_at && counters && rows && phase >= 0 && phase <= 2,
                "downsample_chain_rows: bad arguments");
   for (int a = 0; a < 3; ++a)
     TSMI_REQUIRE(ks[a] == stride[a] && pad[a] == 0 && ks[a] >= 1,
                  "downsample_chain_rows: one output per input needs kernel size == stride and no padding");
-  // counters: 8 per level, [4..8) of a level = the maxima of its INPUT rows
-  if (int e = tsmi_coords_max(s, coords, n, counters + 4, 0)) return e;
-  const int32_t *src = coords;
-  for (int level = 0; level < levels; ++level) {
-    int32_t *ctr = counters + 8 * level;
-    int32_t *bitmap = scratch + bitmap_at[level];
-    int32_t *chunks = scratch + chunks_at[level];
-    int32_t *next_max = level + 1 < levels ? ctr + 8 + 4 : nullptr;
-    if (int e = tsmi_downsample_grid_count(s, src, n, ks, stride, pad, nullptr, ctr + 4, bitmap,
-                                           bitmap_words[level], 0, chunks, ctr, next_max,
-                                           level > 0 ? ctr - 8 : nullptr))
-      return e;
-    int32_t *out = rows + (int64_t)level * n * 4;
-    if (int e = tsmi_downsample_grid_emit(s, ks, stride, pad, nullptr, ctr + 4, nullptr, bitmap,
-                                          bitmap_words[level], chunks, -n, nullptr, nullptr, 0, out, ctr))
-      return e;
-    src = out;
+  Geom g;
+  if (int e = make_geom(&g, ks, stride, pad)) return e;
+  TSMI_REQUIRE((uintptr_t)scratch % 16 == 0, "downsample_chain_rows: scratch must be 16-byte aligned");
+  TSMI_GRID_CHECK(n);
+  // blocks of the launches that walk chunks: the extents are on the device, so a bounded number
+  // per level strides over the chunks there are
+  constexpr int64_t kBlocksPerLevel = 512;
+  ChainLayout lay;
+  lay.levels = levels;
+  lay.first_block[0] = 0;
+  for (int l = 0; l < kChainMaxLevels; ++l) {
+    const int u = l < levels ? l : 0;  // (unused entries repeat level 0)
+    TSMI_REQUIRE(bitmap_words[u] >= kGridChunkWords && bitmap_words[u] % kGridChunkWords == 0 &&
+                     bitmap_words[u] <= (int64_t(1) << 25) && bitmap_at[u] >= 0 && bitmap_at[u] % 4 == 0 &&
+                     chunks_at[u] >= 0,
+                 "downsample_chain_rows: bitmap_words must be a multiple of %d and at most 2^25, bitmaps 16-byte aligned",
+                 kGridChunkWords);
+    lay.bitmap_at[l] = bitmap_at[u];
+    lay.words[l] = bitmap_words[u];
+    lay.chunks_at[l] = chunks_at[u];
+    const int64_t blocks = l < levels ? std::min(bitmap_words[u] / kGridChunkWords, kBlocksPerLevel) : 0;
+    lay.first_block[l + 1] = lay.first_block[l] + (unsigned)blocks;
   }
-  return TSMI_OK;
+  hipStream_t st = (hipStream_t)s;
+  if (phase != 2) {
+    // counters: 8 per level, [4..8) of a level = the maxima of its INPUT rows
+    if (int e = tsmi_coords_max(s, coords, n, counters + 4, 0)) return e;
+    for (int level = 0; level < levels; ++level)
+      hipLaunchKernelGGL(chain_mark_kernel, grid_for(n), dim3(kBlock), 0, st, (const int4 *)coords, n, g, level,
+                         lay, scratch, counters);
+    hipLaunchKernelGGL(chain_count_kernel, dim3(lay.first_block[levels]), dim3(kBlock), 0, st, g, lay,
+                       (const int32_t *)scratch, scratch, (const int32_t *)counters);
+    hipLaunchKernelGGL(chain_scan_kernel, dim3((unsigned)levels), dim3(1024), 0, st, g, lay, scratch, counters);
+  }
+  if (phase != 1)
+    hipLaunchKernelGGL(chain_emit_kernel, dim3(lay.first_block[levels]), dim3(kBlock), 0, st, g, lay, scratch,
+                       (const int32_t *)counters, (int4 *)rows, n);
+  return check_launch("tsmi_downsample_chain_rows");
 }
 
 extern "C" int tsmi_transpose_map(tsmi_stream_t s, const int32_t *map, int64_t n_rows, int kvol,
