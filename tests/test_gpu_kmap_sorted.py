@@ -91,11 +91,48 @@ def test_unsorted_or_repeated_rows_take_the_tables():
     assert backend.coords_ascending(dev(coords[:1])) and backend.coords_ascending(dev(coords[:0]))
 
 
-def test_rows_declared_ready_are_checked_without_waiting_for_the_verdict():
-    """rows_ready(): the first map over such a tensor is built through the tables (the verdict of
+def test_rows_declared_ready_are_checked_on_the_second_stream():
+    """rows_ready(): the check of such rows runs on the device's second stream and its verdict is
+    read at once, while the caller's stream is still busy: ascending rows take the table-free
+    builder from their first map on, unsorted rows the tables, a row outside the packed range
+    raises from the call that looks at the tensor first."""
+    rng = np.random.default_rng(303)
+    coords = ascending(random_coords(rng, 3000, (30, 30, 12)))
+    busy = torch.empty(1 << 30, dtype=torch.int8, device="cuda")
+    assert backend.coords_ascending(backend.rows_ready(dev(coords)))  # (the second stream exists from here on)
+    t = backend.rows_ready(dev(coords))
+    torch.cuda.synchronize()
+    done = torch.cuda.Event()
+    for _ in range(50):
+        busy.fill_(1)  # (some 15 ms of work queued on the caller's stream)
+    done.record()
+    assert backend.coords_ascending(t)
+    assert not done.query()  # the verdict did not wait for the caller's stream
+    kmap = F.build_kernel_map(t, len(coords), 3, 1, 0, mode="hashmap_on_the_fly")
+    assert kmap["in_hashmap"] is None  # (the table-free builder)
+    np.testing.assert_array_equal(kmap["out_in_map"].cpu().numpy(), oracle.kmap_subm(coords, 3))
+    swapped = coords.copy()
+    swapped[[100, 101]] = swapped[[101, 100]]
+    u = backend.rows_ready(dev(swapped))
+    assert not backend.coords_ascending(u)
+    kmap = F.build_kernel_map(u, len(swapped), 3, 1, 0, mode="hashmap_on_the_fly")
+    assert kmap["in_hashmap"] is not None
+    np.testing.assert_array_equal(kmap["out_in_map"].cpu().numpy(), oracle.kmap_subm(swapped, 3))
+    far = coords.copy()
+    far[-1, 2] = 1 << 20  # beyond the 18 bits a packed key holds per axis
+    v = backend.rows_ready(dev(far))
+    with pytest.raises(ValueError, match="range"):
+        backend.coords_ascending(v)
+    assert not backend._pending_verdicts
+
+
+def test_rows_declared_ready_are_checked_without_waiting_for_the_verdict(monkeypatch):
+    """coords_check_aside off: the check of rows_ready() rows is queued on the caller's stream and
+    nobody waits for it.  The first map over such a tensor is built through the tables (the verdict of
     the ordering check is still on its way), equals the oracle's, and later maps take the
     table-free builder once the verdict has been picked up; unsorted rows keep the tables; a row
     outside the packed range raises at the latest when settle_checks() is called."""
+    monkeypatch.setattr(backend, "coords_check_aside", False)
     rng = np.random.default_rng(303)
     coords = ascending(random_coords(rng, 3000, (30, 30, 12)))
     t = backend.rows_ready(dev(coords))
@@ -396,3 +433,48 @@ def test_batch_of_maps_whose_row_counts_are_on_the_device(rows):
     big[1] = 200000
     status = backend._C.tsmi_kmap_sorted_batch(backend._stream(), 1, (ctypes.c_int64 * 22)(*big))
     assert status != 0 and b"samples" in backend._C.tsmi_last_error()
+
+
+def test_root_map_queued_before_the_verdict_of_a_new_tensor(monkeypatch):
+    """The submanifold map over a caller's rows is queued behind the first check of a new tensor,
+    before the host has the verdict, once the tensor before on this stream asked for such a map:
+    one launch per tensor either way, the oracle's map for ascending rows; rows that do not ascend
+    get theirs through the table (the queued search is dropped, and nothing is queued ahead for the
+    next tensor); a map nobody asks for ends the queueing as well."""
+    rng = np.random.default_rng(77)
+    base = ascending(lidar_like_coords(rng, 20000))
+    want = oracle.kmap_subm(base, 3)
+    launches = []
+    real = backend._kmap_sorted_launch
+    monkeypatch.setattr(backend, "_kmap_sorted_launch", lambda *a, **k: (launches.append(a[2]), real(*a, **k))[1])
+    backend._root_geoms.clear()
+    backend._root_maps.clear()
+
+    def build(rows):
+        t = dev(rows)
+        launches.clear()
+        m = F.build_kernel_map(t, len(rows), (3, 3, 3), 1, 0, mode="hashmap_on_the_fly")["out_in_map"]
+        return m.cpu().numpy(), len(launches)
+
+    got, n = build(base)  # learns the geometry
+    np.testing.assert_array_equal(got, want)
+    assert n == 1 and backend._root_geoms and not backend._root_maps
+    for _ in range(2):  # queued before the verdict, taken after it
+        got, n = build(base)
+        np.testing.assert_array_equal(got, want)
+        assert n == 1 and not backend._root_maps
+    shuffled = base[rng.permutation(len(base))]
+    got, n = build(shuffled)
+    np.testing.assert_array_equal(got, oracle.kmap_subm(shuffled, 3))
+    assert n == 1 and not backend._root_maps and not backend._root_geoms  # (the one launch was the dropped one)
+    got, n = build(base)
+    np.testing.assert_array_equal(got, want)
+    assert n == 1 and backend._root_geoms
+    # a new tensor whose map nobody asks for, then another one: nothing queued for it
+    t = dev(base)
+    launches.clear()
+    assert backend.coords_ascending(t) and len(launches) == 1 and len(backend._root_maps) == 1
+    t2 = dev(base)
+    assert backend.coords_ascending(t2) and len(launches) == 1
+    assert not backend._root_maps and not backend._root_geoms
+    torch.cuda.synchronize()

@@ -268,6 +268,10 @@ _range_ok = {}  # id(tensor) -> (weak reference, version, address, ascending: Tr
 # table, which takes any order).  A row outside the packed range of such a tensor raises its
 # ValueError from the call that picks the verdict up (settle_checks() picks up all of them).
 coords_check_deferred = True
+# ... unless the check runs on the device's second stream, where nothing of the caller's stream is
+# in its way: the host then waits for the verdict at once (a kernel and a copy) and rows that
+# ascend take the table-free builders from their first map on.
+coords_check_aside = True
 # The first check of any other tensor is read back at once; the strided chain that followed such
 # rows last time is queued before the host waits for the verdict (False: after it).
 coords_check_overlap = True
@@ -385,56 +389,95 @@ def _declared_ready(coords: torch.Tensor) -> bool:
 def coords_ascending(coords: torch.Tensor) -> bool:
     """Whether the rows of ``coords`` ascend strictly in (b, x, y, z); raises ValueError for a
     row outside the packed key's range.  One kernel and one read-back the first time a tensor
-    is seen, nothing afterwards; for rows declared complete (rows_ready) the verdict is picked
-    up later and False is the answer until then."""
-    global _verdict_slots, _verdict_next
+    is seen, nothing afterwards.  Rows declared complete (rows_ready) are checked on the second
+    stream, so that the read-back waits for nothing else (or, with coords_check_aside off, have
+    their verdict picked up later: False is the answer until then)."""
     if _pending_verdicts:
         settle_checks(block=False)
     hit = _range_entry(coords)
     if hit is not None and hit[3] is not None:
         return hit[3]
     rows = _need(coords, torch.int32, "coords")
+    if coords_check_aside and rows is coords and _declared_ready(coords):
+        return _verdict(coords, _check_aside(rows))
     flags = torch.zeros(1, dtype=torch.int32, device=rows.device)
     _check(_C.tsmi_coords_check(_stream(), _ptr(rows), rows.shape[0], _ptr(flags)))
     if coords_check_deferred and rows is coords and _declared_ready(coords):
-        if _verdict_slots is None:
-            _verdict_slots = torch.zeros(_VERDICT_SLOTS, dtype=torch.int32, pin_memory=True)
-        if len(_pending_verdicts) >= _VERDICT_SLOTS - 1:
-            settle_checks(block=True)  # (every slot is on its way: wait for them)
-        slot = _verdict_next
-        _verdict_next = (slot + 1) % _VERDICT_SLOTS
+        slot = _verdict_slot()
         _verdict_slots[slot:slot + 1].copy_(flags, non_blocking=True)
         event = torch.cuda.Event()
         event.record()
         _pending_verdicts.append((weakref.ref(coords), coords._version, coords.data_ptr(), slot, event))
         _mark_range_ok(coords, ascending=False, origin="user")  # (complete: the caller said so)
         return False
-    if coords_check_overlap and rows is coords:
+    elif coords_check_overlap and rows is coords:
         # The read-back below waits for everything the stream has queued - the whole forward
         # before, in a loop over new tensors - and until it returns the device gets nothing new.
         # What does not depend on the verdict is therefore queued first: the strided chain that
         # followed rows like these last time (any order of rows will do for it, and rows it cannot
         # take are flagged, not followed), on the second stream behind the check.
-        if _verdict_slots is None:
-            _verdict_slots = torch.zeros(_VERDICT_SLOTS, dtype=torch.int32, pin_memory=True)
-        if len(_pending_verdicts) >= _VERDICT_SLOTS - 1:
-            settle_checks(block=True)
-        slot = _verdict_next
-        while any(item[3] == slot for item in _pending_verdicts):  # (a verdict still on its way keeps its slot)
-            slot = (slot + 1) % _VERDICT_SLOTS
-        _verdict_next = (slot + 1) % _VERDICT_SLOTS
+        slot = _verdict_slot()
         _verdict_slots[slot:slot + 1].copy_(flags, non_blocking=True)
         event = torch.cuda.Event()
         event.record()
         strided_lookahead(coords, behind=event)
+        _queue_root_map(coords)
         event.synchronize()
         bits = int(_verdict_slots[slot])
+        if bits and _root_maps:
+            for key in [k for k in _root_maps if k[0] == id(coords)]:
+                _root_maps.pop(key, None)  # (searched over rows that do not ascend)
+            if bits & 1:
+                _root_geoms.pop((coords.device.index, _stream()), None)
     else:
         bits = int(flags.item())
+    return _verdict(coords, bits)
+
+
+def _verdict(coords: torch.Tensor, bits: int) -> bool:
     if bits & 2:
         raise _range_error()
     _mark_range_ok(coords, ascending=not (bits & 1), origin="user")
     return not (bits & 1)
+
+
+def _verdict_slot() -> int:
+    """A free element of the pinned ring the verdicts are copied into."""
+    global _verdict_slots, _verdict_next
+    if _verdict_slots is None:
+        _verdict_slots = torch.zeros(_VERDICT_SLOTS, dtype=torch.int32, pin_memory=True)
+    if len(_pending_verdicts) >= _VERDICT_SLOTS - 1:
+        settle_checks(block=True)  # (every slot is on its way: wait for them)
+    slot = _verdict_next
+    while any(item[3] == slot for item in _pending_verdicts):  # (a verdict still on its way keeps its slot)
+        slot = (slot + 1) % _VERDICT_SLOTS
+    _verdict_next = (slot + 1) % _VERDICT_SLOTS
+    return slot
+
+
+def _check_aside(rows: torch.Tensor) -> int:
+    """The check of rows that are complete (rows_ready), on the device's second stream: the host
+    waits for that stream only - a kernel and a copy - whatever the caller's stream still has
+    queued.  Returns the flags."""
+    dev = rows.device
+    with _state_lock:
+        state = _strided_state(dev)
+        if state.side is None:
+            state.side = torch.cuda.Stream(device=dev)
+        side = state.side
+    slot = _verdict_slot()
+    main = torch.cuda.current_stream(dev)
+    torch.cuda.set_stream(side)
+    try:
+        flags = torch.zeros(1, dtype=torch.int32, device=dev)
+        _check(_C.tsmi_coords_check(_stream(), _ptr(rows), rows.shape[0], _ptr(flags)))
+        _verdict_slots[slot:slot + 1].copy_(flags, non_blocking=True)
+        event = torch.cuda.Event()
+        event.record()
+    finally:
+        torch.cuda.set_stream(main)
+    event.synchronize()
+    return int(_verdict_slots[slot])
 
 
 @functools.lru_cache(maxsize=256)
@@ -452,11 +495,48 @@ def kmap_sorted(in_coords: torch.Tensor, out_coords: torch.Tensor, kernel_size, 
     in_coords = _need(in_coords, torch.int32, "coords")
     out_coords = _need(out_coords, torch.int32, "coords")
     ks, st, pd = _triple(kernel_size), _triple(stride), _triple(pad)
+    if in_coords is out_coords and _root_maps:
+        hit = _root_maps.pop((id(in_coords), ks, st, pd), None)
+        if (hit is not None and hit[0]() is in_coords and hit[1] == in_coords._version
+                and hit[2] == in_coords.data_ptr() and hit[3] == _stream()):
+            return hit[4]
     if kmap_queue_ahead:
         ahead = _map_queued_ahead(in_coords, out_coords, ks, st, pd)
         if ahead is not None:
             return ahead
+    if in_coords is out_coords and _range_origin(in_coords) == "user":
+        _root_geoms[(in_coords.device.index, _stream())] = (ks, st, pd)  # (see _queue_root_map)
     return _kmap_sorted_launch(in_coords, out_coords, ks, st, pd)
+
+
+# The submanifold map over a caller's own rows, queued while their first check is still on its
+# way.  A loop over new coordinate tensors waits for each tensor's check with the device drained,
+# and the first thing the forward then needs is this map; when the stream's last such tensor
+# had ascending rows and asked for the map, it is queued right behind the check of the next one,
+# before the host waits for the verdict: the device builds it while the host wakes up.  Rows
+# that turn out not to ascend make it a wasted launch (the search stays inside the rows whatever
+# their order; its result is dropped).
+_root_geoms = {}  # (device index, stream) -> geometry of the last map built over a caller's ascending rows
+_root_maps = {}   # (id(coords), ks, st, pd) -> (weak reference, version, address, stream, map)
+
+
+def _queue_root_map(coords: torch.Tensor) -> None:
+    stream = _stream()
+    geom = _root_geoms.get((coords.device.index, stream))
+    if geom is None or not kmap_through_sorted or coords.shape[0] == 0:
+        return
+    left = [k for k, v in _root_maps.items() if v[3] == stream]
+    if left:
+        # the map queued for the tensor before was never asked for: another network runs now;
+        # nothing is queued until a forward asks for such a map again
+        for k in left:
+            _root_maps.pop(k, None)
+        _root_geoms.pop((coords.device.index, stream), None)
+        return
+    ks, st, pd = geom
+    omap = _kmap_sorted_launch(coords, coords, ks, st, pd)
+    _remember(_root_maps, (id(coords), ks, st, pd),
+              (weakref.ref(coords), coords._version, coords.data_ptr(), stream, omap), 8)
 
 
 # The maps a network builds over the levels of its strided chain (the submanifold map of every
