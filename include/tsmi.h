@@ -547,6 +547,11 @@ int tsmi_conv_segments_supported(int kvol, int cin, int cout, int dtype);
 int tsmi_pair_segments(tsmi_stream_t s, const int32_t *map, int64_t n_rows, int kvol,
                        int64_t seg_rows, int32_t *pool, int32_t *counts, int32_t *in_rows,
                        int32_t *pos);
+/* `count` calls of tsmi_pair_segments queued by one (the segments of several maps of a network,
+ * built ahead of their layers): args is host int64[8 * count], per build [map, n_rows, kvol,
+ * seg_rows, pool, counts, in_rows, pos] with the pointers as integers.  The builds run one after
+ * the other on the stream and may share a pool. */
+int tsmi_pair_segments_batch(tsmi_stream_t s, int count, const int64_t *args);
 int tsmi_conv_implicit_gemm_segments(tsmi_stream_t s, const void *x, const void *w_packed,
                                      const int32_t *in_rows, const int32_t *counts,
                                      const int32_t *pos, int64_t seg_rows, int64_t n_out, int kvol,

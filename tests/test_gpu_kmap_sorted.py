@@ -91,23 +91,32 @@ def test_unsorted_or_repeated_rows_take_the_tables():
     assert backend.coords_ascending(dev(coords[:1])) and backend.coords_ascending(dev(coords[:0]))
 
 
-def test_rows_declared_ready_are_checked_on_the_second_stream():
-    """rows_ready(): the check of such rows runs on the device's second stream and its verdict is
-    read at once, while the caller's stream is still busy: ascending rows take the table-free
-    builder from their first map on, unsorted rows the tables, a row outside the packed range
-    raises from the call that looks at the tensor first."""
+def test_rows_declared_ready_are_checked_on_the_second_stream(monkeypatch):
+    """rows_ready(): the check of such rows is queued on the device's second stream and the host
+    waits for that stream alone (on a device whose hardware queues are not shared between the two
+    streams the verdict does not wait for what the caller's stream has queued): ascending rows
+    take the table-free builder from their first map on, unsorted rows the tables, a row outside
+    the packed range raises from the call that looks at the tensor first."""
     rng = np.random.default_rng(303)
     coords = ascending(random_coords(rng, 3000, (30, 30, 12)))
-    busy = torch.empty(1 << 30, dtype=torch.int8, device="cuda")
-    assert backend.coords_ascending(backend.rows_ready(dev(coords)))  # (the second stream exists from here on)
+    seen = []
+    real = backend._C.tsmi_coords_check
+    main = backend._stream()
+
+    class Spy:  # (the library object, with the one entry point watched)
+        def __getattr__(self, name):
+            return getattr(real_lib, name)
+
+        def tsmi_coords_check(self, stream, *args):
+            seen.append(stream)
+            return real(stream, *args)
+    real_lib = backend._C
+    monkeypatch.setattr(backend, "_C", Spy())
     t = backend.rows_ready(dev(coords))
-    torch.cuda.synchronize()
-    done = torch.cuda.Event()
-    for _ in range(50):
-        busy.fill_(1)  # (some 15 ms of work queued on the caller's stream)
-    done.record()
     assert backend.coords_ascending(t)
-    assert not done.query()  # the verdict did not wait for the caller's stream
+    state = backend._stream_states[(torch.cuda.current_device(), main)]
+    assert seen == [state.side.cuda_stream] and seen[0] != main
+    assert backend._stream() == main
     kmap = F.build_kernel_map(t, len(coords), 3, 1, 0, mode="hashmap_on_the_fly")
     assert kmap["in_hashmap"] is None  # (the table-free builder)
     np.testing.assert_array_equal(kmap["out_in_map"].cpu().numpy(), oracle.kmap_subm(coords, 3))

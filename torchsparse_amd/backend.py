@@ -109,6 +109,7 @@ def _load():
                                       _i32, _i32, _i32, _i32, _i32, _vp, _vp, _i32, _vp, _vp],
         "tsmi_conv_segments_supported": [_i32, _i32, _i32, _i32],
         "tsmi_pair_segments": [_vp, _vp, _i64, _i32, _i64, _vp, _vp, _vp, _vp],
+        "tsmi_pair_segments_batch": [_vp, _i32, _vp],
         "tsmi_conv_implicit_gemm_segments": [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i32, _i32, _i32,
                                              _i32, _vp, _vp, _i32, _vp, _vp],
         "tsmi_launch_thread_open": [],
@@ -666,7 +667,18 @@ def _launch_maps_early(state, job, coords) -> None:
                  pair_ptr + 16 * slot if counted else 0, pair_ptr + 8 * (2 * _PAIR_SLOTS + slot) if counted else 0,
                  0 if i == 0 else ctr_ptr + 32 * (i - 1), 0 if o == 0 else ctr_ptr + 32 * (o - 1))
     _check(_C.tsmi_kmap_sorted_batch(_stream(), len(todo), (ctypes.c_int64 * len(flat))(*flat)))
-    job.early = (tuple(t[0] for t in todo), todo, buffers, t_buffer, counted, transposed, bound)
+    # (what follows the launch needs no count either: off the host's hands before the counts arrive)
+    if counted:
+        if state.pair_out is None:
+            state.pair_out = state.pair_dev[2 * _PAIR_SLOTS:]
+        state.pair_host.copy_(state.pair_out, non_blocking=True)
+    main = state.main_stream
+    if main is not None:
+        for buf in buffers.values():
+            buf.record_stream(main)  # allocated on the second stream, read and freed on the caller's
+        if t_buffer is not None:
+            t_buffer.record_stream(main)
+    job.early = (tuple(t[0] for t in todo), todo, buffers, t_buffer, counted, transposed, bound, main)
 
 
 def _queue_maps_ahead(state, chain_rows, on_side: bool, job=None) -> None:
@@ -695,7 +707,7 @@ def _queue_maps_ahead(state, chain_rows, on_side: bool, job=None) -> None:
     # between the streams each
     todo, rows_of, t_ints = [], {}, 0
     if early is not None:
-        _, early_todo, buffers, t_buffer, counted, _, _ = early
+        _, early_todo, buffers, t_buffer, counted, _, _, recorded_for = early
         state.maps_early_hits += 1
         for slot, (request, kvol, first, t_first) in enumerate(early_todo):
             i, o, ks, st, pd = request
@@ -724,7 +736,12 @@ def _queue_maps_ahead(state, chain_rows, on_side: bool, job=None) -> None:
     if not todo:
         return
     dev = chain_rows[0].device
-    main = state.maps_main = torch.cuda.current_stream(dev)
+    main = state.main_stream  # (asking torch for the current stream costs 5 us)
+    if main is None or main.cuda_stream != _stream():
+        main = state.main_stream = torch.cuda.current_stream(dev)
+    state.maps_main = main
+    if early is None:
+        recorded_for = None
     torch.cuda.set_stream(state.side)  # (the context manager costs 6 us, two switches 0.8)
     try:
         if early is None:
@@ -740,10 +757,10 @@ def _queue_maps_ahead(state, chain_rows, on_side: bool, job=None) -> None:
         segment_jobs = []
         for a, b, ks, st, pd, kvol, first, t_first, with_segments, slot in todo:
             n_pad = make_divisible(b.shape[0], 128)
-            omap = buffers[kvol][first:first + n_pad]
+            omap = buffers[kvol].narrow(0, first, n_pad)
             omap_t, t_pad = None, make_divisible(a.shape[0], 128)
-            if t_first >= 0:
-                omap_t = t_buffer[t_first:t_first + t_pad * kvol].view(t_pad, kvol)
+            if t_first >= 0:  # (= t_buffer[t_first:t_first + t_pad * kvol].view(t_pad, kvol), in one call)
+                omap_t = t_buffer.as_strided((t_pad, kvol), (kvol, 1), t_buffer.storage_offset() + t_first)
             if early is None:
                 samples = _sorted_samples(a)
                 flat += (a.data_ptr(), a.shape[0], b.data_ptr(), b.shape[0], n_pad,
@@ -761,22 +778,27 @@ def _queue_maps_ahead(state, chain_rows, on_side: bool, job=None) -> None:
             _check(_C.tsmi_kmap_sorted_batch(_stream(), len(todo), (ctypes.c_int64 * len(flat))(*flat)))
         # the pair segments the forward before built over these maps, behind the maps on this
         # stream instead of in front of their first layer on the caller's
-        for omap, n_rows, kvol in segment_jobs:
-            seg = _build_pair_segments(omap, n_rows, kvol, dev)
-            seg.buffer.record_stream(main)
-            _remember(_segments_of, id(omap), (weakref.ref(omap), omap._version, omap.data_ptr(),
-                                               main.cuda_stream, n_rows, seg), 64)
-            state.segments_hits += 1
-        if counted:
-            state.pair_host.copy_(state.pair_dev[2 * _PAIR_SLOTS:], non_blocking=True)
+        if segment_jobs:
+            segs = _build_pair_segments_batch(segment_jobs, dev)
+            segs[0].buffer.record_stream(main)
+            main_handle = main.cuda_stream
+            for (omap, n_rows, kvol), seg in zip(segment_jobs, segs):
+                _remember(_segments_of, id(omap), (weakref.ref(omap), omap._version, omap.data_ptr(),
+                                                   main_handle, n_rows, seg), 64)
+            state.segments_hits += len(segs)
+        if counted and early is None:  # (counts of maps queued before the row counts are on their way already)
+            if state.pair_out is None:
+                state.pair_out = state.pair_dev[2 * _PAIR_SLOTS:]
+            state.pair_host.copy_(state.pair_out, non_blocking=True)
         event = torch.cuda.Event()
         event.record()
     finally:
         torch.cuda.set_stream(main)
-    for buf in buffers.values():
-        buf.record_stream(main)  # allocated on the second stream, read and freed on the caller's
-    if t_buffer is not None:
-        t_buffer.record_stream(main)
+    if recorded_for is None or recorded_for.cuda_stream != main.cuda_stream:
+        for buf in buffers.values():
+            buf.record_stream(main)  # allocated on the second stream, read and freed on the caller's
+        if t_buffer is not None:
+            t_buffer.record_stream(main)
     # (only now: a call that failed above leaves no map behind that was never written)
     state.maps_ahead, state.maps_event = queued, event
     if counted:
@@ -1100,7 +1122,7 @@ class _StridedState:
                  "chain_len", "ahead", "ahead_hits", "host_counters", "pending", "pending_rsv", "root_chain",
                  "lookahead_hits", "side", "grid_event", "grid_event_stream", "grid_old", "level_index", "map_plan",
                  "map_plan_seen", "maps_ahead", "maps_event", "maps_ahead_hits", "maps_main", "transposed_plan",
-                 "maps_early_hits", "level_counts",
+                 "maps_early_hits", "level_counts", "main_stream", "pair_out",
                  "transposed_seen", "transposed_hits", "pair_dev", "pair_host", "pair_event", "pair_vals", "pairs_of",
                  "segments_plan", "segments_seen", "segments_hits")
 
@@ -1130,6 +1152,8 @@ class _StridedState:
         self.maps_event = None    # end of that queue; None once the caller's stream has waited for it
         self.maps_ahead_hits = 0  # maps answered from `maps_ahead` (diagnostic)
         self.maps_early_hits = 0  # forwards whose maps were queued before the counts were read (diagnostic)
+        self.main_stream = None   # torch's object for the stream this state belongs to
+        self.pair_out = None      # the last third of pair_dev (the counts)
         self.level_counts = []    # rows of the levels of the last chain (the root's not among them)
         self.maps_main = None     # the caller's stream object at the time of that queue
         self.transposed_plan = frozenset()  # requests of map_plan whose transposed map was asked for too
@@ -1388,7 +1412,7 @@ def _grid_finish(state, job: _GridJob, rsv_ratio, cap, want_table):
     def emit(level, n_in, capacity):
         n_out = host[8 * level]
         if job.rows is not None:  # emitted before the read-back: the level is a view of its buffer
-            out = job.rows[level, :n_out]
+            out = job.rows.as_strided((n_out, 4), (4, 1), job.rows.storage_offset() + level * n * 4)  # (= rows[level, :n_out])
             tbl = None
             if want_table:
                 _mark_range_ok(out, ascending=True)  # (known: the insert below does not read a flag back)
@@ -1993,28 +2017,38 @@ class PairSegments:
     """Per-offset pair lists of a kernel map (tsmi_pair_segments), in one int32 allocation:
     ``counts`` [K_vol], ``in_rows`` [K_vol, seg_rows], ``pos`` [K_vol, n_rows] (views, made when
     asked for; the convolution works from the addresses)."""
-    __slots__ = ("buffer", "kvol", "n_rows", "seg_rows", "counts_ptr", "in_rows_ptr", "pos_ptr")
+    __slots__ = ("buffer", "first", "kvol", "n_rows", "seg_rows", "counts_ptr", "in_rows_ptr", "pos_ptr")
 
-    def __init__(self, kvol: int, n_rows: int, seg_rows: int, device):
-        self.kvol, self.n_rows, self.seg_rows = kvol, n_rows, seg_rows
+    @staticmethod
+    def elems(kvol: int, n_rows: int, seg_rows: int) -> int:
+        """int32 elements of one set of lists, rounded so that the next set in the same allocation
+        starts 256-byte aligned as well."""
+        return make_divisible(make_divisible(kvol, 64) + kvol * seg_rows + kvol * n_rows, 64)
+
+    def __init__(self, kvol: int, n_rows: int, seg_rows: int, device, buffer=None, first: int = 0):
+        """``buffer`` / ``first``: an int32 allocation shared with other sets and the element
+        this one starts at (a multiple of 64); None: an allocation of its own."""
+        self.kvol, self.n_rows, self.seg_rows, self.first = kvol, n_rows, seg_rows, first
         head = make_divisible(kvol, 64)  # keeps the two lists 256-byte aligned
-        self.buffer = torch.empty(head + kvol * seg_rows + kvol * n_rows, dtype=torch.int32, device=device)
-        self.counts_ptr = self.buffer.data_ptr()
+        if buffer is None:
+            buffer = torch.empty(head + kvol * seg_rows + kvol * n_rows, dtype=torch.int32, device=device)
+        self.buffer = buffer
+        self.counts_ptr = buffer.data_ptr() + 4 * first
         self.in_rows_ptr = self.counts_ptr + 4 * head
         self.pos_ptr = self.in_rows_ptr + 4 * kvol * seg_rows
 
     @property
     def counts(self) -> torch.Tensor:
-        return self.buffer[:self.kvol]
+        return self.buffer[self.first:self.first + self.kvol]
 
     @property
     def in_rows(self) -> torch.Tensor:
-        head = make_divisible(self.kvol, 64)
+        head = self.first + make_divisible(self.kvol, 64)
         return self.buffer[head:head + self.kvol * self.seg_rows].view(self.kvol, self.seg_rows)
 
     @property
     def pos(self) -> torch.Tensor:
-        start = make_divisible(self.kvol, 64) + self.kvol * self.seg_rows
+        start = self.first + make_divisible(self.kvol, 64) + self.kvol * self.seg_rows
         return self.buffer[start:start + self.kvol * self.n_rows].view(self.kvol, self.n_rows)
 
     def __iter__(self):  # (counts, in_rows, pos, seg_rows)
@@ -2040,6 +2074,35 @@ def _build_pair_segments(out_in_map: torch.Tensor, n_rows: int, kvol: int, dev) 
                                      pool.data_ptr() if kvol < 520 else None, seg.counts_ptr,
                                      seg.in_rows_ptr, seg.pos_ptr))
     return seg
+
+
+def _build_pair_segments_batch(jobs, dev):
+    """The segments of several maps (``jobs``: (map, rows, kernel volume)) in one allocation,
+    queued by one call on the current stream."""
+    stream = _stream()
+    sizes = [PairSegments.elems(kvol, n_rows, make_divisible(max(n_rows, 1), 128)) for _, n_rows, kvol in jobs]
+    buffer = torch.empty(sum(sizes), dtype=torch.int32, device=dev)
+    key = (dev.index, stream)
+    pool = _SEGMENT_POOLS.get(key)
+    if pool is None:
+        with _tables_lock:
+            pool = _SEGMENT_POOLS.get(key)
+            if pool is None:
+                pool = _SEGMENT_POOLS[key] = torch.zeros(520, dtype=torch.int32, device=dev)
+    if _pin_sinks:
+        _pin(pool)
+        _pin(buffer)
+    pool_ptr = pool.data_ptr()
+    segs, flat, first = [], [], 0
+    for (omap, n_rows, kvol), size in zip(jobs, sizes):
+        seg = PairSegments(kvol, n_rows, make_divisible(max(n_rows, 1), 128), dev, buffer, first)
+        first += size
+        flat += (omap.data_ptr(), n_rows, kvol, seg.seg_rows, pool_ptr if kvol < 520 else 0, seg.counts_ptr,
+                 seg.in_rows_ptr, seg.pos_ptr)
+        segs.append(seg)
+    with _scratch_lock:  # (the pool is shared by the builds of one stream)
+        _check(_C.tsmi_pair_segments_batch(stream, len(jobs), (ctypes.c_int64 * len(flat))(*flat)))
+    return segs
 
 
 def pair_segments(out_in_map: torch.Tensor, n_rows: int) -> PairSegments:

@@ -2080,6 +2080,19 @@ extern "C" int tsmi_pair_segments(tsmi_stream_t s, const int32_t *map, int64_t n
   return check_launch("tsmi_pair_segments");
 }
 
+extern "C" int tsmi_pair_segments_batch(tsmi_stream_t s, int count, const int64_t *args) {
+  TSMI_REQUIRE(count >= 0 && (count == 0 || args), "pair_segments_batch: bad arguments");
+  for (int i = 0; i < count; ++i) {
+    const int64_t *a = args + 8 * (int64_t)i;
+    TSMI_REQUIRE(a[2] >= 1 && a[2] <= kPairMaxKvol, "pair_segments_batch: bad kernel volume");
+    if (int e = tsmi_pair_segments(s, (const int32_t *)(uintptr_t)a[0], a[1], (int)a[2], a[3],
+                                   (int32_t *)(uintptr_t)a[4], (int32_t *)(uintptr_t)a[5],
+                                   (int32_t *)(uintptr_t)a[6], (int32_t *)(uintptr_t)a[7]))
+      return e;
+  }
+  return TSMI_OK;
+}
+
 // ---- rows of a 3x3x3 map grouped by the planes of the kernel they use ------------------------
 // An implicit-GEMM workgroup multiplies every kernel offset that ANY row of its tile uses; on a
 // surface scan in coordinate order four of five such products are for absent neighbours.  Rows
