@@ -900,7 +900,7 @@ def main():
         other amounts to; the library checks its range and row order - one small kernel and
         one read-back - and every kernel map is rebuilt); "resident": a new tensor every step
         that was complete before the loop and is declared so (backend.rows_ready), so its
-        check is not read back at once; "same": the same tensor every step (the check is
+        check runs on the second stream and waits for nothing the forward before has queued; "same": the same tensor every step (the check is
         remembered, the strided chain runs ahead on the second stream; the maps are rebuilt)."""
         pool = [coords.clone() for _ in range(steps + warmup)] if rows == "resident" else None
         k = [0]
