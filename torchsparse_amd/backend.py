@@ -424,6 +424,7 @@ def coords_ascending(coords: torch.Tensor) -> bool:
         strided_lookahead(coords, behind=event)
         _queue_root_map(coords)
         event.synchronize()
+        _drained[(rows.device.index, _stream())] = weakref.ref(coords)  # (nothing is queued on this stream now)
         bits = int(_verdict_slots[slot])
         if bits and _root_maps:
             for key in [k for k in _root_maps if k[0] == id(coords)]:
@@ -517,6 +518,7 @@ def kmap_sorted(in_coords: torch.Tensor, out_coords: torch.Tensor, kernel_size, 
 # before the host waits for the verdict: the device builds it while the host wakes up.  Rows
 # that turn out not to ascend make it a wasted launch (the search stays inside the rows whatever
 # their order; its result is dropped).
+_drained = {}     # (device index, stream) -> weak reference to the tensor whose check the host last waited for there
 _root_geoms = {}  # (device index, stream) -> geometry of the last map built over a caller's ascending rows
 _root_maps = {}   # (id(coords), ks, st, pd) -> (weak reference, version, address, stream, map)
 
@@ -616,6 +618,9 @@ def _map_queued_ahead(in_coords, out_coords, ks, st, pd) -> Optional[torch.Tenso
 # hides that start-up, the first strided layer finds its map ~0.15 ms earlier.  Only for roots of
 # at most 131,072 rows (larger inputs search through samples gathered per input).
 kmap_queue_before_counts = True
+# A forward that starts with the device drained hands its maps out without the second stream's
+# event traffic (see _queue_maps_ahead).
+kmap_register_on_drained_stream = True
 _EARLY_MAX_ROWS = 131072
 
 
@@ -672,13 +677,15 @@ def _launch_maps_early(state, job, coords) -> None:
         if state.pair_out is None:
             state.pair_out = state.pair_dev[2 * _PAIR_SLOTS:]
         state.pair_host.copy_(state.pair_out, non_blocking=True)
+    event = torch.cuda.Event()
+    event.record()
     main = state.main_stream
     if main is not None:
         for buf in buffers.values():
             buf.record_stream(main)  # allocated on the second stream, read and freed on the caller's
         if t_buffer is not None:
             t_buffer.record_stream(main)
-    job.early = (tuple(t[0] for t in todo), todo, buffers, t_buffer, counted, transposed, bound, main)
+    job.early = (tuple(t[0] for t in todo), todo, buffers, t_buffer, counted, transposed, bound, main, event)
 
 
 def _queue_maps_ahead(state, chain_rows, on_side: bool, job=None) -> None:
@@ -695,8 +702,16 @@ def _queue_maps_ahead(state, chain_rows, on_side: bool, job=None) -> None:
     state.maps_ahead = {}
     state.maps_event = None
     state.pairs_of, state.pair_event, state.pair_vals = {}, None, None
+
+    def behind_rows():
+        # (_grid_finish left the caller's stream in front of the launch that emitted the rows)
+        if job is not None and job.rows_wait_deferred:
+            job.rows_wait_deferred = False
+            if job.rows_event is not None and not job.rows_event.query():
+                torch.cuda.current_stream(chain_rows[0].device).wait_event(job.rows_event)
+
     if not (kmap_queue_ahead and on_side and plan and state.side is not None and kmap_through_sorted):
-        return
+        return behind_rows()
     early = getattr(job, "early", None)
     if early is not None and (early[0] != tuple(r for r in plan if 0 < max(r[0], r[1]) <= job.levels)
                               or any((r in early[5]) != (r in state.transposed_plan) for r in early[0])):
@@ -707,7 +722,7 @@ def _queue_maps_ahead(state, chain_rows, on_side: bool, job=None) -> None:
     # between the streams each
     todo, rows_of, t_ints = [], {}, 0
     if early is not None:
-        _, early_todo, buffers, t_buffer, counted, _, _, recorded_for = early
+        _, early_todo, buffers, t_buffer, counted, _, _, recorded_for, early_event = early
         state.maps_early_hits += 1
         for slot, (request, kvol, first, t_first) in enumerate(early_todo):
             i, o, ks, st, pd = request
@@ -734,7 +749,7 @@ def _queue_maps_ahead(state, chain_rows, on_side: bool, job=None) -> None:
             with_segments = request in state.segments_plan
             todo.append((a, b, ks, st, pd, kvol, first, t_first, with_segments, len(todo)))
     if not todo:
-        return
+        return behind_rows()
     dev = chain_rows[0].device
     main = state.main_stream  # (asking torch for the current stream costs 5 us)
     if main is None or main.cuda_stream != _stream():
@@ -742,7 +757,21 @@ def _queue_maps_ahead(state, chain_rows, on_side: bool, job=None) -> None:
     state.maps_main = main
     if early is None:
         recorded_for = None
-    torch.cuda.set_stream(state.side)  # (the context manager costs 6 us, two switches 0.8)
+    # A forward that began with the device drained (the read-back of a new tensor's check) has the
+    # device waiting for the host here: nothing is to be gained from the second stream, and an event
+    # record plus the wait for it at the first map cost the host 30 us.  The pair segments then go
+    # to the caller's stream, behind the maps, which were queued before the row counts arrived.
+    drained = False
+    if early is not None and _drained:
+        hit = _drained.pop((dev.index, main.cuda_stream), None)
+        drained = kmap_register_on_drained_stream and hit is not None and hit() is chain_rows[0]
+    if drained:
+        if not early_event.query():
+            main.wait_event(early_event)
+        job.rows_wait_deferred = False  # (the maps were queued behind the rows)
+    else:
+        behind_rows()
+        torch.cuda.set_stream(state.side)  # (the context manager costs 6 us, two switches 0.8)
     try:
         if early is None:
             buffers = {kvol: torch.empty((rows, kvol), dtype=torch.int32, device=dev) for kvol, rows in rows_of.items()}
@@ -780,7 +809,8 @@ def _queue_maps_ahead(state, chain_rows, on_side: bool, job=None) -> None:
         # stream instead of in front of their first layer on the caller's
         if segment_jobs:
             segs = _build_pair_segments_batch(segment_jobs, dev)
-            segs[0].buffer.record_stream(main)
+            if not drained:
+                segs[0].buffer.record_stream(main)
             main_handle = main.cuda_stream
             for (omap, n_rows, kvol), seg in zip(segment_jobs, segs):
                 _remember(_segments_of, id(omap), (weakref.ref(omap), omap._version, omap.data_ptr(),
@@ -790,10 +820,14 @@ def _queue_maps_ahead(state, chain_rows, on_side: bool, job=None) -> None:
             if state.pair_out is None:
                 state.pair_out = state.pair_dev[2 * _PAIR_SLOTS:]
             state.pair_host.copy_(state.pair_out, non_blocking=True)
-        event = torch.cuda.Event()
-        event.record()
+        if drained:
+            event = None  # (the caller's stream is behind the maps already)
+        else:
+            event = torch.cuda.Event()
+            event.record()
     finally:
-        torch.cuda.set_stream(main)
+        if not drained:
+            torch.cuda.set_stream(main)
     if recorded_for is None or recorded_for.cuda_stream != main.cuda_stream:
         for buf in buffers.values():
             buf.record_stream(main)  # allocated on the second stream, read and freed on the caller's
@@ -802,7 +836,7 @@ def _queue_maps_ahead(state, chain_rows, on_side: bool, job=None) -> None:
     # (only now: a call that failed above leaves no map behind that was never written)
     state.maps_ahead, state.maps_event = queued, event
     if counted:
-        state.pairs_of, state.pair_event = pairs_of, event
+        state.pairs_of, state.pair_event = pairs_of, early_event if drained else event
 
 
 def _kmap_sorted_launch(in_coords, out_coords, ks, st, pd, omap=None) -> torch.Tensor:
@@ -1252,7 +1286,7 @@ class _GridJob:
     marks and counts of every level queued, the counters on their way to pinned host memory —
     whose second half (emit) needs the counts on the host."""
     __slots__ = ("coords", "geom", "coords_max_host", "fan", "levels", "ctr", "host", "event", "stream", "rows",
-                 "early", "rows_event")
+                 "early", "rows_event", "rows_wait_deferred")
 
 
 def _strided_fan(ks, st) -> int:
@@ -1309,6 +1343,7 @@ def _grid_start(state, coords, ks, st, pd, coords_max_host, fan, ahead, early=Fa
                 part(level, "chunks"), part(level, "counters"), part(level + 1, "in_max")))
     job = _GridJob()
     job.early = job.rows_event = None
+    job.rows_wait_deferred = False
     job.rows = rows
     job.coords, job.geom, job.coords_max_host, job.fan = coords, (ks, st, pd), coords_max_host, fan
     job.levels, job.ctr, job.stream = levels, ctr, s
@@ -1395,7 +1430,11 @@ def _grid_finish(state, job: _GridJob, rsv_ratio, cap, want_table):
         host = job.host.tolist()
         # the rows were emitted behind the counters' copy: a launch or two that the caller's stream,
         # if it is another one, has to be behind as well (usually they are over by now)
-        if job.rows_event is not None and s != _stream() and not job.rows_event.query():
+        # (not where the maps queued behind the rows are about to be waited for: _queue_maps_ahead, drained)
+        hit = _drained.get((dev.index, _stream())) if job.early is not None and _drained else None
+        if hit is not None and hit() is coords and kmap_register_on_drained_stream and levels > 1:
+            job.rows_wait_deferred = True
+        elif job.rows_event is not None and s != _stream() and not job.rows_event.query():
             torch.cuda.current_stream(dev).wait_event(job.rows_event)
     else:
         host = ctr.tolist()
