@@ -606,6 +606,13 @@ def _map_queued_ahead(in_coords, out_coords, ks, st, pd) -> Optional[torch.Tenso
             state.maps_event = None
         state.maps_ahead_hits += 1
         _remember(_map_requests, id(hit[2]), (weakref.ref(hit[2]), state, request, hit[4]), 64)
+        if state.segments_todo is not None and any(j[0] is hit[2] for j in state.segments_todo):
+            jobs, state.segments_todo = state.segments_todo, None
+            main_handle = _stream()
+            for (omap, n_rows, kvol), seg in zip(jobs, _build_pair_segments_batch(jobs, hit[2].device)):
+                _remember(_segments_of, id(omap), (weakref.ref(omap), omap._version, omap.data_ptr(),
+                                                   main_handle, n_rows, seg), 64)
+            state.segments_hits += len(jobs)
         return hit[2]
 
 
@@ -701,6 +708,7 @@ def _queue_maps_ahead(state, chain_rows, on_side: bool, job=None) -> None:
     state.segments_plan, state.segments_seen = frozenset(state.segments_seen), set()
     state.maps_ahead = {}
     state.maps_event = None
+    state.segments_todo = None
     state.pairs_of, state.pair_event, state.pair_vals = {}, None, None
 
     def behind_rows():
@@ -766,9 +774,7 @@ def _queue_maps_ahead(state, chain_rows, on_side: bool, job=None) -> None:
         hit = _drained.pop((dev.index, main.cuda_stream), None)
         drained = kmap_register_on_drained_stream and hit is not None and hit() is chain_rows[0]
     if drained:
-        if not early_event.query():
-            main.wait_event(early_event)
-        job.rows_wait_deferred = False  # (the maps were queued behind the rows)
+        job.rows_wait_deferred = False  # (the maps were queued behind the rows: whoever takes one waits for both)
     else:
         behind_rows()
         torch.cuda.set_stream(state.side)  # (the context manager costs 6 us, two switches 0.8)
@@ -788,13 +794,13 @@ def _queue_maps_ahead(state, chain_rows, on_side: bool, job=None) -> None:
             n_pad = make_divisible(b.shape[0], 128)
             omap = buffers[kvol].narrow(0, first, n_pad)
             omap_t, t_pad = None, make_divisible(a.shape[0], 128)
-            if t_first >= 0:  # (= t_buffer[t_first:t_first + t_pad * kvol].view(t_pad, kvol), in one call)
-                omap_t = t_buffer.as_strided((t_pad, kvol), (kvol, 1), t_buffer.storage_offset() + t_first)
+            if t_first >= 0:  # (where the transposed map lies: the view is cut when a layer asks for it)
+                omap_t = (t_buffer, t_first, t_pad, kvol)
             if early is None:
                 samples = _sorted_samples(a)
                 flat += (a.data_ptr(), a.shape[0], b.data_ptr(), b.shape[0], n_pad,
                          0 if samples is None else samples.data_ptr(), omap.data_ptr(), *ks, *st, *pd,
-                         0 if omap_t is None else omap_t.data_ptr(), t_pad,
+                         0 if omap_t is None else t_buffer.data_ptr() + 4 * t_first, t_pad,
                          pair_ptr + 16 * slot if counted else 0,
                          pair_ptr + 8 * (2 * _PAIR_SLOTS + slot) if counted else 0, 0, 0)
             queued[(id(a), id(b), ks, st, pd)] = (weakref.ref(a), weakref.ref(b), omap, (a._version, b._version),
@@ -807,10 +813,13 @@ def _queue_maps_ahead(state, chain_rows, on_side: bool, job=None) -> None:
             _check(_C.tsmi_kmap_sorted_batch(_stream(), len(todo), (ctypes.c_int64 * len(flat))(*flat)))
         # the pair segments the forward before built over these maps, behind the maps on this
         # stream instead of in front of their first layer on the caller's
+        if segment_jobs and drained:
+            # (on the caller's stream, which is not behind the maps yet: queued when the first of
+            # these maps is taken - the first map taken at all has waited for them by then)
+            state.segments_todo, segment_jobs = segment_jobs, None
         if segment_jobs:
             segs = _build_pair_segments_batch(segment_jobs, dev)
-            if not drained:
-                segs[0].buffer.record_stream(main)
+            segs[0].buffer.record_stream(main)
             main_handle = main.cuda_stream
             for (omap, n_rows, kvol), seg in zip(segment_jobs, segs):
                 _remember(_segments_of, id(omap), (weakref.ref(omap), omap._version, omap.data_ptr(),
@@ -821,7 +830,7 @@ def _queue_maps_ahead(state, chain_rows, on_side: bool, job=None) -> None:
                 state.pair_out = state.pair_dev[2 * _PAIR_SLOTS:]
             state.pair_host.copy_(state.pair_out, non_blocking=True)
         if drained:
-            event = None  # (the caller's stream is behind the maps already)
+            event = early_event
         else:
             event = torch.cuda.Event()
             event.record()
@@ -836,7 +845,7 @@ def _queue_maps_ahead(state, chain_rows, on_side: bool, job=None) -> None:
     # (only now: a call that failed above leaves no map behind that was never written)
     state.maps_ahead, state.maps_event = queued, event
     if counted:
-        state.pairs_of, state.pair_event = pairs_of, early_event if drained else event
+        state.pairs_of, state.pair_event = pairs_of, event
 
 
 def _kmap_sorted_launch(in_coords, out_coords, ks, st, pd, omap=None) -> torch.Tensor:
@@ -1156,7 +1165,7 @@ class _StridedState:
                  "chain_len", "ahead", "ahead_hits", "host_counters", "pending", "pending_rsv", "root_chain",
                  "lookahead_hits", "side", "grid_event", "grid_event_stream", "grid_old", "level_index", "map_plan",
                  "map_plan_seen", "maps_ahead", "maps_event", "maps_ahead_hits", "maps_main", "transposed_plan",
-                 "maps_early_hits", "level_counts", "main_stream", "pair_out",
+                 "maps_early_hits", "level_counts", "main_stream", "pair_out", "segments_todo",
                  "transposed_seen", "transposed_hits", "pair_dev", "pair_host", "pair_event", "pair_vals", "pairs_of",
                  "segments_plan", "segments_seen", "segments_hits")
 
@@ -1188,6 +1197,7 @@ class _StridedState:
         self.maps_early_hits = 0  # forwards whose maps were queued before the counts were read (diagnostic)
         self.main_stream = None   # torch's object for the stream this state belongs to
         self.pair_out = None      # the last third of pair_dev (the counts)
+        self.segments_todo = None  # pair-segment builds left for the first take of one of their maps
         self.level_counts = []    # rows of the levels of the last chain (the root's not among them)
         self.maps_main = None     # the caller's stream object at the time of that queue
         self.transposed_plan = frozenset()  # requests of map_plan whose transposed map was asked for too
@@ -1635,10 +1645,12 @@ def convert_transposed_out_in_map(out_in_map: torch.Tensor, n_rows_t: int, n_row
         # one too; this forward's did if the forward before asked
         hit[1].transposed_seen.add(hit[2])
         ready = hit[3]
-        if ready is not None and ready.shape[0] == n_rows_t:
+        if ready is not None and ready[2] == n_rows_t:
             _map_requests[id(out_in_map)] = hit[:3] + (None,)
             hit[1].transposed_hits += 1
-            return ready
+            t_buffer, t_first, t_pad, kvol = ready
+            # (= t_buffer[t_first:t_first + t_pad * kvol].view(t_pad, kvol), in one call)
+            return t_buffer.as_strided((t_pad, kvol), (kvol, 1), t_buffer.storage_offset() + t_first)
     map_t = out_in_map.new_empty(n_rows_t, kvol)
     _check(_C.tsmi_transpose_map(_stream(), _ptr(out_in_map), n_rows, kvol, _ptr(map_t), n_rows_t))
     return map_t
