@@ -1428,13 +1428,14 @@ def _grid_finish(state, job: _GridJob, rsv_ratio, cap, want_table):
     fan, levels, ctr = job.fan, job.levels, job.ctr
     n = coords.shape[0]
     dev = coords.device
-    buf = state.grid_buf
-    layout, _ = _grid_layout(state.grid_words)
     s = job.stream
-    g = (_i3(ks), _i3(st), _i3(pd))
-    host_max = _I3(*[int(v) for v in job.coords_max_host]) if job.coords_max_host is not None else None
-    buf_ptr, ctr_ptr = buf.data_ptr(), ctr.data_ptr()
-    part = lambda level, what: _grid_part(buf_ptr, ctr_ptr, layout, levels, level, what)  # noqa: E731
+    if job.rows is None:  # (what the emit launches below take; rows emitted already need none of it)
+        buf = state.grid_buf
+        layout, _ = _grid_layout(state.grid_words)
+        g = (_i3(ks), _i3(st), _i3(pd))
+        host_max = _I3(*[int(v) for v in job.coords_max_host]) if job.coords_max_host is not None else None
+        buf_ptr, ctr_ptr = buf.data_ptr(), ctr.data_ptr()
+        part = lambda level, what: _grid_part(buf_ptr, ctr_ptr, layout, levels, level, what)  # noqa: E731
     if job.event is not None:
         job.event.synchronize()
         host = job.host.tolist()
@@ -1511,8 +1512,9 @@ def _grid_finish(state, job: _GridJob, rsv_ratio, cap, want_table):
         if thin:
             _note_level(nxt[0], n_in)
         # the later levels are not flagged on the device; their inputs' maxima are on the host
-        if (host[8 * level + 4] < BATCH_LIMIT and
-                all(host[8 * level + 5 + a] + 2 * pd[a] < COORD_LIMIT for a in range(3))):
+        h = 8 * level
+        if (host[h + 4] < BATCH_LIMIT and host[h + 5] + 2 * pd[0] < COORD_LIMIT
+                and host[h + 6] + 2 * pd[1] < COORD_LIMIT and host[h + 7] + 2 * pd[2] < COORD_LIMIT):
             _mark_range_ok(nxt[0], ascending=True)
         prev = nxt[0]
     # rows emitted before the read-back cleared every bitmap they read, asked for or not
