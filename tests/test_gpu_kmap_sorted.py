@@ -487,3 +487,39 @@ def test_root_map_queued_before_the_verdict_of_a_new_tensor(monkeypatch):
     assert backend.coords_ascending(t2) and len(launches) == 1
     assert not backend._root_maps and not backend._root_geoms
     torch.cuda.synchronize()
+
+
+def test_root_map_of_rows_known_to_be_complete_is_built_on_the_second_stream(monkeypatch):
+    """Once a network's strided chain is queued ahead on the second stream (the rows are known to be
+    complete: declared so, or checked before), the submanifold map over the rows themselves is
+    launched there too, in front of the chain, and the layer that asks for it takes it from there:
+    the oracle's map, one launch per tensor, on the second stream."""
+    rng = np.random.default_rng(99)
+    base = ascending(lidar_like_coords(rng, 20000))
+    want = oracle.kmap_subm(base, 3)
+    want_down, level2 = oracle.kmap_downsample(base, 2, 2, 0)
+    launches = []
+    real = backend._kmap_sorted_launch
+    monkeypatch.setattr(backend, "_kmap_sorted_launch",
+                        lambda *a, **k: (launches.append((a[0] is a[1], backend._stream())), real(*a, **k))[1])
+    backend.release_scratch()
+    backend._root_geoms.clear()
+    backend._root_maps.clear()
+    main = backend._stream()
+    for turn in range(5):
+        t = backend.rows_ready(dev(base))
+        launches.clear()
+        subm = F.build_kernel_map(t, len(base), (3, 3, 3), 1, 0, mode="hashmap_on_the_fly")
+        down = F.build_kernel_map(t, len(base), (2, 2, 2), 2, 0, mode="hashmap_on_the_fly")
+        down2 = F.build_kernel_map(down["coords"], len(level2), (2, 2, 2), 2, 0, mode="hashmap_on_the_fly")
+        np.testing.assert_array_equal(subm["out_in_map"].cpu().numpy(), want)
+        np.testing.assert_array_equal(down["out_in_map"].cpu().numpy(), want_down)
+        np.testing.assert_array_equal(down["coords"].cpu().numpy(), level2)
+        assert down2["out_in_map"].shape[1] == 8
+        roots = [s for is_root, s in launches if is_root]
+        assert len(roots) == 1
+        state = backend._stream_states[(torch.cuda.current_device(), main)]
+        if state.lookahead_hits:  # the chain of this tensor was queued at its submanifold build
+            assert state.side is not None and roots[0] == state.side.cuda_stream
+    assert state.lookahead_hits >= 2 and not backend._root_maps
+    torch.cuda.synchronize()
