@@ -623,6 +623,7 @@ def _map_queued_ahead(in_coords, out_coords, ks, st, pd) -> Optional[torch.Tenso
                 _remember(_segments_of, id(omap), (weakref.ref(omap), omap._version, omap.data_ptr(),
                                                    main_handle, n_rows, seg), 64)
             state.segments_hits += len(jobs)
+            state.segments_ids = tuple(id(j[0]) for j in jobs)
         return hit[2]
 
 
@@ -723,6 +724,13 @@ def _queue_maps_ahead(state, chain_rows, on_side: bool, job=None) -> None:
     state.maps_ahead = {}
     state.maps_event = None
     state.segments_todo = None
+    if state.segments_ids:
+        # (the segments built ahead for the forward before, over maps that are gone: up to 20 MB a forward)
+        for key in state.segments_ids:
+            hit = _segments_of.get(key)
+            if hit is not None and hit[0]() is None:
+                _segments_of.pop(key, None)
+        state.segments_ids = ()
     state.pairs_of, state.pair_event, state.pair_vals = {}, None, None
 
     def behind_rows():
@@ -839,6 +847,7 @@ def _queue_maps_ahead(state, chain_rows, on_side: bool, job=None) -> None:
                 _remember(_segments_of, id(omap), (weakref.ref(omap), omap._version, omap.data_ptr(),
                                                    main_handle, n_rows, seg), 64)
             state.segments_hits += len(segs)
+            state.segments_ids = tuple(id(j[0]) for j in segment_jobs)
         if counted and early is None:  # (counts of maps queued before the row counts are on their way already)
             if state.pair_out is None:
                 state.pair_out = state.pair_dev[2 * _PAIR_SLOTS:]
@@ -1179,7 +1188,7 @@ class _StridedState:
                  "chain_len", "ahead", "ahead_hits", "host_counters", "pending", "pending_rsv", "root_chain",
                  "lookahead_hits", "side", "grid_event", "grid_event_stream", "grid_old", "level_index", "map_plan",
                  "map_plan_seen", "maps_ahead", "maps_event", "maps_ahead_hits", "maps_main", "transposed_plan",
-                 "maps_early_hits", "level_counts", "main_stream", "pair_out", "segments_todo",
+                 "maps_early_hits", "level_counts", "main_stream", "pair_out", "segments_todo", "segments_ids",
                  "transposed_seen", "transposed_hits", "pair_dev", "pair_host", "pair_event", "pair_vals", "pairs_of",
                  "segments_plan", "segments_seen", "segments_hits")
 
@@ -1212,6 +1221,7 @@ class _StridedState:
         self.main_stream = None   # torch's object for the stream this state belongs to
         self.pair_out = None      # the last third of pair_dev (the counts)
         self.segments_todo = None  # pair-segment builds left for the first take of one of their maps
+        self.segments_ids = ()     # ids of the maps whose segments were built ahead last
         self.level_counts = []    # rows of the levels of the last chain (the root's not among them)
         self.maps_main = None     # the caller's stream object at the time of that queue
         self.transposed_plan = frozenset()  # requests of map_plan whose transposed map was asked for too
