@@ -279,6 +279,7 @@ coords_check_overlap = True
 _rows_ready = {}  # id(tensor) -> (weak reference, version, address)
 _pending_verdicts = []  # (weak reference, version, address, pinned slot, event)
 _verdict_slots = None   # pinned int32 ring the verdicts are copied into
+_verdict_host = None    # ... as a numpy array over the same memory (an element read costs 0.2 us against 3)
 _verdict_next = 0
 _VERDICT_SLOTS = 64
 # Kernel maps of ascending inputs are built by binary search over the coordinates themselves
@@ -357,7 +358,7 @@ def settle_checks(block: bool = True) -> None:
             continue
         if block:
             event.synchronize()
-        bits = int(_verdict_slots[slot])
+        bits = int(_verdict_host[slot])
         t = ref()
         if bits & 2:
             bad = True
@@ -425,7 +426,7 @@ def coords_ascending(coords: torch.Tensor) -> bool:
         _queue_root_map(coords)
         event.synchronize()
         _drained[(rows.device.index, _stream())] = weakref.ref(coords)  # (nothing is queued on this stream now)
-        bits = int(_verdict_slots[slot])
+        bits = int(_verdict_host[slot])
         if bits and _root_maps:
             for key in [k for k in _root_maps if k[0] == id(coords)]:
                 _root_maps.pop(key, None)  # (searched over rows that do not ascend)
@@ -445,9 +446,10 @@ def _verdict(coords: torch.Tensor, bits: int) -> bool:
 
 def _verdict_slot() -> int:
     """A free element of the pinned ring the verdicts are copied into."""
-    global _verdict_slots, _verdict_next
+    global _verdict_slots, _verdict_next, _verdict_host
     if _verdict_slots is None:
         _verdict_slots = torch.zeros(_VERDICT_SLOTS, dtype=torch.int32, pin_memory=True)
+        _verdict_host = _verdict_slots.numpy()
     if len(_pending_verdicts) >= _VERDICT_SLOTS - 1:
         settle_checks(block=True)  # (every slot is on its way: wait for them)
     slot = _verdict_next
@@ -479,7 +481,7 @@ def _check_aside(rows: torch.Tensor) -> int:
     finally:
         torch.cuda.set_stream(main)
     event.synchronize()
-    return int(_verdict_slots[slot])
+    return int(_verdict_host[slot])
 
 
 @functools.lru_cache(maxsize=256)
