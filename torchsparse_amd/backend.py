@@ -797,10 +797,8 @@ def _queue_maps_ahead(state, chain_rows, on_side: bool, job=None) -> None:
     if early is not None and _drained:
         hit = _drained.pop((dev.index, main.cuda_stream), None)
         drained = kmap_register_on_drained_stream and hit is not None and hit() is chain_rows[0]
-    if drained:
-        job.rows_wait_deferred = False  # (the maps were queued behind the rows: whoever takes one waits for both)
-    else:
-        behind_rows()
+    behind_rows()  # (by now a query of the event that finds it complete)
+    if not drained:
         torch.cuda.set_stream(state.side)  # (the context manager costs 6 us, two switches 0.8)
     try:
         if early is None:
