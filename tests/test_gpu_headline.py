@@ -415,3 +415,44 @@ def test_minkunet_over_alternating_scans(mods, scan):
     # maps queued once the counts are there
     assert sizes["A"][1] > sizes["B"][1] + sizes["B"][1] // 8 + 1024, sizes
     assert state.maps_early_hits == 4, state.maps_early_hits
+
+
+def test_minkunet_over_small_clouds_of_changing_size(mods):
+    """The look-ahead machinery (chain on the second stream, maps queued with the row counts still
+    on the device and room for an eighth more rows than the forward before) over clouds of a few
+    hundred voxels whose sizes jump up and down from one forward to the next, several batches among
+    them: every forward's nine maps and five levels bit for bit the oracle's, every output that of
+    the same cloud when it was first seen (to 2e-3 of its RMS: the form a wide layer takes may differ)."""
+    ts, backend, spnn, F = mods
+    from torchsparse_amd.backbones import SparseResUNet42
+    from torchsparse_amd.nn.utils import fuse_inference
+    from helpers import random_coords
+    rng = np.random.default_rng(21)
+
+    def cloud(n, shape, batch):
+        c = random_coords(rng, n, shape, batch)
+        return c[np.lexsort((c[:, 3], c[:, 2], c[:, 1], c[:, 0]))]
+    clouds = [cloud(300, (64, 64, 32), 1), cloud(2500, (96, 96, 32), 2), cloud(120, (48, 48, 32), 1),
+              cloud(4000, (128, 96, 48), 3)]
+    tables = [_scan_tables(c) for c in clouds]
+    assert all(t["levels"][16].shape[0] > 0 for t in tables)
+    torch.manual_seed(8)
+    model = fuse_inference(SparseResUNet42(in_channels=4).eval().cuda().half())
+    feats = [torch.randn(len(c), 4, device="cuda", dtype=torch.float16) for c in clouds]
+    backend.release_scratch()
+    first = {}
+    for turn, k in enumerate([0, 0, 0, 1, 1, 2, 3, 3, 0, 2, 1, 3]):
+        with torch.no_grad():
+            x = ts.SparseTensor(feats[k], torch.from_numpy(clouds[k]).cuda())
+            outs = model(x)
+        _check_maps(x._caches, outs, tables[k])
+        got = _f32(outs[-1].feats)
+        if k in first:
+            # (not bit for bit: once a map's pairs have been counted - from the third forward on - a
+            # wide layer may take the other of its two forms, which rounds its sums differently)
+            assert rel_rms(got, first[k]) < 2e-3, (turn, k)
+        else:
+            first[k] = got
+    state, = backend._stream_states.values()
+    assert state.maps_early_hits >= 4, state.maps_early_hits  # (forwards whose levels fit the room given)
+    torch.cuda.synchronize()
