@@ -291,3 +291,43 @@ def test_detection_backbone_every_layer_against_the_oracle(mods):
     assert len(maps) == 8  # four submanifold maps (levels 1, 2, 4, 8) and the four strided ones
     assert outs["out"].coords.shape[0] == maps[((8, 8, 8), (3, 1, 1), (2, 1, 1))][1].shape[0]
     print(f"{n} voxels, worst layer {worst:.2e}")
+
+
+def test_two_networks_alternating_on_one_stream():
+    """A U-Net and a detection backbone take turns on one stream, each forward over a new coordinate
+    tensor: what the library learnt from one network (its strided chain, the maps it asks for, the
+    map over the caller's rows queued ahead of the check's verdict) must not reach the other's
+    results.  Every output bit for bit the one the same network gave on its first forward."""
+    import torchsparse_amd as ts
+    from torchsparse_amd import backend
+    from torchsparse_amd.backbones import SparseResUNet42, VoxelResBackBone8x
+    from torchsparse_amd.nn.utils import fuse_inference
+    from torchsparse_amd.utils import synthetic
+    torch.manual_seed(0)
+    rows_u = synthetic.lidar_scan_voxels(seed=1)
+    rows_d, range_d = synthetic.multisweep_voxels(seed=2)
+    rows_d = rows_d[:120000]
+    rows_d = rows_d[np.lexsort((rows_d[:, 3], rows_d[:, 2], rows_d[:, 1], rows_d[:, 0]))]
+    unet = fuse_inference(SparseResUNet42(in_channels=4).eval().cuda().half())
+    det = fuse_inference(VoxelResBackBone8x(in_channels=5).eval().cuda().half())
+    feats_u = torch.randn(len(rows_u), 4, device="cuda", dtype=torch.float16)
+    feats_d = torch.randn(len(rows_d), 5, device="cuda", dtype=torch.float16)
+
+    def run(kind):
+        with torch.no_grad():
+            if kind == "U":
+                return unet(ts.SparseTensor(feats_u, torch.from_numpy(rows_u).cuda()))[-1].feats.clone()
+            out = det(ts.SparseTensor(feats_d, torch.from_numpy(rows_d).cuda(), spatial_range=range_d))
+            return out["out"].feats.clone()
+
+    backend.release_scratch()
+    first = {}
+    for turn, kind in enumerate("UUUDDDUDUDDUUUDU"):
+        got = run(kind)
+        if kind in first:
+            assert torch.equal(got, first[kind]), (turn, kind)
+        else:
+            first[kind] = got
+    state, = backend._stream_states.values()
+    assert state.lookahead_hits >= 2  # (the U-Net's chain was queued ahead again after the other network's turns)
+    torch.cuda.synchronize()
