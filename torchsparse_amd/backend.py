@@ -402,6 +402,17 @@ def coords_ascending(coords: torch.Tensor) -> bool:
     rows = _need(coords, torch.int32, "coords")
     if coords_check_aside and rows is coords and _declared_ready(coords):
         return _verdict(coords, _check_aside(rows))
+    overlap = coords_check_overlap and rows is coords and not _declared_ready(coords)
+    if overlap:
+        # The read-back below waits for everything the stream has queued - the whole forward
+        # before, in a loop over new tensors - and until it returns the device gets nothing new.
+        # What does not depend on the verdict is therefore queued first: the strided chain that
+        # followed rows like these last time (any order of rows will do for it, and rows it cannot
+        # take are flagged, not followed), on the second stream, behind this point of the caller's
+        # stream - in front of the check, which the chain does not need.
+        ready = torch.cuda.Event()
+        ready.record()
+        strided_lookahead(coords, behind=ready)
     flags = torch.zeros(1, dtype=torch.int32, device=rows.device)
     _check(_C.tsmi_coords_check(_stream(), _ptr(rows), rows.shape[0], _ptr(flags)))
     if coords_check_deferred and rows is coords and _declared_ready(coords):
@@ -412,18 +423,12 @@ def coords_ascending(coords: torch.Tensor) -> bool:
         _pending_verdicts.append((weakref.ref(coords), coords._version, coords.data_ptr(), slot, event))
         _mark_range_ok(coords, ascending=False, origin="user")  # (complete: the caller said so)
         return False
-    elif coords_check_overlap and rows is coords:
-        # The read-back below waits for everything the stream has queued - the whole forward
-        # before, in a loop over new tensors - and until it returns the device gets nothing new.
-        # What does not depend on the verdict is therefore queued first: the strided chain that
-        # followed rows like these last time (any order of rows will do for it, and rows it cannot
-        # take are flagged, not followed), on the second stream behind the check.
+    elif overlap:
         slot = _verdict_slot()
         _verdict_slots[slot:slot + 1].copy_(flags, non_blocking=True)
         event = torch.cuda.Event()
         event.record()
-        strided_lookahead(coords, behind=event)
-        _queue_root_map(coords)
+        _queue_root_map(coords)  # (taken or dropped with the verdict)
         event.synchronize()
         _drained[(rows.device.index, _stream())] = weakref.ref(coords)  # (nothing is queued on this stream now)
         bits = int(_verdict_host[slot])
