@@ -433,8 +433,9 @@ def coords_ascending(coords: torch.Tensor) -> bool:
         _drained[(rows.device.index, _stream())] = weakref.ref(coords)  # (nothing is queued on this stream now)
         bits = int(_verdict_host[slot])
         if bits and _root_maps:
-            for key in [k for k in _root_maps if k[0] == id(coords)]:
-                _root_maps.pop(key, None)  # (searched over rows that do not ascend)
+            with _tables_lock:
+                for key in [k for k in _root_maps if k[0] == id(coords)]:
+                    _root_maps.pop(key, None)  # (searched over rows that do not ascend)
             if bits & 1:
                 _root_geoms.pop((coords.device.index, _stream()), None)
     else:
@@ -540,12 +541,13 @@ def _queue_root_map(coords: torch.Tensor, main=None) -> None:
     geom = _root_geoms.get((coords.device.index, stream))
     if geom is None or not kmap_through_sorted or coords.shape[0] == 0:
         return
-    left = [k for k, v in _root_maps.items() if v[3] == stream]
+    with _tables_lock:  # (another host thread may be adding its own)
+        left = [k for k, v in _root_maps.items() if v[3] == stream]
+        for k in left:
+            _root_maps.pop(k, None)
     if left:
         # the map queued for the tensor before was never asked for: another network runs now;
         # nothing is queued until a forward asks for such a map again
-        for k in left:
-            _root_maps.pop(k, None)
         _root_geoms.pop((coords.device.index, stream), None)
         return
     ks, st, pd = geom
