@@ -456,3 +456,53 @@ def test_minkunet_over_small_clouds_of_changing_size(mods):
     state, = backend._stream_states.values()
     assert state.maps_early_hits >= 4, state.maps_early_hits  # (forwards whose levels fit the room given)
     torch.cuda.synchronize()
+
+
+def test_new_tensors_whose_rows_do_not_ascend_between_tensors_whose_rows_do(mods):
+    """What is queued ahead of a new tensor's verdict (its strided chain, the maps over the chain's
+    levels, the map over the rows themselves) is queued for any tensor; rows that turn out not to
+    ascend take the table builders, the queued chain serves them all the same, the map searched
+    over them is dropped.  Shuffled and sorted clouds in turn through one U-Net: the submanifold
+    map and the first strided map of every forward bit for bit the oracle's for THAT order of rows,
+    outputs those of the same forwards with nothing queued ahead of the verdict."""
+    ts, backend, spnn, F = mods
+    from torchsparse_amd.backbones import SparseResUNet42
+    from torchsparse_amd.nn.utils import fuse_inference
+    from torchsparse_amd.utils.synthetic import lidar_scan_voxels
+    rows = lidar_scan_voxels(seed=5, n_azimuth=700, n_boxes=8)
+    rng = np.random.default_rng(6)
+    perm = rng.permutation(len(rows))
+    clouds = {"s": rows, "u": rows[perm]}
+    torch.manual_seed(9)
+    model = fuse_inference(SparseResUNet42(in_channels=4).eval().cuda().half())
+    base = torch.randn(len(rows), 4, device="cuda", dtype=torch.float16)
+    feats = {"s": base, "u": base[torch.from_numpy(perm).cuda()]}
+    want_maps = {k: (oracle.kmap_subm(c, 3), oracle.kmap_downsample(c, 2, 2, 0)) for k, c in clouds.items()}
+    order = "sssuusuussus"
+
+    def sweep():
+        outs = []
+        backend.release_scratch()
+        for k in order:
+            with torch.no_grad():
+                x = ts.SparseTensor(feats[k], torch.from_numpy(clouds[k]).cuda())
+                y = model(x)[-1].feats
+            kmaps = x._caches.kmaps
+            np.testing.assert_array_equal(kmaps[_key(1, 3, 1)]["out_in_map"].cpu().numpy(), want_maps[k][0])
+            np.testing.assert_array_equal(kmaps[_key(1, 2, 2)]["out_in_map"].cpu().numpy(), want_maps[k][1][0])
+            np.testing.assert_array_equal(kmaps[_key(1, 2, 2)]["coords"].cpu().numpy(), want_maps[k][1][1])
+            outs.append(_f32(y))
+        return outs
+
+    backend.coords_check_overlap = False
+    try:
+        plain = sweep()
+    finally:
+        backend.coords_check_overlap = True
+    ahead = sweep()
+    for turn, (a, b) in enumerate(zip(ahead, plain)):
+        assert rel_rms(a, b) < 2e-3, (turn, order[turn])
+    # the same cloud in the other order of rows: the same features, row for row
+    assert rel_rms(ahead[3], ahead[0][perm]) < 2e-3
+    assert not backend._root_maps
+    torch.cuda.synchronize()
